@@ -1,0 +1,83 @@
+/**
+ *  @brief Thin C ABI over the gfx950 (MI355X) HIP kernels for packed batched dot products.
+ *  @file include/numkong_amd/hip_abi.h
+ *
+ *  Everything in this header is plain C: pointers, sizes and integer codes, no HIP or torch types.
+ *  The C host layer (numkong_amd/csrc/numkong.c, dispatch_*.c, gfx950.c) is the only intended caller;
+ *  it builds the reference-compatible `nk_dots_*` entry points declared in <numkong_amd/dots.h> on top.
+ *
+ *  All `*_async` calls enqueue work on `stream` (a `hipStream_t` passed as `void *`, NULL = default
+ *  stream), require DEVICE-accessible pointers and do not synchronise. They return 0 on success or a
+ *  non-zero HIP error code; `nk_hip_last_error()` returns a thread-local description of the last failure.
+ *
+ *  `dtype` arguments take the `nk_dtype_t` codes of <numkong_amd/dots.h> (reference:
+ *  include/numkong/types.h:923-952): nk_i8_k, nk_u8_k, nk_bf16_k, nk_f16_k, nk_e4m3_k, nk_e5m2_k.
+ */
+#ifndef NUMKONG_AMD_HIP_ABI_H
+#define NUMKONG_AMD_HIP_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#pragma GCC visibility push(default)
+
+/** Number of visible HIP devices; 0 when there is no usable GPU (never raises). */
+int nk_hip_device_count(void);
+
+/** 0 = plain host memory, 1 = device memory, 2 = host memory the device can address (pinned/managed). */
+int nk_hip_pointer_kind(void const *ptr);
+
+/** Device allocation helpers used by the host layer to stage host-resident operands. */
+int nk_hip_malloc(void **ptr, size_t bytes);
+int nk_hip_free(void *ptr);
+int nk_hip_memcpy_h2d(void *dst, void const *src, size_t bytes, void *stream);
+int nk_hip_memcpy_d2h(void *dst, void const *src, size_t bytes, void *stream);
+int nk_hip_memcpy2d_h2d(void *dst, size_t dst_pitch, void const *src, size_t src_pitch, size_t width_bytes,
+                        size_t rows, void *stream);
+int nk_hip_memcpy2d_d2h(void *dst, size_t dst_pitch, void const *src, size_t src_pitch, size_t width_bytes,
+                        size_t rows, void *stream);
+int nk_hip_stream_synchronize(void *stream);
+
+/**
+ *  Bytes of the gfx950 packed image of an (n x k) B matrix: 64-byte header, MFMA-fragment tiles,
+ *  per-column compensation terms. Replaces `nk_dots_packed_size_<T>_<isa>`
+ *  (reference: include/numkong/dots/serial.h:245-271). Returns 0 for an unsupported dtype or when
+ *  n or k do not fit 32 bits.
+ */
+size_t nk_hip_dots_packed_size(int dtype, size_t n, size_t k);
+
+/**
+ *  Pack row-major B (n rows of k elements, `b_stride` bytes apart) into `b_packed`.
+ *  Replaces `nk_dots_pack_<T>_<isa>` (reference: include/numkong/dots/serial.h:286-333).
+ */
+int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_stride, void *b_packed,
+                           void *stream);
+
+/**
+ *  C[m x n] = A[m x k] * B^T with widened accumulators (i32 / u32 / f32), C overwritten.
+ *  Replaces `nk_dots_packed_<T>_<isa>` (reference: include/numkong/dots/serial.h:520-1072).
+ *  A packed image whose header does not match (dtype, n, k) makes every C element 0xFFFFFFFF.
+ */
+int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n,
+                             size_t k, size_t a_stride, size_t c_stride, void *stream);
+
+/** Fill the m x n block of 32-bit outputs with `value` (used for the 0xFF error convention). */
+int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_t value, void *stream);
+
+/** Tile-shape override for experiments: 0 = heuristic, otherwise a configuration index. */
+void nk_hip_set_tile_config(int config);
+
+/** Thread-local text of the last failure in this layer ("" if none). */
+char const *nk_hip_last_error(void);
+
+#pragma GCC visibility pop
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif // NUMKONG_AMD_HIP_ABI_H

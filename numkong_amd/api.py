@@ -1,0 +1,176 @@
+"""ctypes binding of libnumkong_amd.so and the host-side mirror of the reference's Python API.
+
+Reference behaviour mirrored here (python/matrix.c):
+  * ``dots_pack(b, dtype)`` -> ``PackedMatrix``                     (:151-227)
+  * ``dots_packed(a, packed, out=None)`` -> ``C = A @ B.T``          (:324-490)
+  * output dtype per input dtype: i8->i32, u8->u32, floats->f32     (include/numkong/numkong.h:41-45)
+  * shape / dtype / stride validation raising ``ValueError``/``TypeError`` (:162-197, :378-421)
+
+There is no CPU fallback: if the shared library is missing, loading raises; if a call fails on the
+GPU side, ``NumKongAmdError`` is raised with the library's own message.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from dataclasses import dataclass
+from typing import Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+# nk_dtype_t codes (reference: include/numkong/types.h:923-952)
+NK_I8, NK_I32, NK_U8, NK_U32 = 1 << 2, 1 << 4, 1 << 6, 1 << 8
+NK_F32, NK_F16, NK_BF16, NK_E4M3, NK_E5M2 = 1 << 11, 1 << 12, 1 << 13, 1 << 14, 1 << 15
+
+# name -> (nk code, element bytes, output torch dtype name)
+DTYPES = {
+    "i8": (NK_I8, 1, "int32"),
+    "u8": (NK_U8, 1, "int32"),  # u32 results are returned as their int32 bit patterns
+    "bf16": (NK_BF16, 2, "float32"),
+    "f16": (NK_F16, 2, "float32"),
+    "e4m3": (NK_E4M3, 1, "float32"),
+    "e5m2": (NK_E5M2, 1, "float32"),
+}
+
+
+class NumKongAmdError(RuntimeError):
+    """A call into libnumkong_amd.so failed (no GPU, bad packed image, launch error)."""
+
+
+def library_path() -> str:
+    return os.path.join(_HERE, "lib", "libnumkong_amd.so")
+
+
+_LIB: Optional[ctypes.CDLL] = None
+
+
+def library() -> ctypes.CDLL:
+    """Load the in-tree shared library (built by ``make -C numkong_amd/csrc``). Never falls back."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = library_path()
+    if not os.path.exists(path):
+        raise NumKongAmdError(
+            f"{path} is missing: build it with `make -C numkong_amd/csrc` (there is no CPU fallback)"
+        )
+    lib = ctypes.CDLL(path)
+    sz, vp, i32 = ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int
+    for name in DTYPES:
+        getattr(lib, f"nk_dots_packed_size_{name}").restype = sz
+        getattr(lib, f"nk_dots_packed_size_{name}").argtypes = [sz, sz]
+        getattr(lib, f"nk_dots_pack_{name}").restype = None
+        getattr(lib, f"nk_dots_pack_{name}").argtypes = [vp, sz, sz, sz, vp]
+        getattr(lib, f"nk_dots_packed_{name}").restype = None
+        getattr(lib, f"nk_dots_packed_{name}").argtypes = [vp, vp, vp, sz, sz, sz, sz, sz]
+    lib.nk_amd_last_error.restype = ctypes.c_char_p
+    lib.nk_amd_dots_pack_async.restype = i32
+    lib.nk_amd_dots_pack_async.argtypes = [i32, vp, sz, sz, sz, vp, vp]
+    lib.nk_amd_dots_packed_async.restype = i32
+    lib.nk_amd_dots_packed_async.argtypes = [i32, vp, vp, vp, sz, sz, sz, sz, sz, vp]
+    lib.nk_hip_last_error.restype = ctypes.c_char_p
+    lib.nk_hip_set_tile_config.argtypes = [i32]
+    lib.nk_hip_set_tile_config.restype = None
+    lib.nk_hip_device_count.restype = i32
+    lib.nk_capabilities.restype = ctypes.c_uint64
+    lib.nk_capabilities_compiled.restype = ctypes.c_uint64
+    lib.nk_capabilities_available.restype = ctypes.c_uint64
+    lib.nk_find_kernel_punned.restype = None
+    lib.nk_find_kernel_punned.argtypes = [i32, i32, ctypes.c_uint64, ctypes.POINTER(vp), ctypes.POINTER(ctypes.c_uint64)]
+    lib.nk_dispatch_table_update.argtypes = [ctypes.c_uint64]
+    lib.nk_dispatch_table_update.restype = None
+    lib.nk_kernel_output_dtype.argtypes = [i32, i32]
+    lib.nk_kernel_output_dtype.restype = i32
+    _LIB = lib
+    return lib
+
+
+def _check(where: str) -> None:
+    message = library().nk_amd_last_error()
+    if message:
+        raise NumKongAmdError(f"{where}: {message.decode()}")
+
+
+def dots_packed_size(dtype: str, width: int, depth: int) -> int:
+    if dtype not in DTYPES:
+        raise TypeError(f"unsupported dtype {dtype!r}; expected one of {sorted(DTYPES)}")
+    return int(getattr(library(), f"nk_dots_packed_size_{dtype}")(width, depth))
+
+
+@dataclass
+class PackedMatrix:
+    """B packed for the GPU kernels; ``buffer`` is a uint8 CUDA tensor holding the relocatable image."""
+
+    dtype: str
+    width: int  # rows of B = columns of C
+    depth: int
+    buffer: "object"
+
+    @property
+    def nbytes(self) -> int:
+        return int(self.buffer.numel())
+
+
+def _as_matrix(t, dtype: str, what: str):
+    import torch
+
+    if dtype not in DTYPES:
+        raise TypeError(f"unsupported dtype {dtype!r}; expected one of {sorted(DTYPES)}")
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{what} must be a torch.Tensor")
+    if t.dim() != 2:
+        raise ValueError(f"{what} must be 2-dimensional, got {t.dim()} dimensions")
+    if not t.is_cuda:
+        raise ValueError(f"{what} must live on the GPU")
+    if t.element_size() != DTYPES[dtype][1]:
+        raise TypeError(f"{what} has {t.element_size()}-byte elements, dtype {dtype!r} needs {DTYPES[dtype][1]}")
+    if t.shape[1] > 1 and t.stride(1) != 1:
+        raise ValueError(f"{what} rows must be contiguous (stride of the last dimension must be 1)")
+    return t
+
+
+def dots_pack(b, dtype: str) -> PackedMatrix:
+    """Pack row-major ``b`` (width x depth, raw element bits in a same-width torch dtype)."""
+    import torch
+
+    b = _as_matrix(b, dtype, "b")
+    width, depth = int(b.shape[0]), int(b.shape[1])
+    size = dots_packed_size(dtype, width, depth)
+    if size == 0:
+        raise NumKongAmdError("nk_dots_packed_size returned 0 (unsupported dtype or dimensions)")
+    buffer = torch.empty(size, dtype=torch.uint8, device=b.device)
+    stride = int(b.stride(0)) * b.element_size() if width > 1 else depth * b.element_size()
+    getattr(library(), f"nk_dots_pack_{dtype}")(b.data_ptr(), width, depth, stride, buffer.data_ptr())
+    _check("nk_dots_pack_" + dtype)
+    return PackedMatrix(dtype, width, depth, buffer)
+
+
+def dots_packed(a, packed: PackedMatrix, out=None):
+    """``C[height x width] = a @ B.T`` with widened accumulators; ``out`` (optional) is overwritten."""
+    import torch
+
+    if not isinstance(packed, PackedMatrix):
+        raise TypeError("packed must be a PackedMatrix from dots_pack()")
+    a = _as_matrix(a, packed.dtype, "a")
+    height, depth = int(a.shape[0]), int(a.shape[1])
+    if depth != packed.depth:
+        raise ValueError(f"depth mismatch: a has {depth} columns, packed matrix has depth {packed.depth}")
+    out_dtype = getattr(torch, DTYPES[packed.dtype][2])
+    if out is None:
+        out = torch.empty((height, packed.width), dtype=out_dtype, device=a.device)
+    else:
+        if not isinstance(out, torch.Tensor) or not out.is_cuda or out.dim() != 2:
+            raise ValueError("out must be a 2-dimensional GPU tensor")
+        if tuple(out.shape) != (height, packed.width):
+            raise ValueError(f"out has shape {tuple(out.shape)}, expected {(height, packed.width)}")
+        if out.dtype != out_dtype:
+            raise TypeError(f"out must have dtype {out_dtype}")
+        if packed.width > 1 and out.stride(1) != 1:
+            raise ValueError("out rows must be contiguous")
+    a_stride = int(a.stride(0)) * a.element_size() if height > 1 else depth * a.element_size()
+    c_stride = int(out.stride(0)) * 4 if height > 1 else packed.width * 4
+    getattr(library(), f"nk_dots_packed_{packed.dtype}")(
+        a.data_ptr(), packed.buffer.data_ptr(), out.data_ptr(), height, packed.width, depth, a_stride, c_stride
+    )
+    _check("nk_dots_packed_" + packed.dtype)
+    return out

@@ -1,0 +1,83 @@
+/**
+ *  @brief Shared declarations of the dispatch layer: table, error stubs, per-dtype find/init.
+ *  @file numkong_amd/csrc/dispatch.h
+ *
+ *  Mirrors the role of the reference's c/dispatch.h:37-506, reduced to the packed-dots slots
+ *  (reference slots: c/dispatch.h:279-319) for i8, u8, bf16, f16, e4m3, e5m2.
+ */
+#ifndef NUMKONG_AMD_DISPATCH_H
+#define NUMKONG_AMD_DISPATCH_H
+
+#include "numkong_amd/dots.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct {
+    nk_dots_packed_size_punned_t dots_packed_size_i8, dots_packed_size_u8, dots_packed_size_bf16,
+        dots_packed_size_f16, dots_packed_size_e4m3, dots_packed_size_e5m2;
+    nk_dots_pack_punned_t dots_pack_i8, dots_pack_u8, dots_pack_bf16, dots_pack_f16, dots_pack_e4m3, dots_pack_e5m2;
+    nk_dots_packed_punned_t dots_packed_i8, dots_packed_u8, dots_packed_bf16, dots_packed_f16, dots_packed_e4m3,
+        dots_packed_e5m2;
+} nk_implementations_t;
+
+extern nk_implementations_t nk_dispatch_table;
+
+/* Error stubs (reference: c/numkong.c:78-81, 195-216). */
+void nk_error_dense_(void const *a, void const *b, nk_size_t n, void *d);
+nk_size_t nk_error_packed_size_(nk_size_t n, nk_size_t k);
+void nk_error_pack_(void const *b, nk_size_t n, nk_size_t k, nk_size_t b_stride, void *b_packed);
+void nk_error_dots_(void const *a, void const *b_packed, void *c, nk_size_t m, nk_size_t n, nk_size_t k,
+                    nk_size_t a_stride, nk_size_t c_stride);
+
+/* Per-dtype lookup and table initialisation (reference: c/dispatch.h:483-506). */
+#define NK_AMD_DECLARE_DISPATCH_(T)                                                                              \
+    void nk_dispatch_##T##_find_(nk_capability_t viable, nk_kernel_kind_t kind, nk_kernel_punned_t *kernel,      \
+                                 nk_capability_t *used);                                                         \
+    void nk_dispatch_##T##_init_(nk_capability_t caps);
+NK_AMD_DECLARE_DISPATCH_(i8)
+NK_AMD_DECLARE_DISPATCH_(u8)
+NK_AMD_DECLARE_DISPATCH_(bf16)
+NK_AMD_DECLARE_DISPATCH_(f16)
+NK_AMD_DECLARE_DISPATCH_(e4m3)
+NK_AMD_DECLARE_DISPATCH_(e5m2)
+#undef NK_AMD_DECLARE_DISPATCH_
+
+/**
+ *  Body shared by the six dispatch_<T>.c files. The reference walks a ladder of CPU ISAs per dtype
+ *  (c/dispatch_i8.c:9-323); here there is one backend, so the ladder has one rung, and a kind this
+ *  library does not implement falls through to the reference's error fallback (c/dispatch_i8.c:321-322).
+ */
+#define NK_AMD_DEFINE_DISPATCH_(T)                                                                                    \
+    void nk_dispatch_##T##_find_(nk_capability_t v, nk_kernel_kind_t k, nk_kernel_punned_t *m, nk_capability_t *c) { \
+        typedef nk_kernel_punned_t m_t;                                                                               \
+        if (v & nk_cap_gfx950_k) switch (k) {                                                                         \
+            case nk_kernel_dots_packed_size_k:                                                                        \
+                *m = (m_t)&nk_dots_packed_size_##T##_gfx950, *c = nk_cap_gfx950_k;                                    \
+                return;                                                                                               \
+            case nk_kernel_dots_pack_k: *m = (m_t)&nk_dots_pack_##T##_gfx950, *c = nk_cap_gfx950_k; return;          \
+            case nk_kernel_dots_packed_k: *m = (m_t)&nk_dots_packed_##T##_gfx950, *c = nk_cap_gfx950_k; return;      \
+            default: break;                                                                                           \
+            }                                                                                                         \
+        switch (k) {                                                                                                  \
+        case nk_kernel_dots_packed_size_k: *m = (m_t)nk_error_packed_size_, *c = 0; return;                          \
+        case nk_kernel_dots_pack_k: *m = (m_t)nk_error_pack_, *c = 0; return;                                        \
+        case nk_kernel_dots_packed_k: *m = (m_t)nk_error_dots_, *c = 0; return;                                      \
+        default: *m = (m_t)nk_error_dense_, *c = 0; return;                                                          \
+        }                                                                                                             \
+    }                                                                                                                 \
+    void nk_dispatch_##T##_init_(nk_capability_t caps) {                                                              \
+        nk_implementations_t *t = &nk_dispatch_table;                                                                 \
+        nk_capability_t used;                                                                                         \
+        nk_dispatch_##T##_find_(caps, nk_kernel_dots_packed_size_k, (nk_kernel_punned_t *)&t->dots_packed_size_##T,  \
+                                &used);                                                                               \
+        nk_dispatch_##T##_find_(caps, nk_kernel_dots_pack_k, (nk_kernel_punned_t *)&t->dots_pack_##T, &used);         \
+        nk_dispatch_##T##_find_(caps, nk_kernel_dots_packed_k, (nk_kernel_punned_t *)&t->dots_packed_##T, &used);     \
+    }
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif // NUMKONG_AMD_DISPATCH_H

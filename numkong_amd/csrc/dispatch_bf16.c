@@ -1,0 +1,10 @@
+/**
+ *  @brief Dispatch for BF16 packed dots: binds the table slots and `nk_find_kernel_punned` to gfx950.
+ *  @file numkong_amd/csrc/dispatch_bf16.c
+ *
+ *  Counterpart of the reference's c/dispatch_bf16.c (`nk_dispatch_bf16_find_`, `nk_dispatch_bf16_init_`),
+ *  for the kinds nk_kernel_dots_packed_size_k, nk_kernel_dots_pack_k, nk_kernel_dots_packed_k only.
+ */
+#include "dispatch.h"
+
+NK_AMD_DEFINE_DISPATCH_(bf16)

@@ -1,0 +1,749 @@
+/**
+ *  @brief gfx950 (MI355X, CDNA4) kernels for packed batched dot products: C = A * B^T.
+ *  @file numkong_amd/csrc/dots_gfx950.hip
+ *
+ *  The only translation unit that sees HIP. It exports the plain-C functions of
+ *  <numkong_amd/hip_abi.h>; the reference-compatible API is built on top of them in C.
+ *
+ *  Replaces the per-ISA kernels the reference instantiates from
+ *  include/numkong/dots/serial.h:245-333 (pack size, pack) and :520-1072 (packed product) for
+ *  i8, u8, bf16, f16, e4m3, e5m2.
+ *
+ *  Packed image of B (n rows of k elements), all little-endian:
+ *
+ *      [ 64-byte header ][ tiles ][ per-column compensation terms, u32 x 32 x n_tiles ]
+ *
+ *  A "chunk" is 16 consecutive bytes of one B row (16 i8/fp8 values, 8 bf16/f16 values). Rows are grouped
+ *  into tiles of 32; K is padded with zeros to a multiple of 8 chunks (128 bytes) and N with zero rows to
+ *  a multiple of 32. Chunk `c` of row `r` of tile `t` lives at
+ *
+ *      data + ((t * k_chunks + c) * 32 + r) * 16
+ *
+ *  so the 64 lanes of a wavefront that execute one 32x32 MFMA step `q` (lane l supplies row l % 32 and
+ *  chunk 2q + l / 32) read 1024 contiguous bytes at `data + (t * k_chunks + 2q) * 512 + l * 16`: the image
+ *  is the MFMA operand-fragment order, and B goes from HBM to registers with one coalesced 128-bit load
+ *  per lane per step, never through LDS. The same image serves the 16-byte-per-lane MFMAs
+ *  (32x32x32 i8, 32x32x16 bf16/f16), the 8-byte legacy fp8 forms (two MFMAs per chunk) and the
+ *  32-byte f8f6f4 forms (two chunks per MFMA), because a product only needs A and B to agree on which
+ *  k sits in which operand slot.
+ *
+ *  u8 has no unsigned MFMA. B is stored as b' = b ^ 0x80 (signed b - 128), A is turned into
+ *  a' = a ^ 0x80 on its way into LDS, and  sum(a*b) = sum(a'*b') + 128*sum(a) + 128*sum(b')  (mod 2^32)
+ *  with zero padding contributing nothing. 128*sum(b') per column is stored behind the tiles at pack
+ *  time; sum(a) per row is accumulated with v_sad_u8 while A is staged.
+ */
+#include <hip/hip_runtime.h>
+
+#include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "numkong_amd/hip_abi.h"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef long v2l __attribute__((ext_vector_type(2)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+// nk_dtype_t codes (reference: include/numkong/types.h:923-952)
+enum : int {
+    kI8 = 1 << 2,
+    kU8 = 1 << 6,
+    kF16 = 1 << 12,
+    kBF16 = 1 << 13,
+    kE4M3 = 1 << 14,
+    kE5M2 = 1 << 15,
+};
+
+constexpr uint32_t kMagic = 0x35394B4Eu; // "NK95"
+constexpr uint32_t kVersion = 1;
+constexpr int kChunkBytes = 16;   // bytes of K per lane per operand load
+constexpr int kTileRows = 32;     // B rows per tile = MFMA N
+constexpr int kStageChunks = 8;   // chunks of K per pipeline stage (128 bytes per row)
+constexpr int kStageBytes = kStageChunks * kChunkBytes;
+constexpr int kTileChunkBytes = kTileRows * kChunkBytes; // 512: one chunk of all 32 rows of a tile
+
+struct PackedHeader {
+    uint32_t magic;
+    uint32_t version;
+    uint32_t dtype;
+    uint32_t elem_bytes;
+    uint32_t n;        // logical rows of B = columns of C
+    uint32_t k;        // logical depth in elements
+    uint32_t n_tiles;  // ceil(n / 32)
+    uint32_t k_chunks; // padded depth in 16-byte chunks, multiple of 8
+    uint64_t data_offset;
+    uint64_t sums_offset; // u32 x (32 * n_tiles): 128 * sum(b') per column for u8, zeros otherwise
+    uint64_t total_bytes;
+    uint64_t reserved[1];
+};
+static_assert(sizeof(PackedHeader) == 64, "header must stay 64 bytes");
+
+struct Geometry {
+    uint32_t elem_bytes, n, k, n_tiles, k_chunks;
+    uint64_t k_bytes, data_bytes, sums_bytes, total_bytes;
+};
+
+inline int elem_bytes_of(int dtype) {
+    switch (dtype) {
+    case kI8:
+    case kU8:
+    case kE4M3:
+    case kE5M2: return 1;
+    case kF16:
+    case kBF16: return 2;
+    default: return 0;
+    }
+}
+
+inline bool make_geometry(int dtype, size_t n, size_t k, Geometry &g) {
+    int const eb = elem_bytes_of(dtype);
+    if (!eb) return false;
+    if (n > 0x7FFFFFFFull || k > 0x3FFFFFFFull) return false;
+    g.elem_bytes = (uint32_t)eb, g.n = (uint32_t)n, g.k = (uint32_t)k;
+    g.k_bytes = (uint64_t)k * eb;
+    uint64_t const chunks = (g.k_bytes + kChunkBytes - 1) / kChunkBytes;
+    g.k_chunks = (uint32_t)((chunks + kStageChunks - 1) / kStageChunks * kStageChunks);
+    g.n_tiles = (uint32_t)((n + kTileRows - 1) / kTileRows);
+    g.data_bytes = (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes;
+    g.sums_bytes = (uint64_t)g.n_tiles * kTileRows * sizeof(uint32_t);
+    g.total_bytes = sizeof(PackedHeader) + g.data_bytes + g.sums_bytes;
+    return true;
+}
+
+thread_local char g_last_error[256] = "";
+
+int fail(hipError_t e, char const *what) {
+    snprintf(g_last_error, sizeof(g_last_error), "%s: %s", what, hipGetErrorString(e));
+    (void)hipGetLastError();
+    return (int)e ? (int)e : -1;
+}
+int fail_msg(char const *what) {
+    snprintf(g_last_error, sizeof(g_last_error), "%s", what);
+    return -1;
+}
+
+/**
+ *  Load one 16-byte chunk of which only the first `valid` bytes exist (valid may be <= 0 or >= 16),
+ *  with loads no wider than the pointer's known alignment `avec`. Missing bytes read as zero; `xr`
+ *  (0 or 0x80808080) is applied to existing bytes only, so zero padding stays zero for u8.
+ */
+__device__ __forceinline__ v4i load_chunk_guarded(uint8_t const *p, int valid, int avec, uint32_t xr) {
+    v4i out;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        int const rem = valid - 4 * w;
+        uint32_t x = 0;
+        if (rem >= 4 && avec >= 4) { x = *(uint32_t const *)(p + 4 * w) ^ xr; }
+        else if (rem > 0) {
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                if (b < rem) x |= (uint32_t)(uint8_t)(p[4 * w + b] ^ (uint8_t)xr) << (8 * b);
+        }
+        out[w] = (int)x;
+    }
+    return out;
+}
+
+__device__ __forceinline__ uint32_t sum_bytes_u8(v4i v) {
+    uint32_t s = __builtin_amdgcn_sad_u8((uint32_t)v[0], 0u, 0u);
+    s = __builtin_amdgcn_sad_u8((uint32_t)v[1], 0u, s);
+    s = __builtin_amdgcn_sad_u8((uint32_t)v[2], 0u, s);
+    s = __builtin_amdgcn_sad_u8((uint32_t)v[3], 0u, s);
+    return s;
+}
+
+#pragma region Packing
+
+/**
+ *  One thread per 16-byte chunk of the image. A block of 256 threads covers 32 rows x 8 chunks: reads are
+ *  128 contiguous bytes per row, writes are eight 512-byte runs.
+ */
+__global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
+                                                   uint64_t k_bytes, uint32_t k_chunks, uint8_t *__restrict__ data,
+                                                   int avec, uint32_t xr) {
+    uint32_t const groups = k_chunks / kStageChunks;
+    uint32_t const tile = blockIdx.x / groups;
+    uint32_t const group = blockIdx.x % groups;
+    uint32_t const r = threadIdx.x >> 3;
+    uint32_t const c = group * kStageChunks + (threadIdx.x & 7);
+    uint64_t const row = (uint64_t)tile * kTileRows + r;
+    int64_t const left = (int64_t)k_bytes - (int64_t)c * kChunkBytes;
+    int const valid = row < n ? (int)(left > 16 ? 16 : (left < 0 ? 0 : left)) : 0;
+    v4i v = {0, 0, 0, 0};
+    if (valid > 0) {
+        uint8_t const *src = b + row * b_stride + (uint64_t)c * kChunkBytes;
+        if (valid == 16 && avec >= 16) {
+            v = *(v4i const *)src;
+            v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
+        }
+        else { v = load_chunk_guarded(src, valid, avec, xr); }
+    }
+    *(v4i *)(data + (((uint64_t)tile * k_chunks + c) * kTileRows + r) * kChunkBytes) = v;
+}
+
+/**
+ *  Per-column compensation term for u8: 128 * sum of the signed packed bytes of the row (mod 2^32).
+ *  One wavefront per tile: lane l owns row l % 32 and every second chunk starting at l / 32.
+ */
+__global__ __launch_bounds__(64) void column_terms_kernel(uint8_t const *__restrict__ data, uint32_t k_chunks,
+                                                          uint32_t *__restrict__ sums) {
+    uint32_t const tile = blockIdx.x;
+    uint32_t const lane = threadIdx.x;
+    uint8_t const *base = data + (uint64_t)tile * k_chunks * kTileChunkBytes + lane * kChunkBytes;
+    int acc = 0;
+    for (uint32_t c = 0; c < k_chunks; c += 2) {
+        v4i const v = *(v4i const *)(base + (uint64_t)c * kTileChunkBytes);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) acc = __builtin_amdgcn_sdot4(v[w], 0x01010101, acc, false);
+    }
+    acc += __shfl_xor(acc, 32, 64);
+    if (lane < 32) sums[(uint64_t)tile * kTileRows + lane] = (uint32_t)acc * 128u;
+}
+
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t *p, uint64_t count, uint32_t value) {
+    uint64_t const i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) p[i] = value;
+}
+
+__global__ __launch_bounds__(64) void write_header_kernel(PackedHeader *dst, PackedHeader h) {
+    if (threadIdx.x == 0) *dst = h;
+}
+
+__global__ __launch_bounds__(256) void fill_rows_kernel(uint8_t *c, uint32_t m, uint32_t n, uint64_t c_stride,
+                                                        uint32_t value) {
+    uint64_t const i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    uint64_t const row = i / n, col = i % n;
+    if (row < m) *(uint32_t *)(c + row * c_stride + col * 4) = value;
+}
+
+#pragma endregion Packing
+
+#pragma region Element types
+
+struct I8 {
+    typedef v16i acc_t;
+    static constexpr int kDtype = kI8;
+    static constexpr bool kUnsigned = false;
+    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
+    }
+};
+struct U8 : I8 {
+    static constexpr int kDtype = kU8;
+    static constexpr bool kUnsigned = true;
+};
+struct BF16 {
+    typedef v16f acc_t;
+    static constexpr int kDtype = kBF16;
+    static constexpr bool kUnsigned = false;
+    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), acc, 0,
+                                                      0, 0);
+    }
+};
+struct F16 {
+    typedef v16f acc_t;
+    static constexpr int kDtype = kF16;
+    static constexpr bool kUnsigned = false;
+    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), acc, 0, 0,
+                                                     0);
+    }
+};
+struct E4M3 {
+    typedef v16f acc_t;
+    static constexpr int kDtype = kE4M3;
+    static constexpr bool kUnsigned = false;
+    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
+        v2l const al = __builtin_bit_cast(v2l, a), bl = __builtin_bit_cast(v2l, b);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[0], bl[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[1], bl[1], acc, 0, 0, 0);
+    }
+};
+struct E5M2 {
+    typedef v16f acc_t;
+    static constexpr int kDtype = kE5M2;
+    static constexpr bool kUnsigned = false;
+    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
+        v2l const al = __builtin_bit_cast(v2l, a), bl = __builtin_bit_cast(v2l, b);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(al[0], bl[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(al[1], bl[1], acc, 0, 0, 0);
+    }
+};
+
+#pragma endregion Element types
+
+#pragma region Packed product
+
+template <int V>
+struct slot_c {
+    static constexpr int value = V;
+};
+template <int V>
+__device__ __forceinline__ constexpr slot_c<(V ^ 1)> slot_next() {
+    return {};
+}
+
+struct GemmArgs {
+    uint8_t const *a;
+    uint8_t const *bp; // packed image (header first)
+    uint8_t *c;
+    uint64_t a_stride, c_stride, k_bytes;
+    uint32_t m, n, k;
+    uint32_t n_tiles, k_chunks;
+    uint32_t tiles_m, tiles_n;
+    int avec; // widest load the A pointer and stride allow (1, 2, 4, 8 or 16 bytes)
+};
+
+/**
+ *  Workgroup index -> output tile. Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each
+ *  with a private L2, so ids are first regrouped into 8 contiguous ranges (one per XCD) and each range
+ *  walks the tile grid in column-major bands of 8 tile rows: tiles resident on one XCD at the same time
+ *  share A row blocks and B column tiles in that XCD's L2.
+ */
+__device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm,
+                                              uint32_t &tn) {
+    uint32_t const total = tiles_m * tiles_n;
+    uint32_t const per_xcd = total / 8;
+    uint32_t lid = pid;
+    if (pid < per_xcd * 8) lid = (pid % 8) * per_xcd + pid / 8;
+    constexpr uint32_t kBand = 8;
+    uint32_t const width = kBand * tiles_n;
+    uint32_t const band = lid / width;
+    uint32_t const first = band * kBand;
+    uint32_t const rows = tiles_m - first < kBand ? tiles_m - first : kBand;
+    uint32_t const in_band = lid % width;
+    tm = first + in_band % rows;
+    tn = in_band / rows;
+}
+
+/**
+ *  One workgroup of NW wavefronts computes a (32*TM) x (32*TN*NW) tile of C. Every wavefront owns all
+ *  32*TM rows and its own 32*TN columns, so B fragments are loaded by exactly one wavefront straight
+ *  from the packed image into registers, while the shared A block is staged through LDS
+ *  (double-buffered, 128 bytes of K per row per stage, row pitch 144 bytes so that 16 consecutive rows
+ *  start in 16 different 16-byte bank groups).
+ */
+template <class T, int TM, int TN, int NW, bool ALIGNED>
+__global__ __launch_bounds__(NW * 64) void dots_packed_kernel(GemmArgs g) {
+    typedef typename T::acc_t acc_t;
+    constexpr int BM = TM * 32;
+    constexpr int NT = NW * 64;
+    constexpr int kPitch = kStageBytes + 16;
+    constexpr int kStageLds = BM * kPitch;
+    constexpr int kLoads = BM * kStageChunks / NT; // chunks staged per thread per stage
+    static_assert(BM * kStageChunks % NT == 0, "stage must divide evenly among threads");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    uint32_t const tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t tile_m, tile_n;
+    tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    uint32_t const row0 = tile_m * BM;
+    uint32_t const col0 = tile_n * (32 * TN * NW) + wave * (32 * TN);
+
+    // Trust, but verify: the image must have been packed for this dtype and these dimensions.
+    PackedHeader const *header = (PackedHeader const *)g.bp;
+    bool const image_ok = header->magic == kMagic && header->version == kVersion &&
+                          header->dtype == (uint32_t)T::kDtype && header->n == g.n && header->k == g.k &&
+                          header->k_chunks == g.k_chunks && header->n_tiles == g.n_tiles;
+    uint8_t const *data = g.bp + sizeof(PackedHeader);
+    uint32_t const *col_terms = (uint32_t const *)(data + (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes);
+
+    acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+    uint32_t row_sum[kLoads]; // u8 only: sum of the unsigned bytes this thread staged, per staged row
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) row_sum[i] = 0;
+
+    if (image_ok) {
+        // Per-thread A source rows (clamped to the last row: edge tiles recompute it and mask the store).
+        uint8_t const *a_src[kLoads];
+        uint32_t lds_dst[kLoads];
+        uint32_t const chunk_in_stage = tid & 7;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            uint32_t const r = (i * NT + tid) >> 3;
+            uint32_t const row = row0 + r < g.m ? row0 + r : g.m - 1;
+            a_src[i] = g.a + (uint64_t)row * g.a_stride + chunk_in_stage * kChunkBytes;
+            lds_dst[i] = r * kPitch + chunk_in_stage * kChunkBytes;
+        }
+        // Per-wavefront B fragment streams (tile index clamped the same way).
+        uint8_t const *b_src[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
+            b_src[j] = data + (uint64_t)t * g.k_chunks * kTileChunkBytes + lane * kChunkBytes;
+        }
+        uint32_t const a_frag = (lane & 31) * kPitch + (lane >> 5) * kChunkBytes;
+        uint32_t const stages = g.k_chunks / kStageChunks;
+        uint32_t const xr = T::kUnsigned ? 0x80808080u : 0u;
+
+        v4i a_reg[kLoads];
+        v4i b_reg[2][TN][4];
+
+        auto load_a = [&](uint32_t s) {
+            uint64_t const offset = (uint64_t)s * kStageBytes;
+            bool const full = offset + kStageBytes <= g.k_bytes;
+            if (ALIGNED && full) {
+#pragma unroll
+                for (int i = 0; i < kLoads; ++i) {
+                    v4i v = *(v4i const *)(a_src[i] + offset);
+                    if (T::kUnsigned) {
+                        row_sum[i] += sum_bytes_u8(v);
+                        v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
+                    }
+                    a_reg[i] = v;
+                }
+            }
+            else {
+                int64_t const left = (int64_t)g.k_bytes - (int64_t)offset - (int64_t)chunk_in_stage * kChunkBytes;
+                int const valid = (int)(left > 16 ? 16 : (left < 0 ? 0 : left));
+#pragma unroll
+                for (int i = 0; i < kLoads; ++i) {
+                    v4i v = load_chunk_guarded(a_src[i] + offset, valid, g.avec, 0u);
+                    if (T::kUnsigned) {
+                        row_sum[i] += sum_bytes_u8(v);
+                        // Flip only bytes that exist so that the zero padding stays zero.
+#pragma unroll
+                        for (int w = 0; w < 4; ++w) {
+                            int const rem = valid - 4 * w;
+                            uint32_t const mask = rem >= 4 ? 0x80808080u : (rem <= 0 ? 0u : (0x80808080u >> (8 * (4 - rem))));
+                            v[w] ^= (int)mask;
+                        }
+                    }
+                    a_reg[i] = v;
+                }
+            }
+        };
+        auto store_a = [&](uint32_t buffer) {
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i) *(v4i *)(lds + buffer * kStageLds + lds_dst[i]) = a_reg[i];
+        };
+        auto load_b = [&](uint32_t s, auto slot_tag) {
+            constexpr int slot = decltype(slot_tag)::value;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    b_reg[slot][j][q] =
+                        *(v4i const *)(b_src[j] + (uint64_t)s * (kStageChunks * kTileChunkBytes) + q * 2 * kTileChunkBytes);
+        };
+
+        // One pipeline stage with compile-time buffer/register-slot indices (runtime indexing of
+        // register arrays would spill them to scratch).
+        auto stage = [&](auto slot_tag, uint32_t s) {
+            constexpr int slot = decltype(slot_tag)::value;
+            bool const more = s + 1 < stages;
+            if (more) {
+                load_a(s + 1);
+                load_b(s + 1, slot_next<slot>());
+            }
+            uint8_t const *a_lds = lds + slot * kStageLds + a_frag;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                v4i af[TM];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) af[i] = *(v4i const *)(a_lds + i * 32 * kPitch + q * 2 * kChunkBytes);
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[i], b_reg[slot][j][q]);
+            }
+            if (more) store_a(slot ^ 1);
+            __syncthreads();
+        };
+
+        load_a(0);
+        load_b(0, slot_c<0>());
+        store_a(0);
+        __syncthreads();
+        for (uint32_t s = 0; s < stages; s += 2) {
+            stage(slot_c<0>(), s);
+            if (s + 1 < stages) stage(slot_c<1>(), s + 1);
+        }
+    }
+
+    // Epilogue. Accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.
+    uint32_t const half = lane >> 5, col_in_tile = lane & 31;
+    uint32_t *row_terms = (uint32_t *)lds;
+    if (T::kUnsigned && image_ok) {
+        // The 8 threads that staged one row hold its partial byte sums in adjacent lanes.
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            uint32_t s = row_sum[i];
+            s += __shfl_xor(s, 1, 64);
+            s += __shfl_xor(s, 2, 64);
+            s += __shfl_xor(s, 4, 64);
+            if ((tid & 7) == 0) row_terms[(i * NT + tid) >> 3] = s * 128u;
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        uint32_t const col = col0 + j * 32 + col_in_tile;
+        uint32_t col_term = 0;
+        if (T::kUnsigned && image_ok) {
+            uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
+            col_term = col_terms[(uint64_t)t * kTileRows + col_in_tile];
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                uint32_t const r = i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+                uint32_t const row = row0 + r;
+                auto const element = acc[i][j][v]; // a named copy: bit-casting the vector element expression reads lane 0
+                uint32_t bits = __builtin_bit_cast(uint32_t, element);
+                if (T::kUnsigned) bits += row_terms[r] + col_term;
+                if (!image_ok) bits = 0xFFFFFFFFu;
+                if (row < g.m && col < g.n) *(uint32_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 4) = bits;
+            }
+        }
+    }
+}
+
+struct TileConfig {
+    int tm, tn, nw;
+};
+// Index 0 is "choose for me"; 1.. are explicit.
+constexpr TileConfig kConfigs[] = {{0, 0, 0}, {8, 2, 4}, {4, 2, 4}, {4, 1, 4}, {2, 1, 4}};
+constexpr int kConfigCount = sizeof(kConfigs) / sizeof(kConfigs[0]);
+int g_forced_config = 0;
+
+template <class T, int TM, int TN, int NW>
+hipError_t launch_one(GemmArgs &g, hipStream_t stream) {
+    constexpr int BM = TM * 32, BN = TN * NW * 32;
+    constexpr size_t lds_bytes = (size_t)2 * BM * (kStageBytes + 16);
+    g.tiles_m = (g.m + BM - 1) / BM;
+    g.tiles_n = (g.n + BN - 1) / BN;
+    uint64_t const blocks = (uint64_t)g.tiles_m * g.tiles_n;
+    if (blocks > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    bool const aligned = g.avec >= 16;
+    auto kernel = aligned ? dots_packed_kernel<T, TM, TN, NW, true> : dots_packed_kernel<T, TM, TN, NW, false>;
+    if (lds_bytes > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((void const *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)lds_bytes);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(NW * 64), lds_bytes, stream, g);
+    return hipGetLastError();
+}
+
+template <class T>
+hipError_t launch_typed(GemmArgs &g, hipStream_t stream) {
+    int config = g_forced_config;
+    if (config <= 0 || config >= kConfigCount) {
+        // Largest tile that still gives every one of the 256 CUs at least one workgroup.
+        auto tiles = [&](int c) {
+            uint64_t const bm = kConfigs[c].tm * 32, bn = (uint64_t)kConfigs[c].tn * kConfigs[c].nw * 32;
+            return ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
+        };
+        config = kConfigCount - 1;
+        for (int c = 1; c < kConfigCount; ++c)
+            if (tiles(c) >= 256) {
+                config = c;
+                break;
+            }
+    }
+    switch (config) {
+    case 1: return launch_one<T, 8, 2, 4>(g, stream);
+    case 2: return launch_one<T, 4, 2, 4>(g, stream);
+    case 3: return launch_one<T, 4, 1, 4>(g, stream);
+    default: return launch_one<T, 2, 1, 4>(g, stream);
+    }
+}
+
+inline int widest_load(void const *p, size_t stride) {
+    uintptr_t const bits = (uintptr_t)p | (uintptr_t)stride;
+    if (!(bits & 15)) return 16;
+    if (!(bits & 7)) return 8;
+    if (!(bits & 3)) return 4;
+    if (!(bits & 1)) return 2;
+    return 1;
+}
+
+#pragma endregion Packed product
+
+} // namespace
+
+extern "C" {
+
+int nk_hip_device_count(void) {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return count;
+}
+
+int nk_hip_pointer_kind(void const *ptr) {
+    if (!ptr) return 0;
+    hipPointerAttribute_t attributes;
+    memset(&attributes, 0, sizeof(attributes));
+    if (hipPointerGetAttributes(&attributes, ptr) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    switch (attributes.type) {
+    case hipMemoryTypeDevice: return 1;
+    case hipMemoryTypeHost:
+    case hipMemoryTypeManaged: return 2;
+    default: return 0;
+    }
+}
+
+int nk_hip_malloc(void **ptr, size_t bytes) {
+    hipError_t e = hipMalloc(ptr, bytes ? bytes : 1);
+    return e == hipSuccess ? 0 : fail(e, "hipMalloc");
+}
+int nk_hip_free(void *ptr) {
+    hipError_t e = hipFree(ptr);
+    return e == hipSuccess ? 0 : fail(e, "hipFree");
+}
+int nk_hip_memcpy_h2d(void *dst, void const *src, size_t bytes, void *stream) {
+    if (!bytes) return 0;
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream);
+    return e == hipSuccess ? 0 : fail(e, "hipMemcpyAsync(H2D)");
+}
+int nk_hip_memcpy_d2h(void *dst, void const *src, size_t bytes, void *stream) {
+    if (!bytes) return 0;
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream);
+    return e == hipSuccess ? 0 : fail(e, "hipMemcpyAsync(D2H)");
+}
+int nk_hip_memcpy2d_h2d(void *dst, size_t dst_pitch, void const *src, size_t src_pitch, size_t width_bytes,
+                        size_t rows, void *stream) {
+    if (!width_bytes || !rows) return 0;
+    hipError_t e = hipMemcpy2DAsync(dst, dst_pitch, src, src_pitch, width_bytes, rows, hipMemcpyHostToDevice,
+                                    (hipStream_t)stream);
+    return e == hipSuccess ? 0 : fail(e, "hipMemcpy2DAsync(H2D)");
+}
+int nk_hip_memcpy2d_d2h(void *dst, size_t dst_pitch, void const *src, size_t src_pitch, size_t width_bytes,
+                        size_t rows, void *stream) {
+    if (!width_bytes || !rows) return 0;
+    hipError_t e = hipMemcpy2DAsync(dst, dst_pitch, src, src_pitch, width_bytes, rows, hipMemcpyDeviceToHost,
+                                    (hipStream_t)stream);
+    return e == hipSuccess ? 0 : fail(e, "hipMemcpy2DAsync(D2H)");
+}
+int nk_hip_stream_synchronize(void *stream) {
+    hipError_t e = hipStreamSynchronize((hipStream_t)stream);
+    return e == hipSuccess ? 0 : fail(e, "hipStreamSynchronize");
+}
+
+size_t nk_hip_dots_packed_size(int dtype, size_t n, size_t k) {
+    Geometry g;
+    if (!make_geometry(dtype, n, k, g)) return 0;
+    return (size_t)g.total_bytes;
+}
+
+int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_stride, void *b_packed,
+                           void *stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    Geometry g;
+    if (!make_geometry(dtype, n, k, g)) return fail_msg("nk_hip_dots_pack: unsupported dtype or dimensions");
+    if (!b_packed || ((uintptr_t)b_packed & 15)) return fail_msg("nk_hip_dots_pack: b_packed must be 16-byte aligned");
+    if (n && k && !b) return fail_msg("nk_hip_dots_pack: b is NULL");
+    if (g.elem_bytes == 2 && (((uintptr_t)b | b_stride) & 1)) return fail_msg("nk_hip_dots_pack: 16-bit B is misaligned");
+
+    PackedHeader h;
+    memset(&h, 0, sizeof(h));
+    h.magic = kMagic, h.version = kVersion, h.dtype = (uint32_t)dtype, h.elem_bytes = g.elem_bytes;
+    h.n = g.n, h.k = g.k, h.n_tiles = g.n_tiles, h.k_chunks = g.k_chunks;
+    h.data_offset = sizeof(PackedHeader);
+    h.sums_offset = sizeof(PackedHeader) + g.data_bytes;
+    h.total_bytes = g.total_bytes;
+
+    uint8_t *image = (uint8_t *)b_packed;
+    uint8_t *data = image + sizeof(PackedHeader);
+    uint32_t *sums = (uint32_t *)(data + g.data_bytes);
+    hipLaunchKernelGGL(write_header_kernel, dim3(1), dim3(64), 0, stream, (PackedHeader *)image, h);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(e, "write_header_kernel");
+    if (g.n_tiles && g.k_chunks) {
+        uint64_t const blocks = (uint64_t)g.n_tiles * (g.k_chunks / kStageChunks);
+        if (blocks > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_pack: matrix too large");
+        uint32_t const xr = dtype == kU8 ? 0x80808080u : 0u;
+        hipLaunchKernelGGL(pack_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t const *)b,
+                           (uint64_t)b_stride, g.n, g.k_bytes, g.k_chunks, data, widest_load(b, b_stride), xr);
+        e = hipGetLastError();
+        if (e != hipSuccess) return fail(e, "pack_kernel");
+    }
+    if (g.n_tiles) {
+        if (dtype == kU8 && g.k_chunks) {
+            hipLaunchKernelGGL(column_terms_kernel, dim3(g.n_tiles), dim3(64), 0, stream, (uint8_t const *)data,
+                               g.k_chunks, sums);
+        }
+        else {
+            uint64_t const count = (uint64_t)g.n_tiles * kTileRows;
+            hipLaunchKernelGGL(fill_u32_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, stream, sums, count,
+                               0u);
+        }
+        e = hipGetLastError();
+        if (e != hipSuccess) return fail(e, "column_terms_kernel");
+    }
+    return 0;
+}
+
+int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_t value, void *stream) {
+    if (!m || !n) return 0;
+    if (m > 0x7FFFFFFFull || n > 0x7FFFFFFFull) return fail_msg("nk_hip_fill_rows: dimensions too large");
+    uint64_t const count = (uint64_t)m * n;
+    uint64_t const blocks = (count + 255) / 256;
+    if (blocks > 0x7FFFFFFFull) return fail_msg("nk_hip_fill_rows: matrix too large");
+    hipLaunchKernelGGL(fill_rows_kernel, dim3((uint32_t)blocks), dim3(256), 0, (hipStream_t)stream, (uint8_t *)c,
+                       (uint32_t)m, (uint32_t)n, (uint64_t)c_stride, value);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : fail(e, "fill_rows_kernel");
+}
+
+int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n, size_t k,
+                             size_t a_stride, size_t c_stride, void *stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (!m || !n) return 0;
+    Geometry geo;
+    if (!make_geometry(dtype, n, k, geo)) return fail_msg("nk_hip_dots_packed: unsupported dtype or dimensions");
+    if (m > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_packed: too many rows");
+    if (!c || ((uintptr_t)c & 3) || (c_stride & 3)) return fail_msg("nk_hip_dots_packed: c must be 4-byte aligned");
+    if (!b_packed || ((uintptr_t)b_packed & 15)) return fail_msg("nk_hip_dots_packed: b_packed must be 16-byte aligned");
+    if (k == 0) return nk_hip_fill_rows_async(c, m, n, c_stride, 0u, stream_);
+    if (!a) return fail_msg("nk_hip_dots_packed: a is NULL");
+    if (geo.elem_bytes == 2 && (((uintptr_t)a | a_stride) & 1)) return fail_msg("nk_hip_dots_packed: 16-bit A is misaligned");
+
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.a = (uint8_t const *)a, g.bp = (uint8_t const *)b_packed, g.c = (uint8_t *)c;
+    g.a_stride = a_stride, g.c_stride = c_stride, g.k_bytes = geo.k_bytes;
+    g.m = (uint32_t)m, g.n = geo.n, g.k = geo.k, g.n_tiles = geo.n_tiles, g.k_chunks = geo.k_chunks;
+    g.avec = widest_load(a, a_stride);
+
+    hipError_t e;
+    switch (dtype) {
+    case kI8: e = launch_typed<I8>(g, stream); break;
+    case kU8: e = launch_typed<U8>(g, stream); break;
+    case kBF16: e = launch_typed<BF16>(g, stream); break;
+    case kF16: e = launch_typed<F16>(g, stream); break;
+    case kE4M3: e = launch_typed<E4M3>(g, stream); break;
+    case kE5M2: e = launch_typed<E5M2>(g, stream); break;
+    default: return fail_msg("nk_hip_dots_packed: unsupported dtype");
+    }
+    return e == hipSuccess ? 0 : fail(e, "dots_packed_kernel");
+}
+
+void nk_hip_set_tile_config(int config) { g_forced_config = config; }
+
+char const *nk_hip_last_error(void) { return g_last_error; }
+
+} // extern "C"

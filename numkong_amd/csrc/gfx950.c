@@ -1,0 +1,184 @@
+/**
+ *  @brief Host side of the gfx950 backend: operand placement, staging, the reference's error convention.
+ *  @file numkong_amd/csrc/gfx950.c
+ *
+ *  Defines `nk_dots_packed_size_<T>_gfx950`, `nk_dots_pack_<T>_gfx950`, `nk_dots_packed_<T>_gfx950`,
+ *  the backend-suffixed kernels that dispatch_<T>.c binds, in the way the reference names its per-ISA
+ *  kernels (include/numkong/dots.h:361-1877). Plain C over the thin HIP ABI of <numkong_amd/hip_abi.h>.
+ *
+ *  The reference's kernels take caller-owned pointers and return nothing (include/numkong/dots.h:84-98);
+ *  so do these. A pointer the GPU can address is used in place; a plain host pointer is staged through
+ *  a temporary device buffer that lives for the duration of the call (the one hidden allocation of this
+ *  library). Failures follow c/numkong.c:195-216: size 0, pack is a no-op, the product fills C with 0xFF.
+ */
+#include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "dispatch.h"
+#include "numkong_amd/hip_abi.h"
+
+static _Thread_local char nk_amd_error_[256] = "";
+
+static void nk_amd_set_error_(char const *where) {
+    char const *detail = nk_hip_last_error();
+    snprintf(nk_amd_error_, sizeof(nk_amd_error_), "%s: %s", where, detail && detail[0] ? detail : "failed");
+}
+
+char const *nk_amd_last_error(void) { return nk_amd_error_; }
+
+static size_t nk_amd_element_bytes_(nk_dtype_t dtype) {
+    switch (dtype) {
+    case nk_i8_k:
+    case nk_u8_k:
+    case nk_e4m3_k:
+    case nk_e5m2_k: return 1;
+    case nk_f16_k:
+    case nk_bf16_k: return 2;
+    default: return 0;
+    }
+}
+
+static size_t nk_amd_round_up_(size_t x, size_t to) { return (x + to - 1) / to * to; }
+
+/** 0xFF over the m x n outputs only: the reference stub writes n * 8 bytes per row (c/numkong.c:209-216),
+ *  which overruns 4-byte outputs; the convention is kept, the overrun is not. */
+static void nk_amd_fill_error_(void *c, int c_kind, size_t m, size_t n, size_t c_stride) {
+    if (!c || !m || !n) return;
+    if (c_kind == 1) {
+        if (nk_hip_fill_rows_async(c, m, n, c_stride, 0xFFFFFFFFu, NULL) == 0) nk_hip_stream_synchronize(NULL);
+        return;
+    }
+    for (size_t row = 0; row < m; ++row) memset((char *)c + row * c_stride, 0xFF, n * 4);
+}
+
+int nk_amd_dots_pack_async(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t k, nk_size_t b_stride,
+                           void *b_packed, void *stream) {
+    return nk_hip_dots_pack_async((int)dtype, b, n, k, b_stride, b_packed, stream);
+}
+
+int nk_amd_dots_packed_async(nk_dtype_t dtype, void const *a, void const *b_packed, void *c, nk_size_t m, nk_size_t n,
+                             nk_size_t k, nk_size_t a_stride, nk_size_t c_stride, void *stream) {
+    return nk_hip_dots_packed_async((int)dtype, a, b_packed, c, m, n, k, a_stride, c_stride, stream);
+}
+
+static nk_size_t nk_amd_packed_size_(nk_dtype_t dtype, nk_size_t n, nk_size_t k) {
+    return nk_hip_dots_packed_size((int)dtype, n, k);
+}
+
+static void nk_amd_pack_(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t k, nk_size_t b_stride,
+                         void *b_packed) {
+    nk_amd_error_[0] = 0;
+    size_t const element_bytes = nk_amd_element_bytes_(dtype);
+    size_t const total = nk_hip_dots_packed_size((int)dtype, n, k);
+    if (!total || !b_packed) {
+        snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_pack: unsupported dtype or dimensions");
+        return;
+    }
+    if (nk_hip_device_count() <= 0) {
+        snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_pack: no HIP device");
+        return;
+    }
+    int const b_kind = (n && k) ? nk_hip_pointer_kind(b) : 1;
+    int const p_kind = nk_hip_pointer_kind(b_packed);
+    void *staged_b = NULL, *staged_p = NULL;
+    void const *device_b = b;
+    void *device_p = b_packed;
+    size_t device_b_stride = b_stride;
+    int status = 0;
+
+    if (b_kind == 0) {
+        size_t const row_bytes = k * element_bytes;
+        device_b_stride = nk_amd_round_up_(row_bytes, 16);
+        status = nk_hip_malloc(&staged_b, n * device_b_stride);
+        if (!status) status = nk_hip_memcpy2d_h2d(staged_b, device_b_stride, b, b_stride, row_bytes, n, NULL);
+        device_b = staged_b;
+    }
+    if (!status && p_kind == 0) {
+        status = nk_hip_malloc(&staged_p, total);
+        device_p = staged_p;
+    }
+    if (!status) status = nk_hip_dots_pack_async((int)dtype, device_b, n, k, device_b_stride, device_p, NULL);
+    if (!status && staged_p) status = nk_hip_memcpy_d2h(b_packed, staged_p, total, NULL);
+    if (!status) status = nk_hip_stream_synchronize(NULL);
+    if (status) nk_amd_set_error_("nk_dots_pack");
+    if (staged_b) nk_hip_free(staged_b);
+    if (staged_p) nk_hip_free(staged_p);
+}
+
+static void nk_amd_packed_(nk_dtype_t dtype, void const *a, void const *b_packed, void *c, nk_size_t m, nk_size_t n,
+                           nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {
+    nk_amd_error_[0] = 0;
+    if (!m || !n) return;
+    size_t const element_bytes = nk_amd_element_bytes_(dtype);
+    size_t const total = nk_hip_dots_packed_size((int)dtype, n, k);
+    if (nk_hip_device_count() <= 0) {
+        snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_packed: no HIP device");
+        nk_amd_fill_error_(c, 0, m, n, c_stride);
+        return;
+    }
+    int const c_kind = nk_hip_pointer_kind(c);
+    if (!total || !b_packed || !c) {
+        snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_packed: unsupported dtype or dimensions");
+        nk_amd_fill_error_(c, c_kind, m, n, c_stride);
+        return;
+    }
+    int const a_kind = k ? nk_hip_pointer_kind(a) : 1;
+    int const p_kind = nk_hip_pointer_kind(b_packed);
+    void *staged_a = NULL, *staged_p = NULL, *staged_c = NULL;
+    void const *device_a = a, *device_p = b_packed;
+    void *device_c = c;
+    size_t device_a_stride = a_stride, device_c_stride = c_stride;
+    int status = 0;
+
+    if (a_kind == 0) {
+        size_t const row_bytes = k * element_bytes;
+        device_a_stride = nk_amd_round_up_(row_bytes, 16);
+        status = nk_hip_malloc(&staged_a, m * device_a_stride);
+        if (!status) status = nk_hip_memcpy2d_h2d(staged_a, device_a_stride, a, a_stride, row_bytes, m, NULL);
+        device_a = staged_a;
+    }
+    if (!status && p_kind == 0) {
+        status = nk_hip_malloc(&staged_p, total);
+        if (!status) status = nk_hip_memcpy_h2d(staged_p, b_packed, total, NULL);
+        device_p = staged_p;
+    }
+    if (!status && c_kind == 0) {
+        device_c_stride = nk_amd_round_up_(n * 4, 16);
+        status = nk_hip_malloc(&staged_c, m * device_c_stride);
+        device_c = staged_c;
+    }
+    if (!status)
+        status = nk_hip_dots_packed_async((int)dtype, device_a, device_p, device_c, m, n, k, device_a_stride,
+                                          device_c_stride, NULL);
+    if (!status && staged_c) status = nk_hip_memcpy2d_d2h(c, c_stride, staged_c, device_c_stride, n * 4, m, NULL);
+    if (!status) status = nk_hip_stream_synchronize(NULL);
+    if (status) {
+        nk_amd_set_error_("nk_dots_packed");
+        nk_amd_fill_error_(c, c_kind, m, n, c_stride);
+    }
+    if (staged_a) nk_hip_free(staged_a);
+    if (staged_p) nk_hip_free(staged_p);
+    if (staged_c) nk_hip_free(staged_c);
+}
+
+#define NK_AMD_DEFINE_BACKEND_(T, in_t, out_t)                                                                     \
+    nk_size_t nk_dots_packed_size_##T##_gfx950(nk_size_t width, nk_size_t depth) {                                 \
+        return nk_amd_packed_size_(nk_##T##_k, width, depth);                                                      \
+    }                                                                                                              \
+    void nk_dots_pack_##T##_gfx950(in_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,            \
+                                   void *b_packed) {                                                               \
+        nk_amd_pack_(nk_##T##_k, b, width, depth, b_stride, b_packed);                                             \
+    }                                                                                                              \
+    void nk_dots_packed_##T##_gfx950(in_t const *a, void const *b_packed, out_t *c, nk_size_t height,              \
+                                     nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride) {   \
+        nk_amd_packed_(nk_##T##_k, a, b_packed, c, height, width, depth, a_stride, c_stride);                      \
+    }
+
+NK_AMD_DEFINE_BACKEND_(i8, nk_i8_t, nk_i32_t)
+NK_AMD_DEFINE_BACKEND_(u8, nk_u8_t, nk_u32_t)
+NK_AMD_DEFINE_BACKEND_(bf16, nk_bf16_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_(f16, nk_f16_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_(e4m3, nk_e4m3_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_(e5m2, nk_e5m2_t, nk_f32_t)
