@@ -22,10 +22,9 @@
  *  so the 64 lanes of a wavefront that execute one 32x32 MFMA step `q` (lane l supplies row l % 32 and
  *  chunk 2q + l / 32) read 1024 contiguous bytes at `data + (t * k_chunks + 2q) * 512 + l * 16`: the image
  *  is the MFMA operand-fragment order, and B goes from HBM to registers with one coalesced 128-bit load
- *  per lane per step, never through LDS. The same image serves the 16-byte-per-lane MFMAs
- *  (32x32x32 i8, 32x32x16 bf16/f16), the 8-byte legacy fp8 forms (two MFMAs per chunk) and the
- *  32-byte f8f6f4 forms (two chunks per MFMA), because a product only needs A and B to agree on which
- *  k sits in which operand slot.
+ *  per lane per step, never through LDS. Which k sits in which operand slot of the instruction does not
+ *  matter as long as A and B agree, and they do: A fragments are read from LDS with the same rule.
+ *  e4m3 and e5m2 are stored widened to f16 (see packed_bytes_of), so their chunks hold 8 values.
  *
  *  u8 has no unsigned MFMA. B is stored as b' = b ^ 0x80 (signed b - 128), A is turned into
  *  a' = a ^ 0x80 on its way into LDS, and  sum(a*b) = sum(a'*b') + 128*sum(a) + 128*sum(b')  (mod 2^32)
@@ -73,7 +72,7 @@ struct PackedHeader {
     uint32_t magic;
     uint32_t version;
     uint32_t dtype;
-    uint32_t elem_bytes;
+    uint32_t elem_bytes; // bytes per element as stored in the image (2 for fp8, which is widened to f16)
     uint32_t n;        // logical rows of B = columns of C
     uint32_t k;        // logical depth in elements
     uint32_t n_tiles;  // ceil(n / 32)
@@ -86,8 +85,12 @@ struct PackedHeader {
 static_assert(sizeof(PackedHeader) == 64, "header must stay 64 bytes");
 
 struct Geometry {
-    uint32_t elem_bytes, n, k, n_tiles, k_chunks;
-    uint64_t k_bytes, data_bytes, sums_bytes, total_bytes;
+    uint32_t elem_bytes;   // bytes per element in the caller's A and B
+    uint32_t packed_bytes; // bytes per element in the image and in LDS (fp8 is widened to f16)
+    uint32_t n, k, n_tiles, k_chunks;
+    uint64_t k_bytes;      // bytes of one packed row: k * packed_bytes
+    uint64_t k_src_bytes;  // bytes of one source row: k * elem_bytes
+    uint64_t data_bytes, sums_bytes, total_bytes;
 };
 
 inline int elem_bytes_of(int dtype) {
@@ -102,12 +105,19 @@ inline int elem_bytes_of(int dtype) {
     }
 }
 
+/** The fp8 MFMA forms of gfx950 align the products inside one lane's k-group to the largest of them and
+ *  keep only about 14 bits (1 + 2^-14 comes back as 1), far from the f32 accumulation of the reference's
+ *  kernels (dot/serial.h:522-600). e4m3 and e5m2 are therefore widened, exactly, to f16 and run on the f16
+ *  MFMA, whose products and sums are kept to full f32 precision: B at pack time, A on its way into LDS. */
+inline int packed_bytes_of(int dtype) { return (dtype == kE4M3 || dtype == kE5M2) ? 2 : elem_bytes_of(dtype); }
+
 inline bool make_geometry(int dtype, size_t n, size_t k, Geometry &g) {
     int const eb = elem_bytes_of(dtype);
     if (!eb) return false;
     if (n > 0x7FFFFFFFull || k > 0x3FFFFFFFull) return false;
-    g.elem_bytes = (uint32_t)eb, g.n = (uint32_t)n, g.k = (uint32_t)k;
-    g.k_bytes = (uint64_t)k * eb;
+    g.elem_bytes = (uint32_t)eb, g.packed_bytes = (uint32_t)packed_bytes_of(dtype), g.n = (uint32_t)n, g.k = (uint32_t)k;
+    g.k_bytes = (uint64_t)k * g.packed_bytes;
+    g.k_src_bytes = (uint64_t)k * eb;
     uint64_t const chunks = (g.k_bytes + kChunkBytes - 1) / kChunkBytes;
     g.k_chunks = (uint32_t)((chunks + kStageChunks - 1) / kStageChunks * kStageChunks);
     g.n_tiles = (uint32_t)((n + kTileRows - 1) / kTileRows);
@@ -159,31 +169,58 @@ __device__ __forceinline__ uint32_t sum_bytes_u8(v4i v) {
     return s;
 }
 
+/** Eight OCP fp8 values (two dwords) -> eight f16 values, exact for every code incl. subnormals, Inf, NaN. */
+template <bool E5M2>
+__device__ __forceinline__ v4i widen_fp8x8(uint32_t lo, uint32_t hi) {
+    typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+    v2h p0, p1, p2, p3;
+    if (E5M2) {
+        p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(lo, 1.0f, false);
+        p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(lo, 1.0f, true);
+        p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(hi, 1.0f, false);
+        p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(hi, 1.0f, true);
+    }
+    else {
+        p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false);
+        p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, true);
+        p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, false);
+        p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, true);
+    }
+    v4i out;
+    out[0] = __builtin_bit_cast(int, p0), out[1] = __builtin_bit_cast(int, p1);
+    out[2] = __builtin_bit_cast(int, p2), out[3] = __builtin_bit_cast(int, p3);
+    return out;
+}
+
 #pragma region Packing
 
 /**
  *  One thread per 16-byte chunk of the image. A block of 256 threads covers 32 rows x 8 chunks: reads are
- *  128 contiguous bytes per row, writes are eight 512-byte runs.
+ *  128 (64 for fp8) contiguous bytes per row, writes are eight 512-byte runs. WIDEN: 0 copies the
+ *  elements, 1 widens e4m3 to f16, 2 widens e5m2 to f16 (8 source bytes per chunk).
  */
+template <int WIDEN>
 __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
-                                                   uint64_t k_bytes, uint32_t k_chunks, uint8_t *__restrict__ data,
+                                                   uint64_t k_src_bytes, uint32_t k_chunks, uint8_t *__restrict__ data,
                                                    int avec, uint32_t xr) {
+    constexpr int kSrcChunk = WIDEN ? 8 : 16;
     uint32_t const groups = k_chunks / kStageChunks;
     uint32_t const tile = blockIdx.x / groups;
     uint32_t const group = blockIdx.x % groups;
     uint32_t const r = threadIdx.x >> 3;
     uint32_t const c = group * kStageChunks + (threadIdx.x & 7);
     uint64_t const row = (uint64_t)tile * kTileRows + r;
-    int64_t const left = (int64_t)k_bytes - (int64_t)c * kChunkBytes;
-    int const valid = row < n ? (int)(left > 16 ? 16 : (left < 0 ? 0 : left)) : 0;
+    int64_t const left = (int64_t)k_src_bytes - (int64_t)c * kSrcChunk;
+    int const valid = row < n ? (int)(left > kSrcChunk ? kSrcChunk : (left < 0 ? 0 : left)) : 0;
     v4i v = {0, 0, 0, 0};
     if (valid > 0) {
-        uint8_t const *src = b + row * b_stride + (uint64_t)c * kChunkBytes;
-        if (valid == 16 && avec >= 16) {
+        uint8_t const *src = b + row * b_stride + (uint64_t)c * kSrcChunk;
+        if (!WIDEN && valid == 16 && avec >= 16) {
             v = *(v4i const *)src;
             v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
         }
         else { v = load_chunk_guarded(src, valid, avec, xr); }
+        if (WIDEN) v = widen_fp8x8<WIDEN == 2>((uint32_t)v[0], (uint32_t)v[1]);
     }
     *(v4i *)(data + (((uint64_t)tile * k_chunks + c) * kTileRows + r) * kChunkBytes) = v;
 }
@@ -228,6 +265,8 @@ __global__ __launch_bounds__(256) void fill_rows_kernel(uint8_t *c, uint32_t m, 
 #pragma region Element types
 
 struct I8 {
+    static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
+    static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16i acc_t;
     static constexpr int kDtype = kI8;
     static constexpr bool kUnsigned = false;
@@ -240,6 +279,8 @@ struct U8 : I8 {
     static constexpr bool kUnsigned = true;
 };
 struct BF16 {
+    static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
+    static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
     static constexpr int kDtype = kBF16;
     static constexpr bool kUnsigned = false;
@@ -249,6 +290,8 @@ struct BF16 {
     }
 };
 struct F16 {
+    static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
+    static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
     static constexpr int kDtype = kF16;
     static constexpr bool kUnsigned = false;
@@ -257,25 +300,15 @@ struct F16 {
                                                      0);
     }
 };
-struct E4M3 {
-    typedef v16f acc_t;
+struct E4M3 : F16 {
     static constexpr int kDtype = kE4M3;
-    static constexpr bool kUnsigned = false;
-    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
-        v2l const al = __builtin_bit_cast(v2l, a), bl = __builtin_bit_cast(v2l, b);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[0], bl[0], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[1], bl[1], acc, 0, 0, 0);
-    }
+    static constexpr int kSrcChunk = 8;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<false>((uint32_t)v[0], (uint32_t)v[1]); }
 };
-struct E5M2 {
-    typedef v16f acc_t;
+struct E5M2 : F16 {
     static constexpr int kDtype = kE5M2;
-    static constexpr bool kUnsigned = false;
-    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
-        v2l const al = __builtin_bit_cast(v2l, a), bl = __builtin_bit_cast(v2l, b);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(al[0], bl[0], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(al[1], bl[1], acc, 0, 0, 0);
-    }
+    static constexpr int kSrcChunk = 8;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<true>((uint32_t)v[0], (uint32_t)v[1]); }
 };
 
 #pragma endregion Element types
@@ -295,7 +328,7 @@ struct GemmArgs {
     uint8_t const *a;
     uint8_t const *bp; // packed image (header first)
     uint8_t *c;
-    uint64_t a_stride, c_stride, k_bytes;
+    uint64_t a_stride, c_stride, k_src_bytes;
     uint32_t m, n, k;
     uint32_t n_tiles, k_chunks;
     uint32_t tiles_m, tiles_n;
@@ -377,7 +410,7 @@ __global__ __launch_bounds__(NW * 64) void dots_packed_kernel(GemmArgs g) {
         for (int i = 0; i < kLoads; ++i) {
             uint32_t const r = (i * NT + tid) >> 3;
             uint32_t const row = row0 + r < g.m ? row0 + r : g.m - 1;
-            a_src[i] = g.a + (uint64_t)row * g.a_stride + chunk_in_stage * kChunkBytes;
+            a_src[i] = g.a + (uint64_t)row * g.a_stride + chunk_in_stage * T::kSrcChunk;
             lds_dst[i] = r * kPitch + chunk_in_stage * kChunkBytes;
         }
         // Per-wavefront B fragment streams (tile index clamped the same way).
@@ -395,22 +428,28 @@ __global__ __launch_bounds__(NW * 64) void dots_packed_kernel(GemmArgs g) {
         v4i b_reg[2][TN][4];
 
         auto load_a = [&](uint32_t s) {
-            uint64_t const offset = (uint64_t)s * kStageBytes;
-            bool const full = offset + kStageBytes <= g.k_bytes;
+            uint64_t const offset = (uint64_t)s * (kStageChunks * T::kSrcChunk);
+            bool const full = offset + kStageChunks * T::kSrcChunk <= g.k_src_bytes;
             if (ALIGNED && full) {
 #pragma unroll
                 for (int i = 0; i < kLoads; ++i) {
-                    v4i v = *(v4i const *)(a_src[i] + offset);
+                    v4i v = {0, 0, 0, 0};
+                    if (T::kSrcChunk == 16) { v = *(v4i const *)(a_src[i] + offset); }
+                    else {
+                        typedef int v2i __attribute__((ext_vector_type(2)));
+                        v2i const narrow = *(v2i const *)(a_src[i] + offset);
+                        v[0] = narrow[0], v[1] = narrow[1];
+                    }
                     if (T::kUnsigned) {
                         row_sum[i] += sum_bytes_u8(v);
                         v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
                     }
-                    a_reg[i] = v;
+                    a_reg[i] = T::widen(v);
                 }
             }
             else {
-                int64_t const left = (int64_t)g.k_bytes - (int64_t)offset - (int64_t)chunk_in_stage * kChunkBytes;
-                int const valid = (int)(left > 16 ? 16 : (left < 0 ? 0 : left));
+                int64_t const left = (int64_t)g.k_src_bytes - (int64_t)offset - (int64_t)chunk_in_stage * T::kSrcChunk;
+                int const valid = (int)(left > T::kSrcChunk ? T::kSrcChunk : (left < 0 ? 0 : left));
 #pragma unroll
                 for (int i = 0; i < kLoads; ++i) {
                     v4i v = load_chunk_guarded(a_src[i] + offset, valid, g.avec, 0u);
@@ -424,7 +463,7 @@ __global__ __launch_bounds__(NW * 64) void dots_packed_kernel(GemmArgs g) {
                             v[w] ^= (int)mask;
                         }
                     }
-                    a_reg[i] = v;
+                    a_reg[i] = T::widen(v);
                 }
             }
         };
@@ -531,7 +570,7 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream) {
     g.tiles_n = (g.n + BN - 1) / BN;
     uint64_t const blocks = (uint64_t)g.tiles_m * g.tiles_n;
     if (blocks > 0x7FFFFFFFull) return hipErrorInvalidValue;
-    bool const aligned = g.avec >= 16;
+    bool const aligned = g.avec >= T::kSrcChunk;
     auto kernel = aligned ? dots_packed_kernel<T, TM, TN, NW, true> : dots_packed_kernel<T, TM, TN, NW, false>;
     if (lds_bytes > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((void const *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -660,7 +699,7 @@ int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t 
 
     PackedHeader h;
     memset(&h, 0, sizeof(h));
-    h.magic = kMagic, h.version = kVersion, h.dtype = (uint32_t)dtype, h.elem_bytes = g.elem_bytes;
+    h.magic = kMagic, h.version = kVersion, h.dtype = (uint32_t)dtype, h.elem_bytes = g.packed_bytes;
     h.n = g.n, h.k = g.k, h.n_tiles = g.n_tiles, h.k_chunks = g.k_chunks;
     h.data_offset = sizeof(PackedHeader);
     h.sums_offset = sizeof(PackedHeader) + g.data_bytes;
@@ -676,8 +715,9 @@ int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t 
         uint64_t const blocks = (uint64_t)g.n_tiles * (g.k_chunks / kStageChunks);
         if (blocks > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_pack: matrix too large");
         uint32_t const xr = dtype == kU8 ? 0x80808080u : 0u;
-        hipLaunchKernelGGL(pack_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t const *)b,
-                           (uint64_t)b_stride, g.n, g.k_bytes, g.k_chunks, data, widest_load(b, b_stride), xr);
+        auto kernel = dtype == kE4M3 ? pack_kernel<1> : (dtype == kE5M2 ? pack_kernel<2> : pack_kernel<0>);
+        hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride,
+                           g.n, g.k_src_bytes, g.k_chunks, data, widest_load(b, b_stride), xr);
         e = hipGetLastError();
         if (e != hipSuccess) return fail(e, "pack_kernel");
     }
@@ -725,7 +765,7 @@ int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, voi
     GemmArgs g;
     memset(&g, 0, sizeof(g));
     g.a = (uint8_t const *)a, g.bp = (uint8_t const *)b_packed, g.c = (uint8_t *)c;
-    g.a_stride = a_stride, g.c_stride = c_stride, g.k_bytes = geo.k_bytes;
+    g.a_stride = a_stride, g.c_stride = c_stride, g.k_src_bytes = geo.k_src_bytes;
     g.m = (uint32_t)m, g.n = geo.n, g.k = geo.k, g.n_tiles = geo.n_tiles, g.k_chunks = geo.k_chunks;
     g.avec = widest_load(a, a_stride);
 

@@ -1,0 +1,321 @@
+/**
+ *  @brief CPU restatement of NumKong's packed batched dots, serial semantics. TEST INFRASTRUCTURE ONLY.
+ *  @file oracle/dots_oracle.c
+ *
+ *  This file is the checker, not the product: only tests/, __graft_entry__.smoke() and the cpu_baseline
+ *  leg of bench.py may load it. Nothing under numkong_amd/ links, imports or calls it, and the product
+ *  has no CPU fallback.
+ *
+ *  What is restated, and from where (paths relative to the reference checkout):
+ *    - element decode/encode for f16, bf16, e4m3 (OCP E4M3FN), e5m2 (OCP)
+ *          include/numkong/cast/serial.h:586-623, 669-741, 750-784, 810-839, 866-947, 1042-1082, 1109-1180
+ *    - packed size and layout of the serial backend: 64-byte header {columns, depth, padded depth},
+ *      rows padded with zeros, per-column norms behind them
+ *          include/numkong/dots/serial.h:103-108, 245-271, 286-333, instantiated :2493-2599
+ *    - the serial product: integers accumulate exactly in 64 bits and are truncated to 32,
+ *      floats accumulate exact products into 4 f32 lane sums (lane = k mod 4, increasing k) that are
+ *      combined as ((s0 + s1) + s2) + s3; C is overwritten
+ *          include/numkong/dots/serial.h:520-1072, include/numkong/dot/serial.h:376-600
+ *    - the f64 ground truth of the reference's own tests: sum = sum + (f64)a * (f64)b in depth order
+ *          include/numkong/dots.hpp:42-61, test/test_cross.hpp:26-71
+ *
+ *  The conversions are written from the formats' definitions (value = (-1)^s * 2^(e-bias) * 1.m,
+ *  round-to-nearest-even onto the target grid, the overflow/NaN policies listed in the comment tables of
+ *  cast/serial.h), not from the reference's control flow. Every function here is pinned by
+ *  tests/test_oracle.py: against the reference library built from its own sources (oracle/_ref) where
+ *  that exists, against committed vectors produced from it (tests/golden), against torch's float8/
+ *  float16/bfloat16 decoders, and against closed forms (exact integer products, powers of two).
+ *
+ *  Parity unpinned: the per-column norms of FLOAT types in the packed image (the reference computes them
+ *  with nk_reduce_moments_*, whose summation order is not restated here). They are not read by
+ *  dots_packed; this file writes zeros there and the tests compare header + rows only.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+enum {
+    NKO_I8 = 1 << 2,
+    NKO_U8 = 1 << 6,
+    NKO_F16 = 1 << 12,
+    NKO_BF16 = 1 << 13,
+    NKO_E4M3 = 1 << 14,
+    NKO_E5M2 = 1 << 15,
+};
+
+#define NKO_API __attribute__((visibility("default")))
+
+static float bits_to_f32(uint32_t u) {
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+static uint32_t f32_to_bits(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+
+/* Small IEEE-like formats: sign, `ebits` exponent bits with bias, `mbits` mantissa bits. */
+typedef struct {
+    int ebits, mbits, bias;
+    int has_inf;       /* all-ones exponent encodes Inf (m = 0) and NaN (m != 0), as f16 and e5m2 do      */
+    int nan_is_all_ones; /* only exponent and mantissa all ones is NaN, no Inf (E4M3FN)                   */
+    int saturate;      /* overflow (and Inf input) clamps to the largest finite value instead of Inf      */
+    uint32_t nan_code; /* magnitude bits written for a NaN input                                          */
+} small_format_t;
+
+static small_format_t const k_f16 = {5, 10, 15, 1, 0, 0, 0x7E00};
+static small_format_t const k_e4m3 = {4, 3, 7, 0, 1, 1, 0x7F};
+static small_format_t const k_e5m2 = {5, 2, 15, 1, 0, 0, 0x7D};
+
+static float small_decode(small_format_t const *fmt, uint32_t code) {
+    int const total = 1 + fmt->ebits + fmt->mbits;
+    uint32_t const sign = (code >> (total - 1)) & 1;
+    uint32_t const e = (code >> fmt->mbits) & ((1u << fmt->ebits) - 1);
+    uint32_t const m = code & ((1u << fmt->mbits) - 1);
+    uint32_t const e_max = (1u << fmt->ebits) - 1;
+    float magnitude;
+    if (fmt->has_inf && e == e_max) {
+        if (m == 0) magnitude = INFINITY;
+        else {
+            /* quiet NaN; f16 keeps its payload in the top mantissa bits like the reference does */
+            uint32_t payload = fmt->mbits == 10 ? (m << 13) : 0x00400000u;
+            return bits_to_f32((sign << 31) | 0x7F800000u | payload);
+        }
+    }
+    else if (fmt->nan_is_all_ones && e == e_max && m == (1u << fmt->mbits) - 1) {
+        return bits_to_f32((sign << 31) | 0x7FC00000u);
+    }
+    else if (e == 0) { magnitude = ldexpf((float)m, 1 - fmt->bias - fmt->mbits); }
+    else { magnitude = ldexpf((float)((1u << fmt->mbits) | m), (int)e - fmt->bias - fmt->mbits); }
+    return sign ? -magnitude : magnitude;
+}
+
+/* Round-to-nearest-even of a finite f32 onto the format's grid, done on the integer significand. */
+static uint32_t small_encode(small_format_t const *fmt, float x) {
+    int const total = 1 + fmt->ebits + fmt->mbits;
+    uint32_t const bits = f32_to_bits(x);
+    uint32_t const sign = (bits >> 31) << (total - 1);
+    uint32_t const magnitude_bits = bits & 0x7FFFFFFFu;
+    uint32_t const e_max = (1u << fmt->ebits) - 1;
+    uint32_t const max_finite = fmt->has_inf ? ((e_max << fmt->mbits) - 1)        /* largest below Inf   */
+                                             : ((e_max << fmt->mbits) | ((1u << fmt->mbits) - 2)); /* E4M3FN: 0x7E */
+    uint32_t const inf_code = e_max << fmt->mbits;
+    if (magnitude_bits > 0x7F800000u) {
+        if (fmt->mbits == 10) { /* f16 keeps the truncated payload, never letting it become zero */
+            uint32_t payload = (magnitude_bits & 0x007FFFFFu) >> 13;
+            if (!payload) payload = 1;
+            return sign | inf_code | payload;
+        }
+        return sign | fmt->nan_code;
+    }
+    if (magnitude_bits == 0x7F800000u) return sign | (fmt->saturate ? max_finite : inf_code);
+    if (magnitude_bits == 0) return sign;
+
+    int exponent2;
+    float const fraction = frexpf(fabsf(x), &exponent2); /* |x| = fraction * 2^exponent2, fraction in [0.5, 1) */
+    int unbiased = exponent2 - 1;                       /* |x| = 1.f * 2^unbiased */
+    int const min_normal = 1 - fmt->bias;
+    /* quantum = spacing of the grid at this magnitude */
+    int const quantum_exp = (unbiased < min_normal ? min_normal : unbiased) - fmt->mbits;
+    /* |x| / 2^quantum_exp is exactly representable in double; round it to nearest even */
+    double const scaled = ldexp((double)fraction, exponent2 - quantum_exp);
+    double rounded = nearbyint(scaled); /* default rounding mode: to nearest, ties to even */
+    uint64_t q = (uint64_t)rounded;
+    if (q == 0) return sign;
+    /* q is either a subnormal mantissa (< 2^mbits) or a significand in [2^mbits, 2^(mbits+1)] */
+    int overflow = 0;
+    uint32_t code = 0;
+    if (unbiased < min_normal) { code = (uint32_t)q; /* a carry into 2^mbits lands on the first normal by itself */ }
+    else {
+        int e = unbiased + fmt->bias;
+        if (q == (2ull << fmt->mbits)) q >>= 1, e += 1;
+        if ((uint32_t)e > e_max) overflow = 1;
+        else code = ((uint32_t)e << fmt->mbits) | ((uint32_t)q & ((1u << fmt->mbits) - 1));
+    }
+    if (fmt->has_inf) {
+        if (overflow || code >= inf_code) return sign | (fmt->saturate ? max_finite : inf_code);
+    }
+    else if (overflow || code > max_finite) { return sign | max_finite; }
+    return sign | code;
+}
+
+NKO_API float nko_f16_to_f32(uint16_t x) { return small_decode(&k_f16, x); }
+NKO_API uint16_t nko_f32_to_f16(float x) { return (uint16_t)small_encode(&k_f16, x); }
+NKO_API float nko_e4m3_to_f32(uint8_t x) { return small_decode(&k_e4m3, x); }
+NKO_API uint8_t nko_f32_to_e4m3(float x) { return (uint8_t)small_encode(&k_e4m3, x); }
+NKO_API float nko_e5m2_to_f32(uint8_t x) { return small_decode(&k_e5m2, x); }
+NKO_API uint8_t nko_f32_to_e5m2(float x) { return (uint8_t)small_encode(&k_e5m2, x); }
+
+/* bf16 is the top half of an f32; the reference rounds by adding 0x7FFF plus the kept LSB and does not
+ * special-case NaN or overflow (cast/serial.h:768-784), which is restated literally because it defines
+ * the result for every bit pattern. */
+NKO_API float nko_bf16_to_f32(uint16_t x) { return bits_to_f32((uint32_t)x << 16); }
+NKO_API uint16_t nko_f32_to_bf16(float x) {
+    uint32_t u = f32_to_bits(x);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+static int element_bytes(int dtype) {
+    switch (dtype) {
+    case NKO_I8:
+    case NKO_U8:
+    case NKO_E4M3:
+    case NKO_E5M2: return 1;
+    case NKO_F16:
+    case NKO_BF16: return 2;
+    default: return 0;
+    }
+}
+
+/* Value of element `i` of a row as f32 (integers are exact in f32 too: |x| <= 255). */
+static float element_f32(int dtype, void const *row, size_t i) {
+    switch (dtype) {
+    case NKO_I8: return (float)((int8_t const *)row)[i];
+    case NKO_U8: return (float)((uint8_t const *)row)[i];
+    case NKO_F16: return nko_f16_to_f32(((uint16_t const *)row)[i]);
+    case NKO_BF16: return nko_bf16_to_f32(((uint16_t const *)row)[i]);
+    case NKO_E4M3: return nko_e4m3_to_f32(((uint8_t const *)row)[i]);
+    case NKO_E5M2: return nko_e5m2_to_f32(((uint8_t const *)row)[i]);
+    default: return NAN;
+    }
+}
+
+NKO_API void nko_decode(int dtype, void const *src, size_t count, float *dst) {
+    for (size_t i = 0; i < count; ++i) dst[i] = element_f32(dtype, src, i);
+}
+
+NKO_API void nko_encode(int dtype, float const *src, size_t count, void *dst) {
+    for (size_t i = 0; i < count; ++i) switch (dtype) {
+        case NKO_F16: ((uint16_t *)dst)[i] = nko_f32_to_f16(src[i]); break;
+        case NKO_BF16: ((uint16_t *)dst)[i] = nko_f32_to_bf16(src[i]); break;
+        case NKO_E4M3: ((uint8_t *)dst)[i] = nko_f32_to_e4m3(src[i]); break;
+        case NKO_E5M2: ((uint8_t *)dst)[i] = nko_f32_to_e5m2(src[i]); break;
+        default: break;
+        }
+}
+
+#pragma region Serial packed layout
+
+/* Per backend instantiation: values per 128-bit step, and the element width stored in the image
+ * (dots/serial.h:2493-2599; f16 is stored already widened to f32). */
+static size_t serial_step(int dtype) {
+    switch (dtype) {
+    case NKO_F16: return 4;
+    case NKO_BF16: return 8;
+    default: return 16;
+    }
+}
+static size_t serial_packed_element_bytes(int dtype) { return dtype == NKO_F16 ? 4 : (size_t)element_bytes(dtype); }
+
+static size_t serial_padded_depth(int dtype, size_t depth) {
+    size_t const step = serial_step(dtype);
+    size_t padded = (depth + step - 1) / step * step;
+    size_t const stride_bytes = padded * serial_packed_element_bytes(dtype);
+    /* a power-of-two row stride is broken up by one extra step (dots/serial.h:260-265) */
+    if (stride_bytes && !(stride_bytes & (stride_bytes - 1))) padded += step;
+    return padded;
+}
+
+NKO_API size_t nko_serial_packed_size(int dtype, size_t columns, size_t depth) {
+    if (!element_bytes(dtype)) return 0;
+    return 64 + columns * serial_padded_depth(dtype, depth) * serial_packed_element_bytes(dtype) + columns * 4;
+}
+
+NKO_API void nko_serial_pack(int dtype, void const *b, size_t columns, size_t depth, size_t b_stride, void *packed) {
+    size_t const padded = serial_padded_depth(dtype, depth);
+    size_t const width = serial_packed_element_bytes(dtype);
+    uint32_t header[16] = {0};
+    header[0] = (uint32_t)columns, header[1] = (uint32_t)depth, header[2] = (uint32_t)padded;
+    memcpy(packed, header, 64);
+    unsigned char *rows = (unsigned char *)packed + 64;
+    for (size_t j = 0; j < columns; ++j) {
+        unsigned char const *source = (unsigned char const *)b + j * b_stride;
+        unsigned char *target = rows + j * padded * width;
+        memset(target, 0, padded * width);
+        if (dtype == NKO_F16)
+            for (size_t l = 0; l < depth; ++l) ((float *)target)[l] = nko_f16_to_f32(((uint16_t const *)source)[l]);
+        else memcpy(target, source, depth * width);
+    }
+    uint32_t *norms = (uint32_t *)(rows + columns * padded * width);
+    for (size_t j = 0; j < columns; ++j) {
+        uint64_t sum_of_squares = 0;
+        if (dtype == NKO_I8 || dtype == NKO_U8) {
+            unsigned char const *source = (unsigned char const *)b + j * b_stride;
+            for (size_t l = 0; l < depth; ++l) {
+                int64_t const v = dtype == NKO_I8 ? (int64_t)((int8_t const *)source)[l] : (int64_t)source[l];
+                sum_of_squares += (uint64_t)(v * v);
+            }
+        }
+        norms[j] = (uint32_t)sum_of_squares; /* float dtypes: zeros, see "parity unpinned" in the file header */
+    }
+}
+
+#pragma endregion Serial packed layout
+
+#pragma region Products
+
+/** C = A * B^T exactly as the serial backend rounds it, reading an image made by nko_serial_pack. */
+NKO_API void nko_serial_packed(int dtype, void const *a, void const *packed, void *c, size_t rows, size_t columns,
+                               size_t depth, size_t a_stride, size_t c_stride) {
+    uint32_t header[16];
+    memcpy(header, packed, 64);
+    size_t const padded = header[2];
+    size_t const width = serial_packed_element_bytes(dtype);
+    unsigned char const *b_rows = (unsigned char const *)packed + 64;
+    int const image_dtype = dtype == NKO_F16 ? 0 : dtype;
+    for (size_t i = 0; i < rows; ++i) {
+        unsigned char const *a_row = (unsigned char const *)a + i * a_stride;
+        unsigned char *c_row = (unsigned char *)c + i * c_stride;
+        for (size_t j = 0; j < columns; ++j) {
+            unsigned char const *b_row = b_rows + j * padded * width;
+            if (dtype == NKO_I8) {
+                int64_t sum = 0;
+                for (size_t l = 0; l < depth; ++l) sum += (int64_t)((int8_t const *)a_row)[l] * ((int8_t const *)b_row)[l];
+                ((int32_t *)c_row)[j] = (int32_t)sum;
+            }
+            else if (dtype == NKO_U8) {
+                uint64_t sum = 0;
+                for (size_t l = 0; l < depth; ++l) sum += (uint64_t)a_row[l] * b_row[l];
+                ((uint32_t *)c_row)[j] = (uint32_t)sum;
+            }
+            else {
+                float lanes[4] = {0, 0, 0, 0};
+                for (size_t l = 0; l < depth; ++l) {
+                    float const x = element_f32(dtype, a_row, l);
+                    float const y = image_dtype ? element_f32(image_dtype, b_row, l) : ((float const *)b_row)[l];
+                    /* the product of two values with <= 11 significant bits is exact in f32; `volatile`
+                     * keeps the compiler from contracting the multiply-add into one rounding */
+                    volatile float product = x * y;
+                    lanes[l & 3] += product;
+                }
+                ((float *)c_row)[j] = ((lanes[0] + lanes[1]) + lanes[2]) + lanes[3];
+            }
+        }
+    }
+}
+
+/** f64 ground truth from the unpacked B: sum = sum + a * b in depth order (dots.hpp:42-61). Also returns,
+ *  when `magnitude` is not NULL, sum |a * b| per element, the scale of the normwise error. */
+NKO_API void nko_dots_f64(int dtype, void const *a, void const *b, double *c, double *magnitude, size_t rows,
+                          size_t columns, size_t depth, size_t a_stride, size_t b_stride) {
+    for (size_t i = 0; i < rows; ++i) {
+        unsigned char const *a_row = (unsigned char const *)a + i * a_stride;
+        for (size_t j = 0; j < columns; ++j) {
+            unsigned char const *b_row = (unsigned char const *)b + j * b_stride;
+            double sum = 0, absolute = 0;
+            for (size_t l = 0; l < depth; ++l) {
+                double const product = (double)element_f32(dtype, a_row, l) * (double)element_f32(dtype, b_row, l);
+                sum = sum + product;
+                absolute += fabs(product);
+            }
+            c[i * columns + j] = sum;
+            if (magnitude) magnitude[i * columns + j] = absolute;
+        }
+    }
+}
+
+#pragma endregion Products

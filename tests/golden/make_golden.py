@@ -1,0 +1,57 @@
+"""Writes tests/golden/*.npz from the reference library (oracle/_ref/libnumkong.so).
+
+Run in the development container, where the reference checkout exists:  python tests/golden/make_golden.py
+The fixtures are data only: seeded inputs and what the reference's `_serial` kernels (and `nk_cast_serial`)
+returned for them, so that the oracle stays pinned on machines without the reference.
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from tests import support  # noqa: E402
+
+
+def main():
+    oracle, reference = support.load_oracle(), support.load_reference()
+    if reference is None:
+        raise SystemExit("build oracle/_ref first: make -C oracle")
+    out = support.GOLDEN_DIR
+    rng = np.random.default_rng(2024)
+    for dtype in support.FLOAT_DTYPES:
+        codes = np.arange(256 if support.STORAGE[dtype] == np.uint8 else 65536).astype(support.STORAGE[dtype])
+        if len(codes) > 256:
+            codes = np.concatenate([codes[::61], np.array([0x0001, 0x03FF, 0x0400, 0x7BFF, 0x7C00, 0xFC00, 0x7E00, 0x8000,
+                                                           0x7F7F, 0x7F80, 0xFF80, 0x7FC0], np.uint16)])
+        values = np.concatenate([
+            rng.standard_normal(1500).astype(np.float32) * np.float32(s) for s in (1e-6, 1e-3, 1, 300, 5e4)
+        ] + [np.array([0, -0.0, np.inf, -np.inf, np.nan, 448, 449, 464, 465, 480, 57344, 61439.9, 61440, 65504, 65519.9,
+                       65520, 2.0**-9, 2.0**-10, 1.5 * 2.0**-10, 2.0**-16, 2.0**-17, 1.5 * 2.0**-17, 2.0**-24, 2.0**-25,
+                       1.0001 * 2.0**-25, 1e-40, 3e38], np.float32)])
+        np.savez_compressed(os.path.join(out, f"cast_{dtype}.npz"), dtype=dtype, codes=codes,
+                            decoded=reference.cast(codes, dtype, "f32"), values=values,
+                            encoded=reference.cast(values, "f32", dtype))
+    cases = [("ragged", 13, 21, 77, "default"), ("deep", 6, 10, 2049, "default")]
+    for dtype in support.ALL_DTYPES:
+        for tag, m, n, k, kind in cases + ([("fp8", 8, 12, 300, "fp8")] if dtype[0] == "e" else []) + (
+                [("lognormal", 8, 12, 300, "lognormal")] if dtype in ("f16", "bf16") else []):
+            a = support.random_matrix(oracle, dtype, m, k, rng, kind, pad=3)
+            b = support.random_matrix(oracle, dtype, n, k, rng, kind, pad=1)
+            if dtype in support.FLOAT_DTYPES and tag == "ragged":  # hand-placed special values
+                specials = {"e4m3": [0x7F, 0x7E, 0xFE, 0x01, 0x80], "e5m2": [0x7C, 0xFC, 0x7D, 0x7B, 0x01],
+                            "f16": [0x7C00, 0xFC00, 0x7E00, 0x0001, 0x7BFF], "bf16": [0x7F80, 0xFF80, 0x7FC0, 0x0001, 0x7F7F]}[dtype]
+                a = a.copy(); b = b.copy()
+                for i, code in enumerate(specials):
+                    a[i, 5 * i + 1] = code
+                    b[2 * i + 1, 3 * i + 2] = code
+            a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+            np.savez_compressed(os.path.join(out, f"dots_{dtype}_{tag}.npz"), dtype=dtype, a=a, b=b,
+                                c_serial=reference.dots_packed(dtype, a, b),
+                                serial_packed_size=reference.packed_size(dtype, n, k))
+    print("wrote", len(os.listdir(out)) - 1, "fixtures to", out)
+
+
+if __name__ == "__main__":
+    main()

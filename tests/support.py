@@ -1,0 +1,178 @@
+"""Shared helpers for the tests: ctypes views of the oracle and of the reference library, input makers.
+
+The oracle (oracle/liboracle.so) and the reference build (oracle/_ref/libnumkong.so) are loaded here and
+only here; the product under test is numkong_amd/lib/libnumkong_amd.so.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_PATH = os.path.join(ROOT, "oracle", "liboracle.so")
+REFERENCE_PATH = os.path.join(ROOT, "oracle", "_ref", "libnumkong.so")
+GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
+
+# nk_dtype_t codes (reference: include/numkong/types.h:923-952)
+CODES = {"i8": 1 << 2, "u8": 1 << 6, "f32": 1 << 11, "f16": 1 << 12, "bf16": 1 << 13, "e4m3": 1 << 14, "e5m2": 1 << 15}
+STORAGE = {"i8": np.int8, "u8": np.uint8, "f16": np.uint16, "bf16": np.uint16, "e4m3": np.uint8, "e5m2": np.uint8}
+OUTPUT = {"i8": np.int32, "u8": np.uint32, "f16": np.float32, "bf16": np.float32, "e4m3": np.float32, "e5m2": np.float32}
+FLOAT_DTYPES = ("bf16", "f16", "e4m3", "e5m2")
+ALL_DTYPES = ("i8", "u8") + FLOAT_DTYPES
+KIND_SIZE, KIND_PACK, KIND_PACKED = ord("P"), ord("Q"), ord("G")
+CAP_SERIAL = 1
+
+_sz, _vp, _i32 = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int
+
+
+def _ptr(array: np.ndarray) -> int:
+    return array.ctypes.data
+
+
+class Oracle:
+    """This repository's CPU restatement (oracle/dots_oracle.c)."""
+
+    def __init__(self, lib: ctypes.CDLL):
+        self.lib = lib
+        lib.nko_decode.argtypes = [_i32, _vp, _sz, _vp]
+        lib.nko_encode.argtypes = [_i32, _vp, _sz, _vp]
+        lib.nko_serial_packed_size.restype = _sz
+        lib.nko_serial_packed_size.argtypes = [_i32, _sz, _sz]
+        lib.nko_serial_pack.argtypes = [_i32, _vp, _sz, _sz, _sz, _vp]
+        lib.nko_serial_packed.argtypes = [_i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
+        lib.nko_dots_f64.argtypes = [_i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
+
+    def decode(self, dtype: str, codes: np.ndarray) -> np.ndarray:
+        codes = np.ascontiguousarray(codes, dtype=STORAGE[dtype])
+        out = np.empty(codes.shape, dtype=np.float32)
+        self.lib.nko_decode(CODES[dtype], _ptr(codes), codes.size, _ptr(out))
+        return out
+
+    def encode(self, dtype: str, values: np.ndarray) -> np.ndarray:
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        out = np.empty(values.shape, dtype=STORAGE[dtype])
+        self.lib.nko_encode(CODES[dtype], _ptr(values), values.size, _ptr(out))
+        return out
+
+    def packed_size(self, dtype: str, n: int, k: int) -> int:
+        return int(self.lib.nko_serial_packed_size(CODES[dtype], n, k))
+
+    def pack(self, dtype: str, b: np.ndarray) -> np.ndarray:
+        n, k = b.shape
+        packed = np.zeros(self.packed_size(dtype, n, k), dtype=np.uint8)
+        self.lib.nko_serial_pack(CODES[dtype], _ptr(b), n, k, b.strides[0], _ptr(packed))
+        return packed
+
+    def dots_packed(self, dtype: str, a: np.ndarray, b: np.ndarray) -> np.ndarray:
+        """C = A @ B.T with the serial backend's rounding (pack + packed product)."""
+        m, k = a.shape
+        n = b.shape[0]
+        packed = self.pack(dtype, b)
+        c = np.empty((m, n), dtype=OUTPUT[dtype])
+        self.lib.nko_serial_packed(CODES[dtype], _ptr(a), _ptr(packed), _ptr(c), m, n, k, a.strides[0], c.strides[0])
+        return c
+
+    def truth(self, dtype: str, a: np.ndarray, b: np.ndarray):
+        """(f64 ground truth, sum |a*b|) as the reference's own tests compute it."""
+        m, k = a.shape
+        n = b.shape[0]
+        c = np.empty((m, n), dtype=np.float64)
+        mag = np.empty((m, n), dtype=np.float64)
+        self.lib.nko_dots_f64(CODES[dtype], _ptr(a), _ptr(b), _ptr(c), _ptr(mag), m, n, k, a.strides[0], b.strides[0])
+        return c, mag
+
+
+class Reference:
+    """The reference library built from its own sources; kernels are looked up like its bindings do."""
+
+    def __init__(self, lib: ctypes.CDLL):
+        self.lib = lib
+        lib.nk_find_kernel_punned.argtypes = [_i32, _i32, ctypes.c_uint64, ctypes.POINTER(_vp), ctypes.POINTER(ctypes.c_uint64)]
+        lib.nk_capabilities.restype = ctypes.c_uint64
+        lib.nk_cast.argtypes = [_vp, _i32, _sz, _vp, _i32]
+        lib.nk_configure_thread.argtypes = [ctypes.c_uint64]
+        self.capabilities = int(lib.nk_capabilities())
+        lib.nk_configure_thread(self.capabilities)
+
+    def kernel(self, kind: int, dtype: str, viable: int):
+        fn, cap = _vp(), ctypes.c_uint64()
+        self.lib.nk_find_kernel_punned(kind, CODES[dtype], viable, ctypes.byref(fn), ctypes.byref(cap))
+        if not fn.value or not cap.value:
+            raise RuntimeError(f"reference has no kernel kind={chr(kind)} dtype={dtype} viable={viable:#x}")
+        proto = {
+            KIND_SIZE: ctypes.CFUNCTYPE(_sz, _sz, _sz),
+            KIND_PACK: ctypes.CFUNCTYPE(None, _vp, _sz, _sz, _sz, _vp),
+            KIND_PACKED: ctypes.CFUNCTYPE(None, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz),
+        }[kind]
+        return proto(fn.value), int(cap.value)
+
+    def cast(self, values: np.ndarray, from_dtype: str, to_dtype: str, viable: int = CAP_SERIAL) -> np.ndarray:
+        """`nk_cast_serial` by default: the SIMD casts differ from it on NaN payloads and e5m2 overflow."""
+        src_np = np.float32 if from_dtype == "f32" else STORAGE[from_dtype]
+        dst_np = np.float32 if to_dtype == "f32" else STORAGE[to_dtype]
+        values = np.ascontiguousarray(values, dtype=src_np)
+        out = np.empty(values.shape, dtype=dst_np)
+        fn, cap = _vp(), ctypes.c_uint64()
+        self.lib.nk_find_kernel_punned(ord("-"), 0, viable, ctypes.byref(fn), ctypes.byref(cap))
+        if not fn.value or not cap.value:
+            raise RuntimeError("reference has no cast kernel for these capabilities")
+        cast = ctypes.CFUNCTYPE(None, _vp, _i32, _sz, _vp, _i32)(fn.value)
+        cast(_ptr(values), CODES[from_dtype], values.size, _ptr(out), CODES[to_dtype])
+        return out
+
+    def packed_size(self, dtype: str, n: int, k: int, viable: int = CAP_SERIAL) -> int:
+        return int(self.kernel(KIND_SIZE, dtype, viable)[0](n, k))
+
+    def pack(self, dtype: str, b: np.ndarray, viable: int = CAP_SERIAL) -> np.ndarray:
+        n, k = b.shape
+        packed = np.zeros(self.packed_size(dtype, n, k, viable) + 64, dtype=np.uint8)
+        self.kernel(KIND_PACK, dtype, viable)[0](_ptr(b), n, k, b.strides[0], _ptr(packed))
+        return packed
+
+    def dots_packed(self, dtype: str, a: np.ndarray, b: np.ndarray, viable: int = CAP_SERIAL) -> np.ndarray:
+        m, k = a.shape
+        n = b.shape[0]
+        packed = self.pack(dtype, b, viable)
+        c = np.empty((m, n), dtype=OUTPUT[dtype])
+        self.kernel(KIND_PACKED, dtype, viable)[0](_ptr(a), _ptr(packed), _ptr(c), m, n, k, a.strides[0], c.strides[0])
+        return c
+
+
+def load_oracle() -> Oracle:
+    if not os.path.exists(ORACLE_PATH):
+        subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), os.path.join(ROOT, "oracle", "liboracle.so")])
+    return Oracle(ctypes.CDLL(ORACLE_PATH))
+
+
+def load_reference():
+    if not os.path.exists(REFERENCE_PATH):
+        return None
+    return Reference(ctypes.CDLL(REFERENCE_PATH))
+
+
+def random_matrix(oracle: Oracle, dtype: str, rows: int, cols: int, rng: np.random.Generator, kind: str = "default",
+                  pad: int = 0) -> np.ndarray:
+    """Seeded inputs in the storage type of `dtype`; `pad` extra elements per row make strides non-trivial.
+
+    kinds: "default"  ints uniform over the full range, floats N(0,1)
+           "lognormal" floats +-exp(N(0,1))   (reference tests' family, test/test.hpp:204)
+           "fp8"       N(0,1) scaled to half of the largest finite value, 1 % exact zeros
+    """
+    shape = (rows, cols + pad)
+    if dtype == "i8":
+        full = rng.integers(-128, 128, size=shape, dtype=np.int8)
+    elif dtype == "u8":
+        full = rng.integers(0, 256, size=shape, dtype=np.uint8)
+    else:
+        z = rng.standard_normal(shape).astype(np.float32)
+        if kind == "lognormal":
+            z = (np.exp(z) * rng.choice(np.array([-1.0, 1.0], dtype=np.float32), size=shape)).astype(np.float32)
+        elif kind == "fp8":
+            z = z * np.float32(0.5 * (448.0 if dtype == "e4m3" else 57344.0))
+        full = oracle.encode(dtype, z)
+        if kind == "fp8":
+            full[rng.random(shape) < 0.01] = 0
+    return full[:, :cols] if pad else full

@@ -1,0 +1,131 @@
+"""The C-ABI boundary without a GPU: the library loads, exports what include/*.h declares, and its host
+logic (sizes, dispatch, lookup, the error convention) behaves like the reference's c/numkong.c."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import numkong_amd as nk
+from numkong_amd import api
+from tests import support
+
+INCLUDE = os.path.join(support.ROOT, "include", "numkong_amd")
+CAP_GFX950 = 1 << 62
+TYPES = ("i8", "u8", "bf16", "f16", "e4m3", "e5m2")
+
+
+def declared_symbols():
+    names = set()
+    for header in os.listdir(INCLUDE):
+        text = open(os.path.join(INCLUDE, header)).read()
+        names |= set(re.findall(r"\b(nk_(?:hip|amd)_[a-z0-9_]+)\s*\(", text))
+        names |= set(re.findall(r"NK_DYNAMIC[^;(]*?\b(nk_[a-z0-9_]+)\s*\(", text))
+        for t in TYPES:  # the backend-suffixed kernels come from a macro
+            names |= {f"nk_dots_packed_size_{t}_gfx950", f"nk_dots_pack_{t}_gfx950", f"nk_dots_packed_{t}_gfx950"}
+    return {n for n in names if "##" not in n}
+
+
+def test_library_exports_every_declared_symbol():
+    lib = nk.library()
+    names = declared_symbols()
+    assert len(names) >= 18 * 2 + 8 + 15
+    missing = [n for n in sorted(names) if not hasattr(lib, n)]
+    assert not missing, missing
+    for t in TYPES:
+        for stem in ("nk_dots_packed_size_", "nk_dots_pack_", "nk_dots_packed_"):
+            assert hasattr(lib, stem + t)
+
+
+def test_packed_size_formula():
+    """header + ceil(n/32) tiles * padded chunks * 512 B + 128 B of column terms per tile; fp8 stored as f16."""
+    for t, width in (("i8", 1), ("u8", 1), ("bf16", 2), ("f16", 2), ("e4m3", 2), ("e5m2", 2)):
+        for n, k in [(1, 1), (32, 128), (33, 129), (2048, 2048), (8191, 1000), (1048576, 768)]:
+            tiles = -(-n // 32)
+            chunks = -(-(-(-k * width // 16)) // 8) * 8
+            assert nk.dots_packed_size(t, n, k) == 64 + tiles * chunks * 512 + tiles * 128, (t, n, k)
+        assert nk.dots_packed_size(t, 0, 0) == 64
+        assert nk.dots_packed_size(t, 1 << 40, 8) == 0  # dimensions beyond 32 bits are refused, as the error stub does
+    with pytest.raises(TypeError):
+        nk.dots_packed_size("f64", 4, 4)
+
+
+def find(lib, kind, dtype_code, viable):
+    fn, cap = ctypes.c_void_p(), ctypes.c_uint64(123)
+    lib.nk_find_kernel_punned(kind, dtype_code, viable, ctypes.byref(fn), ctypes.byref(cap))
+    return fn.value, cap.value
+
+
+def test_lookup_and_capabilities():
+    lib = nk.library()
+    assert lib.nk_uses_dynamic_dispatch() == 1
+    assert lib.nk_configure_thread(ctypes.c_uint64(lib.nk_capabilities())) == 1
+    assert lib.nk_capabilities_compiled() == (1 | CAP_GFX950)
+    assert lib.nk_capabilities() & 1
+    assert lib.nk_capabilities_available() == lib.nk_capabilities() & lib.nk_capabilities_compiled()
+    for t in TYPES:
+        code = api.DTYPES[t][0]
+        for kind, stem in ((ord("P"), "nk_dots_packed_size_"), (ord("Q"), "nk_dots_pack_"), (ord("G"), "nk_dots_packed_")):
+            fn, cap = find(lib, kind, code, CAP_GFX950 | 1)
+            backend = ctypes.cast(getattr(lib, f"{stem}{t}_gfx950"), ctypes.c_void_p).value
+            assert fn == backend and cap == CAP_GFX950
+            fn, cap = find(lib, kind, code, 1)  # serial only: no kernel behind it here -> error stub, capability 0
+            assert fn and fn != backend and cap == 0
+        fn, cap = find(lib, ord("y"), code, CAP_GFX950)  # symmetric dots: not on this path
+        assert fn and cap == 0
+    assert find(lib, ord("G"), 1 << 10, CAP_GFX950) == (None, 0)  # f64: unknown dtype -> null kernel
+    out = {"i8": 1 << 4, "u8": 1 << 8, "bf16": 1 << 11, "f16": 1 << 11, "e4m3": 1 << 11, "e5m2": 1 << 11}
+    for t, expected in out.items():
+        assert lib.nk_kernel_output_dtype(ord("G"), api.DTYPES[t][0]) == expected
+    assert lib.nk_kernel_output_dtype(ord("i"), api.DTYPES["i8"][0]) == 0
+
+
+def test_error_convention_without_backend():
+    """With the table re-targeted to no capability, the entry points are the reference's error stubs:
+    size 0, pack leaves the buffer alone, the product fills exactly n*4 bytes of each C row with 0xFF."""
+    lib = nk.library()
+    try:
+        lib.nk_dispatch_table_update(0)
+        assert lib.nk_dots_packed_size_i8(5, 7) == 0
+        packed = np.full(256, 0x5A, np.uint8)
+        b = np.ones((5, 7), np.int8)
+        lib.nk_dots_pack_i8(b.ctypes.data, 5, 7, 7, packed.ctypes.data)
+        assert (packed == 0x5A).all()
+        c = np.zeros((3, 8), np.int32)
+        a = np.ones((3, 7), np.int8)
+        lib.nk_dots_packed_i8(a.ctypes.data, packed.ctypes.data, c.ctypes.data, 3, 5, 7, 7, 32)
+        assert (c[:, :5] == -1).all() and (c[:, 5:] == 0).all()
+        f = np.zeros((2, 4), np.float32)
+        lib.nk_dots_packed_bf16(a.ctypes.data, packed.ctypes.data, f.ctypes.data, 2, 3, 2, 4, 16)
+        assert np.isnan(f[:, :3]).all() and (f[:, 3] == 0).all()
+    finally:
+        lib.nk_dispatch_table_update(lib.nk_capabilities_compiled())
+    assert lib.nk_dots_packed_size_i8(5, 7) == 64 + 8 * 512 + 128
+
+
+def test_no_gpu_means_loud_failure_not_fallback():
+    lib = nk.library()
+    if lib.nk_hip_device_count() > 0:
+        pytest.skip("a GPU is present")
+    a = np.ones((2, 16), np.int8)
+    packed = np.zeros(nk.dots_packed_size("i8", 2, 16), np.uint8)
+    lib.nk_dots_pack_i8(a.ctypes.data, 2, 16, 16, packed.ctypes.data)
+    assert b"no HIP device" in lib.nk_amd_last_error()
+    c = np.zeros((2, 2), np.int32)
+    lib.nk_dots_packed_i8(a.ctypes.data, packed.ctypes.data, c.ctypes.data, 2, 2, 16, 16, 8)
+    assert (c == -1).all() and b"no HIP device" in lib.nk_amd_last_error()
+
+
+def test_python_mirror_validates_arguments():
+    import torch
+
+    cpu = torch.zeros(4, 4, dtype=torch.int8)
+    with pytest.raises(ValueError):
+        nk.dots_pack(cpu, "i8")  # must live on the GPU
+    with pytest.raises(TypeError):
+        nk.dots_pack(cpu, "i4")
+    with pytest.raises(TypeError):
+        nk.dots_pack([[1, 2]], "i8")
+    with pytest.raises(TypeError):
+        nk.dots_packed(cpu, object())

@@ -1,0 +1,257 @@
+"""Parity of the gfx950 kernels with the reference semantics, through the C ABI, on a real MI355X.
+
+Integers must be bit-exact (the reference's integer backends all equal the exact product mod 2^32).
+Floats are compared with the f64 ground truth next to the reference's serial kernel as restated by the
+oracle (which tests/test_oracle.py pins bit-for-bit against the reference library):
+
+  normwise error  e = |c - truth| / sum|a*b|   per element, over elements with a finite truth
+  gate:  mean(e_gpu) <= 2 * mean(e_serial)                 (plus 1e-3 ulp of slack when both are ~0)
+         max(e_gpu)  <= 2 * max(max(e_serial), 2^-24)      (one f32 rounding unit of the magnitude sum)
+         NaN, +Inf and -Inf masks identical to the serial kernel's.
+
+The 2^-24 floor keeps the max statistic meaningful on small samples, where both kernels sit at a single
+rounding of the result, and it is what decides e4m3 at depth 8192: there the serial kernel's lane sums stay
+exact far longer than the MFMA's accumulator (one rounding per 8 products at the magnitude of the whole
+running sum), 8e-9 against 3e-8 measured, both far below the floor.
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+import numkong_amd as nk  # noqa: E402
+from numkong_amd import api  # noqa: E402
+from tests import support  # noqa: E402
+from tests.support import ALL_DTYPES, FLOAT_DTYPES, OUTPUT  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+U = 2.0**-24
+
+
+def to_gpu(array):
+    a = np.ascontiguousarray(array)
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.int16)).to(DEV)
+    return torch.from_numpy(a).to(DEV)
+
+
+def gpu_dots(dtype, a, b, config=0):
+    nk.library().nk_hip_set_tile_config(config)
+    try:
+        packed = nk.dots_pack(to_gpu(b), dtype)
+        c = nk.dots_packed(to_gpu(a), packed)
+    finally:
+        nk.library().nk_hip_set_tile_config(0)
+    out = c.cpu().numpy()
+    return out.view(np.uint32) if dtype == "u8" else out
+
+
+def assert_float_gate(dtype, got, serial, truth, magnitude, where=""):
+    assert np.array_equal(np.isnan(got), np.isnan(serial)), f"NaN mask differs {where}"
+    assert np.array_equal(np.isposinf(got), np.isposinf(serial)), f"+Inf mask differs {where}"
+    assert np.array_equal(np.isneginf(got), np.isneginf(serial)), f"-Inf mask differs {where}"
+    finite = np.isfinite(truth) & (magnitude > 0)
+    if not finite.any():
+        return
+    e_gpu = np.abs(got[finite].astype(np.float64) - truth[finite]) / magnitude[finite]
+    e_ref = np.abs(serial[finite].astype(np.float64) - truth[finite]) / magnitude[finite]
+    assert e_gpu.mean() <= 2 * e_ref.mean() + 1e-3 * U, f"mean error {e_gpu.mean():.3e} vs serial {e_ref.mean():.3e} {where}"
+    assert e_gpu.max() <= 2 * max(e_ref.max(), U), f"max error {e_gpu.max():.3e} vs serial {e_ref.max():.3e} {where}"
+
+
+def check(oracle, dtype, a, b, config=0, where=""):
+    got = gpu_dots(dtype, a, b, config)
+    if dtype in ("i8", "u8"):
+        exact = (a.astype(np.int64) @ b.astype(np.int64).T) & 0xFFFFFFFF
+        assert np.array_equal(got.astype(np.int64) & 0xFFFFFFFF, exact), where
+        assert np.array_equal(got.view(np.uint32), oracle.dots_packed(dtype, a, b).view(np.uint32)), where
+    else:
+        truth, magnitude = oracle.truth(dtype, a, b)
+        assert_float_gate(dtype, got, oracle.dots_packed(dtype, a, b), truth, magnitude, where)
+
+
+SHAPES = [(1, 1, 1), (3, 5, 7), (33, 70, 200), (64, 64, 64), (100, 37, 333), (257, 129, 1000), (31, 300, 129), (130, 33, 4100)]
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("config", [0, 1, 2, 3, 4])
+def test_small_shapes_every_tile_config(oracle, dtype, config):
+    rng = np.random.default_rng(100 + config)
+    for m, n, k in SHAPES:
+        a = support.random_matrix(oracle, dtype, m, k, rng)
+        b = support.random_matrix(oracle, dtype, n, k, rng)
+        check(oracle, dtype, a, b, config, f"{dtype} {m}x{n}x{k} config {config}")
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+def test_float_input_families(oracle, dtype):
+    rng = np.random.default_rng(5)
+    kinds = ["lognormal"] + (["fp8"] if dtype[0] == "e" else [])
+    for kind in kinds:
+        for m, n, k in [(48, 80, 1536), (64, 96, 8192)]:
+            a = support.random_matrix(oracle, dtype, m, k, rng, kind)
+            b = support.random_matrix(oracle, dtype, n, k, rng, kind)
+            check(oracle, dtype, a, b, 0, f"{dtype} {kind} {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("name", sorted(f for f in os.listdir(support.GOLDEN_DIR) if f.startswith("dots_")))
+def test_golden_vectors(oracle, name):
+    """Inputs and serial-kernel outputs recorded from the reference library, special values included."""
+    data = np.load(os.path.join(support.GOLDEN_DIR, name))
+    dtype, a, b, c_serial = str(data["dtype"]), data["a"], data["b"], data["c_serial"]
+    got = gpu_dots(dtype, a, b)
+    if dtype in ("i8", "u8"):
+        assert np.array_equal(got.view(np.uint32), c_serial.view(np.uint32))
+    else:
+        truth, magnitude = oracle.truth(dtype, a, b)
+        assert_float_gate(dtype, got, c_serial, truth, magnitude, name)
+
+
+@pytest.mark.parametrize("dtype", ["e4m3", "e5m2"])
+def test_every_fp8_code_decodes_exactly(oracle, dtype):
+    """code * 1.0 through both operand paths (A is widened on its way into LDS, B when it is packed)."""
+    codes = np.arange(256, dtype=np.uint8)
+    expected = oracle.decode(dtype, codes)
+    one = oracle.encode(dtype, np.array([1.0], np.float32))[0]
+    for k in (1, 16, 100):
+        a = np.zeros((256, k), np.uint8)
+        a[:, k - 1] = codes
+        b = np.zeros((3, k), np.uint8)
+        b[:, k - 1] = one
+        for got in (gpu_dots(dtype, a, b)[:, 1], gpu_dots(dtype, b, a)[1, :]):
+            nan = np.isnan(expected)
+            assert np.array_equal(np.isnan(got), nan) and np.array_equal(got[~nan], expected[~nan])
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_subnormals_are_not_flushed(oracle, dtype):
+    tiny = np.array([[1, 2, 3, 0x8001]], np.uint16)  # smallest subnormals
+    big = oracle.encode(dtype, np.array([[1.0, 1.0, 1.0, 2.0]], np.float32))
+    expected = oracle.dots_packed(dtype, tiny, big)
+    assert expected[0, 0] != 0
+    assert np.array_equal(gpu_dots(dtype, tiny, big), expected)
+    assert np.array_equal(gpu_dots(dtype, big, tiny), expected)
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_strides_alignment_and_untouched_padding(oracle, dtype):
+    """Row strides larger than the row, A not 16-byte aligned, C rows wider than n: only m x n is written."""
+    rng = np.random.default_rng(9)
+    lib = nk.library()
+    for m, n, k, pad_a, pad_b, pad_c, skew in [(37, 29, 1000, 13, 7, 3, 1), (64, 130, 63, 3, 0, 5, 0), (5, 130, 2049, 1, 1, 0, 3)]:
+        a_full = support.random_matrix(oracle, dtype, m, k + pad_a + skew, rng)
+        b_full = support.random_matrix(oracle, dtype, n, k + pad_b, rng)
+        a, b = a_full[:, skew:skew + k], b_full[:, :k]
+        ga, gb = to_gpu(a_full), to_gpu(b_full)
+        packed = torch.empty(nk.dots_packed_size(dtype, n, k), dtype=torch.uint8, device=DEV)
+        c = torch.full((m, n + pad_c), 0x5A5A5A5A, dtype=torch.int32, device=DEV)
+        width = a_full.itemsize
+        getattr(lib, f"nk_dots_pack_{dtype}")(gb.data_ptr(), n, k, b_full.shape[1] * width, packed.data_ptr())
+        assert not lib.nk_amd_last_error()
+        getattr(lib, f"nk_dots_packed_{dtype}")(ga.data_ptr() + skew * width, packed.data_ptr(), c.data_ptr(), m, n, k,
+                                               a_full.shape[1] * width, (n + pad_c) * 4)
+        assert not lib.nk_amd_last_error()
+        out = c.cpu().numpy()
+        assert (out[:, n:] == 0x5A5A5A5A).all()
+        got = np.ascontiguousarray(out[:, :n]).view(OUTPUT[dtype])
+        if dtype in ("i8", "u8"):
+            assert np.array_equal(got.view(np.uint32), oracle.dots_packed(dtype, a, b).view(np.uint32))
+        else:
+            truth, magnitude = oracle.truth(dtype, a, b)
+            assert_float_gate(dtype, got, oracle.dots_packed(dtype, a, b), truth, magnitude)
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_host_pointers_are_staged(oracle, dtype):
+    """The reference API takes plain host pointers; so does this one (staged through device buffers)."""
+    rng = np.random.default_rng(21)
+    lib = nk.library()
+    m, n, k = 19, 45, 300
+    a = support.random_matrix(oracle, dtype, m, k, rng, pad=2)
+    b = support.random_matrix(oracle, dtype, n, k, rng, pad=4)
+    packed = np.zeros(nk.dots_packed_size(dtype, n, k), np.uint8)
+    c = np.full((m, n + 2), 7, OUTPUT[dtype])
+    getattr(lib, f"nk_dots_pack_{dtype}")(a.ctypes.data * 0 + b.ctypes.data, n, k, b.strides[0], packed.ctypes.data)
+    assert not lib.nk_amd_last_error()
+    getattr(lib, f"nk_dots_packed_{dtype}")(a.ctypes.data, packed.ctypes.data, c.ctypes.data, m, n, k, a.strides[0], c.strides[0])
+    assert not lib.nk_amd_last_error()
+    assert (c[:, n:] == 7).all()
+    device = gpu_dots(dtype, a, b)
+    assert np.array_equal(np.ascontiguousarray(c[:, :n]).view(np.uint32), device.view(np.uint32))  # same kernel, same bits
+    # a packed image is relocatable bytes: device image == host image
+    image = nk.dots_pack(to_gpu(b), dtype).buffer.cpu().numpy()
+    assert np.array_equal(image, packed)
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_packed_image_layout(oracle, dtype):
+    """header | tiles[(t * k_chunks + c) * 32 + r] of 16 bytes | 128 * sum(b ^ 0x80 as i8) per column (u8)."""
+    rng = np.random.default_rng(33)
+    n, k = 70, 203
+    b = support.random_matrix(oracle, dtype, n, k, rng)
+    image = nk.dots_pack(to_gpu(b), dtype).buffer.cpu().numpy()
+    header = image[:64].view(np.uint32)
+    if dtype in ("e4m3", "e5m2"):  # stored widened to f16, exactly
+        rows = oracle.encode("f16", oracle.decode(dtype, b)).view(np.uint8).reshape(n, -1)
+    elif dtype == "u8":
+        rows = b ^ 0x80
+    else:
+        rows = np.ascontiguousarray(b).view(np.uint8).reshape(n, -1)
+    row_bytes = rows.shape[1]
+    chunks = -(-(-(-row_bytes // 16)) // 8) * 8
+    tiles = -(-n // 32)
+    assert header[0] == 0x35394B4E and header[2] == api.DTYPES[dtype][0] and header[3] == row_bytes // k
+    assert (header[4], header[5], header[6], header[7]) == (n, k, tiles, chunks)
+    padded = np.zeros((tiles * 32, chunks * 16), np.uint8)
+    padded[:n, :row_bytes] = rows
+    expected = padded.reshape(tiles, 32, chunks, 16).transpose(0, 2, 1, 3).reshape(-1)
+    data = image[64:64 + expected.size]
+    assert np.array_equal(data, expected)
+    terms = image[64 + expected.size:].view(np.uint32)
+    assert terms.size == tiles * 32
+    if dtype == "u8":
+        sums = (b.astype(np.int64) - 128).sum(axis=1) * 128
+        assert np.array_equal(terms[:n].astype(np.int64), sums & 0xFFFFFFFF) and (terms[n:] == 0).all()
+    else:
+        assert (terms == 0).all()
+
+
+def test_mismatched_image_poisons_output_and_zero_sizes(oracle):
+    lib = nk.library()
+    b = to_gpu(np.ones((40, 64), np.int8))
+    packed = nk.dots_pack(b, "i8")
+    a = to_gpu(np.ones((8, 64), np.int8))
+    c = torch.zeros((8, 40), dtype=torch.int32, device=DEV)
+    # wrong dtype for this image, and wrong depth: every output becomes 0xFFFFFFFF, nothing else is touched
+    lib.nk_dots_packed_u8(a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(), 8, 40, 64, 64, 160)
+    assert (c.cpu().numpy() == -1).all()
+    c.zero_()
+    lib.nk_dots_packed_i8(a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(), 8, 40, 48, 64, 160)
+    assert (c.cpu().numpy() == -1).all()
+    # m = 0 or n = 0: nothing happens; k = 0: C is zeroed (the reference zeroes C and adds nothing)
+    c.fill_(5)
+    lib.nk_dots_packed_i8(a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(), 0, 40, 64, 64, 160)
+    assert (c.cpu().numpy() == 5).all()
+    empty = torch.zeros(nk.dots_packed_size("i8", 40, 0), dtype=torch.uint8, device=DEV)
+    lib.nk_dots_pack_i8(b.data_ptr(), 40, 0, 64, empty.data_ptr())
+    lib.nk_dots_packed_i8(a.data_ptr(), empty.data_ptr(), c.data_ptr(), 8, 40, 0, 64, 160)
+    assert not lib.nk_amd_last_error() and (c.cpu().numpy() == 0).all()
+
+
+def test_python_mirror_out_argument(oracle):
+    rng = np.random.default_rng(2)
+    a = to_gpu(support.random_matrix(oracle, "bf16", 70, 128, rng))
+    packed = nk.dots_pack(to_gpu(support.random_matrix(oracle, "bf16", 50, 128, rng)), "bf16")
+    fresh = nk.dots_packed(a, packed)
+    out = torch.zeros_like(fresh)
+    assert nk.dots_packed(a, packed, out=out) is out and torch.equal(out, fresh)
+    with pytest.raises(ValueError):
+        nk.dots_packed(a[:, :64], packed)
+    with pytest.raises(ValueError):
+        nk.dots_packed(a, packed, out=torch.zeros(70, 51, device=DEV))
+    with pytest.raises(TypeError):
+        nk.dots_packed(a, packed, out=torch.zeros(70, 50, dtype=torch.int32, device=DEV))

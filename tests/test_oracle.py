@@ -1,0 +1,204 @@
+"""Pins the CPU oracle (oracle/dots_oracle.c) before anything is compared with it.
+
+Checks, in the order of strength:
+  * against the reference library compiled from its own sources (oracle/_ref), when it was built:
+    `nk_cast_serial` for all conversions, `nk_dots_*_serial` for sizes, packed bytes and products, bit for bit;
+  * against vectors committed under tests/golden (made from that library by tests/golden/make_golden.py),
+    so the same facts hold where the reference is absent;
+  * against independent library routines: torch's float8_e4m3fn / float8_e5m2 / float16 / bfloat16 decoders;
+  * against what arithmetic fixes: the 428-byte packed-size example (64 + 7*48 + 7*4), exact integer
+    products from numpy int64, powers of two, f64 matmul of decoded inputs.
+NaN payloads are never compared: the reference's own cast backends disagree on them.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from tests import support
+from tests.support import ALL_DTYPES, FLOAT_DTYPES, STORAGE
+
+
+def same_floats(x, y):
+    x, y = np.asarray(x), np.asarray(y)
+    nan = np.isnan(x)
+    return np.array_equal(nan, np.isnan(y)) and np.array_equal(x[~nan].view(np.uint32), y[~nan].view(np.uint32))
+
+
+def all_codes(dtype):
+    return np.arange(256 if STORAGE[dtype] == np.uint8 else 65536).astype(STORAGE[dtype])
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+def test_decode_matches_torch(oracle, dtype):
+    import torch
+
+    torch_dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "e4m3": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2}[dtype]
+    codes = all_codes(dtype)
+    view = torch.from_numpy(codes.view(np.int16) if codes.itemsize == 2 else codes).view(torch_dtype)
+    assert same_floats(oracle.decode(dtype, codes), view.to(torch.float32).numpy())
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+def test_decode_closed_form(oracle, dtype):
+    """value = (-1)^s * 2^(e-bias) * (1 + m / 2^mbits), subnormals m * 2^(1-bias-mbits), in Python floats."""
+    ebits, mbits, bias = {"bf16": (8, 7, 127), "f16": (5, 10, 15), "e4m3": (4, 3, 7), "e5m2": (5, 2, 15)}[dtype]
+    codes = all_codes(dtype)
+    got = oracle.decode(dtype, codes)
+    for code in codes[:: max(1, len(codes) // 4096)].tolist() + [0, 1, len(codes) // 2 - 1, len(codes) - 1]:
+        s, e, m = code >> (ebits + mbits), (code >> mbits) & ((1 << ebits) - 1), code & ((1 << mbits) - 1)
+        if e == (1 << ebits) - 1 and dtype != "e4m3":
+            expected = float("nan") if m else float("inf")
+        elif dtype == "e4m3" and e == 15 and m == 7:
+            expected = float("nan")
+        elif e == 0:
+            expected = m * 2.0 ** (1 - bias - mbits)
+        else:
+            expected = (1 + m / 2.0**mbits) * 2.0 ** (e - bias)
+        expected = -expected if s else expected
+        assert (np.isnan(got[code]) and np.isnan(expected)) or float(got[code]) == expected, hex(code)
+
+
+def _encode_probe_values(oracle, dtype):
+    rng = np.random.default_rng(1)
+    scales = [1e-8, 1e-6, 1e-3, 1, 100, 1e4, 1e6]
+    values = [rng.standard_normal(20000).astype(np.float32) * np.float32(s) for s in scales]
+    values.append(np.array([0, -0.0, np.inf, -np.inf, np.nan, 448, 449, 464, 465, 480, 57344, 61439.9, 61440, 65504,
+                            65519.9, 65520, 2.0**-9, 2.0**-10, 1.5 * 2.0**-10, 2.0**-16, 2.0**-17, 1.5 * 2.0**-17,
+                            2.0**-24, 2.0**-25, 1.0001 * 2.0**-25, 1e-40, 3e38], dtype=np.float32))
+    grid = np.sort(oracle.decode(dtype, all_codes(dtype)[: len(all_codes(dtype)) // 2]))
+    grid = grid[np.isfinite(grid)]
+    if len(grid) > 4096:
+        grid = grid[:: len(grid) // 4096]
+    mids = ((grid[:-1].astype(np.float64) + grid[1:]) / 2).astype(np.float32)
+    edge = np.concatenate([grid, mids, np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf))])
+    values += [edge, -edge]
+    return np.concatenate(values)
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+def test_conversions_match_reference_serial(oracle, reference, dtype):
+    codes = all_codes(dtype)
+    assert same_floats(oracle.decode(dtype, codes), reference.cast(codes, dtype, "f32"))
+    values = _encode_probe_values(oracle, dtype)
+    assert np.array_equal(oracle.encode(dtype, values), reference.cast(values, "f32", dtype))
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+def test_encode_round_trip_and_ties(oracle, dtype):
+    """Every finite code encodes back to itself; exact midpoints go to the even neighbour; policies on overflow."""
+    codes = all_codes(dtype)
+    values = oracle.decode(dtype, codes)
+    finite = np.isfinite(values)
+    assert np.array_equal(oracle.encode(dtype, values[finite]), codes[finite])
+    half = codes[: len(codes) // 2]
+    grid = oracle.decode(dtype, half)
+    keep = np.isfinite(grid)
+    grid, half = grid[keep], half[keep]
+    mids = (grid[:-1].astype(np.float64) + grid[1:].astype(np.float64)) / 2
+    exact = mids.astype(np.float32).astype(np.float64) == mids
+    encoded = oracle.encode(dtype, mids[exact].astype(np.float32))
+    lower, upper = half[:-1][exact], half[1:][exact]
+    assert np.array_equal(encoded, np.where(lower % 2 == 0, lower, upper))
+    big = np.array([1e30, -1e30, np.inf, -np.inf], dtype=np.float32)
+    expected = {"e4m3": [0x7E, 0xFE, 0x7E, 0xFE], "e5m2": [0x7C, 0xFC, 0x7C, 0xFC], "f16": [0x7C00, 0xFC00, 0x7C00, 0xFC00],
+                "bf16": [0x7149, 0xF149, 0x7F80, 0xFF80]}[dtype]  # bf16: 1e30 is finite in bf16
+    got = oracle.encode(dtype, big).tolist()
+    if dtype == "bf16":
+        assert got[2:] == expected[2:] and abs(float(oracle.decode(dtype, np.array(got[:1], np.uint16))[0]) / 1e30 - 1) < 1e-2
+    else:
+        assert got == expected
+    assert np.isnan(oracle.decode(dtype, oracle.encode(dtype, np.array([np.nan], np.float32)))).all()
+
+
+def test_packed_size_known_answers(oracle):
+    # reference layout: 64 + n * padded_depth * width + n * 4; depth padded to 16 (i8), 8 (bf16), 4 (f16 as f32)
+    assert oracle.packed_size("i8", 7, 37) == 64 + 7 * 48 + 7 * 4 == 428
+    assert oracle.packed_size("i8", 2048, 2048) == 64 + 2048 * (2048 + 16) + 2048 * 4  # power-of-two stride is broken up
+    assert oracle.packed_size("bf16", 4096, 4096) == 64 + 4096 * (4096 + 8) * 2 + 4096 * 4
+    assert oracle.packed_size("f16", 3, 5) == 64 + 3 * (8 + 4) * 4 + 3 * 4  # 5 -> 8 f32 values = 32 B, a power of two -> +4 values
+    assert oracle.packed_size("e4m3", 10, 1000) == 64 + 10 * 1008 + 40
+
+
+SHAPES = [(5, 7, 37, 0, 0), (33, 29, 1000, 13, 7), (64, 64, 64, 0, 0), (1, 1, 1, 0, 0), (16, 130, 63, 3, 0),
+          (37, 48, 2049, 0, 5), (8, 8, 4096, 0, 0)]
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_serial_layout_and_product_match_reference(oracle, reference, dtype):
+    rng = np.random.default_rng(7)
+    for n, k in [(1, 1), (7, 37), (128, 1536), (5, 64), (3, 128), (9, 4096), (4, 2048), (2, 1000), (17, 8192)]:
+        assert oracle.packed_size(dtype, n, k) == reference.packed_size(dtype, n, k)
+    kinds = ["default"] if dtype in ("i8", "u8") else ["default", "lognormal"] + (["fp8"] if dtype[0] == "e" else [])
+    for m, n, k, pad_a, pad_b in SHAPES:
+        for kind in kinds:
+            a = support.random_matrix(oracle, dtype, m, k, rng, kind, pad_a)
+            b = support.random_matrix(oracle, dtype, n, k, rng, kind, pad_b)
+            mine, theirs = oracle.pack(dtype, b), reference.pack(dtype, b)
+            padded = int(mine[8:12].view(np.uint32)[0])
+            body = 64 + n * padded * (4 if dtype == "f16" else a.itemsize)
+            assert np.array_equal(mine[:body], theirs[:body])
+            if dtype in ("i8", "u8"):
+                assert np.array_equal(mine, theirs[: len(mine)])  # integer norms too
+            assert same_floats(oracle.dots_packed(dtype, a, b).view(np.float32), reference.dots_packed(dtype, a, b).view(np.float32))
+
+
+@pytest.mark.parametrize("dtype", ["i8", "u8"])
+def test_integer_product_closed_form(oracle, dtype):
+    rng = np.random.default_rng(11)
+    for m, n, k, pad_a, pad_b in SHAPES + [(3, 5, 70000, 0, 0)]:
+        a = support.random_matrix(oracle, dtype, m, k, rng, pad=pad_a)
+        b = support.random_matrix(oracle, dtype, n, k, rng, pad=pad_b)
+        exact = a.astype(np.int64) @ b.astype(np.int64).T
+        assert np.array_equal(oracle.dots_packed(dtype, a, b).astype(np.int64) & 0xFFFFFFFF, exact & 0xFFFFFFFF)
+    # extremes: every product is (-128)^2 or 255^2
+    k = 4096
+    a = np.full((2, k), -128 if dtype == "i8" else 255, dtype=STORAGE[dtype])
+    assert int(oracle.dots_packed(dtype, a, a)[0, 0]) == k * (16384 if dtype == "i8" else 65025)
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+def test_float_product_properties(oracle, dtype):
+    rng = np.random.default_rng(13)
+    a = support.random_matrix(oracle, dtype, 9, 333, rng)
+    b = support.random_matrix(oracle, dtype, 11, 333, rng)
+    truth, magnitude = oracle.truth(dtype, a, b)
+    decoded = lambda x: oracle.decode(dtype, np.ascontiguousarray(x)).astype(np.float64)
+    assert np.allclose(truth, decoded(a) @ decoded(b).T, rtol=0, atol=1e-12 * magnitude.max())
+    assert np.allclose(magnitude, np.abs(decoded(a)) @ np.abs(decoded(b)).T, rtol=1e-12)
+    serial = oracle.dots_packed(dtype, a, b)
+    assert np.all(np.abs(serial - truth) <= 333 * 2.0**-24 * magnitude)  # f32 accumulation stays within k ulps
+    # powers of two sum exactly: a = b = 2^-3 everywhere -> k / 64
+    one_eighth = oracle.encode(dtype, np.full((2, 256), 0.125, np.float32))
+    assert np.all(oracle.dots_packed(dtype, one_eighth, one_eighth) == 4.0)
+    # a dropped k-tail or a transposed operand would break this asymmetric case
+    a2 = oracle.encode(dtype, np.arange(1, 7, dtype=np.float32).reshape(2, 3))
+    b2 = oracle.encode(dtype, np.array([[1, 0, 0], [0, 1, 0], [0, 0, 1], [1, 1, 1]], np.float32))
+    assert np.array_equal(oracle.dots_packed(dtype, a2, b2), np.array([[1, 2, 3, 6], [4, 5, 6, 15]], np.float32))
+
+
+def test_special_values_follow_ieee(oracle):
+    enc = lambda dtype, *v: oracle.encode(dtype, np.array([v], np.float32))
+    for dtype in ("f16", "bf16", "e5m2"):
+        inf_one, zero_one, one_one = enc(dtype, np.inf, 1), enc(dtype, 0, 1), enc(dtype, 1, 1)
+        assert oracle.dots_packed(dtype, inf_one, one_one)[0, 0] == np.inf
+        assert np.isnan(oracle.dots_packed(dtype, inf_one, zero_one)[0, 0])  # inf * 0
+        assert np.isnan(oracle.dots_packed(dtype, enc(dtype, np.inf, -np.inf), one_one)[0, 0])  # inf - inf
+    assert np.isnan(oracle.dots_packed("e4m3", enc("e4m3", np.nan, 1), enc("e4m3", 1, 1))[0, 0])
+    assert oracle.dots_packed("e4m3", enc("e4m3", np.inf, 0), enc("e4m3", 1, 1))[0, 0] == 448.0  # saturating encoder
+
+
+@pytest.mark.parametrize("name", sorted(f for f in os.listdir(support.GOLDEN_DIR) if f.endswith(".npz")) if os.path.isdir(support.GOLDEN_DIR) else [])
+def test_golden_vectors(oracle, name):
+    """Vectors written from the reference's serial kernels; hold with or without the reference checkout."""
+    data = np.load(os.path.join(support.GOLDEN_DIR, name))
+    if name.startswith("cast_"):
+        dtype = str(data["dtype"])
+        assert same_floats(oracle.decode(dtype, data["codes"]), data["decoded"])
+        assert np.array_equal(oracle.encode(dtype, data["values"]), data["encoded"])
+    else:
+        dtype = str(data["dtype"])
+        a, b = data["a"], data["b"]
+        assert oracle.packed_size(dtype, b.shape[0], b.shape[1]) == int(data["serial_packed_size"])
+        got = oracle.dots_packed(dtype, a, b)
+        assert same_floats(got.view(np.float32), data["c_serial"].view(np.float32))
