@@ -1,0 +1,211 @@
+"""Throughput of the packed batched-dots path on one MI355X, with its roofline and a CPU baseline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype i8] [--shape M N K] [--no-others] [--no-cpu]
+
+One "step" is one packed product C = A * B^T over one synthetic batch (B is packed once, before the timed
+region, as the reference's own benchmark does: bench/bench.hpp:238-255). The headline workload is the
+i8 -> i32 product at M = N = K = 8192; bf16 and e4m3 at the same shape and the HBM-bound retrieval shape
+(1024 queries x 1,048,576 vectors x 768) are measured the same way and reported under "others".
+gso/s = 2*M*N*K / seconds / 1e9 (bench/bench.hpp:257). All operands are resident in HBM before timing.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import queue
+import sys
+import threading
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published dense peaks, in T(FL)OP/s, for the MFMA the dtype runs on; HBM3E in GB/s.
+MFMA_PEAK = {"i8": 5000.0, "u8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "e4m3": 2500.0, "e5m2": 2500.0}
+MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2": "widened to f16, priced against the f16 MFMA peak"}
+HBM_PEAK = 8000.0
+HEADLINE = ("i8", 8192, 8192, 8192)
+OTHERS = [("bf16", 8192, 8192, 8192), ("e4m3", 8192, 8192, 8192), ("i8", 1024, 1 << 20, 768)]
+
+
+def make_operands(dtype, m, n, k, seed=42):
+    """Synthetic inputs of BASELINE's families, generated on the GPU: ints uniform over the full range,
+    bf16/f16 N(0,1), fp8 N(0,1) scaled to half the largest finite value with 1 % zeros."""
+    import torch
+
+    g = torch.Generator(device="cuda:0").manual_seed(seed)
+    def one(rows):
+        if dtype == "i8":
+            return torch.randint(-128, 128, (rows, k), dtype=torch.int8, device="cuda:0", generator=g)
+        if dtype == "u8":
+            return torch.randint(0, 256, (rows, k), dtype=torch.uint8, device="cuda:0", generator=g)
+        z = torch.randn((rows, k), device="cuda:0", generator=g)
+        if dtype == "bf16":
+            return z.to(torch.bfloat16).view(torch.int16)
+        if dtype == "f16":
+            return z.to(torch.float16).view(torch.int16)
+        top = 448.0 if dtype == "e4m3" else 57344.0
+        z = (z * (0.5 * top)).clamp(-top, top)  # torch's cast has no saturation: clamp first
+        z = z * (torch.rand((rows, k), device="cuda:0", generator=g) >= 0.01)
+        return z.to(torch.float8_e4m3fn if dtype == "e4m3" else torch.float8_e5m2).view(torch.uint8)
+    return one(m), one(n)
+
+
+def time_gpu(dtype, m, n, k, steps, warmup):
+    import torch
+
+    import numkong_amd as nk
+    from numkong_amd import api
+
+    lib = nk.library()
+    a, b = make_operands(dtype, m, n, k)
+    packed = nk.dots_pack(b, dtype)
+    del b
+    c = torch.empty((m, n), dtype=torch.int32 if dtype in ("i8", "u8") else torch.float32, device="cuda:0")
+    code, width = api.DTYPES[dtype][0], api.DTYPES[dtype][1]
+    stream = torch.cuda.current_stream().cuda_stream  # the kernel is launched on this stream, so torch events see it
+
+    def step():
+        status = lib.nk_amd_dots_packed_async(code, a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(), m, n, k,
+                                              k * width, n * 4, stream)
+        if status:
+            raise RuntimeError(lib.nk_hip_last_error().decode())
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    wall = time.perf_counter()
+    begin.record()
+    for _ in range(steps):
+        step()
+    end.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - wall) * 1e3 / steps
+    device_ms = begin.elapsed_time(end) / steps
+    ops = 2.0 * m * n * k
+    result = {"ms_per_step": wall, "kernel_ms": device_ms, "gso_per_s": ops / (wall * 1e-3) / 1e9}
+    if m * n >= 64 * k * 8 and dtype in ("i8", "u8") and n >= 1 << 18:  # retrieval shape: HBM-bound on C and the packed stream
+        algorithmic = (m * k + n * k) * width + m * n * 4
+        result["roofline"] = {"bound": "hbm", "achieved": algorithmic / (device_ms * 1e-3) / 1e9, "peak": HBM_PEAK,
+                              "unit": "GB/s", "frac": algorithmic / (device_ms * 1e-3) / 1e9 / HBM_PEAK, "traffic": None}
+    else:
+        achieved = ops / (device_ms * 1e-3) / 1e12
+        result["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK[dtype], "unit": "TFLOP/s",
+                              "frac": achieved / MFMA_PEAK[dtype], "traffic": None}
+        if dtype in MFMA_NOTE:
+            result["roofline"]["note"] = MFMA_NOTE[dtype]
+    del a, packed, c
+    torch.cuda.empty_cache()
+    return result
+
+
+def cpu_baseline(dtype, m, n, k, budget_rows=2048):
+    """The reference's own dots path on the host cores: B packed once, A split into 64-row tiles handed out
+    dynamically to one thread per core (python/matrix.c:466-483, python/matrix.h:18), best-dispatch kernel.
+    Falls back to this repository's scalar oracle on a smaller sample if the reference build is absent."""
+    import numpy as np
+
+    from tests import support
+
+    oracle = support.load_oracle()
+    reference = support.load_reference()
+    rng = np.random.default_rng(42)
+    cores = max(1, min(16, len(os.sched_getaffinity(0))))
+    if reference is None:
+        rows, cols = 16, min(n, 256)
+        a = support.random_matrix(oracle, dtype, rows, k, rng)
+        b = support.random_matrix(oracle, dtype, cols, k, rng)
+        start = time.perf_counter()
+        oracle.dots_packed(dtype, a, b)
+        seconds = time.perf_counter() - start
+        return {"value": 2.0 * rows * cols * k / seconds / 1e9, "unit": "gso/s", "cores": 1, "kind": "port",
+                "sample": f"{rows} x {cols} x {k} of the workload, scalar restatement (reference build not present)"}
+    rows = min(m, budget_rows)
+    a = support.random_matrix(oracle, dtype, rows, k, rng)
+    b = support.random_matrix(oracle, dtype, min(n, 8192), k, rng)
+    cols = b.shape[0]
+    viable = reference.capabilities
+    size_fn, _ = reference.kernel(support.KIND_SIZE, dtype, viable)
+    pack_fn, _ = reference.kernel(support.KIND_PACK, dtype, viable)
+    dots_fn, used = reference.kernel(support.KIND_PACKED, dtype, viable)
+    packed = np.zeros(int(size_fn(cols, k)) + 64, np.uint8)
+    pack_fn(b.ctypes.data, cols, k, b.strides[0], packed.ctypes.data)
+    c = np.empty((rows, cols), support.OUTPUT[dtype])
+    tile = 64
+
+    def run_once():
+        tiles: "queue.SimpleQueue[int]" = queue.SimpleQueue()
+        for start in range(0, rows, tile):
+            tiles.put(start)
+
+        def worker():
+            reference.lib.nk_configure_thread(ctypes.c_uint64(viable))
+            while True:
+                try:
+                    start = tiles.get_nowait()
+                except queue.Empty:
+                    return
+                count = min(tile, rows - start)
+                dots_fn(a.ctypes.data + start * a.strides[0], packed.ctypes.data, c.ctypes.data + start * c.strides[0],
+                        count, cols, k, a.strides[0], c.strides[0])
+
+        threads = [threading.Thread(target=worker) for _ in range(cores)]
+        begin = time.perf_counter()
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        return time.perf_counter() - begin
+
+    run_once()
+    best = min(run_once() for _ in range(3))
+    return {"value": 2.0 * rows * cols * k / best / 1e9, "unit": "gso/s", "cores": cores, "kind": "reference",
+            "kernel_capability": hex(used),
+            "sample": f"{rows} rows of A x {cols} packed rows of B x depth {k}, 64-row tiles over {cores} threads, best of 3"}
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--dtype", default=HEADLINE[0])
+    parser.add_argument("--shape", type=int, nargs=3, default=list(HEADLINE[1:]))
+    parser.add_argument("--no-others", action="store_true")
+    parser.add_argument("--no-cpu", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (rows of A or of B shard without "
+                 "communication); run with --gpus 1")
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    m, n, k = args.shape
+    head = time_gpu(args.dtype, m, n, k, args.steps, args.warmup)
+    line = {
+        "metric": "gso/s and % MFMA peak: i8->i32, bf16->f32, e4m3->f32 packed dots at 8192^3",
+        "value": head["gso_per_s"], "unit": "gso/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": f"{args.dtype} packed dots C = A * B^T, M={m} N={n} K={k}, A row-major in HBM, "
+                               "B packed once outside the timed region, C overwritten"},
+        "kernel_ms": head["kernel_ms"], "roofline": head["roofline"],
+    }
+    if not args.no_others:
+        line["others"] = {}
+        for dtype, om, on, ok in OTHERS:
+            r = time_gpu(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2))
+            line["others"][f"{dtype}_{om}x{on}x{ok}"] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"],
+                                                         "roofline": r["roofline"]}
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(args.dtype, m, n, k)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -38,7 +38,8 @@ class NumKongAmdError(RuntimeError):
 
 
 def library_path() -> str:
-    return os.path.join(_HERE, "lib", "libnumkong_amd.so")
+    """The in-tree build, unless NUMKONG_AMD_LIBRARY names another build of the same library."""
+    return os.environ.get("NUMKONG_AMD_LIBRARY") or os.path.join(_HERE, "lib", "libnumkong_amd.so")
 
 
 _LIB: Optional[ctypes.CDLL] = None

@@ -315,14 +315,14 @@ struct E5M2 : F16 {
 
 #pragma region Packed product
 
+#ifdef NK_TUNE
+__device__ unsigned long long g_debug_clocks[8];
+#endif
+
 template <int V>
 struct slot_c {
     static constexpr int value = V;
 };
-template <int V>
-__device__ __forceinline__ constexpr slot_c<(V ^ 1)> slot_next() {
-    return {};
-}
 
 struct GemmArgs {
     uint8_t const *a;
@@ -358,28 +358,40 @@ __device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, ui
 }
 
 /**
- *  One workgroup of NW wavefronts computes a (32*TM) x (32*TN*NW) tile of C. Every wavefront owns all
- *  32*TM rows and its own 32*TN columns, so B fragments are loaded by exactly one wavefront straight
- *  from the packed image into registers, while the shared A block is staged through LDS
- *  (double-buffered, 128 bytes of K per row per stage, row pitch 144 bytes so that 16 consecutive rows
- *  start in 16 different 16-byte bank groups).
+ *  A persistent workgroup of 4 wavefronts (one per SIMD) walks over (32*TM) x (128*TN) tiles of C. Every
+ *  wavefront owns all 32*TM rows of the tile and its own 32*TN columns: B fragments are loaded by exactly
+ *  one wavefront, straight from the packed image into registers; the shared A block goes through LDS.
+ *  Being persistent lets the stores of one tile drain while the next tile is already being computed.
+ *
+ *  A stage is 128 bytes of (packed-width) K per row = four MFMA k-steps. LDS holds two stages of A, rows
+ *  128 bytes apart, the 16-byte chunk `c` of row `r` stored at chunk position c ^ ((r >> 1) & 7): the 16
+ *  rows that one pass of a ds_read_b128 touches then fall into 16 different 16-byte bank groups (measured:
+ *  SQ_LDS_BANK_CONFLICT = 0).
+ *
+ *  The steady-state loop handles two stages per trip so that every register slot and LDS buffer has a
+ *  compile-time index, and its body is one basic block (no branches: prefetch indices are clamped instead),
+ *  which keeps the compiler's s_waitcnt counting exact. Everything is fetched two stages ahead:
+ *      k-step q MFMAs of (s, q) under the LDS reads of the A fragments of (s, q+1); then the B registers
+ *               just consumed are refilled with B(s+2, q)
+ *      k-step 2 also moves A(s+1), loaded two stages ago, from registers into the other LDS buffer and
+ *               refills those registers with A(s+3)
+ *      before the last k-step: one barrier; the first fragments of stage s+1 are read under its MFMAs
+ *  Stages that are not whole (and an odd last one), and every stage when A is not aligned for vector loads,
+ *  run afterwards through a plain guarded loop.
  */
-template <class T, int TM, int TN, int NW, bool ALIGNED>
-__global__ __launch_bounds__(NW * 64) void dots_packed_kernel(GemmArgs g) {
+template <class T, int TM, int TN, int DBG = 0>
+__global__ __launch_bounds__(256) void dots_packed_kernel(GemmArgs g) {
     typedef typename T::acc_t acc_t;
     constexpr int BM = TM * 32;
-    constexpr int NT = NW * 64;
-    constexpr int kPitch = kStageBytes + 16;
-    constexpr int kStageLds = BM * kPitch;
-    constexpr int kLoads = BM * kStageChunks / NT; // chunks staged per thread per stage
-    static_assert(BM * kStageChunks % NT == 0, "stage must divide evenly among threads");
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int NT = 256;
+    constexpr int kStageLds = BM * kStageBytes;
+    constexpr int kLoads = BM * kStageChunks / NT; // 16-byte LDS chunks per thread per stage = TM
+    constexpr int kSrcStage = kStageChunks * T::kSrcChunk; // source bytes of A per row per stage
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStageLds];
 
-    uint32_t const tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    uint32_t tile_m, tile_n;
-    tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
-    uint32_t const row0 = tile_m * BM;
-    uint32_t const col0 = tile_n * (32 * TN * NW) + wave * (32 * TN);
+    uint32_t const tid = threadIdx.x, lane = tid & 63;
+    // The wavefront index is the same in all lanes; telling the compiler keeps B addressing in scalar registers.
+    uint32_t const wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     // Trust, but verify: the image must have been packed for this dtype and these dimensions.
     PackedHeader const *header = (PackedHeader const *)g.bp;
@@ -389,195 +401,364 @@ __global__ __launch_bounds__(NW * 64) void dots_packed_kernel(GemmArgs g) {
     uint8_t const *data = g.bp + sizeof(PackedHeader);
     uint32_t const *col_terms = (uint32_t const *)(data + (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes);
 
-    acc_t acc[TM][TN];
+    uint32_t const stages = g.k_chunks / kStageChunks;
+    uint32_t const whole = (uint32_t)(g.k_src_bytes / kSrcStage); // stages with all 128 bytes present
+    // Stages the pipelined loop takes. (readfirstlane: the value is uniform, and it must stay in a scalar
+    // register because the stage offsets of the buffer loads derive from it.)
+    uint32_t const fast = __builtin_amdgcn_readfirstlane((g.avec >= T::kSrcChunk ? whole : 0) & ~1u);
+    uint32_t const xr = T::kUnsigned ? 0x80808080u : 0u;
+    uint32_t const a_pos = tid & 7;
+    // A fragment reads: lane l takes row l % 32 of each 32-row block and chunk 2q + l / 32.
+    uint32_t a_frag[4];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+    for (int q = 0; q < 4; ++q) {
+        uint32_t const r = lane & 31, c = 2 * q + (lane >> 5);
+        a_frag[q] = r * kStageBytes + ((c ^ ((r >> 1) & 7)) << 4);
+    }
 
-    uint32_t row_sum[kLoads]; // u8 only: sum of the unsigned bytes this thread staged, per staged row
-#pragma unroll
-    for (int i = 0; i < kLoads; ++i) row_sum[i] = 0;
+    for (uint32_t tile = blockIdx.x; tile < g.tiles_m * g.tiles_n; tile += gridDim.x) {
+        uint32_t tile_m, tile_n;
+        tile_of_block(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+        uint32_t const row0 = tile_m * BM;
+        uint32_t const col0 = tile_n * (128 * TN) + wave * (32 * TN);
 
-    if (image_ok) {
-        // Per-thread A source rows (clamped to the last row: edge tiles recompute it and mask the store).
-        uint8_t const *a_src[kLoads];
-        uint32_t lds_dst[kLoads];
-        uint32_t const chunk_in_stage = tid & 7;
+        acc_t acc[TM][TN];
 #pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            uint32_t const r = (i * NT + tid) >> 3;
-            uint32_t const row = row0 + r < g.m ? row0 + r : g.m - 1;
-            a_src[i] = g.a + (uint64_t)row * g.a_stride + chunk_in_stage * T::kSrcChunk;
-            lds_dst[i] = r * kPitch + chunk_in_stage * kChunkBytes;
-        }
-        // Per-wavefront B fragment streams (tile index clamped the same way).
-        uint8_t const *b_src[TN];
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
-            b_src[j] = data + (uint64_t)t * g.k_chunks * kTileChunkBytes + lane * kChunkBytes;
-        }
-        uint32_t const a_frag = (lane & 31) * kPitch + (lane >> 5) * kChunkBytes;
-        uint32_t const stages = g.k_chunks / kStageChunks;
-        uint32_t const xr = T::kUnsigned ? 0x80808080u : 0u;
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
-        v4i a_reg[kLoads];
-        v4i b_reg[2][TN][4];
+        uint32_t row_sum[kLoads]; // u8 only: sum of the unsigned bytes this thread staged, per staged row
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) row_sum[i] = 0;
 
-        auto load_a = [&](uint32_t s) {
-            uint64_t const offset = (uint64_t)s * (kStageChunks * T::kSrcChunk);
-            bool const full = offset + kStageChunks * T::kSrcChunk <= g.k_src_bytes;
-            if (ALIGNED && full) {
+        if (image_ok) {
+            // A staging: thread t fetches chunk t % 8 of rows i*32 + t/8 and stores it at its swizzled position.
+            uint32_t a_off[kLoads]; // byte offset of the thread's source chunk from the tile's first row
+            uint32_t a_lds[kLoads]; // where it goes in an LDS stage
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i) {
+                uint32_t const r = i * 32 + (tid >> 3);
+                uint32_t const row = row0 + r < g.m ? r : g.m - 1 - row0; // clamp to the last row; the store is masked
+                a_off[i] = row * (uint32_t)g.a_stride + a_pos * T::kSrcChunk;
+                a_lds[i] = r * kStageBytes + ((a_pos ^ ((r >> 1) & 7)) << 4);
+            }
+            uint8_t const *a_tile = g.a + (uint64_t)row0 * g.a_stride;
+
+            // Loads go through buffer descriptors: one scalar descriptor plus a 32-bit per-lane offset is the
+            // cheapest address form to issue (a single address register per lane, no 64-bit vector adds).
+            // B fragment streams of this wavefront: one descriptor per 32-column tile (tile index clamped like
+            // the rows), every lane at offset lane * 16.
+            __amdgpu_buffer_rsrc_t b_rsrc[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
+                b_rsrc[j] = __builtin_amdgcn_make_buffer_rsrc((void *)(data + (uint64_t)t * g.k_chunks * kTileChunkBytes), 0,
+                                                              (int)(g.k_chunks * kTileChunkBytes), 0x00020000);
+            }
+            uint32_t const b_lane = lane * kChunkBytes;
+            __amdgpu_buffer_rsrc_t const a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a_tile, 0, -1, 0x00020000);
+
+            v4i a_reg[2][kLoads];
+            v4i b_reg[2][TN][4];
+            v4i af[2][TM];
+
+            // A(s) -> registers, in four parts so that the loads can be spread over four k-steps.
+            auto load_a = [&](uint32_t s, auto slot_tag, auto part_tag) {
+                constexpr int slot = decltype(slot_tag)::value, part = decltype(part_tag)::value;
+                uint32_t const stage_offset = s * kSrcStage;
 #pragma unroll
                 for (int i = 0; i < kLoads; ++i) {
+                    if (i * 4 / kLoads != part) continue;
                     v4i v = {0, 0, 0, 0};
-                    if (T::kSrcChunk == 16) { v = *(v4i const *)(a_src[i] + offset); }
-                    else {
-                        typedef int v2i __attribute__((ext_vector_type(2)));
-                        v2i const narrow = *(v2i const *)(a_src[i] + offset);
-                        v[0] = narrow[0], v[1] = narrow[1];
+                    if (T::kSrcChunk == 16) {
+                        v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_off[i], stage_offset, 0));
                     }
+                    else {
+                        typedef unsigned v2u __attribute__((ext_vector_type(2)));
+                        v2u const narrow = __builtin_amdgcn_raw_buffer_load_b64(a_rsrc, a_off[i], stage_offset, 0);
+                        v[0] = (int)narrow[0], v[1] = (int)narrow[1];
+                    }
+                    a_reg[slot][i] = v;
+                }
+            };
+            auto load_a_all = [&](uint32_t s, auto slot_tag) {
+                load_a(s, slot_tag, slot_c<0>()), load_a(s, slot_tag, slot_c<1>());
+                load_a(s, slot_tag, slot_c<2>()), load_a(s, slot_tag, slot_c<3>());
+            };
+            // Element-wise work on the staged chunks happens here, after the loads have had time to land.
+            // `real` is 0 for the clamped re-load of the last stage, which must not be counted twice.
+            auto store_a = [&](auto buffer_tag, auto slot_tag, uint32_t real) {
+                constexpr int buffer = decltype(buffer_tag)::value, slot = decltype(slot_tag)::value;
+                uint8_t *dst = lds + buffer * kStageLds;
+#pragma unroll
+                for (int i = 0; i < kLoads; ++i) {
+                    v4i v = a_reg[slot][i];
                     if (T::kUnsigned) {
-                        row_sum[i] += sum_bytes_u8(v);
+                        row_sum[i] += sum_bytes_u8(v) * real;
                         v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
                     }
-                    a_reg[i] = T::widen(v);
+                    *(v4i *)(dst + a_lds[i]) = T::widen(v);
                 }
+            };
+            auto load_b = [&](uint32_t s, auto slot_tag, auto q_tag) {
+                constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    b_reg[slot][j][q] = __builtin_bit_cast(
+                        v4i, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc[j], b_lane + q * 2 * kTileChunkBytes,
+                                                                   s * (kStageChunks * kTileChunkBytes), 0));
+            };
+            auto read_frags = [&](auto buffer_tag, auto q_tag, auto parity_tag) {
+                constexpr int buffer = decltype(buffer_tag)::value, q = decltype(q_tag)::value,
+                              parity = decltype(parity_tag)::value;
+                uint8_t const *src = lds + buffer * kStageLds + a_frag[q];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) af[parity][i] = *(v4i const *)(src + i * 32 * kStageBytes);
+            };
+            auto multiply = [&](auto slot_tag, auto q_tag) {
+                constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[q & 1][i], b_reg[slot][j][q]);
+            };
+            // Scheduling hints for one k-step. Masks: 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write.
+            // Fragment reads go one-to-one with the first TM MFMAs; the global loads of the k-step (TN of B
+            // and a quarter of A) are spread over the remaining MFMAs; k-step 2 also carries the LDS writes.
+            auto schedule_k_step = [&](auto writes_tag) {
+                constexpr bool writes = decltype(writes_tag)::value != 0;
+                constexpr int loads = TN + (kLoads >= 4 ? kLoads / 4 : 1);
+                constexpr int rest = TM * (TN - 1);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+                if constexpr (rest == 0) {
+                    if (writes) __builtin_amdgcn_sched_group_barrier(0x200, kLoads, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x020, loads, 0);
+                }
+                else {
+#pragma unroll
+                    for (int i = 0; i < rest; ++i) {
+                        if (writes && i < kLoads) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                        if (i * loads / rest != (i + 1) * loads / rest || (loads > rest && i == 0))
+                            __builtin_amdgcn_sched_group_barrier(0x020, loads > rest ? loads : 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    }
+                    if (writes && kLoads > rest) __builtin_amdgcn_sched_group_barrier(0x200, kLoads - rest, 0);
+                }
+            };
+            // One stage of the steady state; `P` = stage parity = LDS buffer = register slot.
+            auto stage = [&](auto parity_tag, uint32_t s, uint32_t last) {
+                constexpr int P = decltype(parity_tag)::value;
+                uint32_t const s2 = s + 2 < last ? s + 2 : last, s3 = s + 3 < last ? s + 3 : last;
+                __builtin_amdgcn_sched_barrier(0);
+                if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
+                multiply(slot_c<P>(), slot_c<0>());
+                if (!(DBG & 1)) load_b(s2, slot_c<P>(), slot_c<0>()), load_a(s2, slot_c<P>(), slot_c<2>());
+                schedule_k_step(slot_c<0>());
+                __builtin_amdgcn_sched_barrier(0);
+                if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
+                multiply(slot_c<P>(), slot_c<1>());
+                if (!(DBG & 1)) load_b(s2, slot_c<P>(), slot_c<1>()), load_a(s2, slot_c<P>(), slot_c<3>());
+                schedule_k_step(slot_c<0>());
+                __builtin_amdgcn_sched_barrier(0);
+                if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
+                multiply(slot_c<P>(), slot_c<2>());
+                if (!(DBG & 1)) load_b(s2, slot_c<P>(), slot_c<2>());
+                // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
+                // at the previous barrier); then its registers start being refilled with A(s+3).
+                if (!(DBG & 8)) store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 <= last ? 1u : 0u);
+                if (!(DBG & 1)) load_a(s3, slot_c<P ^ 1>(), slot_c<0>());
+                schedule_k_step(slot_c<1>());
+                __builtin_amdgcn_sched_barrier(0);
+                if (!(DBG & 4)) __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+                if (!(DBG & 2)) read_frags(slot_c<P ^ 1>(), slot_c<0>(), slot_c<0>());
+                multiply(slot_c<P>(), slot_c<3>());
+                if (!(DBG & 1)) load_b(s2, slot_c<P>(), slot_c<3>()), load_a(s3, slot_c<P ^ 1>(), slot_c<1>());
+                schedule_k_step(slot_c<0>());
+            };
+
+            __syncthreads(); // the previous tile's last fragment reads (and row terms) are done
+#ifdef NK_TUNE
+            unsigned long long const debug_c0 = clock64(), debug_w0 = wall_clock64();
+#endif
+            if (fast > 0) {
+                uint32_t const last = fast - 1;
+                load_a_all(0, slot_c<0>());
+                load_b(0, slot_c<0>(), slot_c<0>()), load_b(0, slot_c<0>(), slot_c<1>());
+                load_b(0, slot_c<0>(), slot_c<2>()), load_b(0, slot_c<0>(), slot_c<3>());
+                load_a_all(1, slot_c<1>());
+                load_b(1, slot_c<1>(), slot_c<0>()), load_b(1, slot_c<1>(), slot_c<1>());
+                load_b(1, slot_c<1>(), slot_c<2>()), load_b(1, slot_c<1>(), slot_c<3>());
+                store_a(slot_c<0>(), slot_c<0>(), 1u);
+                // the first half of A(2), as k-steps 2 and 3 of a stage "-1" would have issued it
+                load_a(2 < last ? 2 : last, slot_c<0>(), slot_c<0>()), load_a(2 < last ? 2 : last, slot_c<0>(), slot_c<1>());
+                __syncthreads();
+                read_frags(slot_c<0>(), slot_c<0>(), slot_c<0>());
+                for (uint32_t s = 0; s < fast; s += 2) {
+                    stage(slot_c<0>(), s, last);
+                    stage(slot_c<1>(), s + 1, last);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            else {
-                int64_t const left = (int64_t)g.k_src_bytes - (int64_t)offset - (int64_t)chunk_in_stage * T::kSrcChunk;
+#ifdef NK_TUNE
+            if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + gridDim.x) {
+                g_debug_clocks[0] = clock64() - debug_c0, g_debug_clocks[1] = wall_clock64() - debug_w0;
+                g_debug_clocks[2] = fast;
+            }
+#endif
+
+            // Remaining stages: the ragged end of K, or everything when A cannot be read with vector loads.
+            for (uint32_t s = fast; s < stages; ++s) {
+                __syncthreads();
+                int64_t const left = (int64_t)g.k_src_bytes - (int64_t)s * kSrcStage - (int64_t)a_pos * T::kSrcChunk;
                 int const valid = (int)(left > T::kSrcChunk ? T::kSrcChunk : (left < 0 ? 0 : left));
 #pragma unroll
                 for (int i = 0; i < kLoads; ++i) {
-                    v4i v = load_chunk_guarded(a_src[i] + offset, valid, g.avec, 0u);
+                    v4i v = load_chunk_guarded(a_tile + (uint64_t)s * kSrcStage + a_off[i], valid, g.avec, 0u);
                     if (T::kUnsigned) {
                         row_sum[i] += sum_bytes_u8(v);
-                        // Flip only bytes that exist so that the zero padding stays zero.
 #pragma unroll
-                        for (int w = 0; w < 4; ++w) {
+                        for (int w = 0; w < 4; ++w) { // flip only bytes that exist: the zero padding stays zero
                             int const rem = valid - 4 * w;
                             uint32_t const mask = rem >= 4 ? 0x80808080u : (rem <= 0 ? 0u : (0x80808080u >> (8 * (4 - rem))));
                             v[w] ^= (int)mask;
                         }
                     }
-                    a_reg[i] = T::widen(v);
+                    *(v4i *)(lds + a_lds[i]) = T::widen(v);
+                }
+                load_b(s, slot_c<0>(), slot_c<0>()), load_b(s, slot_c<0>(), slot_c<1>());
+                load_b(s, slot_c<0>(), slot_c<2>()), load_b(s, slot_c<0>(), slot_c<3>());
+                __syncthreads();
+                read_frags(slot_c<0>(), slot_c<0>(), slot_c<0>());
+                read_frags(slot_c<0>(), slot_c<1>(), slot_c<1>());
+                multiply(slot_c<0>(), slot_c<0>());
+                read_frags(slot_c<0>(), slot_c<2>(), slot_c<0>());
+                multiply(slot_c<0>(), slot_c<1>());
+                read_frags(slot_c<0>(), slot_c<3>(), slot_c<1>());
+                multiply(slot_c<0>(), slot_c<2>());
+                multiply(slot_c<0>(), slot_c<3>());
+            }
+        }
+
+        // Epilogue. Accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.
+        uint32_t const half = lane >> 5, col_in_tile = lane & 31;
+        uint32_t *row_terms = (uint32_t *)lds;
+        if (T::kUnsigned && image_ok) {
+            __syncthreads();
+            // The 8 threads that staged one row hold its partial byte sums in adjacent lanes.
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i) {
+                uint32_t s = row_sum[i];
+                s += __shfl_xor(s, 1, 64);
+                s += __shfl_xor(s, 2, 64);
+                s += __shfl_xor(s, 4, 64);
+                if ((tid & 7) == 0) row_terms[i * 32 + (tid >> 3)] = s * 128u;
+            }
+            __syncthreads();
+        }
+        // Stores: a scalar row base (advanced by the row stride with scalar adds) plus one per-lane offset,
+        // so that no 64-bit address ever lives in vector registers. Tiles that touch the matrix edge take
+        // the masked copy of the loop.
+        bool const interior = row0 + BM <= g.m && col0 + 32 * TN <= g.n;
+        uint8_t *c_tile = g.c + (uint64_t)row0 * g.c_stride + (uint64_t)col0 * 4;
+        uint32_t const lane_offset = 4 * half * (uint32_t)g.c_stride + col_in_tile * 4;
+        auto store_all = [&](auto masked_tag) {
+            constexpr bool masked = decltype(masked_tag)::value != 0;
+            uint64_t const row_step = g.c_stride;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                uint32_t col_term = 0;
+                if (T::kUnsigned && image_ok) {
+                    uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
+                    col_term = col_terms[(uint64_t)t * kTileRows + col_in_tile];
+                }
+                bool const col_ok = col0 + j * 32 + col_in_tile < g.n;
+                // Rows come in runs of 4 that start 8 apart: the base advances by one row or by five. The
+                // empty asm keeps it a running scalar (otherwise every row's base is precomputed and the
+                // scalar registers overflow).
+                uint8_t *row_base = c_tile + j * 128;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        int const r_fixed = i * 32 + 8 * (v / 4) + (v % 4); // row of lanes 0..31; lanes 32..63 are 4 rows below
+                        auto const element = acc[i][j][v]; // a named copy: bit-casting the vector element expression reads lane 0
+                        uint32_t bits = __builtin_bit_cast(uint32_t, element);
+                        if (T::kUnsigned) bits += row_terms[r_fixed + 4 * half] + col_term;
+                        if (!image_ok) bits = 0xFFFFFFFFu;
+                        if (!masked || (col_ok && row0 + r_fixed + 4 * half < g.m)) *(uint32_t *)(row_base + lane_offset) = bits;
+                        row_base += (v % 4 == 3 ? 5 : 1) * row_step;
+                        asm volatile("" : "+s"(row_base));
+                    }
                 }
             }
         };
-        auto store_a = [&](uint32_t buffer) {
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) *(v4i *)(lds + buffer * kStageLds + lds_dst[i]) = a_reg[i];
-        };
-        auto load_b = [&](uint32_t s, auto slot_tag) {
-            constexpr int slot = decltype(slot_tag)::value;
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    b_reg[slot][j][q] =
-                        *(v4i const *)(b_src[j] + (uint64_t)s * (kStageChunks * kTileChunkBytes) + q * 2 * kTileChunkBytes);
-        };
-
-        // One pipeline stage with compile-time buffer/register-slot indices (runtime indexing of
-        // register arrays would spill them to scratch).
-        auto stage = [&](auto slot_tag, uint32_t s) {
-            constexpr int slot = decltype(slot_tag)::value;
-            bool const more = s + 1 < stages;
-            if (more) {
-                load_a(s + 1);
-                load_b(s + 1, slot_next<slot>());
-            }
-            uint8_t const *a_lds = lds + slot * kStageLds + a_frag;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                v4i af[TM];
-#pragma unroll
-                for (int i = 0; i < TM; ++i) af[i] = *(v4i const *)(a_lds + i * 32 * kPitch + q * 2 * kChunkBytes);
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[i], b_reg[slot][j][q]);
-            }
-            if (more) store_a(slot ^ 1);
-            __syncthreads();
-        };
-
-        load_a(0);
-        load_b(0, slot_c<0>());
-        store_a(0);
-        __syncthreads();
-        for (uint32_t s = 0; s < stages; s += 2) {
-            stage(slot_c<0>(), s);
-            if (s + 1 < stages) stage(slot_c<1>(), s + 1);
-        }
-    }
-
-    // Epilogue. Accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.
-    uint32_t const half = lane >> 5, col_in_tile = lane & 31;
-    uint32_t *row_terms = (uint32_t *)lds;
-    if (T::kUnsigned && image_ok) {
-        // The 8 threads that staged one row hold its partial byte sums in adjacent lanes.
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            uint32_t s = row_sum[i];
-            s += __shfl_xor(s, 1, 64);
-            s += __shfl_xor(s, 2, 64);
-            s += __shfl_xor(s, 4, 64);
-            if ((tid & 7) == 0) row_terms[(i * NT + tid) >> 3] = s * 128u;
-        }
-        __syncthreads();
-    }
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        uint32_t const col = col0 + j * 32 + col_in_tile;
-        uint32_t col_term = 0;
-        if (T::kUnsigned && image_ok) {
-            uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
-            col_term = col_terms[(uint64_t)t * kTileRows + col_in_tile];
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                uint32_t const r = i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
-                uint32_t const row = row0 + r;
-                auto const element = acc[i][j][v]; // a named copy: bit-casting the vector element expression reads lane 0
-                uint32_t bits = __builtin_bit_cast(uint32_t, element);
-                if (T::kUnsigned) bits += row_terms[r] + col_term;
-                if (!image_ok) bits = 0xFFFFFFFFu;
-                if (row < g.m && col < g.n) *(uint32_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 4) = bits;
-            }
-        }
+        if (interior) store_all(slot_c<0>());
+        else store_all(slot_c<1>());
     }
 }
 
 struct TileConfig {
-    int tm, tn, nw;
+    int tm, tn;
 };
 // Index 0 is "choose for me"; 1.. are explicit.
-constexpr TileConfig kConfigs[] = {{0, 0, 0}, {8, 2, 4}, {4, 2, 4}, {4, 1, 4}, {2, 1, 4}};
+constexpr TileConfig kConfigs[] = {{0, 0}, {8, 2}, {4, 2}, {4, 1}, {2, 1}};
 constexpr int kConfigCount = sizeof(kConfigs) / sizeof(kConfigs[0]);
 int g_forced_config = 0;
+int g_variant = 0; // timing experiments of tuning builds
 
-template <class T, int TM, int TN, int NW>
+int g_cu_count = 0;
+
+template <class T, int TM, int TN>
 hipError_t launch_one(GemmArgs &g, hipStream_t stream) {
-    constexpr int BM = TM * 32, BN = TN * NW * 32;
-    constexpr size_t lds_bytes = (size_t)2 * BM * (kStageBytes + 16);
+    constexpr int BM = TM * 32, BN = TN * 128;
     g.tiles_m = (g.m + BM - 1) / BM;
     g.tiles_n = (g.n + BN - 1) / BN;
-    uint64_t const blocks = (uint64_t)g.tiles_m * g.tiles_n;
-    if (blocks > 0x7FFFFFFFull) return hipErrorInvalidValue;
-    bool const aligned = g.avec >= T::kSrcChunk;
-    auto kernel = aligned ? dots_packed_kernel<T, TM, TN, NW, true> : dots_packed_kernel<T, TM, TN, NW, false>;
-    if (lds_bytes > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute((void const *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)lds_bytes);
-        if (e != hipSuccess) return e;
+    uint64_t const tiles = (uint64_t)g.tiles_m * g.tiles_n;
+    if (tiles > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    // The tile's A offsets are 32-bit: (rows of a tile) * stride must stay below 4 GiB.
+    if ((uint64_t)BM * g.a_stride > 0xFFFFFFFFull) return hipErrorInvalidValue;
+    // So are the per-lane C offsets: 4 rows plus the tile's width.
+    if (4 * (uint64_t)g.c_stride + BN * 4 > 0xFFFFFFFFull) return hipErrorInvalidValue;
+    void (*kernel)(GemmArgs) = dots_packed_kernel<T, TM, TN>;
+#ifdef NK_TUNE // timing experiments that leave parts of the loop out (results are wrong on purpose)
+    if constexpr (TM == 8 && TN == 2 && T::kDtype == kI8) {
+        switch (g_variant >> 2) {
+        case 1: kernel = dots_packed_kernel<T, TM, TN, 1>; break;
+        case 2: kernel = dots_packed_kernel<T, TM, TN, 2>; break;
+        case 3: kernel = dots_packed_kernel<T, TM, TN, 3>; break;
+        case 4: kernel = dots_packed_kernel<T, TM, TN, 4>; break;
+        case 5: kernel = dots_packed_kernel<T, TM, TN, 7>; break;
+        case 6: kernel = dots_packed_kernel<T, TM, TN, 15>; break;
+        case 7: kernel = dots_packed_kernel<T, TM, TN, 8>; break;
+        case 8: kernel = dots_packed_kernel<T, TM, TN, 9>; break;
+        default: break;
+        }
     }
-    hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(NW * 64), lds_bytes, stream, g);
+#endif
+    // Persistent grid: as many workgroups as fit on the device at once (queried once per kernel).
+    static int resident = 0;
+    if (!resident) {
+        int per_cu = 0, device = 0;
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (void const *)kernel, 256, 0);
+        if (e != hipSuccess) return e;
+        if (!g_cu_count) {
+            hipDeviceProp_t properties;
+            if ((e = hipGetDevice(&device)) != hipSuccess) return e;
+            if ((e = hipGetDeviceProperties(&properties, device)) != hipSuccess) return e;
+            g_cu_count = properties.multiProcessorCount;
+        }
+        resident = (per_cu > 0 ? per_cu : 1) * (g_cu_count > 0 ? g_cu_count : 256);
+    }
+    uint32_t const blocks = (uint32_t)(tiles < (uint64_t)resident ? tiles : (uint64_t)resident);
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, g);
     return hipGetLastError();
 }
 
@@ -587,7 +768,7 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream) {
     if (config <= 0 || config >= kConfigCount) {
         // Largest tile that still gives every one of the 256 CUs at least one workgroup.
         auto tiles = [&](int c) {
-            uint64_t const bm = kConfigs[c].tm * 32, bn = (uint64_t)kConfigs[c].tn * kConfigs[c].nw * 32;
+            uint64_t const bm = kConfigs[c].tm * 32, bn = (uint64_t)kConfigs[c].tn * 128;
             return ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
         };
         config = kConfigCount - 1;
@@ -598,10 +779,10 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream) {
             }
     }
     switch (config) {
-    case 1: return launch_one<T, 8, 2, 4>(g, stream);
-    case 2: return launch_one<T, 4, 2, 4>(g, stream);
-    case 3: return launch_one<T, 4, 1, 4>(g, stream);
-    default: return launch_one<T, 2, 1, 4>(g, stream);
+    case 1: return launch_one<T, 8, 2>(g, stream);
+    case 2: return launch_one<T, 4, 2>(g, stream);
+    case 3: return launch_one<T, 4, 1>(g, stream);
+    default: return launch_one<T, 2, 1>(g, stream);
     }
 }
 
@@ -782,7 +963,16 @@ int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, voi
     return e == hipSuccess ? 0 : fail(e, "dots_packed_kernel");
 }
 
-void nk_hip_set_tile_config(int config) { g_forced_config = config; }
+#ifdef NK_TUNE
+__attribute__((visibility("default"))) void nk_hip_debug_clocks(unsigned long long *out) {
+    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_debug_clocks), sizeof(unsigned long long) * 8);
+}
+#endif
+
+void nk_hip_set_tile_config(int config) {
+    g_forced_config = config & 0xFF;
+    g_variant = (config >> 8) & 0xFF;
+}
 
 char const *nk_hip_last_error(void) { return g_last_error; }
 
