@@ -376,8 +376,14 @@ __device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, ui
  *      k-step 2 also moves A(s+1), loaded two stages ago, from registers into the other LDS buffer and
  *               refills those registers with A(s+3)
  *      before the last k-step: one barrier; the first fragments of stage s+1 are read under its MFMAs
- *  Stages that are not whole (and an odd last one), and every stage when A is not aligned for vector loads,
- *  run afterwards through a plain guarded loop.
+ *  An odd last whole stage, a stage that is not whole, and every stage when A is not even dword-aligned, run
+ *  afterwards through a plain guarded loop.
+ *
+ *  A is the MFMA's first operand, so a lane ends up with one column and 16 rows of each 32x32 block and the
+ *  epilogue stores dwords that are contiguous across lanes: 128 bytes per row per instruction, any C
+ *  alignment. (The other orientation, one row and runs of 4 columns per lane stored as 128-bit vectors,
+ *  needs a quarter of the store instructions but writes 32-byte pieces of 32 different rows; it measured
+ *  12 % slower on the square shapes and 9 % slower on the retrieval shape.)
  */
 template <class T, int TM, int TN, int DBG = 0>
 __global__ __launch_bounds__(256) void dots_packed_kernel(GemmArgs g) {
@@ -403,9 +409,10 @@ __global__ __launch_bounds__(256) void dots_packed_kernel(GemmArgs g) {
 
     uint32_t const stages = g.k_chunks / kStageChunks;
     uint32_t const whole = (uint32_t)(g.k_src_bytes / kSrcStage); // stages with all 128 bytes present
-    // Stages the pipelined loop takes. (readfirstlane: the value is uniform, and it must stay in a scalar
+    // Stages the pipelined loop takes: the whole ones, in pairs, when A is at least dword-aligned, which is
+    // all that multi-dword global loads need. (readfirstlane: the value is uniform, and it must stay in a scalar
     // register because the stage offsets of the buffer loads derive from it.)
-    uint32_t const fast = __builtin_amdgcn_readfirstlane((g.avec >= T::kSrcChunk ? whole : 0) & ~1u);
+    uint32_t const fast = __builtin_amdgcn_readfirstlane((g.avec >= 4 ? whole : 0) & ~1u);
     uint32_t const xr = T::kUnsigned ? 0x80808080u : 0u;
     uint32_t const a_pos = tid & 7;
     // A fragment reads: lane l takes row l % 32 of each 32-row block and chunk 2q + l / 32.
@@ -663,39 +670,41 @@ __global__ __launch_bounds__(256) void dots_packed_kernel(GemmArgs g) {
             }
             __syncthreads();
         }
-        // Stores: a scalar row base (advanced by the row stride with scalar adds) plus one per-lane offset,
-        // so that no 64-bit address ever lives in vector registers. Tiles that touch the matrix edge take
-        // the masked copy of the loop.
+        // Stores: a scalar base plus one per-lane offset, so that no 64-bit address ever lives in vector
+        // registers. Tiles that touch the matrix edge take the masked copy of the loop.
         bool const interior = row0 + BM <= g.m && col0 + 32 * TN <= g.n;
         uint8_t *c_tile = g.c + (uint64_t)row0 * g.c_stride + (uint64_t)col0 * 4;
-        uint32_t const lane_offset = 4 * half * (uint32_t)g.c_stride + col_in_tile * 4;
         auto store_all = [&](auto masked_tag) {
             constexpr bool masked = decltype(masked_tag)::value != 0;
             uint64_t const row_step = g.c_stride;
+            {
+                // Lane l holds column l % 32; register v holds row 8 * (v / 4) + 4 * (l / 32) + v % 4.
+                uint32_t const lane_offset = 4 * half * (uint32_t)g.c_stride + col_in_tile * 4;
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                uint32_t col_term = 0;
-                if (T::kUnsigned && image_ok) {
-                    uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
-                    col_term = col_terms[(uint64_t)t * kTileRows + col_in_tile];
-                }
-                bool const col_ok = col0 + j * 32 + col_in_tile < g.n;
-                // Rows come in runs of 4 that start 8 apart: the base advances by one row or by five. The
-                // empty asm keeps it a running scalar (otherwise every row's base is precomputed and the
-                // scalar registers overflow).
-                uint8_t *row_base = c_tile + j * 128;
+                for (int j = 0; j < TN; ++j) {
+                    uint32_t col_term = 0;
+                    if (T::kUnsigned && image_ok) {
+                        uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
+                        col_term = col_terms[(uint64_t)t * kTileRows + col_in_tile];
+                    }
+                    bool const col_ok = col0 + j * 32 + col_in_tile < g.n;
+                    // Rows come in runs of 4 that start 8 apart: the base advances by one row or by five. The
+                    // empty asm keeps it a running scalar (otherwise every row's base is precomputed and the
+                    // scalar registers overflow).
+                    uint8_t *row_base = c_tile + j * 128;
 #pragma unroll
-                for (int i = 0; i < TM; ++i) {
+                    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        int const r_fixed = i * 32 + 8 * (v / 4) + (v % 4); // row of lanes 0..31; lanes 32..63 are 4 rows below
-                        auto const element = acc[i][j][v]; // a named copy: bit-casting the vector element expression reads lane 0
-                        uint32_t bits = __builtin_bit_cast(uint32_t, element);
-                        if (T::kUnsigned) bits += row_terms[r_fixed + 4 * half] + col_term;
-                        if (!image_ok) bits = 0xFFFFFFFFu;
-                        if (!masked || (col_ok && row0 + r_fixed + 4 * half < g.m)) *(uint32_t *)(row_base + lane_offset) = bits;
-                        row_base += (v % 4 == 3 ? 5 : 1) * row_step;
-                        asm volatile("" : "+s"(row_base));
+                        for (int v = 0; v < 16; ++v) {
+                            int const r_fixed = i * 32 + 8 * (v / 4) + (v % 4); // row of lanes 0..31; lanes 32..63 are 4 rows below
+                            auto const element = acc[i][j][v]; // a named copy: bit-casting the vector element expression reads lane 0
+                            uint32_t bits = __builtin_bit_cast(uint32_t, element);
+                            if (T::kUnsigned) bits += row_terms[r_fixed + 4 * half] + col_term;
+                            if (!image_ok) bits = 0xFFFFFFFFu;
+                            if (!masked || (col_ok && row0 + r_fixed + 4 * half < g.m)) *(uint32_t *)(row_base + lane_offset) = bits;
+                            row_base += (v % 4 == 3 ? 5 : 1) * row_step;
+                            asm volatile("" : "+s"(row_base));
+                        }
                     }
                 }
             }
