@@ -177,6 +177,8 @@ def main():
     parser.add_argument("--shape", type=int, nargs=3, default=list(HEADLINE[1:]))
     parser.add_argument("--no-others", action="store_true")
     parser.add_argument("--no-cpu", action="store_true")
+    parser.add_argument("--probe", action="store_true",
+                        help="for rocprofv3 --pmc runs: launch the headline kernel 3 times and a plain 1 GiB copy 3 times, nothing else")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (rows of A or of B shard without "
@@ -186,6 +188,15 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     m, n, k = args.shape
+    if args.probe:
+        source = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").fill_(1)
+        target = torch.empty_like(source)
+        for _ in range(3):
+            target.copy_(source)  # known traffic: 1 GiB read + 1 GiB written per launch
+        torch.cuda.synchronize()
+        del source, target
+        time_gpu(args.dtype, m, n, k, 3, 0)
+        return
     head = time_gpu(args.dtype, m, n, k, args.steps, args.warmup)
     line = {
         "metric": "gso/s and % MFMA peak: i8->i32, bf16->f32, e4m3->f32 packed dots at 8192^3",

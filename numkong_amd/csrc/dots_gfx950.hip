@@ -265,6 +265,7 @@ __global__ __launch_bounds__(256) void fill_rows_kernel(uint8_t *c, uint32_t m, 
 #pragma region Element types
 
 struct I8 {
+    static constexpr int kChunkStages = 0; // > 0: fold the accumulator into a second one every so many stages
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16i acc_t;
@@ -279,6 +280,7 @@ struct U8 : I8 {
     static constexpr bool kUnsigned = true;
 };
 struct BF16 {
+    static constexpr int kChunkStages = 0; // > 0: fold the accumulator into a second one every so many stages
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
@@ -290,6 +292,7 @@ struct BF16 {
     }
 };
 struct F16 {
+    static constexpr int kChunkStages = 0; // > 0: fold the accumulator into a second one every so many stages
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
@@ -300,12 +303,19 @@ struct F16 {
                                                      0);
     }
 };
+/** fp8 products and short sums are exact in f32, so the reference's scalar kernel loses almost nothing
+ *  (dot/serial.h:522-600: 4 lanes, 8e-9 of sum|a*b| at depth 8192), while one MFMA accumulator rounds once
+ *  per 8 products at the magnitude of the whole running sum (3e-8). Folding the accumulator into a second
+ *  one every 16 stages (1024 values) keeps the running sums short and brings the error under the scalar
+ *  kernel's own. */
 struct E4M3 : F16 {
+    static constexpr int kChunkStages = 16;
     static constexpr int kDtype = kE4M3;
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<false>((uint32_t)v[0], (uint32_t)v[1]); }
 };
 struct E5M2 : F16 {
+    static constexpr int kChunkStages = 16;
     static constexpr int kDtype = kE5M2;
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<true>((uint32_t)v[0], (uint32_t)v[1]); }
@@ -322,6 +332,39 @@ __device__ unsigned long long g_debug_clocks[8];
 template <int V>
 struct slot_c {
     static constexpr int value = V;
+};
+
+/** Second-level accumulators: real for the chunked types, empty (no registers) for the others. */
+template <class acc_t, int TM, int TN, bool kChunked>
+struct Totals {
+    acc_t value[TM][TN];
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) value[i][j][v] = 0;
+    }
+    __device__ __forceinline__ void fold(acc_t (&acc)[TM][TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                value[i][j] += acc[i][j];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+            }
+    }
+    __device__ __forceinline__ auto finish(acc_t const (&acc)[TM][TN], int i, int j, int v) const {
+        return acc[i][j][v] + value[i][j][v];
+    }
+};
+template <class acc_t, int TM, int TN>
+struct Totals<acc_t, TM, TN, false> {
+    __device__ __forceinline__ void clear() {}
+    __device__ __forceinline__ void fold(acc_t (&)[TM][TN]) {}
+    __device__ __forceinline__ auto finish(acc_t const (&acc)[TM][TN], int i, int j, int v) const { return acc[i][j][v]; }
 };
 
 struct GemmArgs {
@@ -386,7 +429,7 @@ __device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, ui
  *  12 % slower on the square shapes and 9 % slower on the retrieval shape.)
  */
 template <class T, int TM, int TN, int DBG = 0>
-__global__ __launch_bounds__(256) void dots_packed_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunkStages == 0 ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
     typedef typename T::acc_t acc_t;
     constexpr int BM = TM * 32;
     constexpr int NT = 256;
@@ -436,6 +479,11 @@ __global__ __launch_bounds__(256) void dots_packed_kernel(GemmArgs g) {
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+        // Second-level accumulators of the chunked types (see E4M3).
+        constexpr bool kChunked = T::kChunkStages > 0;
+        Totals<acc_t, TM, TN, kChunked> total;
+        total.clear();
 
         uint32_t row_sum[kLoads]; // u8 only: sum of the unsigned bytes this thread staged, per staged row
 #pragma unroll
@@ -611,6 +659,12 @@ __global__ __launch_bounds__(256) void dots_packed_kernel(GemmArgs g) {
                 for (uint32_t s = 0; s < fast; s += 2) {
                     stage(slot_c<0>(), s, last);
                     stage(slot_c<1>(), s + 1, last);
+                    if constexpr (kChunked) {
+                        if ((s + 2) % T::kChunkStages == 0) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            total.fold(acc);
+                        }
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -697,7 +751,8 @@ __global__ __launch_bounds__(256) void dots_packed_kernel(GemmArgs g) {
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
                             int const r_fixed = i * 32 + 8 * (v / 4) + (v % 4); // row of lanes 0..31; lanes 32..63 are 4 rows below
-                            auto const element = acc[i][j][v]; // a named copy: bit-casting the vector element expression reads lane 0
+                            // a named copy: bit-casting the vector element expression itself reads lane 0
+                            auto const element = total.finish(acc, i, j, v);
                             uint32_t bits = __builtin_bit_cast(uint32_t, element);
                             if (T::kUnsigned) bits += row_terms[r_fixed + 4 * half] + col_term;
                             if (!image_ok) bits = 0xFFFFFFFFu;
@@ -787,8 +842,11 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream) {
                 break;
             }
     }
+    if (T::kChunkStages > 0 && config == 1) config = 2; // two accumulator sets do not fit the 256 x 256 tile
     switch (config) {
-    case 1: return launch_one<T, 8, 2>(g, stream);
+    case 1:
+        if constexpr (T::kChunkStages > 0) return hipErrorInvalidValue;
+        else return launch_one<T, 8, 2>(g, stream);
     case 2: return launch_one<T, 4, 2>(g, stream);
     case 3: return launch_one<T, 4, 1>(g, stream);
     default: return launch_one<T, 2, 1>(g, stream);
