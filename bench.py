@@ -27,6 +27,15 @@ if ROOT not in sys.path:
 MFMA_PEAK = {"i8": 5000.0, "u8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "e4m3": 2500.0, "e5m2": 2500.0}
 MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2": "widened to f16, priced against the f16 MFMA peak"}
 HBM_PEAK = 8000.0
+# HBM-side bytes per launch (L2 <-> fabric) from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --probe`,
+# each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
+# the summaries are under profiles/. Not re-measured by a plain run: counters need the profiler.
+MEASURED_TRAFFIC = {
+    ("i8", 8192, 8192, 8192): 1.0897e9,
+    ("bf16", 8192, 8192, 8192): 1.9516e9,
+    ("e4m3", 8192, 8192, 8192): 1.8823e9,
+    ("i8", 1024, 1 << 20, 768): 5.7180e9,
+}
 HEADLINE = ("i8", 8192, 8192, 8192)
 OTHERS = [("bf16", 8192, 8192, 8192), ("e4m3", 8192, 8192, 8192), ("i8", 1024, 1 << 20, 768)]
 
@@ -91,11 +100,12 @@ def time_gpu(dtype, m, n, k, steps, warmup):
     if m * n >= 64 * k * 8 and dtype in ("i8", "u8") and n >= 1 << 18:  # retrieval shape: HBM-bound on C and the packed stream
         algorithmic = (m * k + n * k) * width + m * n * 4
         result["roofline"] = {"bound": "hbm", "achieved": algorithmic / (device_ms * 1e-3) / 1e9, "peak": HBM_PEAK,
-                              "unit": "GB/s", "frac": algorithmic / (device_ms * 1e-3) / 1e9 / HBM_PEAK, "traffic": None}
+                              "unit": "GB/s", "frac": algorithmic / (device_ms * 1e-3) / 1e9 / HBM_PEAK,
+                              "traffic": MEASURED_TRAFFIC.get((dtype, m, n, k))}
     else:
         achieved = ops / (device_ms * 1e-3) / 1e12
         result["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK[dtype], "unit": "TFLOP/s",
-                              "frac": achieved / MFMA_PEAK[dtype], "traffic": None}
+                              "frac": achieved / MFMA_PEAK[dtype], "traffic": MEASURED_TRAFFIC.get((dtype, m, n, k))}
         if dtype in MFMA_NOTE:
             result["roofline"]["note"] = MFMA_NOTE[dtype]
     del a, packed, c
@@ -178,7 +188,7 @@ def main():
     parser.add_argument("--no-others", action="store_true")
     parser.add_argument("--no-cpu", action="store_true")
     parser.add_argument("--probe", action="store_true",
-                        help="for rocprofv3 --pmc runs: launch the headline kernel 3 times and a plain 1 GiB copy 3 times, nothing else")
+                        help="for rocprofv3 --pmc runs: launch a plain 1 GiB elementwise copy kernel 3 times, then the selected product 3 times, nothing else")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (rows of A or of B shard without "
@@ -192,7 +202,7 @@ def main():
         source = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").fill_(1)
         target = torch.empty_like(source)
         for _ in range(3):
-            target.copy_(source)  # known traffic: 1 GiB read + 1 GiB written per launch
+            torch.add(source, 1, out=target)  # an elementwise kernel of known traffic: 1 GiB read + 1 GiB written
         torch.cuda.synchronize()
         del source, target
         time_gpu(args.dtype, m, n, k, 3, 0)

@@ -264,6 +264,10 @@ __global__ __launch_bounds__(256) void fill_rows_kernel(uint8_t *c, uint32_t m, 
 
 #pragma region Element types
 
+#ifndef NK_HALF_CHUNK_STAGES
+#define NK_HALF_CHUNK_STAGES 0
+#endif
+
 struct I8 {
     static constexpr int kChunkStages = 0; // > 0: fold the accumulator into a second one every so many stages
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
@@ -280,7 +284,7 @@ struct U8 : I8 {
     static constexpr bool kUnsigned = true;
 };
 struct BF16 {
-    static constexpr int kChunkStages = 0; // > 0: fold the accumulator into a second one every so many stages
+    static constexpr int kChunkStages = NK_HALF_CHUNK_STAGES;
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
@@ -292,7 +296,7 @@ struct BF16 {
     }
 };
 struct F16 {
-    static constexpr int kChunkStages = 0; // > 0: fold the accumulator into a second one every so many stages
+    static constexpr int kChunkStages = NK_HALF_CHUNK_STAGES;
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
