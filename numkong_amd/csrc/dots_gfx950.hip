@@ -432,7 +432,7 @@ __device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, ui
  *  needs a quarter of the store instructions but writes 32-byte pieces of 32 different rows; it measured
  *  12 % slower on the square shapes and 9 % slower on the retrieval shape.)
  */
-template <class T, int TM, int TN, int DBG = 0>
+template <class T, int TM, int TN, bool ACROSS, int DBG = 0>
 __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunkStages == 0 ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
     typedef typename T::acc_t acc_t;
     constexpr int BM = TM * 32;
@@ -441,6 +441,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunk
     constexpr int kLoads = BM * kStageChunks / NT; // 16-byte LDS chunks per thread per stage = TM
     constexpr int kSrcStage = kStageChunks * T::kSrcChunk; // source bytes of A per row per stage
     __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStageLds];
+    __shared__ uint32_t row_terms[T::kUnsigned ? BM : 1]; // u8 only: 128 * (sum of the bytes of each A row of the tile)
 
     uint32_t const tid = threadIdx.x, lane = tid & 63;
     // The wavefront index is the same in all lanes; telling the compiler keeps B addressing in scalar registers.
@@ -470,13 +471,245 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunk
         a_frag[q] = r * kStageBytes + ((c ^ ((r >> 1) & 7)) << 4);
     }
 
-    for (uint32_t tile = blockIdx.x; tile < g.tiles_m * g.tiles_n; tile += gridDim.x) {
+    // A staging: thread t fetches chunk t % 8 of rows i*32 + t/8 of a tile and stores it at its swizzled
+    // position. The offsets are the same for every tile: rows past the end of A are cut off by the size of
+    // the tile's buffer descriptor (such loads return zeros, and their outputs are never stored).
+    uint32_t a_off[kLoads]; // byte offset of the thread's source chunk from the tile's first row
+    uint32_t a_lds[kLoads]; // where it goes in an LDS stage
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+        uint32_t const r = i * 32 + (tid >> 3);
+        a_off[i] = r * (uint32_t)g.a_stride + a_pos * T::kSrcChunk;
+        a_lds[i] = r * kStageBytes + ((a_pos ^ ((r >> 1) & 7)) << 4);
+    }
+    uint32_t const b_lane = lane * kChunkBytes;
+
+    // Loads go through buffer descriptors: one scalar descriptor plus a 32-bit per-lane offset is the cheapest
+    // address form to issue (a single address register per lane, no 64-bit vector adds), and a descriptor is
+    // all that has to change from one tile to the next. B fragment streams of this wavefront: one descriptor
+    // per 32-column tile (tile index clamped to the last one), every lane at offset lane * 16.
+    struct TileView {
+        uint32_t row0, col0;
+        uint8_t const *a; // first row of the tile
+        uint32_t a_bytes; // up to the end of its last row that exists
+        uint8_t const *b; // first 32-column tile of this wavefront
+        uint32_t b_bytes; // up to the end of the packed tiles (or as far as 32 bits reach)
+        uint32_t b_tile[TN]; // offsets of the wavefront's tiles from `b`
+    };
+    auto view_of = [&](uint32_t tile) {
+        TileView view;
         uint32_t tile_m, tile_n;
         tile_of_block(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
-        uint32_t const row0 = tile_m * BM;
-        uint32_t const col0 = tile_n * (128 * TN) + wave * (32 * TN);
+        view.row0 = tile_m * BM;
+        view.col0 = tile_n * (128 * TN) + wave * (32 * TN);
+        uint32_t const rows_here = g.m - view.row0 < (uint32_t)BM ? g.m - view.row0 : (uint32_t)BM;
+        view.a = g.a + (uint64_t)view.row0 * g.a_stride;
+        view.a_bytes = (rows_here - 1) * (uint32_t)g.a_stride + (uint32_t)g.k_src_bytes;
+        uint32_t const tile_bytes = g.k_chunks * kTileChunkBytes;
+        uint32_t const first = view.col0 / 32 < g.n_tiles ? view.col0 / 32 : g.n_tiles - 1;
+        view.b = data + (uint64_t)first * tile_bytes;
+        uint64_t const left = (uint64_t)(g.n_tiles - first) * tile_bytes;
+        view.b_bytes = left < 0xFFFFFFFFull ? (uint32_t)left : 0xFFFFFFFFu;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) view.b_tile[j] = (first + j < g.n_tiles ? j : g.n_tiles - 1 - first) * tile_bytes;
+        return view;
+    };
+    auto a_rsrc_of = [](TileView const &view) {
+        return __builtin_amdgcn_make_buffer_rsrc((void *)view.a, 0, (int)view.a_bytes, 0x00020000);
+    };
+    auto b_rsrc_of = [](TileView const &view) {
+        return __builtin_amdgcn_make_buffer_rsrc((void *)view.b, 0, (int)view.b_bytes, 0x00020000);
+    };
 
-        acc_t acc[TM][TN];
+    // When every stage of a tile goes through the pipelined loop, the prefetches of a tile's last stages
+    // fetch the first stages of the workgroup's next tile instead of running dry: the pipeline is primed once
+    // and then runs across tile boundaries, and the stores of one tile drain under the next tile's MFMAs.
+    constexpr bool across = ACROSS; // the host checks that it holds: fast == stages and stages >= 4
+    uint32_t const tile_count = g.tiles_m * g.tiles_n;
+    uint32_t row_sum[kLoads]; // u8 only: sum of the unsigned bytes this thread staged, per staged row
+    uint32_t row_sum_next[kLoads]; // ... of the chunks it staged ahead for the next tile
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) row_sum[i] = 0, row_sum_next[i] = 0;
+    v4i a_reg[2][kLoads];
+    v4i b_reg[2][TN][4];
+    v4i af[2][TM];
+
+    typedef __attribute__((address_space(1))) uint8_t global_u8_t;
+    typedef __attribute__((address_space(1))) uint32_t global_u32_t;
+    if (!image_ok) { // the image was not packed for this call: the reference's error convention, all bits set
+        for (uint32_t tile = blockIdx.x; tile < g.tiles_m * g.tiles_n; tile += gridDim.x) {
+            uint32_t tile_m, tile_n;
+            tile_of_block(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+            for (uint32_t at = tid; at < (uint32_t)BM * 128 * TN; at += NT) {
+                uint32_t const row = tile_m * BM + at / (128 * TN), col = tile_n * (128 * TN) + at % (128 * TN);
+                if (row < g.m && col < g.n) *(global_u32_t *)((global_u8_t *)g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 4) = 0xFFFFFFFFu;
+            }
+        }
+        return;
+    }
+    TileView cur, nxt;
+    acc_t acc[TM][TN];
+    constexpr bool kChunked = T::kChunkStages > 0;
+    Totals<acc_t, TM, TN, kChunked> total; // second-level accumulators of the chunked types (see E4M3)
+
+    // A(s) -> registers, in four parts so that the loads can be spread over four k-steps.
+    auto load_a = [&](TileView const &view, uint32_t s, auto slot_tag, auto part_tag) {
+        constexpr int slot = decltype(slot_tag)::value, part = decltype(part_tag)::value;
+        __amdgpu_buffer_rsrc_t const rsrc = a_rsrc_of(view);
+        uint32_t const stage_offset = s * kSrcStage;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            if (i * 4 / kLoads != part) continue;
+            v4i v = {0, 0, 0, 0};
+            if (T::kSrcChunk == 16) {
+                v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, a_off[i], stage_offset, 0));
+            }
+            else {
+                typedef unsigned v2u __attribute__((ext_vector_type(2)));
+                v2u const narrow = __builtin_amdgcn_raw_buffer_load_b64(rsrc, a_off[i], stage_offset, 0);
+                v[0] = (int)narrow[0], v[1] = (int)narrow[1];
+            }
+            a_reg[slot][i] = v;
+        }
+    };
+    auto load_a_all = [&](TileView const &view, uint32_t s, auto slot_tag) {
+        load_a(view, s, slot_tag, slot_c<0>()), load_a(view, s, slot_tag, slot_c<1>());
+        load_a(view, s, slot_tag, slot_c<2>()), load_a(view, s, slot_tag, slot_c<3>());
+    };
+    // Element-wise work on the staged chunks happens here, after the loads have had time to land.
+    // `mine` is 1 for a stage of this tile and 0 for one staged ahead for the next tile.
+    auto store_a = [&](auto buffer_tag, auto slot_tag, uint32_t mine) {
+        constexpr int buffer = decltype(buffer_tag)::value, slot = decltype(slot_tag)::value;
+        uint8_t *dst = lds + buffer * kStageLds;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            v4i v = a_reg[slot][i];
+            if (T::kUnsigned) {
+                uint32_t const sum = sum_bytes_u8(v);
+                row_sum[i] += sum * mine, row_sum_next[i] += sum * (1u - mine);
+                v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
+            }
+            *(v4i *)(dst + a_lds[i]) = T::widen(v);
+        }
+    };
+    auto load_b = [&](TileView const &view, uint32_t s, auto slot_tag, auto q_tag) {
+        constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
+        __amdgpu_buffer_rsrc_t const rsrc = b_rsrc_of(view);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            b_reg[slot][j][q] = __builtin_bit_cast(
+                v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_lane + q * 2 * kTileChunkBytes,
+                                                           view.b_tile[j] + s * (kStageChunks * kTileChunkBytes), 0));
+    };
+    auto read_frags = [&](auto buffer_tag, auto q_tag, auto parity_tag) {
+        constexpr int buffer = decltype(buffer_tag)::value, q = decltype(q_tag)::value,
+                      parity = decltype(parity_tag)::value;
+        uint8_t const *src = lds + buffer * kStageLds + a_frag[q];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[parity][i] = *(v4i const *)(src + i * 32 * kStageBytes);
+    };
+    auto multiply = [&](auto slot_tag, auto q_tag) {
+        constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[q & 1][i], b_reg[slot][j][q]);
+    };
+    // Scheduling hints for one k-step. Masks: 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write.
+    // Fragment reads go one-to-one with the first TM MFMAs; the global loads of the k-step (TN of B
+    // and a quarter of A) are spread over the remaining MFMAs; k-step 2 also carries the LDS writes.
+    auto schedule_k_step = [&](auto writes_tag) {
+        constexpr bool writes = decltype(writes_tag)::value != 0;
+        constexpr int loads = TN + (kLoads >= 4 ? kLoads / 4 : 1);
+        constexpr int rest = TM * (TN - 1);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        if constexpr (rest == 0) {
+            if (writes) __builtin_amdgcn_sched_group_barrier(0x200, kLoads, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, loads, 0);
+        }
+        else {
+#pragma unroll
+            for (int i = 0; i < rest; ++i) {
+                if (writes && i < kLoads) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                if (i * loads / rest != (i + 1) * loads / rest || (loads > rest && i == 0))
+                    __builtin_amdgcn_sched_group_barrier(0x020, loads > rest ? loads : 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+            if (writes && kLoads > rest) __builtin_amdgcn_sched_group_barrier(0x200, kLoads - rest, 0);
+        }
+    };
+    // One stage of the steady state; `P` = stage parity = LDS buffer = register slot. Stages s+2 and
+    // s+3 are fetched here; past the tile's end they are the first stages of `nxt` (the next tile, or
+    // this one again when nothing follows: loads of valid memory that nobody uses).
+    auto stage = [&](auto parity_tag, uint32_t s) {
+        constexpr int P = decltype(parity_tag)::value;
+        bool const wrap2 = s + 2 >= fast, wrap3 = s + 3 >= fast;
+        uint32_t const s2 = wrap2 ? s + 2 - fast : s + 2, s3 = wrap3 ? s + 3 - fast : s + 3;
+        TileView const &a2 = wrap2 ? nxt : cur, &a3 = wrap3 ? nxt : cur, &b2 = a2;
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
+        multiply(slot_c<P>(), slot_c<0>());
+        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<0>()), load_a(a2, s2, slot_c<P>(), slot_c<2>());
+        schedule_k_step(slot_c<0>());
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
+        multiply(slot_c<P>(), slot_c<1>());
+        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<1>()), load_a(a2, s2, slot_c<P>(), slot_c<3>());
+        schedule_k_step(slot_c<0>());
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
+        multiply(slot_c<P>(), slot_c<2>());
+        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<2>());
+        // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
+        // at the previous barrier); then its registers start being refilled with A(s+3).
+        if (!(DBG & 8)) store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 < fast ? 1u : 0u);
+        if (!(DBG & 1)) load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
+        schedule_k_step(slot_c<1>());
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 4)) __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 2)) read_frags(slot_c<P ^ 1>(), slot_c<0>(), slot_c<0>());
+        multiply(slot_c<P>(), slot_c<3>());
+        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<3>()), load_a(a3, s3, slot_c<P ^ 1>(), slot_c<1>());
+        schedule_k_step(slot_c<0>());
+    };
+
+    // Fills the pipeline for a tile: stages 0 and 1 on their way, A(0) in LDS, its first fragments read.
+    auto prime = [&]() {
+        __syncthreads(); // the previous tile's last fragment reads are done
+        load_a_all(cur, 0, slot_c<0>());
+        load_b(cur, 0, slot_c<0>(), slot_c<0>()), load_b(cur, 0, slot_c<0>(), slot_c<1>());
+        load_b(cur, 0, slot_c<0>(), slot_c<2>()), load_b(cur, 0, slot_c<0>(), slot_c<3>());
+        load_a_all(cur, 1, slot_c<1>());
+        load_b(cur, 1, slot_c<1>(), slot_c<0>()), load_b(cur, 1, slot_c<1>(), slot_c<1>());
+        load_b(cur, 1, slot_c<1>(), slot_c<2>()), load_b(cur, 1, slot_c<1>(), slot_c<3>());
+        store_a(slot_c<0>(), slot_c<0>(), 1u);
+        // the first half of A(2), as k-steps 2 and 3 of a stage "-1" would have issued it
+        // (with two stages in all it is A(0) again, which nobody uses)
+        uint32_t const third = fast > 2 ? 2 : 0;
+        load_a(cur, third, slot_c<0>(), slot_c<0>()), load_a(cur, third, slot_c<0>(), slot_c<1>());
+        __syncthreads();
+        read_frags(slot_c<0>(), slot_c<0>(), slot_c<0>());
+    };
+    if constexpr (across) {
+        cur = view_of(blockIdx.x);
+        prime();
+    }
+
+    for (uint32_t tile = blockIdx.x; tile < tile_count; tile += gridDim.x) {
+#ifdef NK_TUNE
+        unsigned long long const debug_t0 = clock64(), debug_tw0 = wall_clock64();
+        unsigned long long debug_t1 = 0, debug_t2 = 0;
+#endif
+        cur = view_of(tile);
+        bool const has_next = across && tile + gridDim.x < tile_count;
+        nxt = view_of(has_next ? tile + gridDim.x : tile);
+        uint32_t const row0 = cur.row0, col0 = cur.col0;
+
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -484,185 +717,20 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunk
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
-        // Second-level accumulators of the chunked types (see E4M3).
-        constexpr bool kChunked = T::kChunkStages > 0;
-        Totals<acc_t, TM, TN, kChunked> total;
         total.clear();
 
-        uint32_t row_sum[kLoads]; // u8 only: sum of the unsigned bytes this thread staged, per staged row
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i) row_sum[i] = 0;
-
-        if (image_ok) {
-            // A staging: thread t fetches chunk t % 8 of rows i*32 + t/8 and stores it at its swizzled position.
-            uint32_t a_off[kLoads]; // byte offset of the thread's source chunk from the tile's first row
-            uint32_t a_lds[kLoads]; // where it goes in an LDS stage
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) {
-                uint32_t const r = i * 32 + (tid >> 3);
-                uint32_t const row = row0 + r < g.m ? r : g.m - 1 - row0; // clamp to the last row; the store is masked
-                a_off[i] = row * (uint32_t)g.a_stride + a_pos * T::kSrcChunk;
-                a_lds[i] = r * kStageBytes + ((a_pos ^ ((r >> 1) & 7)) << 4);
-            }
-            uint8_t const *a_tile = g.a + (uint64_t)row0 * g.a_stride;
-
-            // Loads go through buffer descriptors: one scalar descriptor plus a 32-bit per-lane offset is the
-            // cheapest address form to issue (a single address register per lane, no 64-bit vector adds).
-            // B fragment streams of this wavefront: one descriptor per 32-column tile (tile index clamped like
-            // the rows), every lane at offset lane * 16.
-            __amdgpu_buffer_rsrc_t b_rsrc[TN];
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
-                b_rsrc[j] = __builtin_amdgcn_make_buffer_rsrc((void *)(data + (uint64_t)t * g.k_chunks * kTileChunkBytes), 0,
-                                                              (int)(g.k_chunks * kTileChunkBytes), 0x00020000);
-            }
-            uint32_t const b_lane = lane * kChunkBytes;
-            __amdgpu_buffer_rsrc_t const a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a_tile, 0, -1, 0x00020000);
-
-            v4i a_reg[2][kLoads];
-            v4i b_reg[2][TN][4];
-            v4i af[2][TM];
-
-            // A(s) -> registers, in four parts so that the loads can be spread over four k-steps.
-            auto load_a = [&](uint32_t s, auto slot_tag, auto part_tag) {
-                constexpr int slot = decltype(slot_tag)::value, part = decltype(part_tag)::value;
-                uint32_t const stage_offset = s * kSrcStage;
-#pragma unroll
-                for (int i = 0; i < kLoads; ++i) {
-                    if (i * 4 / kLoads != part) continue;
-                    v4i v = {0, 0, 0, 0};
-                    if (T::kSrcChunk == 16) {
-                        v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_off[i], stage_offset, 0));
-                    }
-                    else {
-                        typedef unsigned v2u __attribute__((ext_vector_type(2)));
-                        v2u const narrow = __builtin_amdgcn_raw_buffer_load_b64(a_rsrc, a_off[i], stage_offset, 0);
-                        v[0] = (int)narrow[0], v[1] = (int)narrow[1];
-                    }
-                    a_reg[slot][i] = v;
-                }
-            };
-            auto load_a_all = [&](uint32_t s, auto slot_tag) {
-                load_a(s, slot_tag, slot_c<0>()), load_a(s, slot_tag, slot_c<1>());
-                load_a(s, slot_tag, slot_c<2>()), load_a(s, slot_tag, slot_c<3>());
-            };
-            // Element-wise work on the staged chunks happens here, after the loads have had time to land.
-            // `real` is 0 for the clamped re-load of the last stage, which must not be counted twice.
-            auto store_a = [&](auto buffer_tag, auto slot_tag, uint32_t real) {
-                constexpr int buffer = decltype(buffer_tag)::value, slot = decltype(slot_tag)::value;
-                uint8_t *dst = lds + buffer * kStageLds;
-#pragma unroll
-                for (int i = 0; i < kLoads; ++i) {
-                    v4i v = a_reg[slot][i];
-                    if (T::kUnsigned) {
-                        row_sum[i] += sum_bytes_u8(v) * real;
-                        v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
-                    }
-                    *(v4i *)(dst + a_lds[i]) = T::widen(v);
-                }
-            };
-            auto load_b = [&](uint32_t s, auto slot_tag, auto q_tag) {
-                constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    b_reg[slot][j][q] = __builtin_bit_cast(
-                        v4i, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc[j], b_lane + q * 2 * kTileChunkBytes,
-                                                                   s * (kStageChunks * kTileChunkBytes), 0));
-            };
-            auto read_frags = [&](auto buffer_tag, auto q_tag, auto parity_tag) {
-                constexpr int buffer = decltype(buffer_tag)::value, q = decltype(q_tag)::value,
-                              parity = decltype(parity_tag)::value;
-                uint8_t const *src = lds + buffer * kStageLds + a_frag[q];
-#pragma unroll
-                for (int i = 0; i < TM; ++i) af[parity][i] = *(v4i const *)(src + i * 32 * kStageBytes);
-            };
-            auto multiply = [&](auto slot_tag, auto q_tag) {
-                constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[q & 1][i], b_reg[slot][j][q]);
-            };
-            // Scheduling hints for one k-step. Masks: 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write.
-            // Fragment reads go one-to-one with the first TM MFMAs; the global loads of the k-step (TN of B
-            // and a quarter of A) are spread over the remaining MFMAs; k-step 2 also carries the LDS writes.
-            auto schedule_k_step = [&](auto writes_tag) {
-                constexpr bool writes = decltype(writes_tag)::value != 0;
-                constexpr int loads = TN + (kLoads >= 4 ? kLoads / 4 : 1);
-                constexpr int rest = TM * (TN - 1);
-#pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                }
-                if constexpr (rest == 0) {
-                    if (writes) __builtin_amdgcn_sched_group_barrier(0x200, kLoads, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x020, loads, 0);
-                }
-                else {
-#pragma unroll
-                    for (int i = 0; i < rest; ++i) {
-                        if (writes && i < kLoads) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-                        if (i * loads / rest != (i + 1) * loads / rest || (loads > rest && i == 0))
-                            __builtin_amdgcn_sched_group_barrier(0x020, loads > rest ? loads : 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    }
-                    if (writes && kLoads > rest) __builtin_amdgcn_sched_group_barrier(0x200, kLoads - rest, 0);
-                }
-            };
-            // One stage of the steady state; `P` = stage parity = LDS buffer = register slot.
-            auto stage = [&](auto parity_tag, uint32_t s, uint32_t last) {
-                constexpr int P = decltype(parity_tag)::value;
-                uint32_t const s2 = s + 2 < last ? s + 2 : last, s3 = s + 3 < last ? s + 3 : last;
-                __builtin_amdgcn_sched_barrier(0);
-                if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
-                multiply(slot_c<P>(), slot_c<0>());
-                if (!(DBG & 1)) load_b(s2, slot_c<P>(), slot_c<0>()), load_a(s2, slot_c<P>(), slot_c<2>());
-                schedule_k_step(slot_c<0>());
-                __builtin_amdgcn_sched_barrier(0);
-                if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
-                multiply(slot_c<P>(), slot_c<1>());
-                if (!(DBG & 1)) load_b(s2, slot_c<P>(), slot_c<1>()), load_a(s2, slot_c<P>(), slot_c<3>());
-                schedule_k_step(slot_c<0>());
-                __builtin_amdgcn_sched_barrier(0);
-                if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
-                multiply(slot_c<P>(), slot_c<2>());
-                if (!(DBG & 1)) load_b(s2, slot_c<P>(), slot_c<2>());
-                // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
-                // at the previous barrier); then its registers start being refilled with A(s+3).
-                if (!(DBG & 8)) store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 <= last ? 1u : 0u);
-                if (!(DBG & 1)) load_a(s3, slot_c<P ^ 1>(), slot_c<0>());
-                schedule_k_step(slot_c<1>());
-                __builtin_amdgcn_sched_barrier(0);
-                if (!(DBG & 4)) __syncthreads();
-                __builtin_amdgcn_sched_barrier(0);
-                if (!(DBG & 2)) read_frags(slot_c<P ^ 1>(), slot_c<0>(), slot_c<0>());
-                multiply(slot_c<P>(), slot_c<3>());
-                if (!(DBG & 1)) load_b(s2, slot_c<P>(), slot_c<3>()), load_a(s3, slot_c<P ^ 1>(), slot_c<1>());
-                schedule_k_step(slot_c<0>());
-            };
-
-            __syncthreads(); // the previous tile's last fragment reads (and row terms) are done
+        {
 #ifdef NK_TUNE
             unsigned long long const debug_c0 = clock64(), debug_w0 = wall_clock64();
 #endif
             if (fast > 0) {
-                uint32_t const last = fast - 1;
-                load_a_all(0, slot_c<0>());
-                load_b(0, slot_c<0>(), slot_c<0>()), load_b(0, slot_c<0>(), slot_c<1>());
-                load_b(0, slot_c<0>(), slot_c<2>()), load_b(0, slot_c<0>(), slot_c<3>());
-                load_a_all(1, slot_c<1>());
-                load_b(1, slot_c<1>(), slot_c<0>()), load_b(1, slot_c<1>(), slot_c<1>());
-                load_b(1, slot_c<1>(), slot_c<2>()), load_b(1, slot_c<1>(), slot_c<3>());
-                store_a(slot_c<0>(), slot_c<0>(), 1u);
-                // the first half of A(2), as k-steps 2 and 3 of a stage "-1" would have issued it
-                load_a(2 < last ? 2 : last, slot_c<0>(), slot_c<0>()), load_a(2 < last ? 2 : last, slot_c<0>(), slot_c<1>());
-                __syncthreads();
-                read_frags(slot_c<0>(), slot_c<0>(), slot_c<0>());
+                if constexpr (!across) prime();
+#ifdef NK_TUNE
+                debug_t1 = clock64();
+#endif
                 for (uint32_t s = 0; s < fast; s += 2) {
-                    stage(slot_c<0>(), s, last);
-                    stage(slot_c<1>(), s + 1, last);
+                    stage(slot_c<0>(), s);
+                    stage(slot_c<1>(), s + 1);
                     if constexpr (kChunked) {
                         if ((s + 2) % T::kChunkStages == 0) {
                             __builtin_amdgcn_sched_barrier(0);
@@ -673,49 +741,60 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunk
                 __builtin_amdgcn_sched_barrier(0);
             }
 #ifdef NK_TUNE
-            if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + gridDim.x) {
+            if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + (tile_count > 45 * gridDim.x ? 40 : 1) * gridDim.x) {
                 g_debug_clocks[0] = clock64() - debug_c0, g_debug_clocks[1] = wall_clock64() - debug_w0;
                 g_debug_clocks[2] = fast;
+                g_debug_clocks[3] = debug_c0 - debug_t0, g_debug_clocks[4] = debug_t1 - debug_c0;
             }
+            debug_t2 = clock64();
 #endif
 
             // Remaining stages: the ragged end of K, or everything when A cannot be read with vector loads.
-            for (uint32_t s = fast; s < stages; ++s) {
-                __syncthreads();
-                int64_t const left = (int64_t)g.k_src_bytes - (int64_t)s * kSrcStage - (int64_t)a_pos * T::kSrcChunk;
-                int const valid = (int)(left > T::kSrcChunk ? T::kSrcChunk : (left < 0 ? 0 : left));
+            if (!across && fast < stages) {
+                uint8_t const *a_tile = g.a + (uint64_t)row0 * g.a_stride;
+                uint32_t a_slow[kLoads]; // rows clamped to the last one: plain loads have no descriptor to stop them
 #pragma unroll
                 for (int i = 0; i < kLoads; ++i) {
-                    v4i v = load_chunk_guarded(a_tile + (uint64_t)s * kSrcStage + a_off[i], valid, g.avec, 0u);
-                    if (T::kUnsigned) {
-                        row_sum[i] += sum_bytes_u8(v);
-#pragma unroll
-                        for (int w = 0; w < 4; ++w) { // flip only bytes that exist: the zero padding stays zero
-                            int const rem = valid - 4 * w;
-                            uint32_t const mask = rem >= 4 ? 0x80808080u : (rem <= 0 ? 0u : (0x80808080u >> (8 * (4 - rem))));
-                            v[w] ^= (int)mask;
-                        }
-                    }
-                    *(v4i *)(lds + a_lds[i]) = T::widen(v);
+                    uint32_t const r = i * 32 + (tid >> 3);
+                    uint32_t const row = row0 + r < g.m ? r : g.m - 1 - row0;
+                    a_slow[i] = row * (uint32_t)g.a_stride + a_pos * T::kSrcChunk;
                 }
-                load_b(s, slot_c<0>(), slot_c<0>()), load_b(s, slot_c<0>(), slot_c<1>());
-                load_b(s, slot_c<0>(), slot_c<2>()), load_b(s, slot_c<0>(), slot_c<3>());
-                __syncthreads();
-                read_frags(slot_c<0>(), slot_c<0>(), slot_c<0>());
-                read_frags(slot_c<0>(), slot_c<1>(), slot_c<1>());
-                multiply(slot_c<0>(), slot_c<0>());
-                read_frags(slot_c<0>(), slot_c<2>(), slot_c<0>());
-                multiply(slot_c<0>(), slot_c<1>());
-                read_frags(slot_c<0>(), slot_c<3>(), slot_c<1>());
-                multiply(slot_c<0>(), slot_c<2>());
-                multiply(slot_c<0>(), slot_c<3>());
+                for (uint32_t s = fast; s < stages; ++s) {
+                    __syncthreads();
+                    int64_t const left = (int64_t)g.k_src_bytes - (int64_t)s * kSrcStage - (int64_t)a_pos * T::kSrcChunk;
+                    int const valid = (int)(left > T::kSrcChunk ? T::kSrcChunk : (left < 0 ? 0 : left));
+#pragma unroll
+                    for (int i = 0; i < kLoads; ++i) {
+                        v4i v = load_chunk_guarded(a_tile + (uint64_t)s * kSrcStage + a_slow[i], valid, g.avec, 0u);
+                        if (T::kUnsigned) {
+                            row_sum[i] += sum_bytes_u8(v);
+#pragma unroll
+                            for (int w = 0; w < 4; ++w) { // flip only bytes that exist: the zero padding stays zero
+                                int const rem = valid - 4 * w;
+                                uint32_t const mask = rem >= 4 ? 0x80808080u : (rem <= 0 ? 0u : (0x80808080u >> (8 * (4 - rem))));
+                                v[w] ^= (int)mask;
+                            }
+                        }
+                        *(v4i *)(lds + a_lds[i]) = T::widen(v);
+                    }
+                    load_b(cur, s, slot_c<0>(), slot_c<0>()), load_b(cur, s, slot_c<0>(), slot_c<1>());
+                    load_b(cur, s, slot_c<0>(), slot_c<2>()), load_b(cur, s, slot_c<0>(), slot_c<3>());
+                    __syncthreads();
+                    read_frags(slot_c<0>(), slot_c<0>(), slot_c<0>());
+                    read_frags(slot_c<0>(), slot_c<1>(), slot_c<1>());
+                    multiply(slot_c<0>(), slot_c<0>());
+                    read_frags(slot_c<0>(), slot_c<2>(), slot_c<0>());
+                    multiply(slot_c<0>(), slot_c<1>());
+                    read_frags(slot_c<0>(), slot_c<3>(), slot_c<1>());
+                    multiply(slot_c<0>(), slot_c<2>());
+                    multiply(slot_c<0>(), slot_c<3>());
+                }
             }
         }
 
         // Epilogue. Accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.
         uint32_t const half = lane >> 5, col_in_tile = lane & 31;
-        uint32_t *row_terms = (uint32_t *)lds;
-        if (T::kUnsigned && image_ok) {
+        if (T::kUnsigned) {
             __syncthreads();
             // The 8 threads that staged one row hold its partial byte sums in adjacent lanes.
 #pragma unroll
@@ -725,51 +804,59 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunk
                 s += __shfl_xor(s, 2, 64);
                 s += __shfl_xor(s, 4, 64);
                 if ((tid & 7) == 0) row_terms[i * 32 + (tid >> 3)] = s * 128u;
+                row_sum[i] = across ? row_sum_next[i] : 0u, row_sum_next[i] = 0;
             }
             __syncthreads();
         }
-        // Stores: a scalar base plus one per-lane offset, so that no 64-bit address ever lives in vector
-        // registers. Tiles that touch the matrix edge take the masked copy of the loop.
+        // Stores: a scalar base plus one 32-bit per-lane offset, through an explicitly global pointer. (A store
+        // through a generic pointer counts as an LDS operation as well, and with such stores in flight the
+        // loads prefetched for the next tile could only be waited for all at once.) Tiles that touch the
+        // matrix edge take the masked copy of the loop.
         bool const interior = row0 + BM <= g.m && col0 + 32 * TN <= g.n;
-        uint8_t *c_tile = g.c + (uint64_t)row0 * g.c_stride + (uint64_t)col0 * 4;
+        global_u8_t *c_tile = (global_u8_t *)g.c + (uint64_t)row0 * g.c_stride + (uint64_t)col0 * 4;
         auto store_all = [&](auto masked_tag) {
             constexpr bool masked = decltype(masked_tag)::value != 0;
             uint64_t const row_step = g.c_stride;
-            {
-                // Lane l holds column l % 32; register v holds row 8 * (v / 4) + 4 * (l / 32) + v % 4.
-                uint32_t const lane_offset = 4 * half * (uint32_t)g.c_stride + col_in_tile * 4;
+            // Lane l holds column l % 32; register v holds row 8 * (v / 4) + 4 * (l / 32) + v % 4.
+            uint32_t const lane_offset = 4 * half * (uint32_t)g.c_stride + col_in_tile * 4;
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    uint32_t col_term = 0;
-                    if (T::kUnsigned && image_ok) {
-                        uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
-                        col_term = col_terms[(uint64_t)t * kTileRows + col_in_tile];
-                    }
-                    bool const col_ok = col0 + j * 32 + col_in_tile < g.n;
-                    // Rows come in runs of 4 that start 8 apart: the base advances by one row or by five. The
-                    // empty asm keeps it a running scalar (otherwise every row's base is precomputed and the
-                    // scalar registers overflow).
-                    uint8_t *row_base = c_tile + j * 128;
+            for (int j = 0; j < TN; ++j) {
+                uint32_t col_term = 0;
+                if (T::kUnsigned) {
+                    uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
+                    col_term = col_terms[(uint64_t)t * kTileRows + col_in_tile];
+                }
+                bool const col_ok = col0 + j * 32 + col_in_tile < g.n;
+                // Rows come in runs of 4 that start 8 apart: the base advances by one row or by five. The
+                // empty asm keeps it a running scalar (otherwise every row's base is precomputed and the
+                // scalar registers overflow).
+                global_u8_t *row_base = c_tile + j * 128;
 #pragma unroll
-                    for (int i = 0; i < TM; ++i) {
+                for (int i = 0; i < TM; ++i) {
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            int const r_fixed = i * 32 + 8 * (v / 4) + (v % 4); // row of lanes 0..31; lanes 32..63 are 4 rows below
-                            // a named copy: bit-casting the vector element expression itself reads lane 0
-                            auto const element = total.finish(acc, i, j, v);
-                            uint32_t bits = __builtin_bit_cast(uint32_t, element);
-                            if (T::kUnsigned) bits += row_terms[r_fixed + 4 * half] + col_term;
-                            if (!image_ok) bits = 0xFFFFFFFFu;
-                            if (!masked || (col_ok && row0 + r_fixed + 4 * half < g.m)) *(uint32_t *)(row_base + lane_offset) = bits;
-                            row_base += (v % 4 == 3 ? 5 : 1) * row_step;
-                            asm volatile("" : "+s"(row_base));
-                        }
+                    for (int v = 0; v < 16; ++v) {
+                        int const r_fixed = i * 32 + 8 * (v / 4) + (v % 4); // row of lanes 0..31; lanes 32..63 are 4 rows below
+                        // a named copy: bit-casting the vector element expression itself reads lane 0
+                        auto const element = total.finish(acc, i, j, v);
+                        uint32_t bits = __builtin_bit_cast(uint32_t, element);
+                        if (T::kUnsigned) bits += row_terms[r_fixed + 4 * half] + col_term;
+                        if ((!(DBG & 16) || bits == 0x12345678u) && // (timing experiment: almost no stores)
+                            (!masked || (col_ok && row0 + r_fixed + 4 * half < g.m)))
+                            *(global_u32_t *)(row_base + lane_offset) = bits;
+                        row_base += (v % 4 == 3 ? 5 : 1) * row_step;
+                        asm volatile("" : "+s"(row_base));
                     }
                 }
             }
         };
         if (interior) store_all(slot_c<0>());
         else store_all(slot_c<1>());
+#ifdef NK_TUNE
+        if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + (g.tiles_m * g.tiles_n > 45 * gridDim.x ? 40 : 1) * gridDim.x) {
+            g_debug_clocks[5] = clock64() - debug_t2, g_debug_clocks[6] = clock64() - debug_t0;
+            g_debug_clocks[7] = wall_clock64() - debug_tw0;
+        }
+#endif
     }
 }
 
@@ -795,24 +882,29 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream) {
     if ((uint64_t)BM * g.a_stride > 0xFFFFFFFFull) return hipErrorInvalidValue;
     // So are the per-lane C offsets: 4 rows plus the tile's width.
     if (4 * (uint64_t)g.c_stride + BN * 4 > 0xFFFFFFFFull) return hipErrorInvalidValue;
-    void (*kernel)(GemmArgs) = dots_packed_kernel<T, TM, TN>;
+    // The offsets into a wavefront's B tiles are 32-bit as well.
+    if ((uint64_t)(TN + 1) * g.k_chunks * kTileChunkBytes > 0xFFFFFFFFull) return hipErrorInvalidValue;
+    // The pipeline runs across tile boundaries when the pipelined loop takes every stage of a tile: A readable
+    // with dword loads, K a whole and even number of stages, and enough of them to prefetch three ahead.
+    uint32_t const stages = g.k_chunks / kStageChunks;
+    bool const across = g.avec >= 4 && g.k_src_bytes == (uint64_t)stages * kStageChunks * T::kSrcChunk &&
+                        stages % 2 == 0 && stages >= 4 && !(g_variant & 1);
+    void (*kernel)(GemmArgs) = across ? dots_packed_kernel<T, TM, TN, true> : dots_packed_kernel<T, TM, TN, false>;
 #ifdef NK_TUNE // timing experiments that leave parts of the loop out (results are wrong on purpose)
     if constexpr (TM == 8 && TN == 2 && T::kDtype == kI8) {
         switch (g_variant >> 2) {
-        case 1: kernel = dots_packed_kernel<T, TM, TN, 1>; break;
-        case 2: kernel = dots_packed_kernel<T, TM, TN, 2>; break;
-        case 3: kernel = dots_packed_kernel<T, TM, TN, 3>; break;
-        case 4: kernel = dots_packed_kernel<T, TM, TN, 4>; break;
-        case 5: kernel = dots_packed_kernel<T, TM, TN, 7>; break;
-        case 6: kernel = dots_packed_kernel<T, TM, TN, 15>; break;
-        case 7: kernel = dots_packed_kernel<T, TM, TN, 8>; break;
-        case 8: kernel = dots_packed_kernel<T, TM, TN, 9>; break;
+        case 1: kernel = dots_packed_kernel<T, TM, TN, false, 1>; break;
+        case 2: kernel = dots_packed_kernel<T, TM, TN, false, 2>; break;
+        case 3: kernel = dots_packed_kernel<T, TM, TN, false, 4>; break;
+        case 4: kernel = dots_packed_kernel<T, TM, TN, false, 16>; break;
+        case 5: kernel = dots_packed_kernel<T, TM, TN, false, 17>; break;
         default: break;
         }
     }
 #endif
     // Persistent grid: as many workgroups as fit on the device at once (queried once per kernel).
-    static int resident = 0;
+    static int resident_of[2] = {0, 0};
+    int &resident = resident_of[across ? 1 : 0];
     if (!resident) {
         int per_cu = 0, device = 0;
         hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (void const *)kernel, 256, 0);
