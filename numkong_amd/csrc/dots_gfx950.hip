@@ -264,12 +264,25 @@ __global__ __launch_bounds__(256) void fill_rows_kernel(uint8_t *c, uint32_t m, 
 
 #pragma region Element types
 
-#ifndef NK_HALF_CHUNK_STAGES
-#define NK_HALF_CHUNK_STAGES 0
+/**
+ *  Float accumulation. One MFMA accumulator rounds once per 8 products at the magnitude of the whole running
+ *  sum; over a depth of thousands that is 1.4x the error of the reference's scalar kernel for bf16 (4 lanes,
+ *  dot/serial.h:406-439), 3x that of its 16-lane AVX-512 kernels (dot/genoa.h:237-256), and 4x the scalar
+ *  kernel's for fp8, whose products and short sums are exact in f32 (dot/serial.h:522-600). The float types
+ *  therefore fold the accumulator into a second one every `chunk_stages` stages (about an eighth of the depth,
+ *  at most 16 stages = 1024 values): the running sums stay short, and the error drops to that of the reference's
+ *  best kernels (measured ratios next to the tests). Two accumulator sets do not fit the 256 x 256 tile, so
+ *  these types stop at 128 x 256. NK_HALF_SINGLE_ACCUMULATOR builds bf16/f16 without the second set (faster,
+ *  less accurate; for comparison only).
+ */
+#ifdef NK_HALF_SINGLE_ACCUMULATOR
+constexpr bool kHalfChunked = false;
+#else
+constexpr bool kHalfChunked = true;
 #endif
 
 struct I8 {
-    static constexpr int kChunkStages = 0; // > 0: fold the accumulator into a second one every so many stages
+    static constexpr bool kChunked = false; // fold the accumulator into a second one every few stages
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16i acc_t;
@@ -284,7 +297,7 @@ struct U8 : I8 {
     static constexpr bool kUnsigned = true;
 };
 struct BF16 {
-    static constexpr int kChunkStages = NK_HALF_CHUNK_STAGES;
+    static constexpr bool kChunked = kHalfChunked;
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
@@ -296,7 +309,7 @@ struct BF16 {
     }
 };
 struct F16 {
-    static constexpr int kChunkStages = NK_HALF_CHUNK_STAGES;
+    static constexpr bool kChunked = kHalfChunked;
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
@@ -307,19 +320,15 @@ struct F16 {
                                                      0);
     }
 };
-/** fp8 products and short sums are exact in f32, so the reference's scalar kernel loses almost nothing
- *  (dot/serial.h:522-600: 4 lanes, 8e-9 of sum|a*b| at depth 8192), while one MFMA accumulator rounds once
- *  per 8 products at the magnitude of the whole running sum (3e-8). Folding the accumulator into a second
- *  one every 16 stages (1024 values) keeps the running sums short and brings the error under the scalar
- *  kernel's own. */
+/** fp8 runs widened to f16 (exact), on the f16 MFMA; see widen_fp8x8. */
 struct E4M3 : F16 {
-    static constexpr int kChunkStages = 16;
+    static constexpr bool kChunked = true;
     static constexpr int kDtype = kE4M3;
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<false>((uint32_t)v[0], (uint32_t)v[1]); }
 };
 struct E5M2 : F16 {
-    static constexpr int kChunkStages = 16;
+    static constexpr bool kChunked = true;
     static constexpr int kDtype = kE5M2;
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<true>((uint32_t)v[0], (uint32_t)v[1]); }
@@ -380,6 +389,7 @@ struct GemmArgs {
     uint32_t n_tiles, k_chunks;
     uint32_t tiles_m, tiles_n;
     int avec; // widest load the A pointer and stride allow (1, 2, 4, 8 or 16 bytes)
+    uint32_t chunk_stages; // chunked types: stages between folds of the accumulator (even, 2..16)
 };
 
 /**
@@ -433,7 +443,7 @@ __device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, ui
  *  12 % slower on the square shapes and 9 % slower on the retrieval shape.)
  */
 template <class T, int TM, int TN, bool ACROSS, int DBG = 0>
-__global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunkStages == 0 ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChunked ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
     typedef typename T::acc_t acc_t;
     constexpr int BM = TM * 32;
     constexpr int NT = 256;
@@ -549,7 +559,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunk
     }
     TileView cur, nxt;
     acc_t acc[TM][TN];
-    constexpr bool kChunked = T::kChunkStages > 0;
+    constexpr bool kChunked = T::kChunked;
     Totals<acc_t, TM, TN, kChunked> total; // second-level accumulators of the chunked types (see E4M3)
 
     // A(s) -> registers, in four parts so that the loads can be spread over four k-steps.
@@ -728,13 +738,16 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && T::kChunk
 #ifdef NK_TUNE
                 debug_t1 = clock64();
 #endif
+                uint32_t until_fold = g.chunk_stages;
                 for (uint32_t s = 0; s < fast; s += 2) {
                     stage(slot_c<0>(), s);
                     stage(slot_c<1>(), s + 1);
                     if constexpr (kChunked) {
-                        if ((s + 2) % T::kChunkStages == 0) {
+                        until_fold -= 2;
+                        if (until_fold == 0) {
                             __builtin_amdgcn_sched_barrier(0);
                             total.fold(acc);
+                            until_fold = g.chunk_stages;
                         }
                     }
                 }
@@ -931,17 +944,17 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream) {
             uint64_t const bm = kConfigs[c].tm * 32, bn = (uint64_t)kConfigs[c].tn * 128;
             return ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
         };
-        config = kConfigCount - 1;
-        for (int c = 1; c < kConfigCount; ++c)
+        config = 4;
+        for (int c = 1; c <= 4; ++c)
             if (tiles(c) >= 256) {
                 config = c;
                 break;
             }
     }
-    if (T::kChunkStages > 0 && config == 1) config = 2; // two accumulator sets do not fit the 256 x 256 tile
+    if (T::kChunked && config == 1) config = 2; // two accumulator sets do not fit the 256 x 256 tile
     switch (config) {
     case 1:
-        if constexpr (T::kChunkStages > 0) return hipErrorInvalidValue;
+        if constexpr (T::kChunked) return hipErrorInvalidValue;
         else return launch_one<T, 8, 2>(g, stream);
     case 2: return launch_one<T, 4, 2>(g, stream);
     case 3: return launch_one<T, 4, 1>(g, stream);
@@ -1112,6 +1125,11 @@ int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, voi
     g.a_stride = a_stride, g.c_stride = c_stride, g.k_src_bytes = geo.k_src_bytes;
     g.m = (uint32_t)m, g.n = geo.n, g.k = geo.k, g.n_tiles = geo.n_tiles, g.k_chunks = geo.k_chunks;
     g.avec = widest_load(a, a_stride);
+    {
+        // Stages between accumulator folds: about an eighth of the depth, even, between 2 and 16.
+        uint32_t const eighth = (g.k_chunks / kStageChunks / 8) & ~1u;
+        g.chunk_stages = eighth < 2 ? 2 : (eighth > 16 ? 16 : eighth);
+    }
 
     hipError_t e;
     switch (dtype) {

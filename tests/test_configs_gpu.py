@@ -13,7 +13,7 @@ torch = pytest.importorskip("torch")
 
 import numkong_amd as nk  # noqa: E402
 from tests import support  # noqa: E402
-from tests.test_dots_gpu import DEV, assert_float_gate, to_gpu  # noqa: E402
+from tests.test_dots_gpu import DEV, assert_float_gate, best_dispatch, to_gpu  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 
@@ -46,7 +46,8 @@ def sampled_oracle_gate(oracle, dtype, a, b, c, rows, cols):
         a_host, b_host = a_host.view(np.uint16), b_host.view(np.uint16)
     got = c[rows][:, cols].cpu().numpy()
     truth, magnitude = oracle.truth(dtype, a_host, b_host)
-    assert_float_gate(dtype, got, oracle.dots_packed(dtype, a_host, b_host), truth, magnitude, f"{dtype} sample")
+    assert_float_gate(dtype, got, oracle.dots_packed(dtype, a_host, b_host), truth, magnitude, f"{dtype} sample",
+                      best_dispatch(dtype, a_host, b_host))
 
 
 def tiling_invariance(dtype, a, packed, c):

@@ -1,18 +1,20 @@
 """Parity of the gfx950 kernels with the reference semantics, through the C ABI, on a real MI355X.
 
 Integers must be bit-exact (the reference's integer backends all equal the exact product mod 2^32).
-Floats are compared with the f64 ground truth next to the reference's serial kernel as restated by the
-oracle (which tests/test_oracle.py pins bit-for-bit against the reference library):
+Floats are compared with the f64 ground truth next to TWO reference CPU kernels on the same inputs: the serial
+kernel as restated by the oracle (which tests/test_oracle.py pins bit-for-bit against the reference library),
+and, when the reference build oracle/_ref is present, the kernel the reference dispatches to on this host
+(16-lane AVX-512 on the GPU boxes). The gate is the tighter of the two:
 
   normwise error  e = |c - truth| / sum|a*b|   per element, over elements with a finite truth
-  gate:  mean(e_gpu) <= 2 * mean(e_serial)                 (plus 1e-3 ulp of slack when both are ~0)
-         max(e_gpu)  <= 2 * max(max(e_serial), 2^-24)      (one f32 rounding unit of the magnitude sum)
-         NaN, +Inf and -Inf masks identical to the serial kernel's.
+  gate:  mean(e_gpu) <= 2 * mean(e_ref) + 2^-24 / sqrt(count)   (the slack only matters for a handful of outputs)
+         max(e_gpu)  <= 2 * max(max(e_ref), 2^-24)         (one f32 rounding unit of the magnitude sum)
+         NaN, +Inf and -Inf masks identical to the serial kernel's (the reference's AVX-512 e5m2 kernels do
+         not propagate Inf/NaN, so masks are not compared with them and their non-finite outputs are skipped).
 
-The 2^-24 floor keeps the max statistic meaningful on small samples, where both kernels sit at a single
-rounding of the result, and it is what decides e4m3 at depth 8192: there the serial kernel's lane sums stay
-exact far longer than the MFMA's accumulator (one rounding per 8 products at the magnitude of the whole
-running sum), 8e-9 against 3e-8 measured, both far below the floor.
+The 2^-24 floor keeps the max statistic meaningful on small samples, where all kernels sit at a single
+rounding of the result. Measured on 192 x 256 outputs at depth 4096-8192 (GPU / serial, GPU / dispatched, mean
+of the normwise error): bf16 0.52-0.56, 1.13; f16 0.27, 0.52; e4m3 0.96, 1.16; e5m2 0.99, 1.13.
 """
 import ctypes
 import os
@@ -50,17 +52,32 @@ def gpu_dots(dtype, a, b, config=0):
     return out.view(np.uint32) if dtype == "u8" else out
 
 
-def assert_float_gate(dtype, got, serial, truth, magnitude, where=""):
+_REFERENCE = []
+
+
+def best_dispatch(dtype, a, b):
+    """The same product by the kernel the reference library dispatches to on this host, or None without the build."""
+    if not _REFERENCE:
+        _REFERENCE.append(support.load_reference())
+    reference = _REFERENCE[0]
+    return None if reference is None else reference.dots_packed(dtype, a, b, viable=reference.capabilities)
+
+
+def assert_float_gate(dtype, got, serial, truth, magnitude, where="", dispatched=None):
     assert np.array_equal(np.isnan(got), np.isnan(serial)), f"NaN mask differs {where}"
     assert np.array_equal(np.isposinf(got), np.isposinf(serial)), f"+Inf mask differs {where}"
     assert np.array_equal(np.isneginf(got), np.isneginf(serial)), f"-Inf mask differs {where}"
-    finite = np.isfinite(truth) & (magnitude > 0)
-    if not finite.any():
-        return
-    e_gpu = np.abs(got[finite].astype(np.float64) - truth[finite]) / magnitude[finite]
-    e_ref = np.abs(serial[finite].astype(np.float64) - truth[finite]) / magnitude[finite]
-    assert e_gpu.mean() <= 2 * e_ref.mean() + 1e-3 * U, f"mean error {e_gpu.mean():.3e} vs serial {e_ref.mean():.3e} {where}"
-    assert e_gpu.max() <= 2 * max(e_ref.max(), U), f"max error {e_gpu.max():.3e} vs serial {e_ref.max():.3e} {where}"
+    for name, ref in (("serial", serial), ("dispatched", dispatched)):
+        if ref is None:
+            continue
+        finite = np.isfinite(truth) & (magnitude > 0) & np.isfinite(ref)
+        if not finite.any():
+            continue
+        e_gpu = np.abs(got[finite].astype(np.float64) - truth[finite]) / magnitude[finite]
+        e_ref = np.abs(ref[finite].astype(np.float64) - truth[finite]) / magnitude[finite]
+        slack = U / np.sqrt(e_gpu.size)  # the standard error of a mean of single-rounding errors: decides tiny samples only
+        assert e_gpu.mean() <= 2 * e_ref.mean() + slack, f"mean error {e_gpu.mean():.3e} vs {name} {e_ref.mean():.3e} {where}"
+        assert e_gpu.max() <= 2 * max(e_ref.max(), U), f"max error {e_gpu.max():.3e} vs {name} {e_ref.max():.3e} {where}"
 
 
 def check(oracle, dtype, a, b, config=0, where=""):
@@ -71,7 +88,7 @@ def check(oracle, dtype, a, b, config=0, where=""):
         assert np.array_equal(got.view(np.uint32), oracle.dots_packed(dtype, a, b).view(np.uint32)), where
     else:
         truth, magnitude = oracle.truth(dtype, a, b)
-        assert_float_gate(dtype, got, oracle.dots_packed(dtype, a, b), truth, magnitude, where)
+        assert_float_gate(dtype, got, oracle.dots_packed(dtype, a, b), truth, magnitude, where, best_dispatch(dtype, a, b))
 
 
 SHAPES = [(1, 1, 1), (3, 5, 7), (33, 70, 200), (64, 64, 64), (100, 37, 333), (257, 129, 1000), (31, 300, 129), (130, 33, 4100)]
@@ -108,7 +125,7 @@ def test_golden_vectors(oracle, name):
         assert np.array_equal(got.view(np.uint32), c_serial.view(np.uint32))
     else:
         truth, magnitude = oracle.truth(dtype, a, b)
-        assert_float_gate(dtype, got, c_serial, truth, magnitude, name)
+        assert_float_gate(dtype, got, c_serial, truth, magnitude, name, best_dispatch(dtype, a, b))
 
 
 @pytest.mark.parametrize("dtype", ["e4m3", "e5m2"])
