@@ -61,7 +61,7 @@ enum : int {
 };
 
 constexpr uint32_t kMagic = 0x35394B4Eu; // "NK95"
-constexpr uint32_t kVersion = 1;
+constexpr uint32_t kVersion = 2;
 constexpr int kChunkBytes = 16;   // bytes of K per lane per operand load
 constexpr int kTileRows = 32;     // B rows per tile = MFMA N
 constexpr int kStageChunks = 8;   // chunks of K per pipeline stage (128 bytes per row)
@@ -119,7 +119,7 @@ inline bool make_geometry(int dtype, size_t n, size_t k, Geometry &g) {
     g.k_bytes = (uint64_t)k * g.packed_bytes;
     g.k_src_bytes = (uint64_t)k * eb;
     uint64_t const chunks = (g.k_bytes + kChunkBytes - 1) / kChunkBytes;
-    g.k_chunks = (uint32_t)((chunks + kStageChunks - 1) / kStageChunks * kStageChunks);
+    g.k_chunks = (uint32_t)((chunks + 2 * kStageChunks - 1) / (2 * kStageChunks) * (2 * kStageChunks)); // an even number of stages
     g.n_tiles = (uint32_t)((n + kTileRows - 1) / kTileRows);
     g.data_bytes = (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes;
     g.sums_bytes = (uint64_t)g.n_tiles * kTileRows * sizeof(uint32_t);
@@ -433,8 +433,10 @@ __device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, ui
  *      k-step 2 also moves A(s+1), loaded two stages ago, from registers into the other LDS buffer and
  *               refills those registers with A(s+3)
  *      before the last k-step: one barrier; the first fragments of stage s+1 are read under its MFMAs
- *  An odd last whole stage, a stage that is not whole, and every stage when A is not even dword-aligned, run
- *  afterwards through a plain guarded loop.
+ *  The packed image pads K with zeros to an even number of stages; on the A side, the bytes a stage reads
+ *  past the end of a row (the next row's, or nothing past the end of the matrix) are masked to zero on their
+ *  way into LDS, so ragged depths run through the same loop. Only A that is not even dword-aligned takes a
+ *  plain guarded loop instead.
  *
  *  A is the MFMA's first operand, so a lane ends up with one column and 16 rows of each 32x32 block and the
  *  epilogue stores dwords that are contiguous across lanes: 128 bytes per row per instruction, any C
@@ -466,11 +468,10 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     uint32_t const *col_terms = (uint32_t const *)(data + (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes);
 
     uint32_t const stages = g.k_chunks / kStageChunks;
-    uint32_t const whole = (uint32_t)(g.k_src_bytes / kSrcStage); // stages with all 128 bytes present
-    // Stages the pipelined loop takes: the whole ones, in pairs, when A is at least dword-aligned, which is
-    // all that multi-dword global loads need. (readfirstlane: the value is uniform, and it must stay in a scalar
-    // register because the stage offsets of the buffer loads derive from it.)
-    uint32_t const fast = __builtin_amdgcn_readfirstlane((g.avec >= 4 ? whole : 0) & ~1u);
+    // Stages the pipelined loop takes: all of them when A is at least dword-aligned, which is all that
+    // multi-dword global loads need. (readfirstlane: the value is uniform, and it must stay in a scalar register
+    // because the stage offsets of the buffer loads derive from it.)
+    uint32_t const fast = __builtin_amdgcn_readfirstlane(g.avec >= 4 ? stages : 0);
     uint32_t const xr = T::kUnsigned ? 0x80808080u : 0u;
     uint32_t const a_pos = tid & 7;
     // A fragment reads: lane l takes row l % 32 of each 32-row block and chunk 2q + l / 32.
@@ -514,7 +515,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         view.col0 = tile_n * (128 * TN) + wave * (32 * TN);
         uint32_t const rows_here = g.m - view.row0 < (uint32_t)BM ? g.m - view.row0 : (uint32_t)BM;
         view.a = g.a + (uint64_t)view.row0 * g.a_stride;
-        view.a_bytes = (rows_here - 1) * (uint32_t)g.a_stride + (uint32_t)g.k_src_bytes;
+        // (whole dwords: a dword-aligned A never ends in the middle of one that could fault)
+        view.a_bytes = (rows_here - 1) * (uint32_t)g.a_stride + (((uint32_t)g.k_src_bytes + 3u) & ~3u);
         uint32_t const tile_bytes = g.k_chunks * kTileChunkBytes;
         uint32_t const first = view.col0 / 32 < g.n_tiles ? view.col0 / 32 : g.n_tiles - 1;
         view.b = data + (uint64_t)first * tile_bytes;
@@ -588,12 +590,24 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     };
     // Element-wise work on the staged chunks happens here, after the loads have had time to land.
     // `mine` is 1 for a stage of this tile and 0 for one staged ahead for the next tile.
-    auto store_a = [&](auto buffer_tag, auto slot_tag, uint32_t mine) {
+    // `s` is the stage the registers hold: the bytes of its chunk that lie past the end of the row are cleared
+    // (for whole stages the masks come out as all ones; no branch either way).
+    int const a_tail = (int)(uint32_t)g.k_src_bytes - (int)(a_pos * T::kSrcChunk); // bytes of the row from this thread's chunk on, stage 0
+    auto store_a = [&](auto buffer_tag, auto slot_tag, uint32_t s, uint32_t mine) {
         constexpr int buffer = decltype(buffer_tag)::value, slot = decltype(slot_tag)::value;
         uint8_t *dst = lds + buffer * kStageLds;
+        int const left = a_tail - (int)(s * kSrcStage);
+        uint32_t keep[T::kSrcChunk / 4];
+#pragma unroll
+        for (int w = 0; w < T::kSrcChunk / 4; ++w) {
+            int const over = left - 4 * w, bytes = over < 0 ? 0 : (over > 4 ? 4 : over);
+            keep[w] = bytes == 4 ? 0xFFFFFFFFu : ((1u << (8 * bytes)) - 1u);
+        }
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             v4i v = a_reg[slot][i];
+#pragma unroll
+            for (int w = 0; w < T::kSrcChunk / 4; ++w) v[w] &= (int)keep[w];
             if (T::kUnsigned) {
                 uint32_t const sum = sum_bytes_u8(v);
                 row_sum[i] += sum * mine, row_sum_next[i] += sum * (1u - mine);
@@ -676,7 +690,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<2>());
         // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
         // at the previous barrier); then its registers start being refilled with A(s+3).
-        if (!(DBG & 8)) store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 < fast ? 1u : 0u);
+        if (!(DBG & 8)) store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, s + 1 < fast ? 1u : 0u);
         if (!(DBG & 1)) load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
         schedule_k_step(slot_c<1>());
         __builtin_amdgcn_sched_barrier(0);
@@ -697,7 +711,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         load_a_all(cur, 1, slot_c<1>());
         load_b(cur, 1, slot_c<1>(), slot_c<0>()), load_b(cur, 1, slot_c<1>(), slot_c<1>());
         load_b(cur, 1, slot_c<1>(), slot_c<2>()), load_b(cur, 1, slot_c<1>(), slot_c<3>());
-        store_a(slot_c<0>(), slot_c<0>(), 1u);
+        store_a(slot_c<0>(), slot_c<0>(), 0u, 1u);
         // the first half of A(2), as k-steps 2 and 3 of a stage "-1" would have issued it
         // (with two stages in all it is A(0) again, which nobody uses)
         uint32_t const third = fast > 2 ? 2 : 0;
@@ -897,11 +911,10 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream) {
     if (4 * (uint64_t)g.c_stride + BN * 4 > 0xFFFFFFFFull) return hipErrorInvalidValue;
     // The offsets into a wavefront's B tiles are 32-bit as well.
     if ((uint64_t)(TN + 1) * g.k_chunks * kTileChunkBytes > 0xFFFFFFFFull) return hipErrorInvalidValue;
-    // The pipeline runs across tile boundaries when the pipelined loop takes every stage of a tile: A readable
-    // with dword loads, K a whole and even number of stages, and enough of them to prefetch three ahead.
+    // The pipeline runs across tile boundaries when the pipelined loop takes the stages of a tile (A readable
+    // with dword loads) and there are enough of them to prefetch three ahead.
     uint32_t const stages = g.k_chunks / kStageChunks;
-    bool const across = g.avec >= 4 && g.k_src_bytes == (uint64_t)stages * kStageChunks * T::kSrcChunk &&
-                        stages % 2 == 0 && stages >= 4 && !(g_variant & 1);
+    bool const across = g.avec >= 4 && stages >= 4 && !(g_variant & 1);
     void (*kernel)(GemmArgs) = across ? dots_packed_kernel<T, TM, TN, true> : dots_packed_kernel<T, TM, TN, false>;
 #ifdef NK_TUNE // timing experiments that leave parts of the loop out (results are wrong on purpose)
     if constexpr (TM == 8 && TN == 2 && T::kDtype == kI8) {

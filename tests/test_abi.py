@@ -39,11 +39,12 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_packed_size_formula():
-    """header + ceil(n/32) tiles * padded chunks * 512 B + 128 B of column terms per tile; fp8 stored as f16."""
+    """header + ceil(n/32) tiles * chunks (padded to an even number of 8-chunk stages) * 512 B + 128 B of column
+    terms per tile; fp8 stored as f16."""
     for t, width in (("i8", 1), ("u8", 1), ("bf16", 2), ("f16", 2), ("e4m3", 2), ("e5m2", 2)):
         for n, k in [(1, 1), (32, 128), (33, 129), (2048, 2048), (8191, 1000), (1048576, 768)]:
             tiles = -(-n // 32)
-            chunks = -(-(-(-k * width // 16)) // 8) * 8
+            chunks = -(-(-(-k * width // 16)) // 16) * 16
             assert nk.dots_packed_size(t, n, k) == 64 + tiles * chunks * 512 + tiles * 128, (t, n, k)
         assert nk.dots_packed_size(t, 0, 0) == 64
         assert nk.dots_packed_size(t, 1 << 40, 8) == 0  # dimensions beyond 32 bits are refused, as the error stub does
@@ -101,7 +102,7 @@ def test_error_convention_without_backend():
         assert np.isnan(f[:, :3]).all() and (f[:, 3] == 0).all()
     finally:
         lib.nk_dispatch_table_update(lib.nk_capabilities_compiled())
-    assert lib.nk_dots_packed_size_i8(5, 7) == 64 + 8 * 512 + 128
+    assert lib.nk_dots_packed_size_i8(5, 7) == 64 + 16 * 512 + 128
 
 
 def test_no_gpu_means_loud_failure_not_fallback():
