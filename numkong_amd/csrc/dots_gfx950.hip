@@ -453,7 +453,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     constexpr int kLoads = BM * kStageChunks / NT; // 16-byte LDS chunks per thread per stage = TM
     constexpr int kSrcStage = kStageChunks * T::kSrcChunk; // source bytes of A per row per stage
     __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStageLds];
-    __shared__ uint32_t row_terms[T::kUnsigned ? BM : 1]; // u8 only: 128 * (sum of the bytes of each A row of the tile)
+    __shared__ __attribute__((aligned(16))) uint32_t row_terms[T::kUnsigned ? BM : 4]; // u8 only: 128 * (sum of the bytes of each A row of the tile)
+    __shared__ uint32_t row_part[T::kUnsigned ? 2 * BM * kStageChunks : 1]; // u8 only: the partial sums behind them
 
     uint32_t const tid = threadIdx.x, lane = tid & 63;
     // The wavefront index is the same in all lanes; telling the compiler keeps B addressing in scalar registers.
@@ -538,10 +539,17 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // and then runs across tile boundaries, and the stores of one tile drain under the next tile's MFMAs.
     constexpr bool across = ACROSS; // the host checks that it holds: fast == stages and stages >= 4
     uint32_t const tile_count = g.tiles_m * g.tiles_n;
-    uint32_t row_sum[kLoads]; // u8 only: sum of the unsigned bytes this thread staged, per staged row
-    uint32_t row_sum_next[kLoads]; // ... of the chunks it staged ahead for the next tile
+    // u8 only: every thread sums the unsigned bytes it stages, per staged row, in LDS slots of its own (slot
+    // i * 256 + tid: fire-and-forget LDS adds instead of 2 x kLoads registers held through the loop). Two sets:
+    // what is staged ahead for the next tile goes to the other one, and the sets swap roles with every tile.
+    uint32_t sums_here = 0; // offset of the set of the tile being computed
+    if (T::kUnsigned) {
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) row_sum[i] = 0, row_sum_next[i] = 0;
+        for (int i = 0; i < 2 * kLoads; ++i) row_part[i * NT + tid] = 0;
+    }
+    auto add_row_sum = [&](int i, uint32_t value, uint32_t set) {
+        __hip_atomic_fetch_add(&row_part[set + i * NT + tid], value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
     v4i a_reg[2][kLoads];
     v4i b_reg[2][TN][4];
     v4i af[2][TM];
@@ -610,7 +618,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             for (int w = 0; w < T::kSrcChunk / 4; ++w) v[w] &= (int)keep[w];
             if (T::kUnsigned) {
                 uint32_t const sum = sum_bytes_u8(v);
-                row_sum[i] += sum * mine, row_sum_next[i] += sum * (1u - mine);
+                // (without a next tile to stage for, what is staged past the end is dropped)
+                add_row_sum(i, across ? sum : sum * mine, across && !mine ? sums_here ^ (uint32_t)(kLoads * NT) : sums_here);
                 v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
             }
             *(v4i *)(dst + a_lds[i]) = T::widen(v);
@@ -740,14 +749,24 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-
+        // u8: the column terms of this tile are fetched now and used in the epilogue, so that nothing has to
+        // wait for them (a wait for a load is a wait for every store issued before it).
+        uint32_t col_term[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            col_term[j] = 0;
+            if constexpr (T::kUnsigned) {
+                uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
+                col_term[j] = col_terms[(uint64_t)t * kTileRows + (lane & 31)];
+            }
+        }
         total.clear();
 
         {
 #ifdef NK_TUNE
             unsigned long long const debug_c0 = clock64(), debug_w0 = wall_clock64();
 #endif
-            if (fast > 0) {
+            if (across || fast > 0) { // (always, when the pipeline runs across tiles: the host checked)
                 if constexpr (!across) prime();
 #ifdef NK_TUNE
                 debug_t1 = clock64();
@@ -794,7 +813,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                     for (int i = 0; i < kLoads; ++i) {
                         v4i v = load_chunk_guarded(a_tile + (uint64_t)s * kSrcStage + a_slow[i], valid, g.avec, 0u);
                         if (T::kUnsigned) {
-                            row_sum[i] += sum_bytes_u8(v);
+                            add_row_sum(i, sum_bytes_u8(v), sums_here);
 #pragma unroll
                             for (int w = 0; w < 4; ++w) { // flip only bytes that exist: the zero padding stays zero
                                 int const rem = valid - 4 * w;
@@ -823,17 +842,18 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         uint32_t const half = lane >> 5, col_in_tile = lane & 31;
         if (T::kUnsigned) {
             __syncthreads();
-            // The 8 threads that staged one row hold its partial byte sums in adjacent lanes.
+            // The 8 threads that staged a row left its partial byte sums in 8 adjacent slots.
+            if (tid < BM) {
+                uint32_t const *parts = &row_part[sums_here + tid * 8];
+                uint32_t sum = 0;
 #pragma unroll
-            for (int i = 0; i < kLoads; ++i) {
-                uint32_t s = row_sum[i];
-                s += __shfl_xor(s, 1, 64);
-                s += __shfl_xor(s, 2, 64);
-                s += __shfl_xor(s, 4, 64);
-                if ((tid & 7) == 0) row_terms[i * 32 + (tid >> 3)] = s * 128u;
-                row_sum[i] = across ? row_sum_next[i] : 0u, row_sum_next[i] = 0;
+                for (int part = 0; part < 8; ++part) sum += parts[part];
+                row_terms[tid] = sum * 128u;
             }
             __syncthreads();
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i) row_part[sums_here + i * NT + tid] = 0; // own slots: ready for the tile after next
+            sums_here ^= (uint32_t)(kLoads * NT);
         }
         // Stores: a scalar base plus one 32-bit per-lane offset, through an explicitly global pointer. (A store
         // through a generic pointer counts as an LDS operation as well, and with such stores in flight the
@@ -848,16 +868,12 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             uint32_t const lane_offset = 4 * half * (uint32_t)g.c_stride + col_in_tile * 4;
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                uint32_t col_term = 0;
-                if (T::kUnsigned) {
-                    uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
-                    col_term = col_terms[(uint64_t)t * kTileRows + col_in_tile];
-                }
                 bool const col_ok = col0 + j * 32 + col_in_tile < g.n;
                 // Rows come in runs of 4 that start 8 apart: the base advances by one row or by five. The
                 // empty asm keeps it a running scalar (otherwise every row's base is precomputed and the
                 // scalar registers overflow).
                 global_u8_t *row_base = c_tile + j * 128;
+                v4i row_term4 = {0, 0, 0, 0};
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -866,13 +882,20 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                         // a named copy: bit-casting the vector element expression itself reads lane 0
                         auto const element = total.finish(acc, i, j, v);
                         uint32_t bits = __builtin_bit_cast(uint32_t, element);
-                        if (T::kUnsigned) bits += row_terms[r_fixed + 4 * half] + col_term;
+                        if (T::kUnsigned) {
+                            // the terms of 4 consecutive rows in one LDS read
+                            if (v % 4 == 0) row_term4 = *(v4i const *)&row_terms[i * 32 + 8 * (v / 4) + 4 * half];
+                            bits += (uint32_t)row_term4[v % 4] + col_term[j];
+                        }
                         if ((!(DBG & 16) || bits == 0x12345678u) && // (timing experiment: almost no stores)
                             (!masked || (col_ok && row0 + r_fixed + 4 * half < g.m)))
                             *(global_u32_t *)(row_base + lane_offset) = bits;
                         row_base += (v % 4 == 3 ? 5 : 1) * row_step;
                         asm volatile("" : "+s"(row_base));
                     }
+                    // u8 reads a row term per element: keep those reads from being hoisted by the hundred
+                    // (registers are what the prefetched tile is short of here).
+                    if (T::kUnsigned) __builtin_amdgcn_sched_barrier(0);
                 }
             }
         };
