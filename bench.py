@@ -31,10 +31,10 @@ HBM_PEAK = 8000.0
 # each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
 # the summaries are under profiles/. Not re-measured by a plain run: counters need the profiler.
 MEASURED_TRAFFIC = {
-    ("i8", 8192, 8192, 8192): 1.0897e9,
-    ("bf16", 8192, 8192, 8192): 1.9516e9,
-    ("e4m3", 8192, 8192, 8192): 1.8823e9,
-    ("i8", 1024, 1 << 20, 768): 5.7180e9,
+    ("i8", 8192, 8192, 8192): 1.0816e9,
+    ("bf16", 8192, 8192, 8192): 2.4244e9,
+    ("e4m3", 8192, 8192, 8192): 1.8863e9,
+    ("i8", 1024, 1 << 20, 768): 5.4967e9,
 }
 HEADLINE = ("i8", 8192, 8192, 8192)
 OTHERS = [("bf16", 8192, 8192, 8192), ("e4m3", 8192, 8192, 8192), ("i8", 1024, 1 << 20, 768)]
@@ -181,8 +181,8 @@ def cpu_baseline(dtype, m, n, k, budget_rows=2048):
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=20)
-    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--steps", type=int, default=50)
+    parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--dtype", default=HEADLINE[0])
     parser.add_argument("--shape", type=int, nargs=3, default=list(HEADLINE[1:]))
     parser.add_argument("--no-others", action="store_true")
