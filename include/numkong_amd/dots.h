@@ -65,8 +65,8 @@ typedef enum {
     nk_e5m2_k = 1 << 15,
 } nk_dtype_t;
 
-/** Kernel kinds (reference: include/numkong/capabilities.h:178-253; same codes). Only the three dots
- *  kinds resolve to kernels here; every other kind resolves to the error stub with capability 0. */
+/** Kernel kinds (reference: include/numkong/capabilities.h:178-253; same codes). The three dots kinds and the
+ *  two packed distance kinds resolve to kernels here; every other kind resolves to the error stub with capability 0. */
 typedef enum {
     nk_kernel_unknown_k = 0,
     nk_kernel_dot_k = 'i',
@@ -128,6 +128,21 @@ NK_DYNAMIC void nk_dots_packed_e4m3(nk_e4m3_t const *a, void const *b_packed, nk
 NK_DYNAMIC void nk_dots_packed_e5m2(nk_e5m2_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,
                                     nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
 
+/* Distances over the same packed B, in one pass: result[i][j] = angular (1 - cosine) or euclidean distance between
+ * row i of A and row j of B, f32 for all six types. Reference: include/numkong/spatials.h:139-266. */
+#define NK_AMD_DECLARE_SPATIALS_(T, in_t)                                                                              \
+    NK_DYNAMIC void nk_angulars_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *result, nk_size_t rows,     \
+                                           nk_size_t cols, nk_size_t depth, nk_size_t a_stride, nk_size_t r_stride);  \
+    NK_DYNAMIC void nk_euclideans_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *result, nk_size_t rows,   \
+                                             nk_size_t cols, nk_size_t depth, nk_size_t a_stride, nk_size_t r_stride);
+NK_AMD_DECLARE_SPATIALS_(i8, nk_i8_t)
+NK_AMD_DECLARE_SPATIALS_(u8, nk_u8_t)
+NK_AMD_DECLARE_SPATIALS_(bf16, nk_bf16_t)
+NK_AMD_DECLARE_SPATIALS_(f16, nk_f16_t)
+NK_AMD_DECLARE_SPATIALS_(e4m3, nk_e4m3_t)
+NK_AMD_DECLARE_SPATIALS_(e5m2, nk_e5m2_t)
+#undef NK_AMD_DECLARE_SPATIALS_
+
 /* Capability and lookup API. Reference: c/numkong.c:767-768, 831-913. */
 NK_DYNAMIC int nk_uses_dynamic_dispatch(void);
 NK_DYNAMIC int nk_configure_thread(nk_capability_t capabilities);
@@ -149,7 +164,13 @@ NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t i
                                               void *b_packed);                                                         \
     NK_DYNAMIC void nk_dots_packed_##T##_gfx950(in_t const *a, void const *b_packed, out_t *c, nk_size_t height,       \
                                                 nk_size_t width, nk_size_t depth, nk_size_t a_stride,                  \
-                                                nk_size_t c_stride);
+                                                nk_size_t c_stride);                                 \
+    NK_DYNAMIC void nk_angulars_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,  \
+                                                    nk_size_t width, nk_size_t depth, nk_size_t a_stride,                 \
+                                                    nk_size_t c_stride);                                                  \
+    NK_DYNAMIC void nk_euclideans_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height, \
+                                                      nk_size_t width, nk_size_t depth, nk_size_t a_stride,               \
+                                                      nk_size_t c_stride);
 NK_AMD_DECLARE_BACKEND_(i8, nk_i8_t, nk_i32_t)
 NK_AMD_DECLARE_BACKEND_(u8, nk_u8_t, nk_u32_t)
 NK_AMD_DECLARE_BACKEND_(bf16, nk_bf16_t, nk_f32_t)
@@ -174,6 +195,10 @@ NK_DYNAMIC int nk_amd_dots_pack_async(nk_dtype_t dtype, void const *b, nk_size_t
 NK_DYNAMIC int nk_amd_dots_packed_async(nk_dtype_t dtype, void const *a, void const *b_packed, void *c,
                                         nk_size_t height, nk_size_t width, nk_size_t depth, nk_size_t a_stride,
                                         nk_size_t c_stride, void *stream);
+/** `kind` is nk_kernel_angulars_packed_k or nk_kernel_euclideans_packed_k. */
+NK_DYNAMIC int nk_amd_spatials_packed_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void const *a, void const *b_packed,
+                                            void *c, nk_size_t height, nk_size_t width, nk_size_t depth,
+                                            nk_size_t a_stride, nk_size_t c_stride, void *stream);
 
 #ifdef __cplusplus
 }

@@ -44,7 +44,7 @@ int nk_hip_stream_synchronize(void *stream);
 
 /**
  *  Bytes of the gfx950 packed image of an (n x k) B matrix: 64-byte header, MFMA-fragment tiles,
- *  per-column compensation terms. Replaces `nk_dots_packed_size_<T>_<isa>`
+ *  per-column compensation terms, per-column sums of squares. Replaces `nk_dots_packed_size_<T>_<isa>`
  *  (reference: include/numkong/dots/serial.h:245-271). Returns 0 for an unsupported dtype or when
  *  n or k do not fit 32 bits.
  */
@@ -64,6 +64,16 @@ int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t 
  */
 int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n,
                              size_t k, size_t a_stride, size_t c_stride, void *stream);
+
+/**
+ *  Distances instead of dot products, in one pass: C[i][j] = angular (metric 1) or euclidean (metric 2) distance
+ *  between row i of A and row j of B, as f32, from the same MFMA product, the per-column sums of squares that
+ *  `nk_hip_dots_pack_async` leaves in the image and the per-row sums of squares gathered while A is staged.
+ *  Replaces `nk_angulars_packed_<T>_<isa>` / `nk_euclideans_packed_<T>_<isa>`
+ *  (reference: include/numkong/dots/serial.h:2756-2800, include/numkong/spatial/serial.h:257-344).
+ */
+int nk_hip_spatials_packed_async(int dtype, int metric, void const *a, void const *b_packed, void *c, size_t m,
+                                 size_t n, size_t k, size_t a_stride, size_t c_stride, void *stream);
 
 /** Fill the m x n block of 32-bit outputs with `value` (used for the 0xFF error convention). */
 int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_t value, void *stream);

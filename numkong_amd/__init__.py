@@ -10,9 +10,11 @@ from .api import (  # noqa: F401
     DTYPES,
     NumKongAmdError,
     PackedMatrix,
+    angulars_packed,
     dots_pack,
     dots_packed,
     dots_packed_size,
+    euclideans_packed,
     library,
     library_path,
 )

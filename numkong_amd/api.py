@@ -64,11 +64,16 @@ def library() -> ctypes.CDLL:
         getattr(lib, f"nk_dots_pack_{name}").argtypes = [vp, sz, sz, sz, vp]
         getattr(lib, f"nk_dots_packed_{name}").restype = None
         getattr(lib, f"nk_dots_packed_{name}").argtypes = [vp, vp, vp, sz, sz, sz, sz, sz]
+        for stem in ("nk_angulars_packed_", "nk_euclideans_packed_"):
+            getattr(lib, stem + name).restype = None
+            getattr(lib, stem + name).argtypes = [vp, vp, vp, sz, sz, sz, sz, sz]
     lib.nk_amd_last_error.restype = ctypes.c_char_p
     lib.nk_amd_dots_pack_async.restype = i32
     lib.nk_amd_dots_pack_async.argtypes = [i32, vp, sz, sz, sz, vp, vp]
     lib.nk_amd_dots_packed_async.restype = i32
     lib.nk_amd_dots_packed_async.argtypes = [i32, vp, vp, vp, sz, sz, sz, sz, sz, vp]
+    lib.nk_amd_spatials_packed_async.restype = i32
+    lib.nk_amd_spatials_packed_async.argtypes = [i32, i32, vp, vp, vp, sz, sz, sz, sz, sz, vp]
     lib.nk_hip_last_error.restype = ctypes.c_char_p
     lib.nk_hip_set_tile_config.argtypes = [i32]
     lib.nk_hip_set_tile_config.restype = None
@@ -146,8 +151,7 @@ def dots_pack(b, dtype: str) -> PackedMatrix:
     return PackedMatrix(dtype, width, depth, buffer)
 
 
-def dots_packed(a, packed: PackedMatrix, out=None):
-    """``C[height x width] = a @ B.T`` with widened accumulators; ``out`` (optional) is overwritten."""
+def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out):
     import torch
 
     if not isinstance(packed, PackedMatrix):
@@ -156,7 +160,7 @@ def dots_packed(a, packed: PackedMatrix, out=None):
     height, depth = int(a.shape[0]), int(a.shape[1])
     if depth != packed.depth:
         raise ValueError(f"depth mismatch: a has {depth} columns, packed matrix has depth {packed.depth}")
-    out_dtype = getattr(torch, DTYPES[packed.dtype][2])
+    out_dtype = getattr(torch, out_dtype_name)
     if out is None:
         out = torch.empty((height, packed.width), dtype=out_dtype, device=a.device)
     else:
@@ -170,8 +174,24 @@ def dots_packed(a, packed: PackedMatrix, out=None):
             raise ValueError("out rows must be contiguous")
     a_stride = int(a.stride(0)) * a.element_size() if height > 1 else depth * a.element_size()
     c_stride = int(out.stride(0)) * 4 if height > 1 else packed.width * 4
-    getattr(library(), f"nk_dots_packed_{packed.dtype}")(
+    getattr(library(), stem + packed.dtype)(
         a.data_ptr(), packed.buffer.data_ptr(), out.data_ptr(), height, packed.width, depth, a_stride, c_stride
     )
-    _check("nk_dots_packed_" + packed.dtype)
+    _check(stem + packed.dtype)
     return out
+
+
+def dots_packed(a, packed: PackedMatrix, out=None):
+    """``C[height x width] = a @ B.T`` with widened accumulators; ``out`` (optional) is overwritten."""
+    return _packed_product("nk_dots_packed_", DTYPES[packed.dtype][2] if isinstance(packed, PackedMatrix) else "float32",
+                           a, packed, out)
+
+
+def angulars_packed(a, packed: PackedMatrix, out=None):
+    """Angular distances ``1 - cos(a_i, b_j)`` as float32 (reference: ``nk_angulars_packed_<dtype>``)."""
+    return _packed_product("nk_angulars_packed_", "float32", a, packed, out)
+
+
+def euclideans_packed(a, packed: PackedMatrix, out=None):
+    """Euclidean distances ``|a_i - b_j|`` as float32 (reference: ``nk_euclideans_packed_<dtype>``)."""
+    return _packed_product("nk_euclideans_packed_", "float32", a, packed, out)

@@ -20,6 +20,10 @@ typedef struct {
     nk_dots_pack_punned_t dots_pack_i8, dots_pack_u8, dots_pack_bf16, dots_pack_f16, dots_pack_e4m3, dots_pack_e5m2;
     nk_dots_packed_punned_t dots_packed_i8, dots_packed_u8, dots_packed_bf16, dots_packed_f16, dots_packed_e4m3,
         dots_packed_e5m2;
+    nk_dots_packed_punned_t angulars_packed_i8, angulars_packed_u8, angulars_packed_bf16, angulars_packed_f16,
+        angulars_packed_e4m3, angulars_packed_e5m2;
+    nk_dots_packed_punned_t euclideans_packed_i8, euclideans_packed_u8, euclideans_packed_bf16, euclideans_packed_f16,
+        euclideans_packed_e4m3, euclideans_packed_e5m2;
 } nk_implementations_t;
 
 extern nk_implementations_t nk_dispatch_table;
@@ -58,12 +62,18 @@ NK_AMD_DECLARE_DISPATCH_(e5m2)
                 return;                                                                                               \
             case nk_kernel_dots_pack_k: *m = (m_t)&nk_dots_pack_##T##_gfx950, *c = nk_cap_gfx950_k; return;          \
             case nk_kernel_dots_packed_k: *m = (m_t)&nk_dots_packed_##T##_gfx950, *c = nk_cap_gfx950_k; return;      \
+            case nk_kernel_angulars_packed_k: *m = (m_t)&nk_angulars_packed_##T##_gfx950, *c = nk_cap_gfx950_k; return; \
+            case nk_kernel_euclideans_packed_k:                                                                       \
+                *m = (m_t)&nk_euclideans_packed_##T##_gfx950, *c = nk_cap_gfx950_k;                                   \
+                return;                                                                                               \
             default: break;                                                                                           \
             }                                                                                                         \
         switch (k) {                                                                                                  \
         case nk_kernel_dots_packed_size_k: *m = (m_t)nk_error_packed_size_, *c = 0; return;                          \
         case nk_kernel_dots_pack_k: *m = (m_t)nk_error_pack_, *c = 0; return;                                        \
-        case nk_kernel_dots_packed_k: *m = (m_t)nk_error_dots_, *c = 0; return;                                      \
+        case nk_kernel_dots_packed_k:                                                                                 \
+        case nk_kernel_angulars_packed_k:                                                                             \
+        case nk_kernel_euclideans_packed_k: *m = (m_t)nk_error_dots_, *c = 0; return;                                \
         default: *m = (m_t)nk_error_dense_, *c = 0; return;                                                          \
         }                                                                                                             \
     }                                                                                                                 \
@@ -74,6 +84,10 @@ NK_AMD_DECLARE_DISPATCH_(e5m2)
                                 &used);                                                                               \
         nk_dispatch_##T##_find_(caps, nk_kernel_dots_pack_k, (nk_kernel_punned_t *)&t->dots_pack_##T, &used);         \
         nk_dispatch_##T##_find_(caps, nk_kernel_dots_packed_k, (nk_kernel_punned_t *)&t->dots_packed_##T, &used);     \
+        nk_dispatch_##T##_find_(caps, nk_kernel_angulars_packed_k, (nk_kernel_punned_t *)&t->angulars_packed_##T,    \
+                                &used);                                                                               \
+        nk_dispatch_##T##_find_(caps, nk_kernel_euclideans_packed_k,                                                  \
+                                (nk_kernel_punned_t *)&t->euclideans_packed_##T, &used);                              \
     }
 
 #ifdef __cplusplus

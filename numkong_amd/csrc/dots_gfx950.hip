@@ -61,7 +61,7 @@ enum : int {
 };
 
 constexpr uint32_t kMagic = 0x35394B4Eu; // "NK95"
-constexpr uint32_t kVersion = 2;
+constexpr uint32_t kVersion = 3;
 constexpr int kChunkBytes = 16;   // bytes of K per lane per operand load
 constexpr int kTileRows = 32;     // B rows per tile = MFMA N
 constexpr int kStageChunks = 8;   // chunks of K per pipeline stage (128 bytes per row)
@@ -80,7 +80,7 @@ struct PackedHeader {
     uint64_t data_offset;
     uint64_t sums_offset; // u32 x (32 * n_tiles): 128 * sum(b') per column for u8, zeros otherwise
     uint64_t total_bytes;
-    uint64_t reserved[1];
+    uint64_t norms_offset; // u32 or f32 x (32 * n_tiles): sum(b^2) per column (exact mod 2^32 for the integer types)
 };
 static_assert(sizeof(PackedHeader) == 64, "header must stay 64 bytes");
 
@@ -90,7 +90,7 @@ struct Geometry {
     uint32_t n, k, n_tiles, k_chunks;
     uint64_t k_bytes;      // bytes of one packed row: k * packed_bytes
     uint64_t k_src_bytes;  // bytes of one source row: k * elem_bytes
-    uint64_t data_bytes, sums_bytes, total_bytes;
+    uint64_t data_bytes, sums_bytes, norms_bytes, total_bytes;
 };
 
 inline int elem_bytes_of(int dtype) {
@@ -123,7 +123,8 @@ inline bool make_geometry(int dtype, size_t n, size_t k, Geometry &g) {
     g.n_tiles = (uint32_t)((n + kTileRows - 1) / kTileRows);
     g.data_bytes = (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes;
     g.sums_bytes = (uint64_t)g.n_tiles * kTileRows * sizeof(uint32_t);
-    g.total_bytes = sizeof(PackedHeader) + g.data_bytes + g.sums_bytes;
+    g.norms_bytes = g.sums_bytes;
+    g.total_bytes = sizeof(PackedHeader) + g.data_bytes + g.sums_bytes + g.norms_bytes;
     return true;
 }
 
@@ -225,23 +226,69 @@ __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b
     *(v4i *)(data + (((uint64_t)tile * k_chunks + c) * kTileRows + r) * kChunkBytes) = v;
 }
 
+/** Sum of the squares of the 8 values of a 16-byte chunk of bf16 (f32 = bits << 16) or f16, in f64. */
+template <bool BF16_VALUES>
+__device__ __forceinline__ double chunk_sumsq_f64(v4i v) {
+    double sum = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        float lo, hi;
+        if (BF16_VALUES) {
+            lo = __builtin_bit_cast(float, (uint32_t)v[w] << 16), hi = __builtin_bit_cast(float, (uint32_t)v[w] & 0xFFFF0000u);
+        }
+        else {
+            typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+            int const word = v[w]; // a named copy: bit-casting the vector element expression itself reads element 0
+            v2h const pair = __builtin_bit_cast(v2h, word);
+            lo = (float)pair[0], hi = (float)pair[1];
+        }
+        sum = __builtin_fma((double)lo, (double)lo, sum);
+        sum = __builtin_fma((double)hi, (double)hi, sum);
+    }
+    return sum;
+}
+
 /**
- *  Per-column compensation term for u8: 128 * sum of the signed packed bytes of the row (mod 2^32).
+ *  Per-column terms, from the packed tiles: the u8 compensation term (128 * sum of the signed packed bytes of
+ *  the row, mod 2^32; zero for the other types) and the column's sum of squares, which the angular and
+ *  euclidean products need (reference: the norms behind the packed rows, dots/serial.h:326-332): exact mod
+ *  2^32 for the integer types, accumulated in f64 and rounded once to f32 for the float types.
  *  One wavefront per tile: lane l owns row l % 32 and every second chunk starting at l / 32.
+ *  KIND: 0 i8, 1 u8, 2 bf16, 3 f16 (and fp8, stored widened to f16).
  */
-__global__ __launch_bounds__(64) void column_terms_kernel(uint8_t const *__restrict__ data, uint32_t k_chunks,
-                                                          uint32_t *__restrict__ sums) {
+template <int KIND>
+__global__ __launch_bounds__(64) void column_terms_kernel(uint8_t const *__restrict__ data, uint32_t k_chunks, uint32_t k,
+                                                          uint32_t *__restrict__ sums, uint32_t *__restrict__ norms) {
     uint32_t const tile = blockIdx.x;
     uint32_t const lane = threadIdx.x;
     uint8_t const *base = data + (uint64_t)tile * k_chunks * kTileChunkBytes + lane * kChunkBytes;
-    int acc = 0;
+    int sum = 0;
+    uint32_t squares = 0;
+    double squares_f64 = 0;
     for (uint32_t c = 0; c < k_chunks; c += 2) {
         v4i const v = *(v4i const *)(base + (uint64_t)c * kTileChunkBytes);
+        if (KIND == 0) {
 #pragma unroll
-        for (int w = 0; w < 4; ++w) acc = __builtin_amdgcn_sdot4(v[w], 0x01010101, acc, false);
+            for (int w = 0; w < 4; ++w) squares = (uint32_t)__builtin_amdgcn_sdot4(v[w], v[w], (int)squares, false);
+        }
+        else if (KIND == 1) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                sum = __builtin_amdgcn_sdot4(v[w], 0x01010101, sum, false);
+                squares = (uint32_t)__builtin_amdgcn_sdot4(v[w], v[w], (int)squares, false);
+            }
+        }
+        else { squares_f64 += chunk_sumsq_f64<KIND == 2>(v); }
     }
-    acc += __shfl_xor(acc, 32, 64);
-    if (lane < 32) sums[(uint64_t)tile * kTileRows + lane] = (uint32_t)acc * 128u;
+    sum += __shfl_xor(sum, 32, 64);
+    squares += __shfl_xor(squares, 32, 64);
+    squares_f64 += __shfl_xor(squares_f64, 32, 64);
+    // u8 is stored as b - 128 (and its padding as 0): sum(b^2) = sum((b - 128)^2) + 256 * sum(b - 128) + 128^2 * k
+    if (KIND == 1) squares += 256u * (uint32_t)sum + 16384u * k;
+    if (lane < 32) {
+        sums[(uint64_t)tile * kTileRows + lane] = (uint32_t)sum * 128u;
+        norms[(uint64_t)tile * kTileRows + lane] = KIND < 2 ? squares : __builtin_bit_cast(uint32_t, (float)squares_f64);
+    }
 }
 
 __global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t *p, uint64_t count, uint32_t value) {
@@ -286,8 +333,16 @@ struct I8 {
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16i acc_t;
+    typedef uint32_t norm_t; // what a row's sum of squares accumulates in
     static constexpr int kDtype = kI8;
     static constexpr bool kUnsigned = false;
+    /** Sum of the squares of the source values behind one staged chunk (`raw`: as loaded, `wide`: as it goes to LDS). */
+    static __device__ __forceinline__ norm_t sumsq(v4i raw, v4i) {
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum = __builtin_amdgcn_sdot4(raw[w], raw[w], sum, false);
+        return (uint32_t)sum;
+    }
     static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
     }
@@ -295,14 +350,32 @@ struct I8 {
 struct U8 : I8 {
     static constexpr int kDtype = kU8;
     static constexpr bool kUnsigned = true;
+    static __device__ __forceinline__ norm_t sumsq(v4i raw, v4i) {
+        uint32_t sum = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum = __builtin_amdgcn_udot4((uint32_t)raw[w], (uint32_t)raw[w], sum, false);
+        return sum;
+    }
 };
 struct BF16 {
     static constexpr bool kChunked = kHalfChunked;
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
+    typedef double norm_t;
     static constexpr int kDtype = kBF16;
     static constexpr bool kUnsigned = false;
+    /** The 8 products are exact in f32; their short sum is rounded a few times, the long sum runs in f64. */
+    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) {
+        float sum = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            float const lo = __builtin_bit_cast(float, (uint32_t)wide[w] << 16);
+            float const hi = __builtin_bit_cast(float, (uint32_t)wide[w] & 0xFFFF0000u);
+            sum = __builtin_fmaf(lo, lo, sum), sum = __builtin_fmaf(hi, hi, sum);
+        }
+        return (double)sum;
+    }
     static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), acc, 0,
                                                       0, 0);
@@ -313,8 +386,21 @@ struct F16 {
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
+    typedef double norm_t;
     static constexpr int kDtype = kF16;
     static constexpr bool kUnsigned = false;
+    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { // also e4m3 / e5m2, which are f16 by then
+        typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+        float sum = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) { // (mixed-precision fused multiply-adds; the packed f16 dot instruction rounds too early)
+            int const word = wide[w]; // a named copy: bit-casting the vector element expression itself reads element 0
+            v2h const pair = __builtin_bit_cast(v2h, word);
+            float const lo = (float)pair[0], hi = (float)pair[1];
+            sum = __builtin_fmaf(lo, lo, sum), sum = __builtin_fmaf(hi, hi, sum);
+        }
+        return (double)sum;
+    }
     static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), acc, 0, 0,
                                                      0);
@@ -333,6 +419,41 @@ struct E5M2 : F16 {
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<true>((uint32_t)v[0], (uint32_t)v[1]); }
 };
+
+/**
+ *  Distance from a dot product and two sums of squares, as the reference's scalar finalisers compute it
+ *  (spatial/serial.h:257-344): integer inputs are converted to f32 first (the i8 kernels read both norms as
+ *  signed 32-bit integers, the u8 kernels as unsigned); angular = max(1 - dot * rsqrt(qn * tn), 0), and 0 or
+ *  1 when the product of the norms is not positive; euclidean = sqrt(max(qn + tn - 2 * dot, 0)).
+ *  METRIC: 1 angular, 2 euclidean. The hardware's rsqrt (refined by one Newton step) and sqrt (1 ulp) stand in
+ *  for the reference's bit trick and three Newton steps.
+ */
+template <class T, int METRIC>
+__device__ __forceinline__ uint32_t distance_from_dot(uint32_t dot_bits, uint32_t row_norm_bits, uint32_t col_norm_bits) {
+    float dot, query, target;
+    if (T::kDtype == kI8) dot = (float)(int)dot_bits, query = (float)(int)row_norm_bits, target = (float)(int)col_norm_bits;
+    else if (T::kDtype == kU8) dot = (float)dot_bits, query = (float)row_norm_bits, target = (float)col_norm_bits;
+    else {
+        dot = __builtin_bit_cast(float, dot_bits), query = __builtin_bit_cast(float, row_norm_bits);
+        target = __builtin_bit_cast(float, col_norm_bits);
+    }
+    float result;
+    if (METRIC == 1) {
+        float const product = query * target;
+        // the hardware estimate (1 ulp) plus one Newton step with fused residuals: identical rows must cancel to
+        // within a rounding or two, as the reference's three Newton steps do
+        float root = __builtin_amdgcn_rsqf(product);
+        float const residual = __builtin_fmaf(-(product * root), root, 1.0f);
+        root = __builtin_fmaf(root * 0.5f, residual, root);
+        float const unclipped = __builtin_fmaf(-dot, root, 1.0f);
+        result = product > 0 ? (unclipped > 0 ? unclipped : 0.0f) : (dot == 0 ? 0.0f : 1.0f);
+    }
+    else {
+        float const squared = query + target - 2.0f * dot;
+        result = squared > 0 ? __builtin_amdgcn_sqrtf(squared) : 0.0f;
+    }
+    return __builtin_bit_cast(uint32_t, result);
+}
 
 #pragma endregion Element types
 
@@ -389,6 +510,7 @@ struct GemmArgs {
     uint32_t n_tiles, k_chunks;
     uint32_t tiles_m, tiles_n;
     int avec; // widest load the A pointer and stride allow (1, 2, 4, 8 or 16 bytes)
+    int metric; // 0: dot products, 1: angular distances, 2: euclidean distances (kernels built with NORMS)
     uint32_t chunk_stages; // chunked types: stages between folds of the accumulator (even, 2..16)
 };
 
@@ -444,7 +566,7 @@ __device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, ui
  *  needs a quarter of the store instructions but writes 32-byte pieces of 32 different rows; it measured
  *  12 % slower on the square shapes and 9 % slower on the retrieval shape.)
  */
-template <class T, int TM, int TN, bool ACROSS, int DBG = 0>
+template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, int DBG = 0>
 __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChunked ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
     typedef typename T::acc_t acc_t;
     constexpr int BM = TM * 32;
@@ -455,6 +577,9 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStageLds];
     __shared__ __attribute__((aligned(16))) uint32_t row_terms[T::kUnsigned ? BM : 4]; // u8 only: 128 * (sum of the bytes of each A row of the tile)
     __shared__ uint32_t row_part[T::kUnsigned ? 2 * BM * kStageChunks : 1]; // u8 only: the partial sums behind them
+    typedef typename T::norm_t norm_t;
+    __shared__ __attribute__((aligned(16))) uint32_t row_norms[NORMS ? BM : 4]; // distances only: sum of squares of each A row
+    __shared__ norm_t norm_part[NORMS ? 2 * BM * kStageChunks : 1];              // ... and the partial sums behind them
 
     uint32_t const tid = threadIdx.x, lane = tid & 63;
     // The wavefront index is the same in all lanes; telling the compiler keeps B addressing in scalar registers.
@@ -467,6 +592,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                           header->k_chunks == g.k_chunks && header->n_tiles == g.n_tiles;
     uint8_t const *data = g.bp + sizeof(PackedHeader);
     uint32_t const *col_terms = (uint32_t const *)(data + (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes);
+    uint32_t const *col_norms = col_terms + (uint64_t)g.n_tiles * kTileRows;
 
     uint32_t const stages = g.k_chunks / kStageChunks;
     // Stages the pipelined loop takes: all of them when A is at least dword-aligned, which is all that
@@ -550,6 +676,14 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     auto add_row_sum = [&](int i, uint32_t value, uint32_t set) {
         __hip_atomic_fetch_add(&row_part[set + i * NT + tid], value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
+    // Distances: the same bookkeeping for the sums of squares of the rows (u32, or f64 for the float types).
+    if (NORMS) {
+#pragma unroll
+        for (int i = 0; i < 2 * kLoads; ++i) norm_part[i * NT + tid] = 0;
+    }
+    auto add_row_norm = [&](int i, norm_t value, uint32_t set) {
+        __hip_atomic_fetch_add(&norm_part[set + i * NT + tid], value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
     v4i a_reg[2][kLoads];
     v4i b_reg[2][TN][4];
     v4i af[2][TM];
@@ -616,13 +750,20 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             v4i v = a_reg[slot][i];
 #pragma unroll
             for (int w = 0; w < T::kSrcChunk / 4; ++w) v[w] &= (int)keep[w];
+            // (without a next tile to stage for, what is staged past the end is dropped)
+            uint32_t const set = across && !mine ? sums_here ^ (uint32_t)(kLoads * NT) : sums_here;
+            v4i const raw = v;
             if (T::kUnsigned) {
                 uint32_t const sum = sum_bytes_u8(v);
-                // (without a next tile to stage for, what is staged past the end is dropped)
-                add_row_sum(i, across ? sum : sum * mine, across && !mine ? sums_here ^ (uint32_t)(kLoads * NT) : sums_here);
+                add_row_sum(i, across ? sum : sum * mine, set);
                 v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
             }
-            *(v4i *)(dst + a_lds[i]) = T::widen(v);
+            v4i const wide = T::widen(v);
+            if (NORMS) {
+                norm_t const squares = T::sumsq(raw, wide);
+                add_row_norm(i, across || mine ? squares : (norm_t)0, set);
+            }
+            *(v4i *)(dst + a_lds[i]) = wide;
         }
     };
     auto load_b = [&](TileView const &view, uint32_t s, auto slot_tag, auto q_tag) {
@@ -751,14 +892,13 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
         // u8: the column terms of this tile are fetched now and used in the epilogue, so that nothing has to
         // wait for them (a wait for a load is a wait for every store issued before it).
-        uint32_t col_term[TN];
+        uint32_t col_term[TN], col_norm[TN];
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            col_term[j] = 0;
-            if constexpr (T::kUnsigned) {
-                uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
-                col_term[j] = col_terms[(uint64_t)t * kTileRows + (lane & 31)];
-            }
+            col_term[j] = 0, col_norm[j] = 0;
+            uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
+            if constexpr (T::kUnsigned) col_term[j] = col_terms[(uint64_t)t * kTileRows + (lane & 31)];
+            if constexpr (NORMS) col_norm[j] = col_norms[(uint64_t)t * kTileRows + (lane & 31)];
         }
         total.clear();
 
@@ -812,6 +952,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
 #pragma unroll
                     for (int i = 0; i < kLoads; ++i) {
                         v4i v = load_chunk_guarded(a_tile + (uint64_t)s * kSrcStage + a_slow[i], valid, g.avec, 0u);
+                        v4i const raw = v;
                         if (T::kUnsigned) {
                             add_row_sum(i, sum_bytes_u8(v), sums_here);
 #pragma unroll
@@ -821,7 +962,9 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                                 v[w] ^= (int)mask;
                             }
                         }
-                        *(v4i *)(lds + a_lds[i]) = T::widen(v);
+                        v4i const wide = T::widen(v);
+                        if (NORMS) add_row_norm(i, T::sumsq(raw, wide), sums_here);
+                        *(v4i *)(lds + a_lds[i]) = wide;
                     }
                     load_b(cur, s, slot_c<0>(), slot_c<0>()), load_b(cur, s, slot_c<0>(), slot_c<1>());
                     load_b(cur, s, slot_c<0>(), slot_c<2>()), load_b(cur, s, slot_c<0>(), slot_c<3>());
@@ -840,19 +983,32 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
 
         // Epilogue. Accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.
         uint32_t const half = lane >> 5, col_in_tile = lane & 31;
-        if (T::kUnsigned) {
+        if (T::kUnsigned || NORMS) {
             __syncthreads();
-            // The 8 threads that staged a row left its partial byte sums in 8 adjacent slots.
+            // The 8 threads that staged a row left its partial sums in 8 adjacent slots.
             if (tid < BM) {
-                uint32_t const *parts = &row_part[sums_here + tid * 8];
-                uint32_t sum = 0;
+                if (T::kUnsigned) {
+                    uint32_t const *parts = &row_part[sums_here + tid * 8];
+                    uint32_t sum = 0;
 #pragma unroll
-                for (int part = 0; part < 8; ++part) sum += parts[part];
-                row_terms[tid] = sum * 128u;
+                    for (int part = 0; part < 8; ++part) sum += parts[part];
+                    row_terms[tid] = sum * 128u;
+                }
+                if (NORMS) {
+                    norm_t const *parts = &norm_part[sums_here + tid * 8];
+                    norm_t sum = 0;
+#pragma unroll
+                    for (int part = 0; part < 8; ++part) sum += parts[part];
+                    if constexpr (sizeof(norm_t) == 8) row_norms[tid] = __builtin_bit_cast(uint32_t, (float)sum); // f64 -> f32, once
+                    else row_norms[tid] = (uint32_t)sum;
+                }
             }
             __syncthreads();
 #pragma unroll
-            for (int i = 0; i < kLoads; ++i) row_part[sums_here + i * NT + tid] = 0; // own slots: ready for the tile after next
+            for (int i = 0; i < kLoads; ++i) { // own slots: ready for the tile after next
+                if (T::kUnsigned) row_part[sums_here + i * NT + tid] = 0;
+                if (NORMS) norm_part[sums_here + i * NT + tid] = 0;
+            }
             sums_here ^= (uint32_t)(kLoads * NT);
         }
         // Stores: a scalar base plus one 32-bit per-lane offset, through an explicitly global pointer. (A store
@@ -861,8 +1017,9 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         // matrix edge take the masked copy of the loop.
         bool const interior = row0 + BM <= g.m && col0 + 32 * TN <= g.n;
         global_u8_t *c_tile = (global_u8_t *)g.c + (uint64_t)row0 * g.c_stride + (uint64_t)col0 * 4;
-        auto store_all = [&](auto masked_tag) {
+        auto store_all = [&](auto masked_tag, auto metric_tag) {
             constexpr bool masked = decltype(masked_tag)::value != 0;
+            constexpr int metric = decltype(metric_tag)::value;
             uint64_t const row_step = g.c_stride;
             // Lane l holds column l % 32; register v holds row 8 * (v / 4) + 4 * (l / 32) + v % 4.
             uint32_t const lane_offset = 4 * half * (uint32_t)g.c_stride + col_in_tile * 4;
@@ -873,7 +1030,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 // empty asm keeps it a running scalar (otherwise every row's base is precomputed and the
                 // scalar registers overflow).
                 global_u8_t *row_base = c_tile + j * 128;
-                v4i row_term4 = {0, 0, 0, 0};
+                v4i row_term4 = {0, 0, 0, 0}, row_norm4 = {0, 0, 0, 0};
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -887,6 +1044,10 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                             if (v % 4 == 0) row_term4 = *(v4i const *)&row_terms[i * 32 + 8 * (v / 4) + 4 * half];
                             bits += (uint32_t)row_term4[v % 4] + col_term[j];
                         }
+                        if (metric != 0) {
+                            if (v % 4 == 0) row_norm4 = *(v4i const *)&row_norms[i * 32 + 8 * (v / 4) + 4 * half];
+                            bits = distance_from_dot<T, metric == 2 ? 2 : 1>(bits, (uint32_t)row_norm4[v % 4], col_norm[j]);
+                        }
                         if ((!(DBG & 16) || bits == 0x12345678u) && // (timing experiment: almost no stores)
                             (!masked || (col_ok && row0 + r_fixed + 4 * half < g.m)))
                             *(global_u32_t *)(row_base + lane_offset) = bits;
@@ -895,12 +1056,24 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                     }
                     // u8 reads a row term per element: keep those reads from being hoisted by the hundred
                     // (registers are what the prefetched tile is short of here).
-                    if (T::kUnsigned) __builtin_amdgcn_sched_barrier(0);
+                    if (T::kUnsigned || metric != 0) __builtin_amdgcn_sched_barrier(0);
                 }
             }
         };
-        if (interior) store_all(slot_c<0>());
-        else store_all(slot_c<1>());
+        if constexpr (NORMS) { // which distance is a run-time choice: one kernel serves both
+            if (g.metric == 2) {
+                if (interior) store_all(slot_c<0>(), slot_c<2>());
+                else store_all(slot_c<1>(), slot_c<2>());
+            }
+            else {
+                if (interior) store_all(slot_c<0>(), slot_c<1>());
+                else store_all(slot_c<1>(), slot_c<1>());
+            }
+        }
+        else {
+            if (interior) store_all(slot_c<0>(), slot_c<0>());
+            else store_all(slot_c<1>(), slot_c<0>());
+        }
 #ifdef NK_TUNE
         if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + (g.tiles_m * g.tiles_n > 45 * gridDim.x ? 40 : 1) * gridDim.x) {
             g_debug_clocks[5] = clock64() - debug_t2, g_debug_clocks[6] = clock64() - debug_t0;
@@ -938,22 +1111,24 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream) {
     // with dword loads) and there are enough of them to prefetch three ahead.
     uint32_t const stages = g.k_chunks / kStageChunks;
     bool const across = g.avec >= 4 && stages >= 4 && !(g_variant & 1);
-    void (*kernel)(GemmArgs) = across ? dots_packed_kernel<T, TM, TN, true> : dots_packed_kernel<T, TM, TN, false>;
+    bool const norms = g.metric != 0;
+    void (*kernel)(GemmArgs) = norms ? (across ? dots_packed_kernel<T, TM, TN, true, true> : dots_packed_kernel<T, TM, TN, false, true>)
+                                     : (across ? dots_packed_kernel<T, TM, TN, true, false> : dots_packed_kernel<T, TM, TN, false, false>);
 #ifdef NK_TUNE // timing experiments that leave parts of the loop out (results are wrong on purpose)
     if constexpr (TM == 8 && TN == 2 && T::kDtype == kI8) {
         switch (g_variant >> 2) {
-        case 1: kernel = dots_packed_kernel<T, TM, TN, false, 1>; break;
-        case 2: kernel = dots_packed_kernel<T, TM, TN, false, 2>; break;
-        case 3: kernel = dots_packed_kernel<T, TM, TN, false, 4>; break;
-        case 4: kernel = dots_packed_kernel<T, TM, TN, false, 16>; break;
-        case 5: kernel = dots_packed_kernel<T, TM, TN, false, 17>; break;
+        case 1: kernel = dots_packed_kernel<T, TM, TN, false, false, 1>; break;
+        case 2: kernel = dots_packed_kernel<T, TM, TN, false, false, 2>; break;
+        case 3: kernel = dots_packed_kernel<T, TM, TN, false, false, 4>; break;
+        case 4: kernel = dots_packed_kernel<T, TM, TN, false, false, 16>; break;
+        case 5: kernel = dots_packed_kernel<T, TM, TN, false, false, 17>; break;
         default: break;
         }
     }
 #endif
     // Persistent grid: as many workgroups as fit on the device at once (queried once per kernel).
-    static int resident_of[2] = {0, 0};
-    int &resident = resident_of[across ? 1 : 0];
+    static int resident_of[4] = {0, 0, 0, 0};
+    int &resident = resident_of[(across ? 1 : 0) + (norms ? 2 : 0)];
     if (!resident) {
         int per_cu = 0, device = 0;
         hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (void const *)kernel, 256, 0);
@@ -1096,11 +1271,13 @@ int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t 
     h.n = g.n, h.k = g.k, h.n_tiles = g.n_tiles, h.k_chunks = g.k_chunks;
     h.data_offset = sizeof(PackedHeader);
     h.sums_offset = sizeof(PackedHeader) + g.data_bytes;
+    h.norms_offset = h.sums_offset + g.sums_bytes;
     h.total_bytes = g.total_bytes;
 
     uint8_t *image = (uint8_t *)b_packed;
     uint8_t *data = image + sizeof(PackedHeader);
     uint32_t *sums = (uint32_t *)(data + g.data_bytes);
+    uint32_t *norms = sums + (uint64_t)g.n_tiles * kTileRows;
     hipLaunchKernelGGL(write_header_kernel, dim3(1), dim3(64), 0, stream, (PackedHeader *)image, h);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(e, "write_header_kernel");
@@ -1115,12 +1292,13 @@ int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t 
         if (e != hipSuccess) return fail(e, "pack_kernel");
     }
     if (g.n_tiles) {
-        if (dtype == kU8 && g.k_chunks) {
-            hipLaunchKernelGGL(column_terms_kernel, dim3(g.n_tiles), dim3(64), 0, stream, (uint8_t const *)data,
-                               g.k_chunks, sums);
+        if (g.k_chunks) {
+            auto terms = dtype == kI8 ? column_terms_kernel<0>
+                         : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
+            hipLaunchKernelGGL(terms, dim3(g.n_tiles), dim3(64), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);
         }
         else {
-            uint64_t const count = (uint64_t)g.n_tiles * kTileRows;
+            uint64_t const count = 2 * (uint64_t)g.n_tiles * kTileRows; // both arrays, back to back
             hipLaunchKernelGGL(fill_u32_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, stream, sums, count,
                                0u);
         }
@@ -1142,8 +1320,8 @@ int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_
     return e == hipSuccess ? 0 : fail(e, "fill_rows_kernel");
 }
 
-int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n, size_t k,
-                             size_t a_stride, size_t c_stride, void *stream_) {
+static int product_async(int dtype, int metric, void const *a, void const *b_packed, void *c, size_t m, size_t n,
+                         size_t k, size_t a_stride, size_t c_stride, void *stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     if (!m || !n) return 0;
     Geometry geo;
@@ -1161,6 +1339,7 @@ int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, voi
     g.a_stride = a_stride, g.c_stride = c_stride, g.k_src_bytes = geo.k_src_bytes;
     g.m = (uint32_t)m, g.n = geo.n, g.k = geo.k, g.n_tiles = geo.n_tiles, g.k_chunks = geo.k_chunks;
     g.avec = widest_load(a, a_stride);
+    g.metric = metric;
     {
         // Stages between accumulator folds: about an eighth of the depth, even, between 2 and 16.
         uint32_t const eighth = (g.k_chunks / kStageChunks / 8) & ~1u;
@@ -1178,6 +1357,17 @@ int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, voi
     default: return fail_msg("nk_hip_dots_packed: unsupported dtype");
     }
     return e == hipSuccess ? 0 : fail(e, "dots_packed_kernel");
+}
+
+int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n, size_t k,
+                             size_t a_stride, size_t c_stride, void *stream) {
+    return product_async(dtype, 0, a, b_packed, c, m, n, k, a_stride, c_stride, stream);
+}
+
+int nk_hip_spatials_packed_async(int dtype, int metric, void const *a, void const *b_packed, void *c, size_t m, size_t n,
+                                 size_t k, size_t a_stride, size_t c_stride, void *stream) {
+    if (metric != 1 && metric != 2) return fail_msg("nk_hip_spatials_packed: metric must be 1 (angular) or 2 (euclidean)");
+    return product_async(dtype, metric, a, b_packed, c, m, n, k, a_stride, c_stride, stream);
 }
 
 #ifdef NK_TUNE

@@ -63,6 +63,13 @@ int nk_amd_dots_packed_async(nk_dtype_t dtype, void const *a, void const *b_pack
     return nk_hip_dots_packed_async((int)dtype, a, b_packed, c, m, n, k, a_stride, c_stride, stream);
 }
 
+int nk_amd_spatials_packed_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void const *a, void const *b_packed, void *c,
+                                 nk_size_t m, nk_size_t n, nk_size_t k, nk_size_t a_stride, nk_size_t c_stride,
+                                 void *stream) {
+    int const metric = kind == nk_kernel_angulars_packed_k ? 1 : (kind == nk_kernel_euclideans_packed_k ? 2 : 0);
+    return nk_hip_spatials_packed_async((int)dtype, metric, a, b_packed, c, m, n, k, a_stride, c_stride, stream);
+}
+
 static nk_size_t nk_amd_packed_size_(nk_dtype_t dtype, nk_size_t n, nk_size_t k) {
     return nk_hip_dots_packed_size((int)dtype, n, k);
 }
@@ -107,8 +114,9 @@ static void nk_amd_pack_(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t
     if (staged_p) nk_hip_free(staged_p);
 }
 
-static void nk_amd_packed_(nk_dtype_t dtype, void const *a, void const *b_packed, void *c, nk_size_t m, nk_size_t n,
-                           nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {
+/** `metric`: 0 dot products, 1 angular distances, 2 euclidean distances; all outputs are 4 bytes wide. */
+static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void const *b_packed, void *c, nk_size_t m,
+                           nk_size_t n, nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {
     nk_amd_error_[0] = 0;
     if (!m || !n) return;
     size_t const element_bytes = nk_amd_element_bytes_(dtype);
@@ -149,9 +157,12 @@ static void nk_amd_packed_(nk_dtype_t dtype, void const *a, void const *b_packed
         status = nk_hip_malloc(&staged_c, m * device_c_stride);
         device_c = staged_c;
     }
-    if (!status)
+    if (!status && metric == 0)
         status = nk_hip_dots_packed_async((int)dtype, device_a, device_p, device_c, m, n, k, device_a_stride,
                                           device_c_stride, NULL);
+    if (!status && metric != 0)
+        status = nk_hip_spatials_packed_async((int)dtype, metric, device_a, device_p, device_c, m, n, k, device_a_stride,
+                                              device_c_stride, NULL);
     if (!status && staged_c) status = nk_hip_memcpy2d_d2h(c, c_stride, staged_c, device_c_stride, n * 4, m, NULL);
     if (!status) status = nk_hip_stream_synchronize(NULL);
     if (status) {
@@ -173,7 +184,17 @@ static void nk_amd_packed_(nk_dtype_t dtype, void const *a, void const *b_packed
     }                                                                                                              \
     void nk_dots_packed_##T##_gfx950(in_t const *a, void const *b_packed, out_t *c, nk_size_t height,              \
                                      nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride) {   \
-        nk_amd_packed_(nk_##T##_k, a, b_packed, c, height, width, depth, a_stride, c_stride);                      \
+        nk_amd_packed_(nk_##T##_k, 0, a, b_packed, c, height, width, depth, a_stride, c_stride);                   \
+    }                                                                                                              \
+    void nk_angulars_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,       \
+                                         nk_size_t width, nk_size_t depth, nk_size_t a_stride,                     \
+                                         nk_size_t c_stride) {                                                     \
+        nk_amd_packed_(nk_##T##_k, 1, a, b_packed, c, height, width, depth, a_stride, c_stride);                   \
+    }                                                                                                              \
+    void nk_euclideans_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,     \
+                                           nk_size_t width, nk_size_t depth, nk_size_t a_stride,                   \
+                                           nk_size_t c_stride) {                                                   \
+        nk_amd_packed_(nk_##T##_k, 2, a, b_packed, c, height, width, depth, a_stride, c_stride);                   \
     }
 
 NK_AMD_DEFINE_BACKEND_(i8, nk_i8_t, nk_i32_t)

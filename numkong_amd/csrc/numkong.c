@@ -4,7 +4,7 @@
  *
  *  Counterpart of the reference's c/numkong.c for this path: the table (c/numkong.c:231), the
  *  `nk_dots_packed_size_T` / `nk_dots_pack_T` / `nk_dots_packed_T` trampolines (c/numkong.c:347-364,
- *  instantiated :628-671), the error stubs (:78-81, :195-216), the capability and lookup API
+ *  instantiated :628-671) and the `nk_angulars_packed_T` / `nk_euclideans_packed_T` ones next to them, the error stubs (:78-81, :195-216), the capability and lookup API
  *  (:767-768, :831-913) and initialisation when the library is loaded (:916-919).
  */
 #include <string.h>
@@ -53,6 +53,15 @@ void nk_error_dots_(void const *a, void const *b_packed, void *c, nk_size_t m, n
     NK_DYNAMIC void nk_dots_packed_##T(in_t const *a, void const *b_packed, out_t *c, nk_size_t m, nk_size_t n, \
                                        nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {                   \
         nk_dispatch_table.dots_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                         \
+    }                                                                                                           \
+    NK_DYNAMIC void nk_angulars_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t m,      \
+                                           nk_size_t n, nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) { \
+        nk_dispatch_table.angulars_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                     \
+    }                                                                                                           \
+    NK_DYNAMIC void nk_euclideans_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t m,    \
+                                             nk_size_t n, nk_size_t k, nk_size_t a_stride,                      \
+                                             nk_size_t c_stride) {                                              \
+        nk_dispatch_table.euclideans_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                   \
     }
 
 NK_AMD_DISPATCH_CROSS_(i8, nk_i8_t, nk_i32_t)
@@ -110,6 +119,17 @@ NK_DYNAMIC void nk_find_kernel_punned(nk_kernel_kind_t kind, nk_dtype_t dtype, n
 }
 
 NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t input) {
+    if (kind == nk_kernel_angulars_packed_k || kind == nk_kernel_euclideans_packed_k) {
+        switch (input) { /* reference: include/numkong/numkong.h:46-51; f32 for every type served here */
+        case nk_i8_k:
+        case nk_u8_k:
+        case nk_bf16_k:
+        case nk_f16_k:
+        case nk_e4m3_k:
+        case nk_e5m2_k: return nk_f32_k;
+        default: return nk_dtype_unknown_k;
+        }
+    }
     if (kind != nk_kernel_dots_packed_k) return nk_dtype_unknown_k;
     switch (input) {
     case nk_i8_k: return nk_i32_k;

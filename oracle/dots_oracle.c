@@ -26,9 +26,21 @@
  *  that exists, against committed vectors produced from it (tests/golden), against torch's float8/
  *  float16/bfloat16 decoders, and against closed forms (exact integer products, powers of two).
  *
- *  Parity unpinned: the per-column norms of FLOAT types in the packed image (the reference computes them
- *  with nk_reduce_moments_*, whose summation order is not restated here). They are not read by
- *  dots_packed; this file writes zeros there and the tests compare header + rows only.
+ *    - the packed distances on top of the packed product: per-row and per-column sums of squares
+ *      (integers exact, truncated to 32 bits; floats as the serial Neumaier-compensated f32 sum of
+ *      include/numkong/reduce/serial.h:223-300), the scalar reciprocal square root (bit trick + three Newton
+ *      steps, include/numkong/scalar/serial.h:22-33) and the finalisers angular = max(1 - dot * rsqrt(qn * tn), 0)
+ *      / euclidean = sqrt(max(qn + tn - 2 * dot, 0)) with their corner cases
+ *          include/numkong/spatial/serial.h:257-344, include/numkong/dots/serial.h:2756-2800
+ *      Pinned bit for bit against nk_angulars_packed_{i8,u8}_serial / nk_euclideans_packed_{i8,u8}_serial (where
+ *      every input of the finaliser is an exact integer), and for the float types, whose norms the reference
+ *      takes from whatever nk_reduce_moments_* kernel its dispatch picks on the host, to within 4 f32 ulp of
+ *      the serial kernels' results.
+ *
+ *  Parity unpinned: the per-column norms of FLOAT types in the serial packed image as stored bytes (the
+ *  reference computes them with the host-dispatched nk_reduce_moments_*, whose summation order is not restated
+ *  here). They are not read by dots_packed; nko_serial_pack writes zeros there and the tests compare header +
+ *  rows only. nko_serial_spatials takes its norms from the unpacked rows instead.
  */
 #include <math.h>
 #include <stddef.h>
@@ -319,3 +331,130 @@ NKO_API void nko_dots_f64(int dtype, void const *a, void const *b, double *c, do
 }
 
 #pragma endregion Products
+
+#pragma region Packed distances
+
+/** Sum of squares of one row. Floats: Neumaier-compensated f32 running sum, as nk_reduce_moments_<T>_serial
+ *  (reduce/serial.h:223-300); integers: exact in 64 bits, truncated to 32 (dots/serial.h:154-164). Returned as
+ *  the bits of the f32 or of the u32. */
+static uint32_t row_sumsq_bits(int dtype, void const *row, size_t depth) {
+    if (dtype == NKO_I8 || dtype == NKO_U8) {
+        uint64_t sum = 0;
+        for (size_t l = 0; l < depth; ++l) {
+            int64_t const v = dtype == NKO_I8 ? (int64_t)((int8_t const *)row)[l] : (int64_t)((uint8_t const *)row)[l];
+            sum += (uint64_t)(v * v);
+        }
+        return (uint32_t)sum;
+    }
+    volatile float running = 0, compensation = 0; /* volatile: every operation rounds to f32, in this order */
+    for (size_t l = 0; l < depth; ++l) {
+        float const value = element_f32(dtype, row, l);
+        volatile float squared = value * value;
+        volatile float tentative = running + squared;
+        if (running >= squared) {
+            volatile float lost = (running - tentative);
+            lost = lost + squared;
+            compensation = compensation + lost;
+        }
+        else {
+            volatile float lost = (squared - tentative);
+            lost = lost + running;
+            compensation = compensation + lost;
+        }
+        running = tentative;
+    }
+    return f32_to_bits(running + compensation);
+}
+
+NKO_API void nko_row_sumsq(int dtype, void const *x, size_t rows, size_t depth, size_t stride, uint32_t *out_bits) {
+    for (size_t i = 0; i < rows; ++i) out_bits[i] = row_sumsq_bits(dtype, (unsigned char const *)x + i * stride, depth);
+}
+
+/** scalar/serial.h:22-31: the bit-trick estimate refined by three Newton steps, all in f32. */
+static float serial_rsqrt(float number) {
+    volatile float y = bits_to_f32(0x5F375A86u - (f32_to_bits(number) >> 1));
+    for (int step = 0; step < 3; ++step) {
+        volatile float t = 0.5f * number;
+        t = t * y;
+        t = t * y;
+        t = 1.5f - t;
+        y = y * t;
+    }
+    return y;
+}
+
+/** spatial/serial.h:257-344. `dot`, `query` and `target` arrive as 32-bit patterns: f32 for the float types,
+ *  i32 for i8 (the i8 finalisers read both norms as signed), u32 for u8. */
+static float serial_from_dot(int dtype, int metric, uint32_t dot_bits, uint32_t query_bits, uint32_t target_bits) {
+    float dot, query, target;
+    if (dtype == NKO_I8) dot = (float)(int32_t)dot_bits, query = (float)(int32_t)query_bits, target = (float)(int32_t)target_bits;
+    else if (dtype == NKO_U8) dot = (float)dot_bits, query = (float)query_bits, target = (float)target_bits;
+    else dot = bits_to_f32(dot_bits), query = bits_to_f32(query_bits), target = bits_to_f32(target_bits);
+    if (metric == 1) {
+        volatile float product = query * target;
+        if (product > 0) {
+            volatile float normalized = dot * serial_rsqrt(product);
+            volatile float result = 1.0f - normalized;
+            return result > 0 ? result : 0.0f;
+        }
+        return dot == 0 ? 0.0f : 1.0f;
+    }
+    volatile float squared = query + target;
+    volatile float twice = 2.0f * dot;
+    squared = squared - twice;
+    if (!(squared > 0)) return 0.0f;
+    volatile float root = squared * serial_rsqrt(squared); /* scalar/serial.h:33 */
+    return root;
+}
+
+/** nk_angulars_packed_<T>_serial (metric 1) / nk_euclideans_packed_<T>_serial (metric 2) from unpacked B:
+ *  the serial product, then the finaliser per element with the row's and the column's sum of squares. */
+NKO_API void nko_serial_spatials(int dtype, int metric, void const *a, void const *b, float *c, size_t rows,
+                                 size_t columns, size_t depth, size_t a_stride, size_t b_stride, size_t c_stride) {
+    size_t const image_bytes = nko_serial_packed_size(dtype, columns, depth) + 64;
+    unsigned char *image = (unsigned char *)__builtin_malloc(image_bytes);
+    uint32_t *target_norms = (uint32_t *)__builtin_malloc(columns * sizeof(uint32_t) + 4);
+    nko_serial_pack(dtype, b, columns, depth, b_stride, image);
+    nko_row_sumsq(dtype, b, columns, depth, b_stride, target_norms);
+    nko_serial_packed(dtype, a, image, c, rows, columns, depth, a_stride, c_stride);
+    for (size_t i = 0; i < rows; ++i) {
+        uint32_t const query_norm = row_sumsq_bits(dtype, (unsigned char const *)a + i * a_stride, depth);
+        uint32_t *row = (uint32_t *)((unsigned char *)c + i * c_stride);
+        for (size_t j = 0; j < columns; ++j)
+            row[j] = f32_to_bits(serial_from_dot(dtype, metric, row[j], query_norm, target_norms[j]));
+    }
+    __builtin_free(image);
+    __builtin_free(target_norms);
+}
+
+/** f64 ground truth of the distances from the unpacked operands (test/test_cross.hpp:290-427 computes its
+ *  references the same way: f64 dot and norms, then the formula). */
+NKO_API void nko_spatials_f64(int dtype, int metric, void const *a, void const *b, double *c, size_t rows, size_t columns,
+                              size_t depth, size_t a_stride, size_t b_stride) {
+    for (size_t i = 0; i < rows; ++i) {
+        unsigned char const *a_row = (unsigned char const *)a + i * a_stride;
+        double query = 0;
+        for (size_t l = 0; l < depth; ++l) query += (double)element_f32(dtype, a_row, l) * (double)element_f32(dtype, a_row, l);
+        for (size_t j = 0; j < columns; ++j) {
+            unsigned char const *b_row = (unsigned char const *)b + j * b_stride;
+            double dot = 0, target = 0;
+            for (size_t l = 0; l < depth; ++l) {
+                double const x = element_f32(dtype, a_row, l), y = element_f32(dtype, b_row, l);
+                dot += x * y, target += y * y;
+            }
+            double result;
+            if (metric == 1) {
+                double const product = query * target;
+                result = product > 0 ? 1.0 - dot / sqrt(product) : (dot == 0 ? 0.0 : 1.0);
+                if (result < 0) result = 0;
+            }
+            else {
+                double const squared = query + target - 2.0 * dot;
+                result = squared > 0 ? sqrt(squared) : 0.0;
+            }
+            c[i * columns + j] = result;
+        }
+    }
+}
+
+#pragma endregion Packed distances

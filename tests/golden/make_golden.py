@@ -20,7 +20,8 @@ def main():
         raise SystemExit("build oracle/_ref first: make -C oracle")
     out = support.GOLDEN_DIR
     rng = np.random.default_rng(2024)
-    for dtype in support.FLOAT_DTYPES:
+    only = sys.argv[1] if len(sys.argv) > 1 else ""  # e.g. "spatials": rewrite only the files of that family
+    for dtype in support.FLOAT_DTYPES if only in ("", "cast", "dots") else []:
         codes = np.arange(256 if support.STORAGE[dtype] == np.uint8 else 65536).astype(support.STORAGE[dtype])
         if len(codes) > 256:
             codes = np.concatenate([codes[::61], np.array([0x0001, 0x03FF, 0x0400, 0x7BFF, 0x7C00, 0xFC00, 0x7E00, 0x8000,
@@ -34,7 +35,7 @@ def main():
                             decoded=reference.cast(codes, dtype, "f32"), values=values,
                             encoded=reference.cast(values, "f32", dtype))
     cases = [("ragged", 13, 21, 77, "default"), ("deep", 6, 10, 2049, "default")]
-    for dtype in support.ALL_DTYPES:
+    for dtype in support.ALL_DTYPES if only in ("", "cast", "dots") else []:
         for tag, m, n, k, kind in cases + ([("fp8", 8, 12, 300, "fp8")] if dtype[0] == "e" else []) + (
                 [("lognormal", 8, 12, 300, "lognormal")] if dtype in ("f16", "bf16") else []):
             a = support.random_matrix(oracle, dtype, m, k, rng, kind, pad=3)
@@ -50,6 +51,20 @@ def main():
             np.savez_compressed(os.path.join(out, f"dots_{dtype}_{tag}.npz"), dtype=dtype, a=a, b=b,
                                 c_serial=reference.dots_packed(dtype, a, b),
                                 serial_packed_size=reference.packed_size(dtype, n, k))
+    # Packed distances: finite inputs, one zero row and one pair of identical rows, serial kernels of the reference.
+    rng = np.random.default_rng(2025)
+    for dtype in support.ALL_DTYPES:
+        m, n, k = 12, 10, 203
+        a = np.ascontiguousarray(support.random_matrix(oracle, dtype, m, k, rng))
+        b = np.ascontiguousarray(support.random_matrix(oracle, dtype, n, k, rng))
+        if dtype == "e5m2":  # the encoder overflows to Inf; keep the distances finite
+            a = np.where((a & 0x7F) > 0x7B, (a & 0x80) | 0x7B, a).astype(a.dtype)
+            b = np.where((b & 0x7F) > 0x7B, (b & 0x80) | 0x7B, b).astype(b.dtype)
+        a[1] = 0
+        b[2] = a[3]
+        np.savez_compressed(os.path.join(out, f"spatials_{dtype}.npz"), dtype=dtype, a=a, b=b,
+                            angulars_serial=reference.spatials_packed(support.KIND_ANGULARS, dtype, a, b),
+                            euclideans_serial=reference.spatials_packed(support.KIND_EUCLIDEANS, dtype, a, b))
     print("wrote", len(os.listdir(out)) - 1, "fixtures to", out)
 
 

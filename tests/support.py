@@ -23,6 +23,9 @@ OUTPUT = {"i8": np.int32, "u8": np.uint32, "f16": np.float32, "bf16": np.float32
 FLOAT_DTYPES = ("bf16", "f16", "e4m3", "e5m2")
 ALL_DTYPES = ("i8", "u8") + FLOAT_DTYPES
 KIND_SIZE, KIND_PACK, KIND_PACKED = ord("P"), ord("Q"), ord("G")
+KIND_ANGULARS, KIND_EUCLIDEANS = ord("N"), ord("E")  # packed distances: same prototype as the packed product
+METRICS = {"angular": 1, "euclidean": 2}
+METRIC_KINDS = {"angular": KIND_ANGULARS, "euclidean": KIND_EUCLIDEANS}
 CAP_SERIAL = 1
 
 _sz, _vp, _i32 = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int
@@ -44,6 +47,9 @@ class Oracle:
         lib.nko_serial_pack.argtypes = [_i32, _vp, _sz, _sz, _sz, _vp]
         lib.nko_serial_packed.argtypes = [_i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
         lib.nko_dots_f64.argtypes = [_i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
+        lib.nko_row_sumsq.argtypes = [_i32, _vp, _sz, _sz, _sz, _vp]
+        lib.nko_serial_spatials.argtypes = [_i32, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz]
+        lib.nko_spatials_f64.argtypes = [_i32, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
 
     def decode(self, dtype: str, codes: np.ndarray) -> np.ndarray:
         codes = np.ascontiguousarray(codes, dtype=STORAGE[dtype])
@@ -73,6 +79,30 @@ class Oracle:
         packed = self.pack(dtype, b)
         c = np.empty((m, n), dtype=OUTPUT[dtype])
         self.lib.nko_serial_packed(CODES[dtype], _ptr(a), _ptr(packed), _ptr(c), m, n, k, a.strides[0], c.strides[0])
+        return c
+
+    def row_sumsq(self, dtype: str, x: np.ndarray) -> np.ndarray:
+        """Per-row sum of squares as the serial backend computes it: u32 for the integer types, f32 otherwise."""
+        out = np.empty(x.shape[0], dtype=np.uint32)
+        self.lib.nko_row_sumsq(CODES[dtype], _ptr(x), x.shape[0], x.shape[1], x.strides[0], _ptr(out))
+        return out if dtype in ("i8", "u8") else out.view(np.float32)
+
+    def spatials_packed(self, metric: str, dtype: str, a: np.ndarray, b: np.ndarray) -> np.ndarray:
+        """`nk_angulars_packed_<dtype>_serial` ("angular") / `nk_euclideans_packed_<dtype>_serial` ("euclidean")."""
+        m, k = a.shape
+        n = b.shape[0]
+        c = np.empty((m, n), dtype=np.float32)
+        self.lib.nko_serial_spatials(CODES[dtype], METRICS[metric], _ptr(a), _ptr(b), _ptr(c), m, n, k, a.strides[0],
+                                     b.strides[0], c.strides[0])
+        return c
+
+    def spatials_truth(self, metric: str, dtype: str, a: np.ndarray, b: np.ndarray) -> np.ndarray:
+        """The distances from f64 dots and f64 norms."""
+        m, k = a.shape
+        n = b.shape[0]
+        c = np.empty((m, n), dtype=np.float64)
+        self.lib.nko_spatials_f64(CODES[dtype], METRICS[metric], _ptr(a), _ptr(b), _ptr(c), m, n, k, a.strides[0],
+                                  b.strides[0])
         return c
 
     def truth(self, dtype: str, a: np.ndarray, b: np.ndarray):
@@ -106,6 +136,8 @@ class Reference:
             KIND_SIZE: ctypes.CFUNCTYPE(_sz, _sz, _sz),
             KIND_PACK: ctypes.CFUNCTYPE(None, _vp, _sz, _sz, _sz, _vp),
             KIND_PACKED: ctypes.CFUNCTYPE(None, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz),
+            KIND_ANGULARS: ctypes.CFUNCTYPE(None, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz),
+            KIND_EUCLIDEANS: ctypes.CFUNCTYPE(None, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz),
         }[kind]
         return proto(fn.value), int(cap.value)
 
@@ -138,6 +170,15 @@ class Reference:
         packed = self.pack(dtype, b, viable)
         c = np.empty((m, n), dtype=OUTPUT[dtype])
         self.kernel(KIND_PACKED, dtype, viable)[0](_ptr(a), _ptr(packed), _ptr(c), m, n, k, a.strides[0], c.strides[0])
+        return c
+
+    def spatials_packed(self, kind: int, dtype: str, a: np.ndarray, b: np.ndarray, viable: int = CAP_SERIAL) -> np.ndarray:
+        """`nk_angulars_packed_<dtype>` / `nk_euclideans_packed_<dtype>` of the chosen backend, f32 results."""
+        m, k = a.shape
+        n = b.shape[0]
+        packed = self.pack(dtype, b, viable)
+        c = np.empty((m, n), dtype=np.float32)
+        self.kernel(kind, dtype, viable)[0](_ptr(a), _ptr(packed), _ptr(c), m, n, k, a.strides[0], c.strides[0])
         return c
 
 

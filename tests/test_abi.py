@@ -24,28 +24,30 @@ def declared_symbols():
         names |= set(re.findall(r"NK_DYNAMIC[^;(]*?\b(nk_[a-z0-9_]+)\s*\(", text))
         for t in TYPES:  # the backend-suffixed kernels come from a macro
             names |= {f"nk_dots_packed_size_{t}_gfx950", f"nk_dots_pack_{t}_gfx950", f"nk_dots_packed_{t}_gfx950"}
+            names |= {f"nk_angulars_packed_{t}_gfx950", f"nk_euclideans_packed_{t}_gfx950"}
+            names |= {f"nk_angulars_packed_{t}", f"nk_euclideans_packed_{t}"}  # also declared through a macro
     return {n for n in names if "##" not in n}
 
 
 def test_library_exports_every_declared_symbol():
     lib = nk.library()
     names = declared_symbols()
-    assert len(names) >= 18 * 2 + 8 + 15
+    assert len(names) >= 30 * 2 + 8 + 15
     missing = [n for n in sorted(names) if not hasattr(lib, n)]
     assert not missing, missing
     for t in TYPES:
-        for stem in ("nk_dots_packed_size_", "nk_dots_pack_", "nk_dots_packed_"):
+        for stem in ("nk_dots_packed_size_", "nk_dots_pack_", "nk_dots_packed_", "nk_angulars_packed_", "nk_euclideans_packed_"):
             assert hasattr(lib, stem + t)
 
 
 def test_packed_size_formula():
     """header + ceil(n/32) tiles * chunks (padded to an even number of 8-chunk stages) * 512 B + 128 B of column
-    terms per tile; fp8 stored as f16."""
+    terms and 128 B of column sums of squares per tile; fp8 stored as f16."""
     for t, width in (("i8", 1), ("u8", 1), ("bf16", 2), ("f16", 2), ("e4m3", 2), ("e5m2", 2)):
         for n, k in [(1, 1), (32, 128), (33, 129), (2048, 2048), (8191, 1000), (1048576, 768)]:
             tiles = -(-n // 32)
             chunks = -(-(-(-k * width // 16)) // 16) * 16
-            assert nk.dots_packed_size(t, n, k) == 64 + tiles * chunks * 512 + tiles * 128, (t, n, k)
+            assert nk.dots_packed_size(t, n, k) == 64 + tiles * chunks * 512 + tiles * 256, (t, n, k)
         assert nk.dots_packed_size(t, 0, 0) == 64
         assert nk.dots_packed_size(t, 1 << 40, 8) == 0  # dimensions beyond 32 bits are refused, as the error stub does
     with pytest.raises(TypeError):
@@ -102,7 +104,7 @@ def test_error_convention_without_backend():
         assert np.isnan(f[:, :3]).all() and (f[:, 3] == 0).all()
     finally:
         lib.nk_dispatch_table_update(lib.nk_capabilities_compiled())
-    assert lib.nk_dots_packed_size_i8(5, 7) == 64 + 16 * 512 + 128
+    assert lib.nk_dots_packed_size_i8(5, 7) == 64 + 16 * 512 + 256
 
 
 def test_no_gpu_means_loud_failure_not_fallback():

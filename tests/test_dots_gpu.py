@@ -212,7 +212,8 @@ def test_host_pointers_are_staged(oracle, dtype):
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
 def test_packed_image_layout(oracle, dtype):
-    """header | tiles[(t * k_chunks + c) * 32 + r] of 16 bytes | 128 * sum(b ^ 0x80 as i8) per column (u8)."""
+    """header | tiles[(t * k_chunks + c) * 32 + r] of 16 bytes | 128 * sum(b ^ 0x80 as i8) per column (u8) | sum(b^2)
+    per column."""
     rng = np.random.default_rng(33)
     n, k = 70, 203
     b = support.random_matrix(oracle, dtype, n, k, rng)
@@ -234,13 +235,20 @@ def test_packed_image_layout(oracle, dtype):
     expected = padded.reshape(tiles, 32, chunks, 16).transpose(0, 2, 1, 3).reshape(-1)
     data = image[64:64 + expected.size]
     assert np.array_equal(data, expected)
-    terms = image[64 + expected.size:].view(np.uint32)
-    assert terms.size == tiles * 32
+    tail = image[64 + expected.size:].view(np.uint32)
+    assert tail.size == 2 * tiles * 32
+    terms, norms = tail[:tiles * 32], tail[tiles * 32:]
     if dtype == "u8":
         sums = (b.astype(np.int64) - 128).sum(axis=1) * 128
         assert np.array_equal(terms[:n].astype(np.int64), sums & 0xFFFFFFFF) and (terms[n:] == 0).all()
     else:
         assert (terms == 0).all()
+    # per-column sums of squares: exact (mod 2^32) for the integer types, f64-accumulated and rounded once otherwise
+    if dtype in ("i8", "u8"):
+        assert np.array_equal(norms[:n].astype(np.int64), (b.astype(np.int64) ** 2).sum(axis=1) & 0xFFFFFFFF)
+    else:
+        exact = (oracle.decode(dtype, b).astype(np.float64) ** 2).sum(axis=1)
+        assert np.array_equal(norms[:n].view(np.float32), exact.astype(np.float32))
 
 
 def test_mismatched_image_poisons_output_and_zero_sizes(oracle):

@@ -143,6 +143,100 @@ def test_serial_layout_and_product_match_reference(oracle, reference, dtype):
             assert same_floats(oracle.dots_packed(dtype, a, b).view(np.float32), reference.dots_packed(dtype, a, b).view(np.float32))
 
 
+def finite_inputs(oracle, dtype, rows, cols, rng):
+    """Seeded rows without Inf/NaN codes (the e5m2 encoder overflows to Inf; distances are gated on finite inputs)."""
+    x = support.random_matrix(oracle, dtype, rows, cols, rng)
+    if dtype == "e5m2":
+        x = np.where((x & 0x7F) > 0x7B, (x & 0x80) | 0x7B, x).astype(x.dtype)
+    return x
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_row_sums_of_squares_match_reference_serial(oracle, reference, dtype):
+    """nk_reduce_moments_<T>_serial: exact integers, Neumaier-compensated f32 for the float types, bit for bit."""
+    if reference is None:
+        pytest.skip("reference build not present")
+    rng = np.random.default_rng(21)
+    moments, _ = reference_moments(reference, dtype)
+    for rows, cols in [(3, 1), (5, 37), (4, 1000), (2, 8192)]:
+        x = finite_inputs(oracle, dtype, rows, cols, rng)
+        mine = oracle.row_sumsq(dtype, x)
+        for i in range(rows):
+            assert mine[i:i + 1].view(np.uint32)[0] == moments(x[i]), (dtype, rows, cols, i)
+
+
+def reference_moments(reference, dtype):
+    import ctypes
+
+    fn, cap = ctypes.c_void_p(), ctypes.c_uint64()
+    reference.lib.nk_find_kernel_punned(ord("R"), support.CODES[dtype], support.CAP_SERIAL, ctypes.byref(fn), ctypes.byref(cap))
+    assert fn.value and cap.value
+    call = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p)(fn.value)
+
+    def sumsq_bits(row):
+        row = np.ascontiguousarray(row)
+        total, squares = np.zeros(1, np.uint64), np.zeros(1, np.uint64)
+        call(row.ctypes.data, row.size, row.itemsize, total.ctypes.data, squares.ctypes.data)
+        # integers: u64 sum of squares, truncated like dots/serial.h:154-164; floats: the f32 in the low half
+        return int(squares[0]) & 0xFFFFFFFF
+
+    return sumsq_bits, int(cap.value)
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_packed_distances_match_reference_serial(oracle, reference, dtype, metric):
+    """Integer types: every input of the finaliser is an exact integer, so the restated reciprocal square root
+    and formulas must reproduce nk_{angulars,euclideans}_packed_<T>_serial bit for bit. Float types: the reference
+    takes its norms from the host-dispatched nk_reduce_moments_*, one rounding away from the serial sum at most,
+    which the finaliser turns into a few roundings: within 8 * 2^-24 absolute for angular, and of the sum of the two
+    norms under the root for euclidean (where identical rows cancel to a residue of that size)."""
+    if reference is None:
+        pytest.skip("reference build not present")
+    rng = np.random.default_rng(22)
+    for m, n, k in [(1, 1, 1), (5, 7, 37), (33, 21, 300), (16, 16, 1024), (9, 4, 4099)]:
+        a, b = finite_inputs(oracle, dtype, m, k, rng), finite_inputs(oracle, dtype, n, k, rng)
+        if m > 4:
+            a[1] = 0  # a zero row: the "product of norms is not positive" branch
+            b[2] = a[3][:k] if n > 2 else b[0]  # identical rows: distance 0 up to rounding
+        mine = oracle.spatials_packed(metric, dtype, a, b)
+        ref = reference.spatials_packed(support.METRIC_KINDS[metric], dtype, a, b)
+        if dtype in ("i8", "u8"):
+            assert np.array_equal(mine.view(np.uint32), ref.view(np.uint32)), (dtype, metric, m, n, k)
+        else:
+            u = 2.0 ** -24
+            if metric == "angular":  # 1 - x with |x| <= 1: absolute roundings
+                assert np.abs(mine.astype(np.float64) - ref).max() <= 8 * u, (dtype, metric, m, n, k)
+            else:  # sqrt(qn + tn - 2 dot): roundings of the size of the norms, under the root
+                norms = oracle.row_sumsq(dtype, a).astype(np.float64)[:, None] + oracle.row_sumsq(dtype, b).astype(np.float64)[None, :]
+                gap = np.abs(mine.astype(np.float64) ** 2 - ref.astype(np.float64) ** 2)
+                close = np.abs(mine.astype(np.float64) - ref) <= 8 * u * np.abs(ref)  # a few ulp of the distance itself,
+                assert (close | (gap <= 8 * u * np.maximum(norms, 1e-30))).all(), (dtype, metric, m, n, k)  # or a cancelled residue
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_packed_distances_closed_forms(oracle, dtype, metric):
+    """Known answers that need no reference: orthogonal rows are at angular 1 / euclidean sqrt(|a|^2 + |b|^2),
+    a row against itself at 0, against its double (same direction) at angular 0 / euclidean |a|, zero rows at 0."""
+    one = {"i8": 1, "u8": 1, "bf16": 0x3F80, "f16": 0x3C00, "e4m3": 0x38, "e5m2": 0x3C}[dtype]
+    two = {"i8": 2, "u8": 2, "bf16": 0x4000, "f16": 0x4000, "e4m3": 0x40, "e5m2": 0x40}[dtype]
+    k = 64
+    rows = np.zeros((4, k), dtype=support.STORAGE[dtype])
+    rows[0, :16] = one   # |.|^2 = 16
+    rows[1, 16:32] = one  # orthogonal to row 0
+    rows[2, :16] = two   # row 0 doubled
+    got = oracle.spatials_packed(metric, dtype, rows, rows)
+    truth = oracle.spatials_truth(metric, dtype, rows, rows)
+    if metric == "angular":
+        expected = np.array([[0, 1, 0, 1], [1, 0, 1, 1], [0, 1, 0, 1], [1, 1, 1, 0]], dtype=np.float64)
+        expected[0, 3] = expected[3, 0] = expected[1, 3] = expected[3, 1] = expected[2, 3] = expected[3, 2] = 0  # zero norm and zero dot
+    else:
+        expected = np.array([[0, np.sqrt(32), 4, 4], [np.sqrt(32), 0, np.sqrt(80), 4], [4, np.sqrt(80), 0, 8], [4, 4, 8, 0]])
+    assert np.allclose(truth, expected, atol=1e-12)
+    assert np.allclose(got, expected, atol=2e-6)
+
+
 @pytest.mark.parametrize("dtype", ["i8", "u8"])
 def test_integer_product_closed_form(oracle, dtype):
     rng = np.random.default_rng(11)
@@ -196,6 +290,19 @@ def test_golden_vectors(oracle, name):
         dtype = str(data["dtype"])
         assert same_floats(oracle.decode(dtype, data["codes"]), data["decoded"])
         assert np.array_equal(oracle.encode(dtype, data["values"]), data["encoded"])
+    elif name.startswith("spatials_"):
+        dtype = str(data["dtype"])
+        a, b = data["a"], data["b"]
+        u = 2.0 ** -24
+        norms = oracle.row_sumsq(dtype, a).astype(np.float64)[:, None] + oracle.row_sumsq(dtype, b).astype(np.float64)[None, :]
+        for metric, key in (("angular", "angulars_serial"), ("euclidean", "euclideans_serial")):
+            mine, ref = oracle.spatials_packed(metric, dtype, a, b).astype(np.float64), data[key].astype(np.float64)
+            if dtype in ("i8", "u8"):
+                assert np.array_equal(mine, ref), (dtype, metric)
+            elif metric == "angular":
+                assert np.abs(mine - ref).max() <= 8 * u
+            else:
+                assert ((np.abs(mine - ref) <= 8 * u * np.abs(ref)) | (np.abs(mine ** 2 - ref ** 2) <= 8 * u * norms)).all()
     else:
         dtype = str(data["dtype"])
         a, b = data["a"], data["b"]

@@ -1,0 +1,199 @@
+"""Parity of the packed angular / euclidean distances with the reference, through the C ABI, on a real MI355X.
+
+`nk_angulars_packed_<T>` and `nk_euclideans_packed_<T>` (reference: include/numkong/spatials.h:139-266,
+include/numkong/dots/serial.h:2756-2800) run the packed product and then finalise every element with the
+row's and the column's sum of squares. All outputs are f32, also for the integer types, so nothing here can
+be bit-exact across backends (the reference's own backends differ in their square roots); the gate is the
+one of the float products, against the f64 truth next to TWO reference kernels on the same inputs, the serial
+one (oracle restatement, pinned in tests/test_oracle.py) and, when oracle/_ref is present, the host-dispatched one:
+
+  angular    e = |x - truth|                               (x = 1 - cos is at most 2: absolute error)
+  euclidean  e = |x^2 - truth^2| / (|a|^2 + |b|^2)          (robust where identical rows cancel to ~0)
+  gate:      mean(e_gpu) <= 2 * mean(e_ref) + 2^-24 / sqrt(count),   max(e_gpu) <= 2 * max(max(e_ref), 2 * 2^-24)
+
+The floor under the max: four f32 roundings enter every result whatever the kernel (the dot, the two norms, their
+product or sum), so where identical rows cancel, any kernel, the reference's included, lands anywhere within
+three or four units of 2^-24 of the truth; which one is luck, and a single such element decides the max.
+
+Measured on 192 x 256 outputs at depth 4096: GPU / serial and GPU / dispatched mean-error ratios between 0.24
+and 1.10 for all six types and both distances.
+"""
+import os
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+import numkong_amd as nk  # noqa: E402
+from numkong_amd import api  # noqa: E402
+from tests import support  # noqa: E402
+from tests.support import ALL_DTYPES  # noqa: E402
+from tests.test_dots_gpu import DEV, U, to_gpu  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+METRICS = ["angular", "euclidean"]
+GPU_CALL = {"angular": nk.angulars_packed, "euclidean": nk.euclideans_packed}
+_REFERENCE = []
+
+
+def reference_library():
+    if not _REFERENCE:
+        _REFERENCE.append(support.load_reference())
+    return _REFERENCE[0]
+
+
+def finite_inputs(oracle, dtype, rows, cols, rng, kind="default"):
+    x = support.random_matrix(oracle, dtype, rows, cols, rng, kind)
+    if dtype == "e5m2":  # the reference-rule encoder overflows to Inf: keep the distances finite
+        x = np.where((x & 0x7F) > 0x7B, (x & 0x80) | 0x7B, x).astype(x.dtype)
+    return x
+
+
+def errors(metric, values, truth, norms):
+    values = values.astype(np.float64)
+    if metric == "angular":
+        return np.abs(values - truth)
+    return np.abs(values ** 2 - truth ** 2) / np.maximum(norms, 1e-300)
+
+
+def assert_distance_gate(oracle, metric, dtype, a, b, got, where=""):
+    truth = oracle.spatials_truth(metric, dtype, a, b)
+    decoded_a = a.astype(np.float64) if dtype in ("i8", "u8") else oracle.decode(dtype, a).astype(np.float64)
+    decoded_b = b.astype(np.float64) if dtype in ("i8", "u8") else oracle.decode(dtype, b).astype(np.float64)
+    norms = (decoded_a ** 2).sum(axis=1)[:, None] + (decoded_b ** 2).sum(axis=1)[None, :]
+    assert np.isfinite(got).all(), where
+    e_gpu = errors(metric, got, truth, norms)
+    references = [("serial", oracle.spatials_packed(metric, dtype, a, b))]
+    if reference_library() is not None:
+        reference = reference_library()
+        references.append(("dispatched", reference.spatials_packed(support.METRIC_KINDS[metric], dtype, a, b,
+                                                                   viable=reference.capabilities)))
+    for name, ref in references:
+        e_ref = errors(metric, ref, truth, norms)
+        slack = U / np.sqrt(e_gpu.size)
+        assert e_gpu.mean() <= 2 * e_ref.mean() + slack, f"mean error {e_gpu.mean():.3e} vs {name} {e_ref.mean():.3e} {where}"
+        assert e_gpu.max() <= 2 * max(e_ref.max(), 2 * U), f"max error {e_gpu.max():.3e} vs {name} {e_ref.max():.3e} {where}"
+
+
+def gpu_distances(metric, dtype, a, b, config=0):
+    nk.library().nk_hip_set_tile_config(config)
+    try:
+        return GPU_CALL[metric](to_gpu(a), nk.dots_pack(to_gpu(b), dtype)).cpu().numpy()
+    finally:
+        nk.library().nk_hip_set_tile_config(0)
+
+
+SHAPES = [(1, 1, 1), (3, 5, 7), (33, 70, 200), (64, 64, 64), (100, 37, 333), (257, 129, 1000), (130, 33, 4100)]
+
+
+@pytest.mark.parametrize("metric", METRICS)
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("config", [0, 1, 2, 3, 4])
+def test_small_shapes_every_tile_config(oracle, dtype, metric, config):
+    rng = np.random.default_rng(300 + config)
+    for m, n, k in SHAPES:
+        a, b = finite_inputs(oracle, dtype, m, k, rng), finite_inputs(oracle, dtype, n, k, rng)
+        if m > 4 and n > 4:
+            a[1] = 0         # zero row: distances 0 (angular, zero dot) and |b|
+            b[2] = a[3]      # identical rows: both distances cancel to ~0
+            b[4] = 0
+        got = gpu_distances(metric, dtype, a, b, config)
+        assert_distance_gate(oracle, metric, dtype, a, b, got, f"{dtype} {metric} {m}x{n}x{k} config {config}")
+        if m > 4 and n > 4:
+            assert got[1, 4] == 0  # two zero rows
+            if metric == "angular":
+                assert (got[1] == 0).all()  # a zero row has dot 0 with everything: the reference returns 0 there
+
+
+@pytest.mark.parametrize("metric", METRICS)
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_deep_rows(oracle, dtype, metric):
+    """Depth 8192: the sums of squares run over 64 to 128 pipeline stages."""
+    rng = np.random.default_rng(31)
+    a, b = finite_inputs(oracle, dtype, 48, 8192, rng), finite_inputs(oracle, dtype, 80, 8192, rng)
+    assert_distance_gate(oracle, metric, dtype, a, b, gpu_distances(metric, dtype, a, b), f"{dtype} {metric} deep")
+
+
+@pytest.mark.parametrize("name", sorted(f for f in os.listdir(support.GOLDEN_DIR) if f.startswith("spatials_")))
+def test_golden_vectors(oracle, name):
+    """Inputs and serial-kernel outputs recorded from the reference library."""
+    data = np.load(os.path.join(support.GOLDEN_DIR, name))
+    dtype, a, b = str(data["dtype"]), data["a"], data["b"]
+    for metric, key in (("angular", "angulars_serial"), ("euclidean", "euclideans_serial")):
+        got = gpu_distances(metric, dtype, a, b)
+        assert_distance_gate(oracle, metric, dtype, a, b, got, name)
+        recorded = data[key].astype(np.float64)
+        if metric == "angular":
+            assert np.abs(got - recorded).max() <= 16 * U
+        else:
+            assert np.abs(got - recorded).max() <= 16 * U * max(1.0, float(np.abs(recorded).max())) + 0.02  # cancelled rows
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_c_abi_strides_host_pointers_and_async(oracle, dtype):
+    """Same calling convention as the packed product: byte strides, host or device pointers, caller's stream."""
+    rng = np.random.default_rng(41)
+    lib = nk.library()
+    m, n, k, pad = 37, 61, 515, 5
+    a_full = finite_inputs(oracle, dtype, m, k + pad, rng)
+    b = np.ascontiguousarray(finite_inputs(oracle, dtype, n, k, rng))
+    a = np.ascontiguousarray(a_full[:, :k])
+    width = a.itemsize
+    # host pointers, padded strides on both sides
+    size = getattr(lib, f"nk_dots_packed_size_{dtype}")(n, k)
+    packed = np.zeros(size, np.uint8)
+    getattr(lib, f"nk_dots_pack_{dtype}")(b.ctypes.data, n, k, b.strides[0], packed.ctypes.data)
+    for metric in METRICS:
+        c = np.full((m, n + 3), np.float32(-7.0))
+        getattr(lib, f"nk_{metric}s_packed_{dtype}")(a_full.ctypes.data, packed.ctypes.data, c.ctypes.data, m, n, k,
+                                                     a_full.strides[0], c.strides[0])
+        assert not lib.nk_amd_last_error()
+        assert (c[:, n:] == -7.0).all()
+        assert_distance_gate(oracle, metric, dtype, a, b, np.ascontiguousarray(c[:, :n]), f"{dtype} {metric} host")
+        # asynchronous form on the caller's stream, device pointers
+        ga, gp = to_gpu(a), torch.from_numpy(packed).to(DEV)
+        gc = torch.empty((m, n), dtype=torch.float32, device=DEV)
+        kind = support.METRIC_KINDS[metric]
+        status = lib.nk_amd_spatials_packed_async(kind, api.DTYPES[dtype][0], ga.data_ptr(), gp.data_ptr(), gc.data_ptr(), m, n,
+                                                  k, k * width, n * 4, torch.cuda.current_stream().cuda_stream)
+        assert status == 0, lib.nk_hip_last_error()
+        torch.cuda.synchronize()
+        # (not bit-identical to the staged call for the float types: rows 1030 bytes apart are not dword-aligned and
+        # take the plain loop, which sums in another order than the pipelined one the 16-byte-padded staging gets)
+        assert_distance_gate(oracle, metric, dtype, a, b, gc.cpu().numpy(), f"{dtype} {metric} async")
+        if dtype in ("i8", "u8"):
+            assert np.array_equal(gc.cpu().numpy().view(np.uint32), np.ascontiguousarray(c[:, :n]).view(np.uint32))
+
+
+def test_mismatched_image_poisons_output(oracle):
+    """An image packed for another depth: every output is all ones (NaN), as the reference's error stub leaves them."""
+    rng = np.random.default_rng(43)
+    a = to_gpu(finite_inputs(oracle, "bf16", 9, 128, rng))
+    packed = nk.dots_pack(to_gpu(finite_inputs(oracle, "bf16", 11, 256, rng)), "bf16")
+    c = torch.zeros((9, 11), dtype=torch.float32, device=DEV)
+    status = nk.library().nk_amd_spatials_packed_async(support.KIND_ANGULARS, api.DTYPES["bf16"][0], a.data_ptr(),
+                                                       packed.buffer.data_ptr(), c.data_ptr(), 9, 11, 128, 256, 44,
+                                                       torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert status == 0 and (c.cpu().numpy().view(np.uint32) == 0xFFFFFFFF).all()
+    with pytest.raises(ValueError):
+        nk.euclideans_packed(a, packed)  # the Python mirror checks the depth first
+
+
+@pytest.mark.parametrize("dtype", ["i8", "bf16"])
+def test_retrieval_shape_sampled(oracle, dtype):
+    """1024 queries against 131,072 vectors of dimension 768, angular: sampled rows x columns against the oracle,
+    plus the property that every distance lies in [0, 2] and a vector is at distance ~0 from itself."""
+    m, n, k = 1024, 1 << 17, 768
+    rng = np.random.default_rng(47)
+    queries = finite_inputs(oracle, dtype, m, k, rng)
+    database = finite_inputs(oracle, dtype, n, k, rng)
+    database[5::4099] = queries[7]  # plant copies of one query
+    packed = nk.dots_pack(to_gpu(database), dtype)
+    c = nk.angulars_packed(to_gpu(queries), packed)
+    assert float(c.min()) >= 0 and float(c.max()) <= 2
+    assert float(c[7, 5::4099].max()) <= 4 * U * 4
+    rows, cols = np.arange(3, m, 97), np.concatenate([np.arange(1, n, 1571), [n - 1]])
+    got = c[torch.from_numpy(rows).to(DEV)][:, torch.from_numpy(cols).to(DEV)].cpu().numpy()
+    assert_distance_gate(oracle, "angular", dtype, queries[rows], database[cols], got, f"{dtype} retrieval sample")
