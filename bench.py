@@ -31,13 +31,16 @@ HBM_PEAK = 8000.0
 # each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
 # the summaries are under profiles/. Not re-measured by a plain run: counters need the profiler.
 MEASURED_TRAFFIC = {
-    ("i8", 8192, 8192, 8192): 1.0816e9,
-    ("bf16", 8192, 8192, 8192): 2.4244e9,
-    ("e4m3", 8192, 8192, 8192): 1.8863e9,
-    ("i8", 1024, 1 << 20, 768): 5.4967e9,
+    ("i8", 8192, 8192, 8192): 1.0834e9,
+    ("bf16", 8192, 8192, 8192): 2.4219e9,
+    ("e4m3", 8192, 8192, 8192): 1.8864e9,
+    ("i8", 1024, 1 << 20, 768): 5.5013e9,
+    ("i8", 1024, 1 << 20, 768, "angular"): 5.3795e9,
 }
 HEADLINE = ("i8", 8192, 8192, 8192)
-OTHERS = [("bf16", 8192, 8192, 8192), ("e4m3", 8192, 8192, 8192), ("i8", 1024, 1 << 20, 768)]
+OTHERS = [("bf16", 8192, 8192, 8192, "dots"), ("e4m3", 8192, 8192, 8192, "dots"), ("i8", 1024, 1 << 20, 768, "dots"),
+          ("i8", 1024, 1 << 20, 768, "angular")]
+KINDS = {"angular": ord("N"), "euclidean": ord("E")}  # nk_kernel_angulars_packed_k, nk_kernel_euclideans_packed_k
 
 
 def make_operands(dtype, m, n, k, seed=42):
@@ -63,7 +66,7 @@ def make_operands(dtype, m, n, k, seed=42):
     return one(m), one(n)
 
 
-def time_gpu(dtype, m, n, k, steps, warmup):
+def time_gpu(dtype, m, n, k, steps, warmup, metric="dots"):
     import torch
 
     import numkong_amd as nk
@@ -73,13 +76,17 @@ def time_gpu(dtype, m, n, k, steps, warmup):
     a, b = make_operands(dtype, m, n, k)
     packed = nk.dots_pack(b, dtype)
     del b
-    c = torch.empty((m, n), dtype=torch.int32 if dtype in ("i8", "u8") else torch.float32, device="cuda:0")
+    c = torch.empty((m, n), dtype=torch.int32 if dtype in ("i8", "u8") and metric == "dots" else torch.float32, device="cuda:0")
     code, width = api.DTYPES[dtype][0], api.DTYPES[dtype][1]
     stream = torch.cuda.current_stream().cuda_stream  # the kernel is launched on this stream, so torch events see it
 
     def step():
-        status = lib.nk_amd_dots_packed_async(code, a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(), m, n, k,
-                                              k * width, n * 4, stream)
+        if metric == "dots":
+            status = lib.nk_amd_dots_packed_async(code, a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(), m, n, k,
+                                                  k * width, n * 4, stream)
+        else:  # the same product with the distance finaliser fused into its epilogue
+            status = lib.nk_amd_spatials_packed_async(KINDS[metric], code, a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(),
+                                                      m, n, k, k * width, n * 4, stream)
         if status:
             raise RuntimeError(lib.nk_hip_last_error().decode())
 
@@ -101,11 +108,12 @@ def time_gpu(dtype, m, n, k, steps, warmup):
         algorithmic = (m * k + n * k) * width + m * n * 4
         result["roofline"] = {"bound": "hbm", "achieved": algorithmic / (device_ms * 1e-3) / 1e9, "peak": HBM_PEAK,
                               "unit": "GB/s", "frac": algorithmic / (device_ms * 1e-3) / 1e9 / HBM_PEAK,
-                              "traffic": MEASURED_TRAFFIC.get((dtype, m, n, k))}
+                              "traffic": MEASURED_TRAFFIC.get((dtype, m, n, k) if metric == "dots" else (dtype, m, n, k, metric))}
     else:
         achieved = ops / (device_ms * 1e-3) / 1e12
         result["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK[dtype], "unit": "TFLOP/s",
-                              "frac": achieved / MFMA_PEAK[dtype], "traffic": MEASURED_TRAFFIC.get((dtype, m, n, k))}
+                              "frac": achieved / MFMA_PEAK[dtype],
+                              "traffic": MEASURED_TRAFFIC.get((dtype, m, n, k) if metric == "dots" else (dtype, m, n, k, metric))}
         if dtype in MFMA_NOTE:
             result["roofline"]["note"] = MFMA_NOTE[dtype]
     del a, packed, c
@@ -185,6 +193,8 @@ def main():
     parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--dtype", default=HEADLINE[0])
     parser.add_argument("--shape", type=int, nargs=3, default=list(HEADLINE[1:]))
+    parser.add_argument("--metric", default="dots", choices=["dots", "angular", "euclidean"],
+                        help="what the timed call computes: the packed product, or one of the packed distances on top of it")
     parser.add_argument("--no-others", action="store_true")
     parser.add_argument("--no-cpu", action="store_true")
     parser.add_argument("--probe", action="store_true",
@@ -205,23 +215,23 @@ def main():
             torch.add(source, 1, out=target)  # an elementwise kernel of known traffic: 1 GiB read + 1 GiB written
         torch.cuda.synchronize()
         del source, target
-        time_gpu(args.dtype, m, n, k, 3, 0)
+        time_gpu(args.dtype, m, n, k, 3, 0, args.metric)
         return
-    head = time_gpu(args.dtype, m, n, k, args.steps, args.warmup)
+    head = time_gpu(args.dtype, m, n, k, args.steps, args.warmup, args.metric)
     line = {
         "metric": "gso/s and % MFMA peak: i8->i32, bf16->f32, e4m3->f32 packed dots at 8192^3",
         "value": head["gso_per_s"], "unit": "gso/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": f"{args.dtype} packed dots C = A * B^T, M={m} N={n} K={k}, A row-major in HBM, "
+        "config": {"workload": f"{args.dtype} packed {args.metric} C = A * B^T, M={m} N={n} K={k}, A row-major in HBM, "
                                "B packed once outside the timed region, C overwritten"},
         "kernel_ms": head["kernel_ms"], "roofline": head["roofline"],
     }
     if not args.no_others:
         line["others"] = {}
-        for dtype, om, on, ok in OTHERS:
-            r = time_gpu(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2))
-            line["others"][f"{dtype}_{om}x{on}x{ok}"] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"],
+        for dtype, om, on, ok, metric in OTHERS:
+            r = time_gpu(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2), metric)
+            line["others"][f"{dtype}_{om}x{on}x{ok}" + ("" if metric == "dots" else "_" + metric)] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"],
                                                          "roofline": r["roofline"]}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.dtype, m, n, k)

@@ -55,6 +55,10 @@ def library() -> ctypes.CDLL:
         raise NumKongAmdError(
             f"{path} is missing: build it with `make -C numkong_amd/csrc` (there is no CPU fallback)"
         )
+    try:  # torch ships its own HIP runtime: load it first, so that the library binds to the same one
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = ctypes.CDLL(path)
     sz, vp, i32 = ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int
     for name in DTYPES:

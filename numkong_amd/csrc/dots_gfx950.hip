@@ -421,35 +421,37 @@ struct E5M2 : F16 {
 };
 
 /**
- *  Distance from a dot product and two sums of squares, as the reference's scalar finalisers compute it
+ *  Distances from a dot product and two sums of squares, as the reference's scalar finalisers compute them
  *  (spatial/serial.h:257-344): integer inputs are converted to f32 first (the i8 kernels read both norms as
  *  signed 32-bit integers, the u8 kernels as unsigned); angular = max(1 - dot * rsqrt(qn * tn), 0), and 0 or
  *  1 when the product of the norms is not positive; euclidean = sqrt(max(qn + tn - 2 * dot, 0)).
- *  METRIC: 1 angular, 2 euclidean. The hardware's rsqrt (refined by one Newton step) and sqrt (1 ulp) stand in
- *  for the reference's bit trick and three Newton steps.
  */
+template <class T>
+__device__ __forceinline__ float norm_as_f32(uint32_t bits) {
+    if (T::kDtype == kI8) return (float)(int)bits;
+    if (T::kDtype == kU8) return (float)bits;
+    return __builtin_bit_cast(float, bits);
+}
+
+/** METRIC: 1 angular, 2 euclidean. `query` and `target` are the row's and the column's sums of squares as f32
+ *  (converted once per row and once per column of a tile). The reciprocal square root is the hardware's estimate
+ *  (1 ulp) refined by one Newton step with fused residuals: identical rows must cancel to within a rounding or
+ *  two, as the reference's three Newton steps do (splitting it into a factor per row and a factor per column
+ *  would save half of the operations and lose exactly that). */
 template <class T, int METRIC>
-__device__ __forceinline__ uint32_t distance_from_dot(uint32_t dot_bits, uint32_t row_norm_bits, uint32_t col_norm_bits) {
-    float dot, query, target;
-    if (T::kDtype == kI8) dot = (float)(int)dot_bits, query = (float)(int)row_norm_bits, target = (float)(int)col_norm_bits;
-    else if (T::kDtype == kU8) dot = (float)dot_bits, query = (float)row_norm_bits, target = (float)col_norm_bits;
-    else {
-        dot = __builtin_bit_cast(float, dot_bits), query = __builtin_bit_cast(float, row_norm_bits);
-        target = __builtin_bit_cast(float, col_norm_bits);
-    }
+__device__ __forceinline__ uint32_t distance_from_dot(uint32_t dot_bits, float query, float target) {
+    float const dot = T::kDtype == kI8 ? (float)(int)dot_bits : (T::kDtype == kU8 ? (float)dot_bits : __builtin_bit_cast(float, dot_bits));
     float result;
     if (METRIC == 1) {
         float const product = query * target;
-        // the hardware estimate (1 ulp) plus one Newton step with fused residuals: identical rows must cancel to
-        // within a rounding or two, as the reference's three Newton steps do
         float root = __builtin_amdgcn_rsqf(product);
         float const residual = __builtin_fmaf(-(product * root), root, 1.0f);
         root = __builtin_fmaf(root * 0.5f, residual, root);
-        float const unclipped = __builtin_fmaf(-dot, root, 1.0f);
-        result = product > 0 ? (unclipped > 0 ? unclipped : 0.0f) : (dot == 0 ? 0.0f : 1.0f);
+        float const unclipped = __builtin_fmaxf(__builtin_fmaf(-dot, root, 1.0f), 0.0f);
+        result = product > 0 ? unclipped : (dot == 0 ? 0.0f : 1.0f);
     }
     else {
-        float const squared = query + target - 2.0f * dot;
+        float const squared = __builtin_fmaf(-2.0f, dot, query + target);
         result = squared > 0 ? __builtin_amdgcn_sqrtf(squared) : 0.0f;
     }
     return __builtin_bit_cast(uint32_t, result);
@@ -999,8 +1001,10 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                     norm_t sum = 0;
 #pragma unroll
                     for (int part = 0; part < 8; ++part) sum += parts[part];
-                    if constexpr (sizeof(norm_t) == 8) row_norms[tid] = __builtin_bit_cast(uint32_t, (float)sum); // f64 -> f32, once
-                    else row_norms[tid] = (uint32_t)sum;
+                    uint32_t bits;
+                    if constexpr (sizeof(norm_t) == 8) bits = __builtin_bit_cast(uint32_t, (float)sum); // f64 -> f32, once
+                    else bits = (uint32_t)sum;
+                    row_norms[tid] = __builtin_bit_cast(uint32_t, norm_as_f32<T>(bits));
                 }
             }
             __syncthreads();
@@ -1031,6 +1035,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 // scalar registers overflow).
                 global_u8_t *row_base = c_tile + j * 128;
                 v4i row_term4 = {0, 0, 0, 0}, row_norm4 = {0, 0, 0, 0};
+                float const col_value = metric != 0 ? norm_as_f32<T>(col_norm[j]) : 0.0f;
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -1046,7 +1051,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                         }
                         if (metric != 0) {
                             if (v % 4 == 0) row_norm4 = *(v4i const *)&row_norms[i * 32 + 8 * (v / 4) + 4 * half];
-                            bits = distance_from_dot<T, metric == 2 ? 2 : 1>(bits, (uint32_t)row_norm4[v % 4], col_norm[j]);
+                            int const row_bits = row_norm4[v % 4];
+                            bits = distance_from_dot<T, metric == 2 ? 2 : 1>(bits, __builtin_bit_cast(float, row_bits), col_value);
                         }
                         if ((!(DBG & 16) || bits == 0x12345678u) && // (timing experiment: almost no stores)
                             (!masked || (col_ok && row0 + r_fixed + 4 * half < g.m)))
@@ -1161,6 +1167,10 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream) {
                 config = c;
                 break;
             }
+        // Distances over a shallow depth are bound by the epilogue (a finaliser and a store per output): two
+        // workgroups per CU of 128 x 128 tiles overlap it with the other's loop better than one large tile does
+        // (measured on 1024 x 1,048,576 x 768: 2.17 against 2.33 ms angular, 1.98 against 2.07 ms euclidean).
+        if (g.metric != 0 && config < 3 && g.k_chunks / kStageChunks <= 8 && tiles(3) >= 256) config = 3;
     }
     if (T::kChunked && config == 1) config = 2; // two accumulator sets do not fit the 256 x 256 tile
     switch (config) {
