@@ -7,6 +7,11 @@ region, as the reference's own benchmark does: bench/bench.hpp:238-255). The hea
 i8 -> i32 product at M = N = K = 8192; bf16 and e4m3 at the same shape and the HBM-bound retrieval shape
 (1024 queries x 1,048,576 vectors x 768) are measured the same way and reported under "others".
 gso/s = 2*M*N*K / seconds / 1e9 (bench/bench.hpp:257). All operands are resident in HBM before timing.
+
+The symmetric kinds (`--metric symmetric`, `symmetric-angular`, `symmetric-euclidean`; N vectors of depth K, M is
+ignored) time the whole call as the reference's benchmark does (bench/bench.hpp:397-438): packing the vectors,
+building the tile list and the triangular product, into a workspace allocated once; they count N*(N+1)*K scalar
+operations per call, the upper triangle only.
 """
 from __future__ import annotations
 
@@ -39,8 +44,10 @@ MEASURED_TRAFFIC = {
 }
 HEADLINE = ("i8", 8192, 8192, 8192)
 OTHERS = [("bf16", 8192, 8192, 8192, "dots"), ("e4m3", 8192, 8192, 8192, "dots"), ("i8", 1024, 1 << 20, 768, "dots"),
-          ("i8", 1024, 1 << 20, 768, "angular")]
+          ("i8", 1024, 1 << 20, 768, "angular"), ("i8", 8192, 8192, 8192, "symmetric"), ("bf16", 8192, 8192, 8192, "symmetric")]
 KINDS = {"angular": ord("N"), "euclidean": ord("E")}  # nk_kernel_angulars_packed_k, nk_kernel_euclideans_packed_k
+# nk_kernel_dots_symmetric_k, nk_kernel_angulars_symmetric_k, nk_kernel_euclideans_symmetric_k
+SYMMETRIC_KINDS = {"symmetric": ord("y"), "symmetric-angular": ord("n"), "symmetric-euclidean": ord("D")}
 
 
 def make_operands(dtype, m, n, k, seed=42):
@@ -66,12 +73,59 @@ def make_operands(dtype, m, n, k, seed=42):
     return one(m), one(n)
 
 
+def time_symmetric(dtype, n, k, steps, warmup, metric):
+    """All pairs of n vectors of depth k, upper triangle: one call packs, lists its tiles and multiplies."""
+    import torch
+
+    import numkong_amd as nk
+    from numkong_amd import api
+
+    lib = nk.library()
+    vectors, _ = make_operands(dtype, n, 1, k)
+    code, width = api.DTYPES[dtype][0], api.DTYPES[dtype][1]
+    result = torch.zeros((n, n), dtype=torch.int32 if dtype in ("i8", "u8") and metric == "symmetric" else torch.float32,
+                         device="cuda:0")
+    workspace_bytes = lib.nk_amd_symmetric_workspace_size(code, n, k, 0, n)
+    workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        status = lib.nk_amd_symmetric_async(SYMMETRIC_KINDS[metric], code, vectors.data_ptr(), n, k, k * width,
+                                            result.data_ptr(), n * 4, 0, n, workspace.data_ptr(), workspace_bytes, stream)
+        if status:
+            raise RuntimeError(lib.nk_hip_last_error().decode())
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    wall = time.perf_counter()
+    begin.record()
+    for _ in range(steps):
+        step()
+    end.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - wall) * 1e3 / steps
+    device_ms = begin.elapsed_time(end) / steps
+    ops = 1.0 * n * (n + 1) * k
+    achieved = ops / (device_ms * 1e-3) / 1e12
+    out = {"ms_per_step": wall, "kernel_ms": device_ms, "gso_per_s": ops / (wall * 1e-3) / 1e9,
+           "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK[dtype], "unit": "TFLOP/s",
+                        "frac": achieved / MFMA_PEAK[dtype], "traffic": MEASURED_TRAFFIC.get((dtype, n, n, k, metric)),
+                        "note": "whole call (pack + tile list + product) over the operations of the upper triangle"}}
+    del vectors, result, workspace
+    torch.cuda.empty_cache()
+    return out
+
+
 def time_gpu(dtype, m, n, k, steps, warmup, metric="dots"):
     import torch
 
     import numkong_amd as nk
     from numkong_amd import api
 
+    if metric in SYMMETRIC_KINDS:
+        return time_symmetric(dtype, n, k, steps, warmup, metric)
     lib = nk.library()
     a, b = make_operands(dtype, m, n, k)
     packed = nk.dots_pack(b, dtype)
@@ -193,8 +247,9 @@ def main():
     parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--dtype", default=HEADLINE[0])
     parser.add_argument("--shape", type=int, nargs=3, default=list(HEADLINE[1:]))
-    parser.add_argument("--metric", default="dots", choices=["dots", "angular", "euclidean"],
-                        help="what the timed call computes: the packed product, or one of the packed distances on top of it")
+    parser.add_argument("--metric", default="dots", choices=["dots", "angular", "euclidean"] + sorted(SYMMETRIC_KINDS),
+                        help="what the timed call computes: the packed product, one of the packed distances on top of it, or "
+                             "one of the symmetric kinds over N vectors of depth K")
     parser.add_argument("--no-others", action="store_true")
     parser.add_argument("--no-cpu", action="store_true")
     parser.add_argument("--probe", action="store_true",
@@ -223,15 +278,18 @@ def main():
         "value": head["gso_per_s"], "unit": "gso/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": f"{args.dtype} packed {args.metric} C = A * B^T, M={m} N={n} K={k}, A row-major in HBM, "
-                               "B packed once outside the timed region, C overwritten"},
+        "config": {"workload": (f"{args.dtype} {args.metric} all pairs of N={n} vectors of depth K={k}, upper triangle, vectors "
+                                "row-major in HBM, packed inside the timed call") if args.metric in SYMMETRIC_KINDS else
+                               (f"{args.dtype} packed {args.metric} C = A * B^T, M={m} N={n} K={k}, A row-major in HBM, "
+                                "B packed once outside the timed region, C overwritten")},
         "kernel_ms": head["kernel_ms"], "roofline": head["roofline"],
     }
     if not args.no_others:
         line["others"] = {}
         for dtype, om, on, ok, metric in OTHERS:
             r = time_gpu(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2), metric)
-            line["others"][f"{dtype}_{om}x{on}x{ok}" + ("" if metric == "dots" else "_" + metric)] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"],
+            name = f"{dtype}_{on}x{ok}_{metric}" if metric in SYMMETRIC_KINDS else f"{dtype}_{om}x{on}x{ok}" + ("" if metric == "dots" else "_" + metric)
+            line["others"][name] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"],
                                                          "roofline": r["roofline"]}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.dtype, m, n, k)

@@ -66,7 +66,8 @@ typedef enum {
 } nk_dtype_t;
 
 /** Kernel kinds (reference: include/numkong/capabilities.h:178-253; same codes). The three dots kinds and the
- *  two packed distance kinds resolve to kernels here; every other kind resolves to the error stub with capability 0. */
+ *  two packed distance kinds, and the three symmetric kinds, resolve to kernels here; every other kind resolves to
+ *  the error stub with capability 0. */
 typedef enum {
     nk_kernel_unknown_k = 0,
     nk_kernel_dot_k = 'i',
@@ -76,6 +77,8 @@ typedef enum {
     nk_kernel_dots_symmetric_k = 'y',
     nk_kernel_angulars_packed_k = 'N',
     nk_kernel_euclideans_packed_k = 'E',
+    nk_kernel_angulars_symmetric_k = 'n',
+    nk_kernel_euclideans_symmetric_k = 'D',
 } nk_kernel_kind_t;
 
 /** Capability mask (reference: include/numkong/capabilities.h:258-304). Bit 0 keeps its reference meaning
@@ -92,6 +95,9 @@ typedef void (*nk_dots_pack_punned_t)(void const *b, nk_size_t columns, nk_size_
                                       void *b_packed);
 typedef void (*nk_dots_packed_punned_t)(void const *a, void const *b_packed, void *c, nk_size_t rows, nk_size_t columns,
                                         nk_size_t depth, nk_size_t a_stride_bytes, nk_size_t c_stride_bytes);
+typedef void (*nk_dots_symmetric_punned_t)(void const *vectors, nk_size_t vectors_count, nk_size_t depth,
+                                           nk_size_t stride_bytes, void *result, nk_size_t result_stride_bytes,
+                                           nk_size_t row_start, nk_size_t row_count);
 typedef void (*nk_kernel_punned_t)(void *);
 
 /* Bytes of the packed image of an (width x depth) B. Reference: include/numkong/dots.h:172-195. */
@@ -143,6 +149,30 @@ NK_AMD_DECLARE_SPATIALS_(e4m3, nk_e4m3_t)
 NK_AMD_DECLARE_SPATIALS_(e5m2, nk_e5m2_t)
 #undef NK_AMD_DECLARE_SPATIALS_
 
+/* All pairs of one set of vectors: result[i][j] for i in [row_start, row_start + row_count), j >= i, is the dot
+ * product (widened, as above) or the angular / euclidean distance (f32) of vectors i and j; the distance of a vector
+ * from itself is exactly 0. Only that upper triangle of the window is written; a caller that wants the full matrix
+ * mirrors it (python/distance.c:865-872) and splits the rows among its threads with the window arguments. Reference:
+ * include/numkong/dots.h:298-359, include/numkong/spatials.h:76-120, 245-275; include/numkong/dots/serial.h:2361-2435,
+ * 2802-2878 for the semantics. */
+#define NK_AMD_DECLARE_SYMMETRIC_(T, in_t, out_t)                                                                      \
+    NK_DYNAMIC void nk_dots_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,              \
+                                          nk_size_t stride, out_t *result, nk_size_t result_stride,                   \
+                                          nk_size_t row_start, nk_size_t row_count);                                  \
+    NK_DYNAMIC void nk_angulars_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,          \
+                                              nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,            \
+                                              nk_size_t row_start, nk_size_t row_count);                              \
+    NK_DYNAMIC void nk_euclideans_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,        \
+                                                nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,          \
+                                                nk_size_t row_start, nk_size_t row_count);
+NK_AMD_DECLARE_SYMMETRIC_(i8, nk_i8_t, nk_i32_t)
+NK_AMD_DECLARE_SYMMETRIC_(u8, nk_u8_t, nk_u32_t)
+NK_AMD_DECLARE_SYMMETRIC_(bf16, nk_bf16_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(f16, nk_f16_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(e4m3, nk_e4m3_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(e5m2, nk_e5m2_t, nk_f32_t)
+#undef NK_AMD_DECLARE_SYMMETRIC_
+
 /* Capability and lookup API. Reference: c/numkong.c:767-768, 831-913. */
 NK_DYNAMIC int nk_uses_dynamic_dispatch(void);
 NK_DYNAMIC int nk_configure_thread(nk_capability_t capabilities);
@@ -170,7 +200,16 @@ NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t i
                                                     nk_size_t c_stride);                                                  \
     NK_DYNAMIC void nk_euclideans_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height, \
                                                       nk_size_t width, nk_size_t depth, nk_size_t a_stride,               \
-                                                      nk_size_t c_stride);
+                                                      nk_size_t c_stride);                                                \
+    NK_DYNAMIC void nk_dots_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,         \
+                                                   nk_size_t stride, out_t *result, nk_size_t result_stride,              \
+                                                   nk_size_t row_start, nk_size_t row_count);                             \
+    NK_DYNAMIC void nk_angulars_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,     \
+                                                       nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,       \
+                                                       nk_size_t row_start, nk_size_t row_count);                         \
+    NK_DYNAMIC void nk_euclideans_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,   \
+                                                         nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,     \
+                                                         nk_size_t row_start, nk_size_t row_count);
 NK_AMD_DECLARE_BACKEND_(i8, nk_i8_t, nk_i32_t)
 NK_AMD_DECLARE_BACKEND_(u8, nk_u8_t, nk_u32_t)
 NK_AMD_DECLARE_BACKEND_(bf16, nk_bf16_t, nk_f32_t)
@@ -199,6 +238,19 @@ NK_DYNAMIC int nk_amd_dots_packed_async(nk_dtype_t dtype, void const *a, void co
 NK_DYNAMIC int nk_amd_spatials_packed_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void const *a, void const *b_packed,
                                             void *c, nk_size_t height, nk_size_t width, nk_size_t depth,
                                             nk_size_t a_stride, nk_size_t c_stride, void *stream);
+
+/**
+ *  The symmetric kinds on the caller's stream. They pack the window's vectors first, so they need scratch memory:
+ *  `workspace` is device memory, 256-byte aligned, of at least `nk_amd_symmetric_workspace_size` bytes for the same
+ *  arguments, and belongs to the call until the stream has run it. `kind` is nk_kernel_dots_symmetric_k,
+ *  nk_kernel_angulars_symmetric_k or nk_kernel_euclideans_symmetric_k.
+ */
+NK_DYNAMIC nk_size_t nk_amd_symmetric_workspace_size(nk_dtype_t dtype, nk_size_t vectors_count, nk_size_t depth,
+                                                     nk_size_t row_start, nk_size_t row_count);
+NK_DYNAMIC int nk_amd_symmetric_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void const *vectors,
+                                      nk_size_t vectors_count, nk_size_t depth, nk_size_t stride, void *result,
+                                      nk_size_t result_stride, nk_size_t row_start, nk_size_t row_count, void *workspace,
+                                      nk_size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

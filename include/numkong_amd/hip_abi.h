@@ -75,6 +75,21 @@ int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, voi
 int nk_hip_spatials_packed_async(int dtype, int metric, void const *a, void const *b_packed, void *c, size_t m,
                                  size_t n, size_t k, size_t a_stride, size_t c_stride, void *stream);
 
+/**
+ *  All pairs of one set of `n` vectors: result[i][j] for i in [row_start, row_start + row_count) and j >= i only,
+ *  the dot product (metric 0), angular (1) or euclidean (2) distance of vectors i and j; distances on the diagonal
+ *  are exactly 0. The vectors from the 32-row boundary at or below `row_start` to the end are packed into the
+ *  workspace as the B of an ordinary product, the window's rows are its A, and a tile list (built on the device, in
+ *  the workspace too) leaves out the tiles left of the diagonal. `workspace`: device memory, 256-byte aligned, at
+ *  least `nk_hip_symmetric_workspace_size` bytes for the same arguments; in use until the stream has run the call.
+ *  Replaces `nk_dots_symmetric_<T>_<isa>`, `nk_angulars_symmetric_<T>_<isa>`, `nk_euclideans_symmetric_<T>_<isa>`
+ *  (reference: include/numkong/dots/serial.h:2361-2435, 2802-2878).
+ */
+size_t nk_hip_symmetric_workspace_size(int dtype, size_t n, size_t k, size_t row_start, size_t row_count);
+int nk_hip_symmetric_async(int dtype, int metric, void const *vectors, size_t n, size_t k, size_t stride, void *result,
+                           size_t result_stride, size_t row_start, size_t row_count, void *workspace,
+                           size_t workspace_bytes, void *stream);
+
 /** Fill the m x n block of 32-bit outputs with `value` (used for the 0xFF error convention). */
 int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_t value, void *stream);
 

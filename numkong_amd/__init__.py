@@ -11,10 +11,13 @@ from .api import (  # noqa: F401
     NumKongAmdError,
     PackedMatrix,
     angulars_packed,
+    angulars_symmetric,
     dots_pack,
     dots_packed,
     dots_packed_size,
+    dots_symmetric,
     euclideans_packed,
+    euclideans_symmetric,
     library,
     library_path,
 )

@@ -3,6 +3,8 @@
 Reference behaviour mirrored here (python/matrix.c):
   * ``dots_pack(b, dtype)`` -> ``PackedMatrix``                     (:151-227)
   * ``dots_packed(a, packed, out=None)`` -> ``C = A @ B.T``          (:324-490)
+  * ``dots_symmetric(vectors, dtype, out=None, start_row=None, end_row=None)`` and the two distance forms:
+    upper triangle of all pairs of one set of vectors                (:492-622)
   * output dtype per input dtype: i8->i32, u8->u32, floats->f32     (include/numkong/numkong.h:41-45)
   * shape / dtype / stride validation raising ``ValueError``/``TypeError`` (:162-197, :378-421)
 
@@ -71,6 +73,13 @@ def library() -> ctypes.CDLL:
         for stem in ("nk_angulars_packed_", "nk_euclideans_packed_"):
             getattr(lib, stem + name).restype = None
             getattr(lib, stem + name).argtypes = [vp, vp, vp, sz, sz, sz, sz, sz]
+        for stem in ("nk_dots_symmetric_", "nk_angulars_symmetric_", "nk_euclideans_symmetric_"):
+            getattr(lib, stem + name).restype = None
+            getattr(lib, stem + name).argtypes = [vp, sz, sz, sz, vp, sz, sz, sz]
+    lib.nk_amd_symmetric_workspace_size.restype = sz
+    lib.nk_amd_symmetric_workspace_size.argtypes = [i32, sz, sz, sz, sz]
+    lib.nk_amd_symmetric_async.restype = i32
+    lib.nk_amd_symmetric_async.argtypes = [i32, i32, vp, sz, sz, sz, vp, sz, sz, sz, vp, sz, vp]
     lib.nk_amd_last_error.restype = ctypes.c_char_p
     lib.nk_amd_dots_pack_async.restype = i32
     lib.nk_amd_dots_pack_async.argtypes = [i32, vp, sz, sz, sz, vp, vp]
@@ -199,3 +208,50 @@ def angulars_packed(a, packed: PackedMatrix, out=None):
 def euclideans_packed(a, packed: PackedMatrix, out=None):
     """Euclidean distances ``|a_i - b_j|`` as float32 (reference: ``nk_euclideans_packed_<dtype>``)."""
     return _packed_product("nk_euclideans_packed_", "float32", a, packed, out)
+
+
+def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_row, end_row):
+    import torch
+
+    vectors = _as_matrix(vectors, dtype, "vectors")
+    count, depth = int(vectors.shape[0]), int(vectors.shape[1])
+    out_dtype = getattr(torch, out_dtype_name)
+    if out is None:
+        # (the reference leaves what it does not write uninitialised; zeros are easier on the eye)
+        out = torch.zeros((count, count), dtype=out_dtype, device=vectors.device)
+    else:
+        if not isinstance(out, torch.Tensor) or not out.is_cuda or out.dim() != 2:
+            raise ValueError("out must be a 2-dimensional GPU tensor")
+        if tuple(out.shape) != (count, count):
+            raise ValueError(f"out has shape {tuple(out.shape)}, expected {(count, count)}")
+        if out.dtype != out_dtype:
+            raise TypeError(f"out must have dtype {out_dtype}")
+        if count > 1 and out.stride(1) != 1:
+            raise ValueError("out rows must be contiguous")
+    first = 0 if start_row is None else int(start_row)
+    last = count if end_row is None else int(end_row)
+    if first < 0 or last < 0 or first > count or last > count or first > last:
+        raise ValueError(f"Invalid row range [{first}, {last}) for {count} vectors")
+    stride = int(vectors.stride(0)) * vectors.element_size() if count > 1 else depth * vectors.element_size()
+    out_stride = int(out.stride(0)) * 4 if count > 1 else count * 4
+    getattr(library(), stem + dtype)(vectors.data_ptr(), count, depth, stride, out.data_ptr(), out_stride, first, last - first)
+    _check(stem + dtype)
+    return out
+
+
+def dots_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
+    """Upper triangle (diagonal included) of ``vectors @ vectors.T`` for the rows ``[start_row, end_row)``, widened as
+    in ``dots_packed``; the rest of ``out`` is left as it was (zeros when allocated here)."""
+    if dtype not in DTYPES:
+        raise TypeError(f"unsupported dtype {dtype!r}; expected one of {sorted(DTYPES)}")
+    return _symmetric("nk_dots_symmetric_", DTYPES[dtype][2], vectors, dtype, out, start_row, end_row)
+
+
+def angulars_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
+    """Upper triangle of the pairwise angular distances as float32; the diagonal is exactly 0."""
+    return _symmetric("nk_angulars_symmetric_", "float32", vectors, dtype, out, start_row, end_row)
+
+
+def euclideans_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
+    """Upper triangle of the pairwise euclidean distances as float32; the diagonal is exactly 0."""
+    return _symmetric("nk_euclideans_symmetric_", "float32", vectors, dtype, out, start_row, end_row)

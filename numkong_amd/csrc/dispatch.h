@@ -2,8 +2,8 @@
  *  @brief Shared declarations of the dispatch layer: table, error stubs, per-dtype find/init.
  *  @file numkong_amd/csrc/dispatch.h
  *
- *  Mirrors the role of the reference's c/dispatch.h:37-506, reduced to the packed-dots slots
- *  (reference slots: c/dispatch.h:279-319) for i8, u8, bf16, f16, e4m3, e5m2.
+ *  Mirrors the role of the reference's c/dispatch.h:37-506, reduced to the packed-dots, packed-distance and symmetric slots
+ *  (reference slots: c/dispatch.h:279-336, 353-380) for i8, u8, bf16, f16, e4m3, e5m2.
  */
 #ifndef NUMKONG_AMD_DISPATCH_H
 #define NUMKONG_AMD_DISPATCH_H
@@ -24,6 +24,12 @@ typedef struct {
         angulars_packed_e4m3, angulars_packed_e5m2;
     nk_dots_packed_punned_t euclideans_packed_i8, euclideans_packed_u8, euclideans_packed_bf16, euclideans_packed_f16,
         euclideans_packed_e4m3, euclideans_packed_e5m2;
+    nk_dots_symmetric_punned_t dots_symmetric_i8, dots_symmetric_u8, dots_symmetric_bf16, dots_symmetric_f16,
+        dots_symmetric_e4m3, dots_symmetric_e5m2;
+    nk_dots_symmetric_punned_t angulars_symmetric_i8, angulars_symmetric_u8, angulars_symmetric_bf16,
+        angulars_symmetric_f16, angulars_symmetric_e4m3, angulars_symmetric_e5m2;
+    nk_dots_symmetric_punned_t euclideans_symmetric_i8, euclideans_symmetric_u8, euclideans_symmetric_bf16,
+        euclideans_symmetric_f16, euclideans_symmetric_e4m3, euclideans_symmetric_e5m2;
 } nk_implementations_t;
 
 extern nk_implementations_t nk_dispatch_table;
@@ -34,6 +40,8 @@ nk_size_t nk_error_packed_size_(nk_size_t n, nk_size_t k);
 void nk_error_pack_(void const *b, nk_size_t n, nk_size_t k, nk_size_t b_stride, void *b_packed);
 void nk_error_dots_(void const *a, void const *b_packed, void *c, nk_size_t m, nk_size_t n, nk_size_t k,
                     nk_size_t a_stride, nk_size_t c_stride);
+void nk_error_dots_symmetric_(void const *vectors, nk_size_t n_vectors, nk_size_t depth, nk_size_t stride, void *result,
+                              nk_size_t result_stride, nk_size_t row_start, nk_size_t row_count);
 
 /* Per-dtype lookup and table initialisation (reference: c/dispatch.h:483-506). */
 #define NK_AMD_DECLARE_DISPATCH_(T)                                                                              \
@@ -66,6 +74,13 @@ NK_AMD_DECLARE_DISPATCH_(e5m2)
             case nk_kernel_euclideans_packed_k:                                                                       \
                 *m = (m_t)&nk_euclideans_packed_##T##_gfx950, *c = nk_cap_gfx950_k;                                   \
                 return;                                                                                               \
+            case nk_kernel_dots_symmetric_k: *m = (m_t)&nk_dots_symmetric_##T##_gfx950, *c = nk_cap_gfx950_k; return; \
+            case nk_kernel_angulars_symmetric_k:                                                                      \
+                *m = (m_t)&nk_angulars_symmetric_##T##_gfx950, *c = nk_cap_gfx950_k;                                  \
+                return;                                                                                               \
+            case nk_kernel_euclideans_symmetric_k:                                                                    \
+                *m = (m_t)&nk_euclideans_symmetric_##T##_gfx950, *c = nk_cap_gfx950_k;                                \
+                return;                                                                                               \
             default: break;                                                                                           \
             }                                                                                                         \
         switch (k) {                                                                                                  \
@@ -74,6 +89,9 @@ NK_AMD_DECLARE_DISPATCH_(e5m2)
         case nk_kernel_dots_packed_k:                                                                                 \
         case nk_kernel_angulars_packed_k:                                                                             \
         case nk_kernel_euclideans_packed_k: *m = (m_t)nk_error_dots_, *c = 0; return;                                \
+        case nk_kernel_dots_symmetric_k:                                                                              \
+        case nk_kernel_angulars_symmetric_k:                                                                          \
+        case nk_kernel_euclideans_symmetric_k: *m = (m_t)nk_error_dots_symmetric_, *c = 0; return;                   \
         default: *m = (m_t)nk_error_dense_, *c = 0; return;                                                          \
         }                                                                                                             \
     }                                                                                                                 \
@@ -88,6 +106,12 @@ NK_AMD_DECLARE_DISPATCH_(e5m2)
                                 &used);                                                                               \
         nk_dispatch_##T##_find_(caps, nk_kernel_euclideans_packed_k,                                                  \
                                 (nk_kernel_punned_t *)&t->euclideans_packed_##T, &used);                              \
+        nk_dispatch_##T##_find_(caps, nk_kernel_dots_symmetric_k, (nk_kernel_punned_t *)&t->dots_symmetric_##T,      \
+                                &used);                                                                               \
+        nk_dispatch_##T##_find_(caps, nk_kernel_angulars_symmetric_k,                                                 \
+                                (nk_kernel_punned_t *)&t->angulars_symmetric_##T, &used);                             \
+        nk_dispatch_##T##_find_(caps, nk_kernel_euclideans_symmetric_k,                                               \
+                                (nk_kernel_punned_t *)&t->euclideans_symmetric_##T, &used);                           \
     }
 
 #ifdef __cplusplus

@@ -253,19 +253,22 @@ __device__ __forceinline__ double chunk_sumsq_f64(v4i v) {
  *  the row, mod 2^32; zero for the other types) and the column's sum of squares, which the angular and
  *  euclidean products need (reference: the norms behind the packed rows, dots/serial.h:326-332): exact mod
  *  2^32 for the integer types, accumulated in f64 and rounded once to f32 for the float types.
- *  One wavefront per tile: lane l owns row l % 32 and every second chunk starting at l / 32.
+ *  Four wavefronts per tile: lane l of wavefront w owns row l % 32 and every eighth chunk starting at 2 w + l / 32.
  *  KIND: 0 i8, 1 u8, 2 bf16, 3 f16 (and fp8, stored widened to f16).
  */
 template <int KIND>
-__global__ __launch_bounds__(64) void column_terms_kernel(uint8_t const *__restrict__ data, uint32_t k_chunks, uint32_t k,
-                                                          uint32_t *__restrict__ sums, uint32_t *__restrict__ norms) {
+__global__ __launch_bounds__(256) void column_terms_kernel(uint8_t const *__restrict__ data, uint32_t k_chunks, uint32_t k,
+                                                           uint32_t *__restrict__ sums, uint32_t *__restrict__ norms) {
+    __shared__ int part_sum[8][32];
+    __shared__ uint32_t part_squares[8][32];
+    __shared__ double part_f64[8][32];
     uint32_t const tile = blockIdx.x;
-    uint32_t const lane = threadIdx.x;
-    uint8_t const *base = data + (uint64_t)tile * k_chunks * kTileChunkBytes + lane * kChunkBytes;
+    uint32_t const first = threadIdx.x >> 5, row = threadIdx.x & 31; // chunk residue mod 8, row of the tile
+    uint8_t const *base = data + (uint64_t)tile * k_chunks * kTileChunkBytes + row * kChunkBytes;
     int sum = 0;
     uint32_t squares = 0;
     double squares_f64 = 0;
-    for (uint32_t c = 0; c < k_chunks; c += 2) {
+    for (uint32_t c = first; c < k_chunks; c += 8) {
         v4i const v = *(v4i const *)(base + (uint64_t)c * kTileChunkBytes);
         if (KIND == 0) {
 #pragma unroll
@@ -280,14 +283,16 @@ __global__ __launch_bounds__(64) void column_terms_kernel(uint8_t const *__restr
         }
         else { squares_f64 += chunk_sumsq_f64<KIND == 2>(v); }
     }
-    sum += __shfl_xor(sum, 32, 64);
-    squares += __shfl_xor(squares, 32, 64);
-    squares_f64 += __shfl_xor(squares_f64, 32, 64);
-    // u8 is stored as b - 128 (and its padding as 0): sum(b^2) = sum((b - 128)^2) + 256 * sum(b - 128) + 128^2 * k
-    if (KIND == 1) squares += 256u * (uint32_t)sum + 16384u * k;
-    if (lane < 32) {
-        sums[(uint64_t)tile * kTileRows + lane] = (uint32_t)sum * 128u;
-        norms[(uint64_t)tile * kTileRows + lane] = KIND < 2 ? squares : __builtin_bit_cast(uint32_t, (float)squares_f64);
+    part_sum[first][row] = sum, part_squares[first][row] = squares, part_f64[first][row] = squares_f64;
+    __syncthreads();
+    if (threadIdx.x < 32) {
+        sum = 0, squares = 0, squares_f64 = 0;
+#pragma unroll
+        for (int part = 0; part < 8; ++part) sum += part_sum[part][row], squares += part_squares[part][row], squares_f64 += part_f64[part][row];
+        // u8 is stored as b - 128 (and its padding as 0): sum(b^2) = sum((b - 128)^2) + 256 * sum(b - 128) + 128^2 * k
+        if (KIND == 1) squares += 256u * (uint32_t)sum + 16384u * k;
+        sums[(uint64_t)tile * kTileRows + row] = (uint32_t)sum * 128u;
+        norms[(uint64_t)tile * kTileRows + row] = KIND < 2 ? squares : __builtin_bit_cast(uint32_t, (float)squares_f64);
     }
 }
 
@@ -300,11 +305,12 @@ __global__ __launch_bounds__(64) void write_header_kernel(PackedHeader *dst, Pac
     if (threadIdx.x == 0) *dst = h;
 }
 
+/** `tri_mask` all ones: only the elements with col >= row + tri_shift (on or right of a diagonal); 0: all of them. */
 __global__ __launch_bounds__(256) void fill_rows_kernel(uint8_t *c, uint32_t m, uint32_t n, uint64_t c_stride,
-                                                        uint32_t value) {
+                                                        uint32_t value, uint32_t tri_shift, uint32_t tri_mask) {
     uint64_t const i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     uint64_t const row = i / n, col = i % n;
-    if (row < m) *(uint32_t *)(c + row * c_stride + col * 4) = value;
+    if (row < m && (((uint32_t)row + tri_shift) & tri_mask) <= (uint32_t)col) *(uint32_t *)(c + row * c_stride + col * 4) = value;
 }
 
 #pragma endregion Packing
@@ -451,8 +457,14 @@ __device__ __forceinline__ uint32_t distance_from_dot(uint32_t dot_bits, float q
         result = product > 0 ? unclipped : (dot == 0 ? 0.0f : 1.0f);
     }
     else {
+        // The hardware's reciprocal square root is good to about one unit in the last place; one Newton step on
+        // the root itself (residual by a fused multiply-add) leaves it correctly rounded but for rare ties, as
+        // the square roots of the reference's vector kernels are.
         float const squared = __builtin_fmaf(-2.0f, dot, query + target);
-        result = squared > 0 ? __builtin_amdgcn_sqrtf(squared) : 0.0f;
+        float const inverse = __builtin_amdgcn_rsqf(squared);
+        float root = squared * inverse;
+        root = __builtin_fmaf(__builtin_fmaf(-root, root, squared), 0.5f * inverse, root);
+        result = squared > 0 ? root : 0.0f;
     }
     return __builtin_bit_cast(uint32_t, result);
 }
@@ -503,6 +515,8 @@ struct Totals<acc_t, TM, TN, false> {
     __device__ __forceinline__ auto finish(acc_t const (&acc)[TM][TN], int i, int j, int v) const { return acc[i][j][v]; }
 };
 
+constexpr uint32_t kTileBand = 8; // tile rows per band of the walk over the tile grid
+
 struct GemmArgs {
     uint8_t const *a;
     uint8_t const *bp; // packed image (header first)
@@ -514,6 +528,11 @@ struct GemmArgs {
     int avec; // widest load the A pointer and stride allow (1, 2, 4, 8 or 16 bytes)
     int metric; // 0: dot products, 1: angular distances, 2: euclidean distances (kernels built with NORMS)
     uint32_t chunk_stages; // chunked types: stages between folds of the accumulator (even, 2..16)
+    // Symmetric products (C = A x A^T, upper triangle): only elements with col >= row + tri_shift are stored
+    // (`tri_mask` all ones; 0 switches the test off), and the tiles to compute come as a list.
+    uint32_t tri_shift, tri_mask;
+    uint32_t tile_count;       // tiles_m * tiles_n, or the length of the list
+    uint32_t const *tile_list; // (tile row, tile column) pairs in walking order, or NULL for the full grid
 };
 
 /**
@@ -522,13 +541,19 @@ struct GemmArgs {
  *  walks the tile grid in column-major bands of 8 tile rows: tiles resident on one XCD at the same time
  *  share A row blocks and B column tiles in that XCD's L2.
  */
-__device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm,
-                                              uint32_t &tn) {
-    uint32_t const total = tiles_m * tiles_n;
+__device__ __forceinline__ void tile_of_block(uint32_t pid, GemmArgs const &g, uint32_t &tm, uint32_t &tn) {
+    uint32_t const tiles_m = g.tiles_m, tiles_n = g.tiles_n;
+    uint32_t const total = g.tile_count;
     uint32_t const per_xcd = total / 8;
     uint32_t lid = pid;
     if (pid < per_xcd * 8) lid = (pid % 8) * per_xcd + pid / 8;
-    constexpr uint32_t kBand = 8;
+    if (g.tile_list) { // a triangular grid: the same walk with the tiles left of the diagonal left out, listed
+        typedef __attribute__((address_space(4))) uint32_t const constant_u32_t;
+        constant_u32_t *entry = (constant_u32_t *)g.tile_list + 2 * (uint64_t)lid;
+        tm = entry[0], tn = entry[1];
+        return;
+    }
+    constexpr uint32_t kBand = kTileBand;
     uint32_t const width = kBand * tiles_n;
     uint32_t const band = lid / width;
     uint32_t const first = band * kBand;
@@ -536,6 +561,68 @@ __device__ __forceinline__ void tile_of_block(uint32_t pid, uint32_t tiles_m, ui
     uint32_t const in_band = lid % width;
     tm = first + in_band % rows;
     tn = in_band / rows;
+}
+
+/** First tile column of tile row `t` that holds an element on or right of the diagonal col = row + shift; tiles
+ *  are 2^bm_log2 rows by 2^bn_log2 columns. */
+__host__ __device__ inline uint32_t first_live_tile(uint32_t t, uint32_t bm_log2, uint32_t bn_log2, uint32_t shift) {
+    return ((t << bm_log2) + shift) >> bn_log2;
+}
+
+/**
+ *  The tile list of a triangular grid, in the order of `tile_of_block`: bands of kTileBand tile rows, column
+ *  by column within a band, top to bottom within a column, and only tiles with something on or right of the
+ *  diagonal. One workgroup: the bands' sizes are scanned 256 at a time, then every band is filled by all threads,
+ *  a column each. A band's first columns form a staircase (row t joins at column first_live_tile(t)); the cells
+ *  left of column c number the sum over its rows of max(0, c - first_live_tile(t)).
+ */
+__global__ __launch_bounds__(256) void triangle_tiles_kernel(uint32_t tiles_m, uint32_t tiles_n, uint32_t bm_log2,
+                                                             uint32_t bn_log2, uint32_t shift, uint32_t *band_start,
+                                                             uint32_t *list) {
+    __shared__ uint32_t scan[256];
+    __shared__ uint32_t base;
+    uint32_t const tid = threadIdx.x;
+    uint32_t const bands = (tiles_m + kTileBand - 1) / kTileBand;
+    if (tid == 0) base = 0, band_start[0] = 0;
+    __syncthreads();
+    for (uint32_t chunk = 0; chunk < bands; chunk += 256) {
+        uint32_t const band = chunk + tid;
+        uint32_t count = 0;
+        if (band < bands) {
+            uint32_t const first = band * kTileBand, last = first + kTileBand < tiles_m ? first + kTileBand : tiles_m;
+            for (uint32_t t = first; t < last; ++t) {
+                uint32_t const from = first_live_tile(t, bm_log2, bn_log2, shift);
+                count += from < tiles_n ? tiles_n - from : 0;
+            }
+        }
+        scan[tid] = count;
+        __syncthreads();
+        for (uint32_t step = 1; step < 256; step *= 2) {
+            uint32_t const below = tid >= step ? scan[tid - step] : 0;
+            __syncthreads();
+            scan[tid] += below;
+            __syncthreads();
+        }
+        if (band < bands) band_start[band + 1] = base + scan[tid];
+        __syncthreads();
+        if (tid == 255) base += scan[255];
+        __syncthreads();
+    }
+    for (uint32_t band = 0; band < bands; ++band) {
+        uint32_t const first = band * kTileBand, last = first + kTileBand < tiles_m ? first + kTileBand : tiles_m;
+        uint32_t joins[kTileBand]; // where each row of the band joins (past the grid for rows that do not exist)
+#pragma unroll
+        for (uint32_t i = 0; i < kTileBand; ++i) joins[i] = first + i < last ? first_live_tile(first + i, bm_log2, bn_log2, shift) : 0xFFFFFFFFu;
+        uint32_t const start = band_start[band];
+        for (uint32_t column = joins[0] + tid; column < tiles_n; column += 256) {
+            uint32_t at = start;
+#pragma unroll
+            for (uint32_t i = 0; i < kTileBand; ++i) at += column > joins[i] ? column - joins[i] : 0;
+#pragma unroll
+            for (uint32_t i = 0; i < kTileBand; ++i)
+                if (joins[i] <= column) list[2 * (uint64_t)at] = first + i, list[2 * (uint64_t)at + 1] = column, ++at;
+        }
+    }
 }
 
 /**
@@ -639,7 +726,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     auto view_of = [&](uint32_t tile) {
         TileView view;
         uint32_t tile_m, tile_n;
-        tile_of_block(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+        tile_of_block(tile, g, tile_m, tile_n);
         view.row0 = tile_m * BM;
         view.col0 = tile_n * (128 * TN) + wave * (32 * TN);
         uint32_t const rows_here = g.m - view.row0 < (uint32_t)BM ? g.m - view.row0 : (uint32_t)BM;
@@ -666,7 +753,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // fetch the first stages of the workgroup's next tile instead of running dry: the pipeline is primed once
     // and then runs across tile boundaries, and the stores of one tile drain under the next tile's MFMAs.
     constexpr bool across = ACROSS; // the host checks that it holds: fast == stages and stages >= 4
-    uint32_t const tile_count = g.tiles_m * g.tiles_n;
+    uint32_t const tile_count = g.tile_count;
     // u8 only: every thread sums the unsigned bytes it stages, per staged row, in LDS slots of its own (slot
     // i * 256 + tid: fire-and-forget LDS adds instead of 2 x kLoads registers held through the loop). Two sets:
     // what is staged ahead for the next tile goes to the other one, and the sets swap roles with every tile.
@@ -693,12 +780,12 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     typedef __attribute__((address_space(1))) uint8_t global_u8_t;
     typedef __attribute__((address_space(1))) uint32_t global_u32_t;
     if (!image_ok) { // the image was not packed for this call: the reference's error convention, all bits set
-        for (uint32_t tile = blockIdx.x; tile < g.tiles_m * g.tiles_n; tile += gridDim.x) {
+        for (uint32_t tile = blockIdx.x; tile < g.tile_count; tile += gridDim.x) {
             uint32_t tile_m, tile_n;
-            tile_of_block(tile, g.tiles_m, g.tiles_n, tile_m, tile_n);
+            tile_of_block(tile, g, tile_m, tile_n);
             for (uint32_t at = tid; at < (uint32_t)BM * 128 * TN; at += NT) {
                 uint32_t const row = tile_m * BM + at / (128 * TN), col = tile_n * (128 * TN) + at % (128 * TN);
-                if (row < g.m && col < g.n) *(global_u32_t *)((global_u8_t *)g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 4) = 0xFFFFFFFFu;
+                if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col) *(global_u32_t *)((global_u8_t *)g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 4) = 0xFFFFFFFFu;
             }
         }
         return;
@@ -947,6 +1034,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                     uint32_t const row = row0 + r < g.m ? r : g.m - 1 - row0;
                     a_slow[i] = row * (uint32_t)g.a_stride + a_pos * T::kSrcChunk;
                 }
+                uint32_t until_fold = g.chunk_stages;
                 for (uint32_t s = fast; s < stages; ++s) {
                     __syncthreads();
                     int64_t const left = (int64_t)g.k_src_bytes - (int64_t)s * kSrcStage - (int64_t)a_pos * T::kSrcChunk;
@@ -979,6 +1067,12 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                     read_frags(slot_c<0>(), slot_c<3>(), slot_c<1>());
                     multiply(slot_c<0>(), slot_c<2>());
                     multiply(slot_c<0>(), slot_c<3>());
+                    if constexpr (kChunked) { // the same two-level accumulation as the pipelined loop
+                        if (--until_fold == 0) {
+                            total.fold(acc);
+                            until_fold = g.chunk_stages;
+                        }
+                    }
                 }
             }
         }
@@ -1019,17 +1113,31 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         // through a generic pointer counts as an LDS operation as well, and with such stores in flight the
         // loads prefetched for the next tile could only be waited for all at once.) Tiles that touch the
         // matrix edge take the masked copy of the loop.
-        bool const interior = row0 + BM <= g.m && col0 + 32 * TN <= g.n;
-        global_u8_t *c_tile = (global_u8_t *)g.c + (uint64_t)row0 * g.c_stride + (uint64_t)col0 * 4;
+        // Of a triangular grid, a wavefront's part of a tile is stored whole (all of it right of the diagonal), not
+        // at all (all of it left), or through the masked copy.
+        // What only the stores need is read from the kernel's arguments again, here, rather than held in a dozen
+        // scalar registers through the loop (the empty asm hides from the compiler that it is the same memory).
+        typedef __attribute__((address_space(4))) GemmArgs const late_args_t;
+        late_args_t *late = (late_args_t *)__builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("" : "+s"(late));
+        bool const interior = row0 + BM <= late->m && col0 + 32 * TN <= late->n &&
+                              (((row0 + (BM - 1) + late->tri_shift) & late->tri_mask) <= col0);
+        bool const nothing = ((row0 + late->tri_shift) & late->tri_mask) > col0 + (32 * TN - 1);
+        global_u8_t *c_tile = (global_u8_t *)late->c + (uint64_t)row0 * late->c_stride + (uint64_t)col0 * 4;
         auto store_all = [&](auto masked_tag, auto metric_tag) {
             constexpr bool masked = decltype(masked_tag)::value != 0;
             constexpr int metric = decltype(metric_tag)::value;
-            uint64_t const row_step = g.c_stride;
+            uint64_t const row_step = late->c_stride;
             // Lane l holds column l % 32; register v holds row 8 * (v / 4) + 4 * (l / 32) + v % 4.
-            uint32_t const lane_offset = 4 * half * (uint32_t)g.c_stride + col_in_tile * 4;
+            uint32_t const lane_offset = 4 * half * (uint32_t)late->c_stride + col_in_tile * 4;
+            // Masked tiles: rows of the matrix from this lane's first one on, and how far right of the diagonal
+            // col = row + tri_shift its first element lies (element (r, 32 j) from there is stored when
+            // r - 32 j <= that distance; without a triangle everything is).
+            int const rows_left = (int)(late->m - row0 - 4 * half);
+            int const diagonal = late->tri_mask ? (int)(col0 + col_in_tile) - (int)(row0 + 4 * half + late->tri_shift) : 0x7FFFFFFF;
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                bool const col_ok = col0 + j * 32 + col_in_tile < g.n;
+                bool const col_ok = col0 + j * 32 + col_in_tile < late->n;
                 // Rows come in runs of 4 that start 8 apart: the base advances by one row or by five. The
                 // empty asm keeps it a running scalar (otherwise every row's base is precomputed and the
                 // scalar registers overflow).
@@ -1054,8 +1162,13 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                             int const row_bits = row_norm4[v % 4];
                             bits = distance_from_dot<T, metric == 2 ? 2 : 1>(bits, __builtin_bit_cast(float, row_bits), col_value);
                         }
-                        if ((!(DBG & 16) || bits == 0x12345678u) && // (timing experiment: almost no stores)
-                            (!masked || (col_ok && row0 + r_fixed + 4 * half < g.m)))
+                        bool keep = true;
+                        if (masked) {
+                            keep = col_ok && r_fixed < rows_left && r_fixed - j * 32 <= diagonal;
+                            // a vector's distance from itself is exactly 0 (dots/serial.h:2871-2876)
+                            if (metric != 0 && r_fixed - j * 32 == diagonal) bits = 0;
+                        }
+                        if ((!(DBG & 16) || bits == 0x12345678u) && keep) // (timing experiment: almost no stores)
                             *(global_u32_t *)(row_base + lane_offset) = bits;
                         row_base += (v % 4 == 3 ? 5 : 1) * row_step;
                         asm volatile("" : "+s"(row_base));
@@ -1066,8 +1179,9 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 }
             }
         };
-        if constexpr (NORMS) { // which distance is a run-time choice: one kernel serves both
-            if (g.metric == 2) {
+        if (nothing) {}
+        else if constexpr (NORMS) { // which distance is a run-time choice: one kernel serves both
+            if (late->metric == 2) {
                 if (interior) store_all(slot_c<0>(), slot_c<2>());
                 else store_all(slot_c<1>(), slot_c<2>());
             }
@@ -1081,7 +1195,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             else store_all(slot_c<1>(), slot_c<0>());
         }
 #ifdef NK_TUNE
-        if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + (g.tiles_m * g.tiles_n > 45 * gridDim.x ? 40 : 1) * gridDim.x) {
+        if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + (g.tile_count > 45 * gridDim.x ? 40 : 1) * gridDim.x) {
             g_debug_clocks[5] = clock64() - debug_t2, g_debug_clocks[6] = clock64() - debug_t0;
             g_debug_clocks[7] = wall_clock64() - debug_tw0;
         }
@@ -1100,13 +1214,49 @@ int g_variant = 0; // timing experiments of tuning builds
 
 int g_cu_count = 0;
 
+/** Scratch memory of a triangular grid: the first tile of every band, then the list itself. */
+struct TriangleScratch {
+    uint32_t *words;
+    size_t bytes;
+};
+
+/** Tiles of a bm x bn grid over m x n outputs with something on or right of the diagonal col = row + shift. */
+inline uint32_t log2_of(uint32_t power_of_two) { return (uint32_t)__builtin_ctz(power_of_two); }
+inline uint64_t live_tiles(uint64_t m, uint64_t n, uint32_t bm, uint32_t bn, uint32_t shift) {
+    uint32_t const tiles_m = (uint32_t)((m + bm - 1) / bm), tiles_n = (uint32_t)((n + bn - 1) / bn);
+    uint64_t count = 0;
+    for (uint32_t t = 0; t < tiles_m; ++t) {
+        uint32_t const from = first_live_tile(t, log2_of(bm), log2_of(bn), shift);
+        count += from < tiles_n ? tiles_n - from : 0;
+    }
+    return count;
+}
+inline size_t triangle_scratch_bytes(uint64_t m, uint64_t n, uint32_t bm, uint32_t bn, uint32_t shift) {
+    uint64_t const bands = ((m + bm - 1) / bm + kTileBand - 1) / kTileBand;
+    return (size_t)(((bands + 1 + 1) & ~1ull) * 4 + live_tiles(m, n, bm, bn, shift) * 8);
+}
+
 template <class T, int TM, int TN>
-hipError_t launch_one(GemmArgs &g, hipStream_t stream) {
+hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle) {
     constexpr int BM = TM * 32, BN = TN * 128;
     g.tiles_m = (g.m + BM - 1) / BM;
     g.tiles_n = (g.n + BN - 1) / BN;
-    uint64_t const tiles = (uint64_t)g.tiles_m * g.tiles_n;
+    uint64_t tiles = (uint64_t)g.tiles_m * g.tiles_n;
     if (tiles > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    g.tile_list = nullptr;
+    if (triangle) {
+        tiles = live_tiles(g.m, g.n, BM, BN, g.tri_shift);
+        if (!tiles) return hipSuccess;
+        if (triangle_scratch_bytes(g.m, g.n, BM, BN, g.tri_shift) > triangle->bytes) return hipErrorInvalidValue;
+        uint32_t const bands = (g.tiles_m + kTileBand - 1) / kTileBand;
+        uint32_t *list = triangle->words + ((bands + 1 + 1) & ~1u);
+        hipLaunchKernelGGL(triangle_tiles_kernel, dim3(1), dim3(256), 0, stream, g.tiles_m, g.tiles_n,
+                           log2_of(BM), log2_of(BN), g.tri_shift, triangle->words, list);
+        hipError_t const e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        g.tile_list = list;
+    }
+    g.tile_count = (uint32_t)tiles;
     // The tile's A offsets are 32-bit: (rows of a tile) * stride must stay below 4 GiB.
     if ((uint64_t)BM * g.a_stride > 0xFFFFFFFFull) return hipErrorInvalidValue;
     // So are the per-lane C offsets: 4 rows plus the tile's width.
@@ -1153,12 +1303,13 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream) {
 }
 
 template <class T>
-hipError_t launch_typed(GemmArgs &g, hipStream_t stream) {
+hipError_t launch_typed(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle) {
     int config = g_forced_config;
     if (config <= 0 || config >= kConfigCount) {
         // Largest tile that still gives every one of the 256 CUs at least one workgroup.
         auto tiles = [&](int c) {
             uint64_t const bm = kConfigs[c].tm * 32, bn = (uint64_t)kConfigs[c].tn * 128;
+            if (triangle) return live_tiles(g.m, g.n, (uint32_t)bm, (uint32_t)bn, g.tri_shift);
             return ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
         };
         config = 4;
@@ -1176,10 +1327,10 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream) {
     switch (config) {
     case 1:
         if constexpr (T::kChunked) return hipErrorInvalidValue;
-        else return launch_one<T, 8, 2>(g, stream);
-    case 2: return launch_one<T, 4, 2>(g, stream);
-    case 3: return launch_one<T, 4, 1>(g, stream);
-    default: return launch_one<T, 2, 1>(g, stream);
+        else return launch_one<T, 8, 2>(g, stream, triangle);
+    case 2: return launch_one<T, 4, 2>(g, stream, triangle);
+    case 3: return launch_one<T, 4, 1>(g, stream, triangle);
+    default: return launch_one<T, 2, 1>(g, stream, triangle);
     }
 }
 
@@ -1266,8 +1417,9 @@ size_t nk_hip_dots_packed_size(int dtype, size_t n, size_t k) {
     return (size_t)g.total_bytes;
 }
 
-int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_stride, void *b_packed,
-                           void *stream_) {
+/** `terms`: also the per-column terms after the tiles (only the u8 product and the distances read them). */
+static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_stride, void *b_packed, void *stream_,
+                      bool terms) {
     hipStream_t stream = (hipStream_t)stream_;
     Geometry g;
     if (!make_geometry(dtype, n, k, g)) return fail_msg("nk_hip_dots_pack: unsupported dtype or dimensions");
@@ -1301,11 +1453,11 @@ int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t 
         e = hipGetLastError();
         if (e != hipSuccess) return fail(e, "pack_kernel");
     }
-    if (g.n_tiles) {
+    if (g.n_tiles && terms) {
         if (g.k_chunks) {
-            auto terms = dtype == kI8 ? column_terms_kernel<0>
-                         : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
-            hipLaunchKernelGGL(terms, dim3(g.n_tiles), dim3(64), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);
+            auto kernel = dtype == kI8 ? column_terms_kernel<0>
+                          : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
+            hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(256), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);
         }
         else {
             uint64_t const count = 2 * (uint64_t)g.n_tiles * kTileRows; // both arrays, back to back
@@ -1318,6 +1470,11 @@ int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t 
     return 0;
 }
 
+int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_stride, void *b_packed,
+                           void *stream) {
+    return pack_async(dtype, b, n, k, b_stride, b_packed, stream, true);
+}
+
 int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_t value, void *stream) {
     if (!m || !n) return 0;
     if (m > 0x7FFFFFFFull || n > 0x7FFFFFFFull) return fail_msg("nk_hip_fill_rows: dimensions too large");
@@ -1325,13 +1482,16 @@ int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_
     uint64_t const blocks = (count + 255) / 256;
     if (blocks > 0x7FFFFFFFull) return fail_msg("nk_hip_fill_rows: matrix too large");
     hipLaunchKernelGGL(fill_rows_kernel, dim3((uint32_t)blocks), dim3(256), 0, (hipStream_t)stream, (uint8_t *)c,
-                       (uint32_t)m, (uint32_t)n, (uint64_t)c_stride, value);
+                       (uint32_t)m, (uint32_t)n, (uint64_t)c_stride, value, 0u, 0u);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : fail(e, "fill_rows_kernel");
 }
 
+/** `triangle`: NULL for the full m x n product; otherwise only the outputs with col >= row + shift are computed
+ *  and stored, over a tile list built in that scratch memory. */
 static int product_async(int dtype, int metric, void const *a, void const *b_packed, void *c, size_t m, size_t n,
-                         size_t k, size_t a_stride, size_t c_stride, void *stream_) {
+                         size_t k, size_t a_stride, size_t c_stride, void *stream_,
+                         TriangleScratch const *triangle = nullptr, uint32_t shift = 0) {
     hipStream_t stream = (hipStream_t)stream_;
     if (!m || !n) return 0;
     Geometry geo;
@@ -1339,7 +1499,15 @@ static int product_async(int dtype, int metric, void const *a, void const *b_pac
     if (m > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_packed: too many rows");
     if (!c || ((uintptr_t)c & 3) || (c_stride & 3)) return fail_msg("nk_hip_dots_packed: c must be 4-byte aligned");
     if (!b_packed || ((uintptr_t)b_packed & 15)) return fail_msg("nk_hip_dots_packed: b_packed must be 16-byte aligned");
-    if (k == 0) return nk_hip_fill_rows_async(c, m, n, c_stride, 0u, stream_);
+    if (k == 0 && !triangle) return nk_hip_fill_rows_async(c, m, n, c_stride, 0u, stream_);
+    if (k == 0) {
+        uint64_t const blocks = ((uint64_t)m * n + 255) / 256;
+        if (blocks > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_symmetric: matrix too large");
+        hipLaunchKernelGGL(fill_rows_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t *)c, (uint32_t)m,
+                           (uint32_t)n, (uint64_t)c_stride, 0u, shift, 0xFFFFFFFFu);
+        hipError_t const e = hipGetLastError();
+        return e == hipSuccess ? 0 : fail(e, "fill_rows_kernel");
+    }
     if (!a) return fail_msg("nk_hip_dots_packed: a is NULL");
     if (geo.elem_bytes == 2 && (((uintptr_t)a | a_stride) & 1)) return fail_msg("nk_hip_dots_packed: 16-bit A is misaligned");
 
@@ -1350,6 +1518,7 @@ static int product_async(int dtype, int metric, void const *a, void const *b_pac
     g.m = (uint32_t)m, g.n = geo.n, g.k = geo.k, g.n_tiles = geo.n_tiles, g.k_chunks = geo.k_chunks;
     g.avec = widest_load(a, a_stride);
     g.metric = metric;
+    if (triangle) g.tri_shift = shift, g.tri_mask = 0xFFFFFFFFu;
     {
         // Stages between accumulator folds: about an eighth of the depth, even, between 2 and 16.
         uint32_t const eighth = (g.k_chunks / kStageChunks / 8) & ~1u;
@@ -1358,12 +1527,12 @@ static int product_async(int dtype, int metric, void const *a, void const *b_pac
 
     hipError_t e;
     switch (dtype) {
-    case kI8: e = launch_typed<I8>(g, stream); break;
-    case kU8: e = launch_typed<U8>(g, stream); break;
-    case kBF16: e = launch_typed<BF16>(g, stream); break;
-    case kF16: e = launch_typed<F16>(g, stream); break;
-    case kE4M3: e = launch_typed<E4M3>(g, stream); break;
-    case kE5M2: e = launch_typed<E5M2>(g, stream); break;
+    case kI8: e = launch_typed<I8>(g, stream, triangle); break;
+    case kU8: e = launch_typed<U8>(g, stream, triangle); break;
+    case kBF16: e = launch_typed<BF16>(g, stream, triangle); break;
+    case kF16: e = launch_typed<F16>(g, stream, triangle); break;
+    case kE4M3: e = launch_typed<E4M3>(g, stream, triangle); break;
+    case kE5M2: e = launch_typed<E5M2>(g, stream, triangle); break;
     default: return fail_msg("nk_hip_dots_packed: unsupported dtype");
     }
     return e == hipSuccess ? 0 : fail(e, "dots_packed_kernel");
@@ -1378,6 +1547,57 @@ int nk_hip_spatials_packed_async(int dtype, int metric, void const *a, void cons
                                  size_t k, size_t a_stride, size_t c_stride, void *stream) {
     if (metric != 1 && metric != 2) return fail_msg("nk_hip_spatials_packed: metric must be 1 (angular) or 2 (euclidean)");
     return product_async(dtype, metric, a, b_packed, c, m, n, k, a_stride, c_stride, stream);
+}
+
+/** What one symmetric call covers: rows [row_start, row_end) of the result, and of those the columns from
+ *  `col_begin` (the start of the 32-row tile of the packed image that holds row_start) to the end. */
+struct SymmetricWindow {
+    size_t row_end, col_begin, columns, image_bytes, scratch_bytes;
+};
+static bool symmetric_window(int dtype, size_t n, size_t k, size_t row_start, size_t row_count, SymmetricWindow &w) {
+    w.row_end = row_count < n - row_start ? row_start + row_count : n;
+    w.col_begin = row_start / kTileRows * kTileRows;
+    w.columns = n - w.col_begin;
+    Geometry geo;
+    if (!make_geometry(dtype, w.columns, k, geo)) return false;
+    w.image_bytes = (size_t)((geo.total_bytes + 255) & ~255ull);
+    w.scratch_bytes = 0;
+    uint32_t const shift = (uint32_t)(row_start - w.col_begin);
+    for (int c = 1; c < kConfigCount; ++c) {
+        size_t const bytes = triangle_scratch_bytes(w.row_end - row_start, w.columns, kConfigs[c].tm * 32,
+                                                    kConfigs[c].tn * 128, shift);
+        if (bytes > w.scratch_bytes) w.scratch_bytes = bytes;
+    }
+    return true;
+}
+
+size_t nk_hip_symmetric_workspace_size(int dtype, size_t n, size_t k, size_t row_start, size_t row_count) {
+    if (row_start >= n || !row_count) return 0;
+    SymmetricWindow w;
+    if (!symmetric_window(dtype, n, k, row_start, row_count, w)) return 0;
+    return w.image_bytes + w.scratch_bytes;
+}
+
+int nk_hip_symmetric_async(int dtype, int metric, void const *vectors, size_t n, size_t k, size_t stride, void *result,
+                           size_t result_stride, size_t row_start, size_t row_count, void *workspace,
+                           size_t workspace_bytes, void *stream) {
+    if (metric < 0 || metric > 2) return fail_msg("nk_hip_symmetric: metric must be 0 (dots), 1 (angular) or 2 (euclidean)");
+    if (row_start >= n || !row_count) return 0;
+    SymmetricWindow w;
+    if (!symmetric_window(dtype, n, k, row_start, row_count, w)) return fail_msg("nk_hip_symmetric: unsupported dtype or dimensions");
+    if (!workspace || ((uintptr_t)workspace & 255)) return fail_msg("nk_hip_symmetric: workspace must be 256-byte aligned");
+    if (workspace_bytes < w.image_bytes + w.scratch_bytes) return fail_msg("nk_hip_symmetric: workspace too small");
+    if (!result || ((uintptr_t)result & 3) || (result_stride & 3)) return fail_msg("nk_hip_symmetric: result must be 4-byte aligned");
+    if (k && !vectors) return fail_msg("nk_hip_symmetric: vectors is NULL");
+    // The columns of the window, packed as the B of an ordinary product; the rows of the window are its A.
+    uint8_t const *rows = (uint8_t const *)vectors;
+    int status = pack_async(dtype, rows + w.col_begin * stride, w.columns, k, stride, workspace, stream,
+                            metric != 0 || dtype == kU8);
+    if (status) return status;
+    TriangleScratch const scratch = {(uint32_t *)((uint8_t *)workspace + w.image_bytes), w.scratch_bytes};
+    uint8_t *c = (uint8_t *)result + row_start * result_stride + w.col_begin * 4;
+    return product_async(dtype, metric, rows + row_start * stride, workspace, c, w.row_end - row_start, w.columns, k, stride,
+                         result_stride, stream, &scratch, (uint32_t)(row_start - w.col_begin));
 }
 
 #ifdef NK_TUNE

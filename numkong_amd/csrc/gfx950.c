@@ -2,8 +2,8 @@
  *  @brief Host side of the gfx950 backend: operand placement, staging, the reference's error convention.
  *  @file numkong_amd/csrc/gfx950.c
  *
- *  Defines `nk_dots_packed_size_<T>_gfx950`, `nk_dots_pack_<T>_gfx950`, `nk_dots_packed_<T>_gfx950`,
- *  the backend-suffixed kernels that dispatch_<T>.c binds, in the way the reference names its per-ISA
+ *  Defines `nk_dots_packed_size_<T>_gfx950`, `nk_dots_pack_<T>_gfx950`, `nk_dots_packed_<T>_gfx950`, the packed
+ *  distances and the symmetric kinds on top of them: the backend-suffixed kernels that dispatch_<T>.c binds, in the way the reference names its per-ISA
  *  kernels (include/numkong/dots.h:361-1877). Plain C over the thin HIP ABI of <numkong_amd/hip_abi.h>.
  *
  *  The reference's kernels take caller-owned pointers and return nothing (include/numkong/dots.h:84-98);
@@ -174,6 +174,100 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
     if (staged_c) nk_hip_free(staged_c);
 }
 
+nk_size_t nk_amd_symmetric_workspace_size(nk_dtype_t dtype, nk_size_t vectors_count, nk_size_t depth,
+                                          nk_size_t row_start, nk_size_t row_count) {
+    return nk_hip_symmetric_workspace_size((int)dtype, vectors_count, depth, row_start, row_count);
+}
+
+static int nk_amd_symmetric_metric_(nk_kernel_kind_t kind) {
+    switch (kind) {
+    case nk_kernel_dots_symmetric_k: return 0;
+    case nk_kernel_angulars_symmetric_k: return 1;
+    case nk_kernel_euclideans_symmetric_k: return 2;
+    default: return -1;
+    }
+}
+
+int nk_amd_symmetric_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void const *vectors, nk_size_t vectors_count,
+                           nk_size_t depth, nk_size_t stride, void *result, nk_size_t result_stride, nk_size_t row_start,
+                           nk_size_t row_count, void *workspace, nk_size_t workspace_bytes, void *stream) {
+    return nk_hip_symmetric_async((int)dtype, nk_amd_symmetric_metric_(kind), vectors, vectors_count, depth, stride,
+                                  result, result_stride, row_start, row_count, workspace, workspace_bytes, stream);
+}
+
+/** 0xFF over the whole n x n result, as the reference's stub does (c/numkong.c:218-227), 4 bytes per output. */
+static void nk_amd_fill_symmetric_error_(void *result, int kind, size_t n, size_t result_stride) {
+    nk_amd_fill_error_(result, kind, n, n, result_stride);
+}
+
+/**
+ *  The symmetric kinds: rows [row_start, row_start + row_count) of the upper triangle of the n x n result.
+ *  Host operands are staged: the vectors from the window's first 32-row boundary on, and the window of the result
+ *  both ways, so that what the kernel does not write (left of the diagonal) comes back as the caller had it.
+ */
+static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors, nk_size_t n, nk_size_t k,
+                              nk_size_t stride, void *result, nk_size_t result_stride, nk_size_t row_start,
+                              nk_size_t row_count) {
+    nk_amd_error_[0] = 0;
+    if (!n || !row_count || row_start >= n) return;
+    size_t const element_bytes = nk_amd_element_bytes_(dtype);
+    if (nk_hip_device_count() <= 0) {
+        snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_symmetric: no HIP device");
+        nk_amd_fill_symmetric_error_(result, 0, n, result_stride);
+        return;
+    }
+    int const r_kind = nk_hip_pointer_kind(result);
+    size_t const workspace_bytes = nk_hip_symmetric_workspace_size((int)dtype, n, k, row_start, row_count);
+    if (!workspace_bytes || !result) {
+        snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_symmetric: unsupported dtype or dimensions");
+        nk_amd_fill_symmetric_error_(result, r_kind, n, result_stride);
+        return;
+    }
+    size_t const row_end = row_count < n - row_start ? row_start + row_count : n;
+    size_t const first = row_start / 32 * 32; /* vectors and result columns from here on take part */
+    int const v_kind = k ? nk_hip_pointer_kind(vectors) : 1;
+    void *staged_v = NULL, *staged_r = NULL, *workspace = NULL;
+    /* device views, addressed as if they started at vector 0 / result element (0, 0) */
+    char const *device_v = (char const *)vectors;
+    char *device_r = (char *)result;
+    size_t device_stride = stride, device_r_stride = result_stride;
+    int status = nk_hip_malloc(&workspace, workspace_bytes);
+
+    if (!status && v_kind == 0) {
+        size_t const row_bytes = k * element_bytes;
+        device_stride = nk_amd_round_up_(row_bytes, 16);
+        status = nk_hip_malloc(&staged_v, (n - first) * device_stride);
+        if (!status)
+            status = nk_hip_memcpy2d_h2d(staged_v, device_stride, (char const *)vectors + first * stride, stride,
+                                         row_bytes, n - first, NULL);
+        device_v = (char const *)staged_v - first * device_stride;
+    }
+    char *host_window = (char *)result + row_start * result_stride + first * 4;
+    if (!status && r_kind == 0) {
+        device_r_stride = nk_amd_round_up_((n - first) * 4, 16);
+        status = nk_hip_malloc(&staged_r, (row_end - row_start) * device_r_stride);
+        if (!status)
+            status = nk_hip_memcpy2d_h2d(staged_r, device_r_stride, host_window, result_stride, (n - first) * 4,
+                                         row_end - row_start, NULL);
+        device_r = (char *)staged_r - row_start * device_r_stride - first * 4;
+    }
+    if (!status)
+        status = nk_hip_symmetric_async((int)dtype, metric, device_v, n, k, device_stride, device_r, device_r_stride,
+                                        row_start, row_count, workspace, workspace_bytes, NULL);
+    if (!status && staged_r)
+        status = nk_hip_memcpy2d_d2h(host_window, result_stride, staged_r, device_r_stride, (n - first) * 4,
+                                     row_end - row_start, NULL);
+    if (!status) status = nk_hip_stream_synchronize(NULL);
+    else (void)nk_hip_stream_synchronize(NULL);
+    if (status) {
+        nk_amd_set_error_("nk_dots_symmetric");
+        nk_amd_fill_symmetric_error_(result, r_kind, n, result_stride);
+    }
+    if (staged_v) nk_hip_free(staged_v);
+    if (staged_r) nk_hip_free(staged_r);
+    if (workspace) nk_hip_free(workspace);
+}
+
 #define NK_AMD_DEFINE_BACKEND_(T, in_t, out_t)                                                                     \
     nk_size_t nk_dots_packed_size_##T##_gfx950(nk_size_t width, nk_size_t depth) {                                 \
         return nk_amd_packed_size_(nk_##T##_k, width, depth);                                                      \
@@ -195,6 +289,24 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
                                            nk_size_t width, nk_size_t depth, nk_size_t a_stride,                   \
                                            nk_size_t c_stride) {                                                   \
         nk_amd_packed_(nk_##T##_k, 2, a, b_packed, c, height, width, depth, a_stride, c_stride);                   \
+    }                                                                                                              \
+    void nk_dots_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,             \
+                                        nk_size_t stride, out_t *result, nk_size_t result_stride,                  \
+                                        nk_size_t row_start, nk_size_t row_count) {                                \
+        nk_amd_symmetric_(nk_##T##_k, 0, vectors, vectors_count, depth, stride, result, result_stride, row_start,  \
+                          row_count);                                                                              \
+    }                                                                                                              \
+    void nk_angulars_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,         \
+                                            nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,           \
+                                            nk_size_t row_start, nk_size_t row_count) {                            \
+        nk_amd_symmetric_(nk_##T##_k, 1, vectors, vectors_count, depth, stride, result, result_stride, row_start,  \
+                          row_count);                                                                              \
+    }                                                                                                              \
+    void nk_euclideans_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,       \
+                                              nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,         \
+                                              nk_size_t row_start, nk_size_t row_count) {                          \
+        nk_amd_symmetric_(nk_##T##_k, 2, vectors, vectors_count, depth, stride, result, result_stride, row_start,  \
+                          row_count);                                                                              \
     }
 
 NK_AMD_DEFINE_BACKEND_(i8, nk_i8_t, nk_i32_t)

@@ -4,7 +4,8 @@
  *
  *  Counterpart of the reference's c/numkong.c for this path: the table (c/numkong.c:231), the
  *  `nk_dots_packed_size_T` / `nk_dots_pack_T` / `nk_dots_packed_T` trampolines (c/numkong.c:347-364,
- *  instantiated :628-671) and the `nk_angulars_packed_T` / `nk_euclideans_packed_T` ones next to them, the error stubs (:78-81, :195-216), the capability and lookup API
+ *  instantiated :628-671), the `nk_angulars_packed_T` / `nk_euclideans_packed_T` ones next to them and the three
+ *  symmetric kinds, the error stubs (:78-81, :195-227), the capability and lookup API
  *  (:767-768, :831-913) and initialisation when the library is loaded (:916-919).
  */
 #include <string.h>
@@ -42,6 +43,13 @@ void nk_error_dots_(void const *a, void const *b_packed, void *c, nk_size_t m, n
     for (nk_size_t row = 0; row < m; ++row) nk_fill_error_((char *)c + row * c_stride, n * 4);
 }
 
+/** The reference's stub poisons the whole n x n result, whatever the window (c/numkong.c:218-227). */
+void nk_error_dots_symmetric_(void const *vectors, nk_size_t n_vectors, nk_size_t depth, nk_size_t stride, void *result,
+                              nk_size_t result_stride, nk_size_t row_start, nk_size_t row_count) {
+    (void)row_start, (void)row_count;
+    nk_error_dots_(vectors, 0, result, n_vectors, n_vectors, depth, stride, result_stride);
+}
+
 #define NK_AMD_DISPATCH_CROSS_(T, in_t, out_t)                                                                  \
     NK_DYNAMIC nk_size_t nk_dots_packed_size_##T(nk_size_t n, nk_size_t k) {                                    \
         return nk_dispatch_table.dots_packed_size_##T(n, k);                                                    \
@@ -62,6 +70,23 @@ void nk_error_dots_(void const *a, void const *b_packed, void *c, nk_size_t m, n
                                              nk_size_t n, nk_size_t k, nk_size_t a_stride,                      \
                                              nk_size_t c_stride) {                                              \
         nk_dispatch_table.euclideans_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                   \
+    }                                                                                                           \
+    NK_DYNAMIC void nk_dots_symmetric_##T(in_t const *vectors, nk_size_t n, nk_size_t k, nk_size_t stride,      \
+                                          out_t *result, nk_size_t result_stride, nk_size_t row_start,          \
+                                          nk_size_t row_count) {                                                \
+        nk_dispatch_table.dots_symmetric_##T(vectors, n, k, stride, result, result_stride, row_start, row_count); \
+    }                                                                                                           \
+    NK_DYNAMIC void nk_angulars_symmetric_##T(in_t const *vectors, nk_size_t n, nk_size_t k, nk_size_t stride,  \
+                                              nk_f32_t *result, nk_size_t result_stride, nk_size_t row_start,   \
+                                              nk_size_t row_count) {                                            \
+        nk_dispatch_table.angulars_symmetric_##T(vectors, n, k, stride, result, result_stride, row_start,       \
+                                                 row_count);                                                    \
+    }                                                                                                           \
+    NK_DYNAMIC void nk_euclideans_symmetric_##T(in_t const *vectors, nk_size_t n, nk_size_t k, nk_size_t stride, \
+                                                nk_f32_t *result, nk_size_t result_stride, nk_size_t row_start, \
+                                                nk_size_t row_count) {                                          \
+        nk_dispatch_table.euclideans_symmetric_##T(vectors, n, k, stride, result, result_stride, row_start,     \
+                                                   row_count);                                                  \
     }
 
 NK_AMD_DISPATCH_CROSS_(i8, nk_i8_t, nk_i32_t)
@@ -119,7 +144,8 @@ NK_DYNAMIC void nk_find_kernel_punned(nk_kernel_kind_t kind, nk_dtype_t dtype, n
 }
 
 NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t input) {
-    if (kind == nk_kernel_angulars_packed_k || kind == nk_kernel_euclideans_packed_k) {
+    if (kind == nk_kernel_angulars_packed_k || kind == nk_kernel_euclideans_packed_k ||
+        kind == nk_kernel_angulars_symmetric_k || kind == nk_kernel_euclideans_symmetric_k) {
         switch (input) { /* reference: include/numkong/numkong.h:46-51; f32 for every type served here */
         case nk_i8_k:
         case nk_u8_k:
@@ -130,7 +156,7 @@ NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t i
         default: return nk_dtype_unknown_k;
         }
     }
-    if (kind != nk_kernel_dots_packed_k) return nk_dtype_unknown_k;
+    if (kind != nk_kernel_dots_packed_k && kind != nk_kernel_dots_symmetric_k) return nk_dtype_unknown_k;
     switch (input) {
     case nk_i8_k: return nk_i32_k;
     case nk_u8_k: return nk_u32_k;

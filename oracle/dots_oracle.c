@@ -37,6 +37,13 @@
  *      takes from whatever nk_reduce_moments_* kernel its dispatch picks on the host, to within 4 f32 ulp of
  *      the serial kernels' results.
  *
+ *    - the symmetric kinds (all pairs of one set of vectors, upper triangle of a row window): the same per-pair
+ *      arithmetic as the packed kinds, the diagonal of the distances exactly 0
+ *          include/numkong/dots/serial.h:2039-2435, 2802-2878
+ *      Pinned against nk_dots_symmetric_<T>_serial (bit for bit, all six types) and
+ *      nk_{angulars,euclideans}_symmetric_<T>_serial (bit for bit for i8/u8, float types as above), over windows that
+ *      start and end off the reference's 32- and 128-row blocks, and against the packed restatement with B = A.
+ *
  *  Parity unpinned: the per-column norms of FLOAT types in the serial packed image as stored bytes (the
  *  reference computes them with the host-dispatched nk_reduce_moments_*, whose summation order is not restated
  *  here). They are not read by dots_packed; nko_serial_pack writes zeros there and the tests compare header +
@@ -458,3 +465,55 @@ NKO_API void nko_spatials_f64(int dtype, int metric, void const *a, void const *
 }
 
 #pragma endregion Packed distances
+
+#pragma region Symmetric kinds
+
+/** One serial dot product of two unpacked rows, as 32 result bits: the arithmetic of nko_serial_packed. The
+ *  symmetric kernels run the same per-pair state machines as the packed ones (dots/serial.h:2499-2603 name the
+ *  same init/update/finalize functions for both; f16 goes through nk_dot_f16x8_*_serial, dot/serial.h:345-374,
+ *  which keeps the same four lane sums, lane = k mod 4, as the f32x4 path of its packed kernel). */
+static uint32_t serial_dot_bits(int dtype, void const *a_row, void const *b_row, size_t depth) {
+    if (dtype == NKO_I8) {
+        int64_t sum = 0;
+        for (size_t l = 0; l < depth; ++l) sum += (int64_t)((int8_t const *)a_row)[l] * ((int8_t const *)b_row)[l];
+        return (uint32_t)(int32_t)sum;
+    }
+    if (dtype == NKO_U8) {
+        uint64_t sum = 0;
+        for (size_t l = 0; l < depth; ++l) sum += (uint64_t)((uint8_t const *)a_row)[l] * ((uint8_t const *)b_row)[l];
+        return (uint32_t)sum;
+    }
+    float lanes[4] = {0, 0, 0, 0};
+    for (size_t l = 0; l < depth; ++l) {
+        volatile float product = element_f32(dtype, a_row, l) * element_f32(dtype, b_row, l); /* exact, see above */
+        lanes[l & 3] += product;
+    }
+    return f32_to_bits(((lanes[0] + lanes[1]) + lanes[2]) + lanes[3]);
+}
+
+/** nk_dots_symmetric_<T>_serial (metric 0), nk_angulars_symmetric_<T>_serial (1), nk_euclideans_symmetric_<T>_serial
+ *  (2): for the rows i of [row_start, row_start + row_count) and the columns j >= i only, result[i][j] = the dot
+ *  product of vectors i and j (dots/serial.h:2361-2435: upper triangle, the rest of the result is not this call's),
+ *  or its finaliser with the two vectors' sums of squares for j > i and exactly 0 on the diagonal
+ *  (dots/serial.h:2802-2878). Everything else in `result` is left alone. */
+NKO_API void nko_serial_symmetric(int dtype, int metric, void const *vectors, size_t count, size_t depth, size_t stride,
+                                  void *result, size_t result_stride, size_t row_start, size_t row_count) {
+    size_t const row_end = row_start + row_count < count ? row_start + row_count : count;
+    uint32_t *norms = NULL;
+    if (metric) {
+        norms = (uint32_t *)__builtin_malloc(count * sizeof(uint32_t) + 4);
+        nko_row_sumsq(dtype, vectors, count, depth, stride, norms);
+    }
+    for (size_t i = row_start; i < row_end; ++i) {
+        unsigned char const *a_row = (unsigned char const *)vectors + i * stride;
+        uint32_t *out = (uint32_t *)((unsigned char *)result + i * result_stride);
+        for (size_t j = i; j < count; ++j) {
+            uint32_t const dot = serial_dot_bits(dtype, a_row, (unsigned char const *)vectors + j * stride, depth);
+            if (!metric) out[j] = dot;
+            else out[j] = i == j ? 0u : f32_to_bits(serial_from_dot(dtype, metric, dot, norms[i], norms[j]));
+        }
+    }
+    if (norms) __builtin_free(norms);
+}
+
+#pragma endregion Symmetric kinds

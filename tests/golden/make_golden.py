@@ -20,7 +20,7 @@ def main():
         raise SystemExit("build oracle/_ref first: make -C oracle")
     out = support.GOLDEN_DIR
     rng = np.random.default_rng(2024)
-    only = sys.argv[1] if len(sys.argv) > 1 else ""  # e.g. "spatials": rewrite only the files of that family
+    only = sys.argv[1] if len(sys.argv) > 1 else ""  # e.g. "spatials" or "symmetric": rewrite only that family's files
     for dtype in support.FLOAT_DTYPES if only in ("", "cast", "dots") else []:
         codes = np.arange(256 if support.STORAGE[dtype] == np.uint8 else 65536).astype(support.STORAGE[dtype])
         if len(codes) > 256:
@@ -53,7 +53,7 @@ def main():
                                 serial_packed_size=reference.packed_size(dtype, n, k))
     # Packed distances: finite inputs, one zero row and one pair of identical rows, serial kernels of the reference.
     rng = np.random.default_rng(2025)
-    for dtype in support.ALL_DTYPES:
+    for dtype in support.ALL_DTYPES if only in ("", "spatials") else []:
         m, n, k = 12, 10, 203
         a = np.ascontiguousarray(support.random_matrix(oracle, dtype, m, k, rng))
         b = np.ascontiguousarray(support.random_matrix(oracle, dtype, n, k, rng))
@@ -65,6 +65,24 @@ def main():
         np.savez_compressed(os.path.join(out, f"spatials_{dtype}.npz"), dtype=dtype, a=a, b=b,
                             angulars_serial=reference.spatials_packed(support.KIND_ANGULARS, dtype, a, b),
                             euclideans_serial=reference.spatials_packed(support.KIND_EUCLIDEANS, dtype, a, b))
+    # Symmetric kinds: 45 vectors, the window of rows [5, 39) (off the reference's 4- and 32-row blocks); only the
+    # elements the call owns are kept (row in the window, column >= row), the rest of the arrays is zero.
+    rng = np.random.default_rng(2026)
+    for dtype in support.ALL_DTYPES if only in ("", "symmetric") else []:
+        count, depth, row_start, row_count = 45, 203, 5, 34
+        vectors = np.ascontiguousarray(support.random_matrix(oracle, dtype, count, depth, rng))
+        if dtype == "e5m2":
+            vectors = np.where((vectors & 0x7F) > 0x7B, (vectors & 0x80) | 0x7B, vectors).astype(vectors.dtype)
+        vectors[7] = 0
+        vectors[30] = vectors[11]
+        i, j = np.arange(count)[:, None], np.arange(count)[None, :]
+        own = (i >= row_start) & (i < row_start + row_count) & (j >= i)
+        results = {metric: np.where(own, reference.symmetric(metric, dtype, vectors, row_start, row_count), 0)
+                   for metric in ("dots", "angular", "euclidean")}
+        np.savez_compressed(os.path.join(out, f"symmetric_{dtype}.npz"), dtype=dtype, vectors=vectors, row_start=row_start,
+                            row_count=row_count, dots_serial=results["dots"].astype(support.OUTPUT[dtype]),
+                            angulars_serial=results["angular"].astype(np.float32),
+                            euclideans_serial=results["euclidean"].astype(np.float32))
     print("wrote", len(os.listdir(out)) - 1, "fixtures to", out)
 
 

@@ -24,6 +24,9 @@ FLOAT_DTYPES = ("bf16", "f16", "e4m3", "e5m2")
 ALL_DTYPES = ("i8", "u8") + FLOAT_DTYPES
 KIND_SIZE, KIND_PACK, KIND_PACKED = ord("P"), ord("Q"), ord("G")
 KIND_ANGULARS, KIND_EUCLIDEANS = ord("N"), ord("E")  # packed distances: same prototype as the packed product
+# symmetric kinds (vectors, count, depth, stride, result, result_stride, row_start, row_count), by metric
+SYMMETRIC_KINDS = {"dots": ord("y"), "angular": ord("n"), "euclidean": ord("D")}
+SYMMETRIC_METRICS = {"dots": 0, "angular": 1, "euclidean": 2}
 METRICS = {"angular": 1, "euclidean": 2}
 METRIC_KINDS = {"angular": KIND_ANGULARS, "euclidean": KIND_EUCLIDEANS}
 CAP_SERIAL = 1
@@ -50,6 +53,7 @@ class Oracle:
         lib.nko_row_sumsq.argtypes = [_i32, _vp, _sz, _sz, _sz, _vp]
         lib.nko_serial_spatials.argtypes = [_i32, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz]
         lib.nko_spatials_f64.argtypes = [_i32, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
+        lib.nko_serial_symmetric.argtypes = [_i32, _i32, _vp, _sz, _sz, _sz, _vp, _sz, _sz, _sz]
 
     def decode(self, dtype: str, codes: np.ndarray) -> np.ndarray:
         codes = np.ascontiguousarray(codes, dtype=STORAGE[dtype])
@@ -105,6 +109,18 @@ class Oracle:
                                   b.strides[0])
         return c
 
+    def symmetric(self, metric: str, dtype: str, vectors: np.ndarray, row_start: int = 0, row_count=None,
+                  out: np.ndarray = None) -> np.ndarray:
+        """`nk_{dots,angulars,euclideans}_symmetric_<dtype>_serial` into `out` (count x count; fresh and zeroed when
+        not given): only result[i][j], i in the row window, j >= i, is written."""
+        count, depth = vectors.shape
+        if out is None:
+            out = np.zeros((count, count), dtype=OUTPUT[dtype] if metric == "dots" else np.float32)
+        rows = count - row_start if row_count is None else row_count
+        self.lib.nko_serial_symmetric(CODES[dtype], SYMMETRIC_METRICS[metric], _ptr(vectors), count, depth,
+                                      vectors.strides[0], _ptr(out), out.strides[0], row_start, rows)
+        return out
+
     def truth(self, dtype: str, a: np.ndarray, b: np.ndarray):
         """(f64 ground truth, sum |a*b|) as the reference's own tests compute it."""
         m, k = a.shape
@@ -138,6 +154,9 @@ class Reference:
             KIND_PACKED: ctypes.CFUNCTYPE(None, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz),
             KIND_ANGULARS: ctypes.CFUNCTYPE(None, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz),
             KIND_EUCLIDEANS: ctypes.CFUNCTYPE(None, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz),
+            SYMMETRIC_KINDS["dots"]: ctypes.CFUNCTYPE(None, _vp, _sz, _sz, _sz, _vp, _sz, _sz, _sz),
+            SYMMETRIC_KINDS["angular"]: ctypes.CFUNCTYPE(None, _vp, _sz, _sz, _sz, _vp, _sz, _sz, _sz),
+            SYMMETRIC_KINDS["euclidean"]: ctypes.CFUNCTYPE(None, _vp, _sz, _sz, _sz, _vp, _sz, _sz, _sz),
         }[kind]
         return proto(fn.value), int(cap.value)
 
@@ -180,6 +199,17 @@ class Reference:
         c = np.empty((m, n), dtype=np.float32)
         self.kernel(kind, dtype, viable)[0](_ptr(a), _ptr(packed), _ptr(c), m, n, k, a.strides[0], c.strides[0])
         return c
+
+    def symmetric(self, metric: str, dtype: str, vectors: np.ndarray, row_start: int = 0, row_count=None,
+                  out: np.ndarray = None, viable: int = CAP_SERIAL) -> np.ndarray:
+        """The chosen backend's symmetric kernel into `out` (count x count; fresh and zeroed when not given)."""
+        count, depth = vectors.shape
+        if out is None:
+            out = np.zeros((count, count), dtype=OUTPUT[dtype] if metric == "dots" else np.float32)
+        rows = count - row_start if row_count is None else row_count
+        self.kernel(SYMMETRIC_KINDS[metric], dtype, viable)[0](_ptr(vectors), count, depth, vectors.strides[0], _ptr(out),
+                                                               out.strides[0], row_start, rows)
+        return out
 
 
 def load_oracle() -> Oracle:

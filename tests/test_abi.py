@@ -26,17 +26,20 @@ def declared_symbols():
             names |= {f"nk_dots_packed_size_{t}_gfx950", f"nk_dots_pack_{t}_gfx950", f"nk_dots_packed_{t}_gfx950"}
             names |= {f"nk_angulars_packed_{t}_gfx950", f"nk_euclideans_packed_{t}_gfx950"}
             names |= {f"nk_angulars_packed_{t}", f"nk_euclideans_packed_{t}"}  # also declared through a macro
+            for family in ("dots", "angulars", "euclideans"):
+                names |= {f"nk_{family}_symmetric_{t}", f"nk_{family}_symmetric_{t}_gfx950"}
     return {n for n in names if "##" not in n}
 
 
 def test_library_exports_every_declared_symbol():
     lib = nk.library()
     names = declared_symbols()
-    assert len(names) >= 30 * 2 + 8 + 15
+    assert len(names) >= 30 * 2 + 36 + 8 + 19
     missing = [n for n in sorted(names) if not hasattr(lib, n)]
     assert not missing, missing
     for t in TYPES:
-        for stem in ("nk_dots_packed_size_", "nk_dots_pack_", "nk_dots_packed_", "nk_angulars_packed_", "nk_euclideans_packed_"):
+        for stem in ("nk_dots_packed_size_", "nk_dots_pack_", "nk_dots_packed_", "nk_angulars_packed_", "nk_euclideans_packed_",
+                     "nk_dots_symmetric_", "nk_angulars_symmetric_", "nk_euclideans_symmetric_"):
             assert hasattr(lib, stem + t)
 
 
@@ -75,12 +78,21 @@ def test_lookup_and_capabilities():
             assert fn == backend and cap == CAP_GFX950
             fn, cap = find(lib, kind, code, 1)  # serial only: no kernel behind it here -> error stub, capability 0
             assert fn and fn != backend and cap == 0
-        fn, cap = find(lib, ord("y"), code, CAP_GFX950)  # symmetric dots: not on this path
+        for kind, stem in ((ord("y"), "nk_dots_symmetric_"), (ord("n"), "nk_angulars_symmetric_"),
+                           (ord("D"), "nk_euclideans_symmetric_")):
+            fn, cap = find(lib, kind, code, CAP_GFX950)
+            assert fn == ctypes.cast(getattr(lib, f"{stem}{t}_gfx950"), ctypes.c_void_p).value and cap == CAP_GFX950
+            fn, cap = find(lib, kind, code, 1)
+            assert fn and cap == 0
+        fn, cap = find(lib, ord("Y"), code, CAP_GFX950)  # symmetric hamming distances: not on this path
         assert fn and cap == 0
     assert find(lib, ord("G"), 1 << 10, CAP_GFX950) == (None, 0)  # f64: unknown dtype -> null kernel
     out = {"i8": 1 << 4, "u8": 1 << 8, "bf16": 1 << 11, "f16": 1 << 11, "e4m3": 1 << 11, "e5m2": 1 << 11}
     for t, expected in out.items():
         assert lib.nk_kernel_output_dtype(ord("G"), api.DTYPES[t][0]) == expected
+        assert lib.nk_kernel_output_dtype(ord("y"), api.DTYPES[t][0]) == expected
+        assert lib.nk_kernel_output_dtype(ord("n"), api.DTYPES[t][0]) == 1 << 11
+        assert lib.nk_kernel_output_dtype(ord("D"), api.DTYPES[t][0]) == 1 << 11
     assert lib.nk_kernel_output_dtype(ord("i"), api.DTYPES["i8"][0]) == 0
 
 
@@ -102,6 +114,10 @@ def test_error_convention_without_backend():
         f = np.zeros((2, 4), np.float32)
         lib.nk_dots_packed_bf16(a.ctypes.data, packed.ctypes.data, f.ctypes.data, 2, 3, 2, 4, 16)
         assert np.isnan(f[:, :3]).all() and (f[:, 3] == 0).all()
+        # the symmetric stub poisons the whole count x count result, whatever the window (c/numkong.c:218-227)
+        g = np.zeros((5, 6), np.int32)
+        lib.nk_dots_symmetric_i8(b.ctypes.data, 5, 7, 7, g.ctypes.data, 24, 1, 2)
+        assert (g[:, :5] == -1).all() and (g[:, 5] == 0).all()
     finally:
         lib.nk_dispatch_table_update(lib.nk_capabilities_compiled())
     assert lib.nk_dots_packed_size_i8(5, 7) == 64 + 16 * 512 + 256
@@ -118,6 +134,24 @@ def test_no_gpu_means_loud_failure_not_fallback():
     c = np.zeros((2, 2), np.int32)
     lib.nk_dots_packed_i8(a.ctypes.data, packed.ctypes.data, c.ctypes.data, 2, 2, 16, 16, 8)
     assert (c == -1).all() and b"no HIP device" in lib.nk_amd_last_error()
+    c[:] = 0
+    lib.nk_dots_symmetric_i8(a.ctypes.data, 2, 16, 16, c.ctypes.data, 8, 0, 2)
+    assert (c == -1).all() and b"no HIP device" in lib.nk_amd_last_error()
+
+
+def test_symmetric_workspace_size():
+    """The packed image of the vectors from the window's 32-row boundary on, rounded up to 256 bytes, plus the tile
+    list: at most 8 bytes per 64 x 128 tile of the window and a word per 8 tile rows."""
+    lib = nk.library()
+    for t in TYPES:
+        code = api.DTYPES[t][0]
+        for n, k, start, rows in [(100, 64, 0, 100), (1000, 300, 37, 411), (8192, 1024, 4096, 4096)]:
+            size = lib.nk_amd_symmetric_workspace_size(code, n, k, start, rows)
+            image = nk.dots_packed_size(t, n - start // 32 * 32, k)
+            tiles = -(-min(rows, n - start) // 64) * -(-(n - start // 32 * 32) // 128)
+            assert (image + 255) // 256 * 256 < size <= (image + 255) // 256 * 256 + 8 * tiles + 4 * (tiles // 8 + 4) + 8
+        assert lib.nk_amd_symmetric_workspace_size(code, 100, 64, 100, 5) == 0  # an empty window needs nothing
+        assert lib.nk_amd_symmetric_workspace_size(code, 100, 64, 0, 0) == 0
 
 
 def test_python_mirror_validates_arguments():
@@ -132,3 +166,7 @@ def test_python_mirror_validates_arguments():
         nk.dots_pack([[1, 2]], "i8")
     with pytest.raises(TypeError):
         nk.dots_packed(cpu, object())
+    with pytest.raises(ValueError):
+        nk.dots_symmetric(cpu, "i8")  # must live on the GPU
+    with pytest.raises(TypeError):
+        nk.angulars_symmetric(cpu, "f64")

@@ -8,12 +8,16 @@ and, when the reference build oracle/_ref is present, the kernel the reference d
 
   normwise error  e = |c - truth| / sum|a*b|   per element, over elements with a finite truth
   gate:  mean(e_gpu) <= 2 * mean(e_ref) + 2^-24 / sqrt(count)   (the slack only matters for a handful of outputs)
-         max(e_gpu)  <= 2 * max(max(e_ref), 2^-24)         (one f32 rounding unit of the magnitude sum)
+         max(e_gpu)  <= 2 * max(max(e_ref), floor)         floor = 2^-24 against the serial kernel (one f32 rounding unit
+                                                            of the magnitude sum), 2.5 * 2^-24 against the dispatched one
          NaN, +Inf and -Inf masks identical to the serial kernel's (the reference's AVX-512 e5m2 kernels do
          not propagate Inf/NaN, so masks are not compared with them and their non-finite outputs are skipped).
 
-The 2^-24 floor keeps the max statistic meaningful on small samples, where all kernels sit at a single
-rounding of the result. Measured on 192 x 256 outputs at depth 4096-8192 (GPU / serial, GPU / dispatched, mean
+The floor keeps the max statistic meaningful where all kernels sit at a few roundings of the result: on small
+samples, and at shallow depths against the 16-lane AVX-512 kernels, whose lanes each add only depth / 16 products
+and round to nearest where the MFMA's 16-product sums truncate. Measured over 490,000 outputs at depth 130, in
+units of 2^-24 (mean, 99.99th percentile, max): bf16 GPU 0.095, 1.95, 3.71; serial 0.088, 1.49, 2.50; dispatched
+0.080, 1.28, 1.98. The means agree; only the largest few outputs in a million differ. Measured on 192 x 256 outputs at depth 4096-8192 (GPU / serial, GPU / dispatched, mean
 of the normwise error): bf16 0.52-0.56, 1.13; f16 0.27, 0.52; e4m3 0.96, 1.16; e5m2 0.99, 1.13.
 """
 import ctypes
@@ -77,7 +81,8 @@ def assert_float_gate(dtype, got, serial, truth, magnitude, where="", dispatched
         e_ref = np.abs(ref[finite].astype(np.float64) - truth[finite]) / magnitude[finite]
         slack = U / np.sqrt(e_gpu.size)  # the standard error of a mean of single-rounding errors: decides tiny samples only
         assert e_gpu.mean() <= 2 * e_ref.mean() + slack, f"mean error {e_gpu.mean():.3e} vs {name} {e_ref.mean():.3e} {where}"
-        assert e_gpu.max() <= 2 * max(e_ref.max(), U), f"max error {e_gpu.max():.3e} vs {name} {e_ref.max():.3e} {where}"
+        floor = U if name == "serial" else 2.5 * U
+        assert e_gpu.max() <= 2 * max(e_ref.max(), floor), f"max error {e_gpu.max():.3e} vs {name} {e_ref.max():.3e} {where}"
 
 
 def check(oracle, dtype, a, b, config=0, where=""):

@@ -237,6 +237,88 @@ def test_packed_distances_closed_forms(oracle, dtype, metric):
     assert np.allclose(got, expected, atol=2e-6)
 
 
+def upper_window(count, row_start, row_count):
+    """Mask of what a symmetric call owns: rows of the window, columns on or right of the diagonal."""
+    i, j = np.arange(count)[:, None], np.arange(count)[None, :]
+    return (i >= row_start) & (i < row_start + row_count) & (j >= i)
+
+
+# (count, depth, row_start, row_count): windows that start and end off the reference's 4-, 32- and 128-row blocks
+SYMMETRIC_CASES = [(1, 1, 0, 1), (7, 37, 0, 7), (45, 300, 0, 45), (45, 300, 5, 17), (150, 70, 0, 150), (150, 70, 33, 100),
+                   (150, 70, 128, 500), (70, 1030, 64, 6)]
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_symmetric_dots_match_reference_serial(oracle, reference, dtype):
+    """nk_dots_symmetric_<T>_serial, bit for bit, on the elements the call owns (the reference may also write a few
+    below the diagonal when a window ends inside one of its 32-row blocks; those are not part of the contract)."""
+    if reference is None:
+        pytest.skip("reference build not present")
+    rng = np.random.default_rng(61)
+    for count, depth, row_start, row_count in SYMMETRIC_CASES:
+        vectors = finite_inputs(oracle, dtype, count, depth, rng)
+        mine = oracle.symmetric("dots", dtype, vectors, row_start, row_count)
+        ref = reference.symmetric("dots", dtype, vectors, row_start, row_count)
+        own = upper_window(count, row_start, row_count)
+        assert np.array_equal(mine.view(np.uint32)[own], ref.view(np.uint32)[own]), (dtype, count, depth, row_start)
+        assert not mine[~own].any()  # the restatement writes nothing else
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_symmetric_distances_match_reference_serial(oracle, reference, dtype, metric):
+    """nk_{angulars,euclideans}_symmetric_<T>_serial: integers bit for bit, floats to the tolerance of the packed
+    distances above (the same host-dispatched norms enter); the diagonal is exactly 0 in both."""
+    if reference is None:
+        pytest.skip("reference build not present")
+    rng = np.random.default_rng(62)
+    for count, depth, row_start, row_count in SYMMETRIC_CASES:
+        # (the reference's distance kinds do not clamp a window that runs past the last vector, unlike its dots
+        # kind, dots/serial.h:2380 against :2815-2821: such a call is outside its contract and is not made here)
+        row_count = min(row_count, count - row_start)
+        vectors = finite_inputs(oracle, dtype, count, depth, rng)
+        if count > 40:
+            vectors[2] = 0
+            vectors[9] = vectors[40]  # identical vectors off the diagonal
+        mine = oracle.symmetric(metric, dtype, vectors, row_start, row_count)
+        ref = reference.symmetric(metric, dtype, vectors, row_start, row_count)
+        own = upper_window(count, row_start, row_count)
+        assert not mine[~own].any()
+        assert not np.diag(mine).any() and not np.diag(ref)[row_start:row_start + row_count].any()
+        if dtype in ("i8", "u8"):
+            assert np.array_equal(mine.view(np.uint32)[own], ref.view(np.uint32)[own]), (dtype, metric, count, row_start)
+            continue
+        u = 2.0 ** -24
+        x, y = mine.astype(np.float64)[own], ref.astype(np.float64)[own]
+        if metric == "angular":
+            assert np.abs(x - y).max() <= 8 * u
+        else:
+            squares = oracle.row_sumsq(dtype, vectors).astype(np.float64)
+            norms = (squares[:, None] + squares[None, :])[own]
+            assert ((np.abs(x - y) <= 8 * u * np.abs(y)) | (np.abs(x * x - y * y) <= 8 * u * np.maximum(norms, 1e-30))).all()
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_symmetric_equals_packed_with_both_sides_the_same(oracle, dtype):
+    """Needs no reference: the upper triangle of the symmetric kinds is the packed kinds with B = A (same per-pair
+    arithmetic), the diagonal of the distances is 0, and the row windows tile the full call."""
+    rng = np.random.default_rng(63)
+    vectors = finite_inputs(oracle, dtype, 53, 129, rng)
+    upper = np.triu(np.ones((53, 53), dtype=bool))
+    full = oracle.symmetric("dots", dtype, vectors)
+    assert np.array_equal(full[upper].view(np.uint32), oracle.dots_packed(dtype, vectors, vectors)[upper].view(np.uint32))
+    pieces = np.zeros_like(full)
+    for start, rows in ((0, 10), (10, 1), (11, 31), (42, 100)):
+        oracle.symmetric("dots", dtype, vectors, start, rows, out=pieces)
+    assert np.array_equal(pieces.view(np.uint32), full.view(np.uint32))
+    for metric in ("angular", "euclidean"):
+        got = oracle.symmetric(metric, dtype, vectors)
+        packed = oracle.spatials_packed(metric, dtype, vectors, vectors)
+        strict = np.triu(np.ones((53, 53), dtype=bool), 1)
+        assert np.array_equal(got[strict].view(np.uint32), packed[strict].view(np.uint32))
+        assert not np.diag(got).any()
+
+
 @pytest.mark.parametrize("dtype", ["i8", "u8"])
 def test_integer_product_closed_form(oracle, dtype):
     rng = np.random.default_rng(11)
@@ -290,6 +372,22 @@ def test_golden_vectors(oracle, name):
         dtype = str(data["dtype"])
         assert same_floats(oracle.decode(dtype, data["codes"]), data["decoded"])
         assert np.array_equal(oracle.encode(dtype, data["values"]), data["encoded"])
+    elif name.startswith("symmetric_"):
+        dtype, vectors = str(data["dtype"]), data["vectors"]
+        row_start, row_count = int(data["row_start"]), int(data["row_count"])
+        u = 2.0 ** -24
+        squares = oracle.row_sumsq(dtype, vectors).astype(np.float64)
+        norms = squares[:, None] + squares[None, :]
+        mine = oracle.symmetric("dots", dtype, vectors, row_start, row_count)
+        assert same_floats(mine.view(np.float32), data["dots_serial"].view(np.float32))
+        for metric, key in (("angular", "angulars_serial"), ("euclidean", "euclideans_serial")):
+            mine, ref = oracle.symmetric(metric, dtype, vectors, row_start, row_count).astype(np.float64), data[key].astype(np.float64)
+            if dtype in ("i8", "u8"):
+                assert np.array_equal(mine, ref), (dtype, metric)
+            elif metric == "angular":
+                assert np.abs(mine - ref).max() <= 8 * u
+            else:
+                assert ((np.abs(mine - ref) <= 8 * u * np.abs(ref)) | (np.abs(mine ** 2 - ref ** 2) <= 8 * u * norms)).all()
     elif name.startswith("spatials_"):
         dtype = str(data["dtype"])
         a, b = data["a"], data["b"]
