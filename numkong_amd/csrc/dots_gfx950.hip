@@ -203,8 +203,9 @@ __device__ __forceinline__ v4i widen_fp8x8(uint32_t lo, uint32_t hi) {
 template <int WIDEN>
 __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
                                                    uint64_t k_src_bytes, uint32_t k_chunks, uint8_t *__restrict__ data,
-                                                   int avec, uint32_t xr) {
+                                                   int avec, uint32_t xr, PackedHeader header) {
     constexpr int kSrcChunk = WIDEN ? 8 : 16;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *(PackedHeader *)(data - sizeof(PackedHeader)) = header; // (64 bytes in front of the tiles)
     uint32_t const groups = k_chunks / kStageChunks;
     uint32_t const tile = blockIdx.x / groups;
     uint32_t const group = blockIdx.x % groups;
@@ -572,13 +573,22 @@ __host__ __device__ inline uint32_t first_live_tile(uint32_t t, uint32_t bm_log2
 /**
  *  The tile list of a triangular grid, in the order of `tile_of_block`: bands of kTileBand tile rows, column
  *  by column within a band, top to bottom within a column, and only tiles with something on or right of the
- *  diagonal. One workgroup: the bands' sizes are scanned 256 at a time, then every band is filled by all threads,
- *  a column each. A band's first columns form a staircase (row t joins at column first_live_tile(t)); the cells
+ *  diagonal. One workgroup per list: the bands' sizes are scanned 256 at a time, then every band is filled by all
+ *  threads, a column each. A band's first columns form a staircase (row t joins at column first_live_tile(t)); the cells
  *  left of column c number the sum over its rows of max(0, c - first_live_tile(t)).
  */
-__global__ __launch_bounds__(256) void triangle_tiles_kernel(uint32_t tiles_m, uint32_t tiles_n, uint32_t bm_log2,
-                                                             uint32_t bn_log2, uint32_t shift, uint32_t *band_start,
-                                                             uint32_t *list) {
+struct TriangleGrid {
+    uint32_t tiles_m, tiles_n, bm_log2, bn_log2, shift;
+    uint32_t *band_start, *list;
+};
+struct TriangleGrids {
+    TriangleGrid grid[2];
+};
+__global__ __launch_bounds__(256) void triangle_tiles_kernel(TriangleGrids grids) {
+    TriangleGrid const &mine = grids.grid[blockIdx.x]; // one workgroup per list
+    uint32_t const tiles_m = mine.tiles_m, tiles_n = mine.tiles_n, bm_log2 = mine.bm_log2, bn_log2 = mine.bn_log2,
+                   shift = mine.shift;
+    uint32_t *band_start = mine.band_start, *list = mine.list;
     __shared__ uint32_t scan[256];
     __shared__ uint32_t base;
     uint32_t const tid = threadIdx.x;
@@ -1236,8 +1246,10 @@ inline size_t triangle_scratch_bytes(uint64_t m, uint64_t n, uint32_t bm, uint32
     return (size_t)(((bands + 1 + 1) & ~1ull) * 4 + live_tiles(m, n, bm, bn, shift) * 8);
 }
 
+/** `slots_only`: do not launch, only report how many workgroups of the kernel this call would use are resident on
+ *  the device at once. */
 template <class T, int TM, int TN>
-hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle) {
+hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle, int *slots_only = nullptr) {
     constexpr int BM = TM * 32, BN = TN * 128;
     g.tiles_m = (g.m + BM - 1) / BM;
     g.tiles_n = (g.n + BN - 1) / BN;
@@ -1249,12 +1261,7 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
         if (!tiles) return hipSuccess;
         if (triangle_scratch_bytes(g.m, g.n, BM, BN, g.tri_shift) > triangle->bytes) return hipErrorInvalidValue;
         uint32_t const bands = (g.tiles_m + kTileBand - 1) / kTileBand;
-        uint32_t *list = triangle->words + ((bands + 1 + 1) & ~1u);
-        hipLaunchKernelGGL(triangle_tiles_kernel, dim3(1), dim3(256), 0, stream, g.tiles_m, g.tiles_n,
-                           log2_of(BM), log2_of(BN), g.tri_shift, triangle->words, list);
-        hipError_t const e = hipGetLastError();
-        if (e != hipSuccess) return e;
-        g.tile_list = list;
+        g.tile_list = triangle->words + ((bands + 1 + 1) & ~1u); // (written by the caller's triangle_tiles_kernel)
     }
     g.tile_count = (uint32_t)tiles;
     // The tile's A offsets are 32-bit: (rows of a tile) * stride must stay below 4 GiB.
@@ -1297,41 +1304,114 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
         }
         resident = (per_cu > 0 ? per_cu : 1) * (g_cu_count > 0 ? g_cu_count : 256);
     }
+    if (slots_only) {
+        *slots_only = resident;
+        return hipSuccess;
+    }
     uint32_t const blocks = (uint32_t)(tiles < (uint64_t)resident ? tiles : (uint64_t)resident);
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, g);
     return hipGetLastError();
 }
 
 template <class T>
+hipError_t launch_config(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle, int config,
+                         int *slots_only = nullptr) {
+    switch (config) {
+    case 1:
+        if constexpr (T::kChunked) return hipErrorInvalidValue;
+        else return launch_one<T, 8, 2>(g, stream, triangle, slots_only);
+    case 2: return launch_one<T, 4, 2>(g, stream, triangle, slots_only);
+    case 3: return launch_one<T, 4, 1>(g, stream, triangle, slots_only);
+    default: return launch_one<T, 2, 1>(g, stream, triangle, slots_only);
+    }
+}
+
+template <class T>
 hipError_t launch_typed(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle) {
-    int config = g_forced_config;
-    if (config <= 0 || config >= kConfigCount) {
-        // Largest tile that still gives every one of the 256 CUs at least one workgroup.
-        auto tiles = [&](int c) {
-            uint64_t const bm = kConfigs[c].tm * 32, bn = (uint64_t)kConfigs[c].tn * 128;
-            if (triangle) return live_tiles(g.m, g.n, (uint32_t)bm, (uint32_t)bn, g.tri_shift);
-            return ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
-        };
-        config = 4;
-        for (int c = 1; c <= 4; ++c)
-            if (tiles(c) >= 256) {
-                config = c;
+    int config = g_forced_config & 0x7F;
+    bool const chosen_here = config <= 0 || config >= kConfigCount;
+    auto tiles_of = [&](GemmArgs const &args, int c) {
+        uint64_t const bm = kConfigs[c].tm * 32, bn = (uint64_t)kConfigs[c].tn * 128;
+        if (triangle) return live_tiles(args.m, args.n, (uint32_t)bm, (uint32_t)bn, args.tri_shift);
+        return ((args.m + bm - 1) / bm) * ((args.n + bn - 1) / bn);
+    };
+    // Largest tile that still gives every one of the 256 CUs at least one workgroup.
+    auto choose = [&](GemmArgs const &args, int first) {
+        int best = 4;
+        for (int c = first; c <= 4; ++c)
+            if (tiles_of(args, c) >= 256) {
+                best = c;
                 break;
             }
         // Distances over a shallow depth are bound by the epilogue (a finaliser and a store per output): two
         // workgroups per CU of 128 x 128 tiles overlap it with the other's loop better than one large tile does
         // (measured on 1024 x 1,048,576 x 768: 2.17 against 2.33 ms angular, 1.98 against 2.07 ms euclidean).
-        if (g.metric != 0 && config < 3 && g.k_chunks / kStageChunks <= 8 && tiles(3) >= 256) config = 3;
+        if (args.metric != 0 && best < 3 && args.k_chunks / kStageChunks <= 8 && tiles_of(args, 3) >= 256) best = 3;
+        if (T::kChunked && best == 1) best = 2; // two accumulator sets do not fit the 256 x 256 tile
+        return best;
+    };
+    if (chosen_here) config = choose(g, 1);
+    if (T::kChunked && config == 1) config = 2;
+    // Where the tile list of a launch goes (the same arithmetic as launch_one's) and what it holds.
+    auto grid_of = [](GemmArgs const &args, int c, TriangleScratch const &scratch) {
+        uint32_t const bm = kConfigs[c].tm * 32, bn = kConfigs[c].tn * 128;
+        TriangleGrid grid;
+        grid.tiles_m = (args.m + bm - 1) / bm, grid.tiles_n = (args.n + bn - 1) / bn;
+        grid.bm_log2 = log2_of(bm), grid.bn_log2 = log2_of(bn), grid.shift = args.tri_shift;
+        uint32_t const bands = (grid.tiles_m + kTileBand - 1) / kTileBand;
+        grid.band_start = scratch.words, grid.list = scratch.words + ((bands + 1 + 1) & ~1u);
+        return grid;
+    };
+
+    // A triangular grid rarely fills a whole number of rounds of the persistent workgroups, and a last round that
+    // is mostly empty costs as much as a full one. When that last round would be less than half full, the tile rows
+    // from the top that fill whole rounds go to this tile shape and the rows below them, the narrow end of the
+    // triangle, to a second launch with small tiles that spreads them over the whole device.
+    if (triangle && (chosen_here || (g_forced_config & 0x80)) && config < 4) {
+        int slots = 0;
+        GemmArgs probe = g;
+        hipError_t e = launch_config<T>(probe, stream, triangle, config, &slots);
+        if (e != hipSuccess) return e;
+        uint64_t const live = tiles_of(g, config);
+        uint64_t const rounds = slots > 0 ? live / (uint64_t)slots : 0, rest = slots > 0 ? live % (uint64_t)slots : 0;
+        if (rounds >= 1 && rest > 0 && rest * 2 <= (uint64_t)slots) {
+            uint32_t const bm = kConfigs[config].tm * 32, bn = kConfigs[config].tn * 128;
+            uint32_t const tiles_m = (g.m + bm - 1) / bm, tiles_n = (g.n + bn - 1) / bn;
+            uint64_t count = 0;
+            uint32_t keep = 0; // tile rows that stay with the large tiles
+            for (; keep < tiles_m; ++keep) {
+                uint32_t const from = first_live_tile(keep, log2_of(bm), log2_of(bn), g.tri_shift);
+                uint64_t const here = from < tiles_n ? tiles_n - from : 0;
+                if (count + here > rounds * (uint64_t)slots) break;
+                count += here;
+            }
+            if (keep > 0 && keep < tiles_m) {
+                GemmArgs top = g, bottom = g;
+                top.m = keep * bm;
+                bottom.m = g.m - top.m;
+                bottom.a += (uint64_t)top.m * g.a_stride, bottom.c += (uint64_t)top.m * g.c_stride;
+                bottom.tri_shift = g.tri_shift + top.m;
+                // each launch builds its tile list in its own half of the scratch memory
+                size_t const half = triangle->bytes / 2 / 8 * 8;
+                TriangleScratch const first_half = {triangle->words, half}, second_half = {triangle->words + half / 4, half};
+                int const small = choose(bottom, config + 1);
+                TriangleGrids grids;
+                grids.grid[0] = grid_of(top, config, first_half), grids.grid[1] = grid_of(bottom, small, second_half);
+                hipLaunchKernelGGL(triangle_tiles_kernel, dim3(2), dim3(256), 0, stream, grids);
+                if ((e = hipGetLastError()) != hipSuccess) return e;
+                if ((e = launch_config<T>(top, stream, &first_half, config)) != hipSuccess) return e;
+                return launch_config<T>(bottom, stream, &second_half, small);
+            }
+        }
     }
-    if (T::kChunked && config == 1) config = 2; // two accumulator sets do not fit the 256 x 256 tile
-    switch (config) {
-    case 1:
-        if constexpr (T::kChunked) return hipErrorInvalidValue;
-        else return launch_one<T, 8, 2>(g, stream, triangle);
-    case 2: return launch_one<T, 4, 2>(g, stream, triangle);
-    case 3: return launch_one<T, 4, 1>(g, stream, triangle);
-    default: return launch_one<T, 2, 1>(g, stream, triangle);
+    if (triangle && tiles_of(g, config) > 0) {
+        TriangleGrids grids;
+        grids.grid[0] = grids.grid[1] = grid_of(g, config, *triangle);
+        hipLaunchKernelGGL(triangle_tiles_kernel, dim3(1), dim3(256), 0, stream, grids);
+        hipError_t const e = hipGetLastError();
+        if (e != hipSuccess) return e;
     }
+    return launch_config<T>(g, stream, triangle, config);
 }
 
 inline int widest_load(void const *p, size_t stride) {
@@ -1440,16 +1520,18 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
     uint8_t *data = image + sizeof(PackedHeader);
     uint32_t *sums = (uint32_t *)(data + g.data_bytes);
     uint32_t *norms = sums + (uint64_t)g.n_tiles * kTileRows;
-    hipLaunchKernelGGL(write_header_kernel, dim3(1), dim3(64), 0, stream, (PackedHeader *)image, h);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fail(e, "write_header_kernel");
+    hipError_t e = hipSuccess;
+    if (!(g.n_tiles && g.k_chunks)) { // nothing to pack: the header alone
+        hipLaunchKernelGGL(write_header_kernel, dim3(1), dim3(64), 0, stream, (PackedHeader *)image, h);
+        if ((e = hipGetLastError()) != hipSuccess) return fail(e, "write_header_kernel");
+    }
     if (g.n_tiles && g.k_chunks) {
         uint64_t const blocks = (uint64_t)g.n_tiles * (g.k_chunks / kStageChunks);
         if (blocks > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_pack: matrix too large");
         uint32_t const xr = dtype == kU8 ? 0x80808080u : 0u;
         auto kernel = dtype == kE4M3 ? pack_kernel<1> : (dtype == kE5M2 ? pack_kernel<2> : pack_kernel<0>);
         hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride,
-                           g.n, g.k_src_bytes, g.k_chunks, data, widest_load(b, b_stride), xr);
+                           g.n, g.k_src_bytes, g.k_chunks, data, widest_load(b, b_stride), xr, h);
         e = hipGetLastError();
         if (e != hipSuccess) return fail(e, "pack_kernel");
     }
@@ -1568,6 +1650,7 @@ static bool symmetric_window(int dtype, size_t n, size_t k, size_t row_start, si
                                                     kConfigs[c].tn * 128, shift);
         if (bytes > w.scratch_bytes) w.scratch_bytes = bytes;
     }
+    w.scratch_bytes = 2 * ((w.scratch_bytes + 7) & ~(size_t)7); // room for the lists of two launches (see launch_typed)
     return true;
 }
 
@@ -1607,7 +1690,7 @@ __attribute__((visibility("default"))) void nk_hip_debug_clocks(unsigned long lo
 #endif
 
 void nk_hip_set_tile_config(int config) {
-    g_forced_config = config & 0xFF;
+    g_forced_config = config & 0xFF; // (bit 7: a forced shape may still hand the narrow end of a triangle to small tiles)
     g_variant = (config >> 8) & 0xFF;
 }
 
