@@ -1,0 +1,1440 @@
+/**
+ *  @brief gfx950 (MI355X, CDNA4) kernels for packed batched dot products: C = A * B^T.
+ *  @file numkong_amd/csrc/dots_gfx950.hpp
+ *
+ *  Everything the HIP translation units share: the packed image, the packing kernels, the element types and the
+ *  product kernel with its launch logic. dots_gfx950.hip holds the plain-C entry points of <numkong_amd/hip_abi.h>;
+ *  dots_gfx950_<T>.hip instantiate the product kernels of one element type each, so that they compile side by side.
+ *
+ *  Replaces the per-ISA kernels the reference instantiates from
+ *  include/numkong/dots/serial.h:245-333 (pack size, pack) and :520-1072 (packed product) for
+ *  i8, u8, bf16, f16, e4m3, e5m2.
+ *
+ *  Packed image of B (n rows of k elements), all little-endian:
+ *
+ *      [ 64-byte header ][ tiles ][ per-column compensation terms, u32 x 32 x n_tiles ]
+ *
+ *  A "chunk" is 16 consecutive bytes of one B row (16 i8/fp8 values, 8 bf16/f16 values). Rows are grouped
+ *  into tiles of 32; K is padded with zeros to a multiple of 8 chunks (128 bytes) and N with zero rows to
+ *  a multiple of 32. Chunk `c` of row `r` of tile `t` lives at
+ *
+ *      data + ((t * k_chunks + c) * 32 + r) * 16
+ *
+ *  so the 64 lanes of a wavefront that execute one 32x32 MFMA step `q` (lane l supplies row l % 32 and
+ *  chunk 2q + l / 32) read 1024 contiguous bytes at `data + (t * k_chunks + 2q) * 512 + l * 16`: the image
+ *  is the MFMA operand-fragment order, and B goes from HBM to registers with one coalesced 128-bit load
+ *  per lane per step, never through LDS. Which k sits in which operand slot of the instruction does not
+ *  matter as long as A and B agree, and they do: A fragments are read from LDS with the same rule.
+ *  e4m3 and e5m2 are stored widened to f16 (see packed_bytes_of), so their chunks hold 8 values.
+ *
+ *  u8 has no unsigned MFMA. B is stored as b' = b ^ 0x80 (signed b - 128), A is turned into
+ *  a' = a ^ 0x80 on its way into LDS, and  sum(a*b) = sum(a'*b') + 128*sum(a) + 128*sum(b')  (mod 2^32)
+ *  with zero padding contributing nothing. 128*sum(b') per column is stored behind the tiles at pack
+ *  time; sum(a) per row is accumulated with v_sad_u8 while A is staged.
+ */#ifndef NUMKONG_AMD_DOTS_GFX950_HPP
+#define NUMKONG_AMD_DOTS_GFX950_HPP
+
+#include <hip/hip_runtime.h>
+
+#include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "numkong_amd/hip_abi.h"
+
+/** What crosses translation units: the product's arguments, its scratch memory, one launcher per element type. */
+namespace nk_gfx950 {
+
+constexpr uint32_t kTileBand = 8; // tile rows per band of the walk over the tile grid
+
+struct GemmArgs {
+    uint8_t const *a;
+    uint8_t const *bp; // packed image (header first)
+    uint8_t *c;
+    uint64_t a_stride, c_stride, k_src_bytes;
+    uint32_t m, n, k;
+    uint32_t n_tiles, k_chunks;
+    uint32_t tiles_m, tiles_n;
+    int avec; // widest load the A pointer and stride allow (1, 2, 4, 8 or 16 bytes)
+    int metric; // 0: dot products, 1: angular distances, 2: euclidean distances (kernels built with NORMS)
+    uint32_t chunk_stages; // chunked types: stages between folds of the accumulator (even, 2..16)
+    // Symmetric products (C = A x A^T, upper triangle): only elements with col >= row + tri_shift are stored
+    // (`tri_mask` all ones; 0 switches the test off), and the tiles to compute come as a list.
+    uint32_t tri_shift, tri_mask;
+    uint32_t tile_count;       // tiles_m * tiles_n, or the length of the list
+    uint32_t const *tile_list; // (tile row, tile column) pairs in walking order, or NULL for the full grid
+};
+
+/** Scratch memory of a triangular grid: the first tile of every band, then the list itself. */
+struct TriangleScratch {
+    uint32_t *words;
+    size_t bytes;
+};
+
+/** The product (or its triangular form) for one element type: picks the tile shape and launches. Defined in
+ *  dots_gfx950_<T>.hip. */
+hipError_t launch_i8(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_u8(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_bf16(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_f16(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_e4m3(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_e5m2(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+
+extern int g_forced_config; // 0: the heuristic picks the tile shape; see nk_hip_set_tile_config
+extern int g_variant;       // timing experiments of tuning builds
+extern int g_cu_count;      // compute units of the device, asked once
+
+} // namespace nk_gfx950
+
+namespace {
+
+using namespace nk_gfx950;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef long v2l __attribute__((ext_vector_type(2)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+// nk_dtype_t codes (reference: include/numkong/types.h:923-952)
+enum : int {
+    kI8 = 1 << 2,
+    kU8 = 1 << 6,
+    kF16 = 1 << 12,
+    kBF16 = 1 << 13,
+    kE4M3 = 1 << 14,
+    kE5M2 = 1 << 15,
+};
+
+constexpr uint32_t kMagic = 0x35394B4Eu; // "NK95"
+constexpr uint32_t kVersion = 3;
+constexpr int kChunkBytes = 16;   // bytes of K per lane per operand load
+constexpr int kTileRows = 32;     // B rows per tile = MFMA N
+constexpr int kStageChunks = 8;   // chunks of K per pipeline stage (128 bytes per row)
+constexpr int kStageBytes = kStageChunks * kChunkBytes;
+constexpr int kTileChunkBytes = kTileRows * kChunkBytes; // 512: one chunk of all 32 rows of a tile
+
+struct PackedHeader {
+    uint32_t magic;
+    uint32_t version;
+    uint32_t dtype;
+    uint32_t elem_bytes; // bytes per element as stored in the image (2 for fp8, which is widened to f16)
+    uint32_t n;        // logical rows of B = columns of C
+    uint32_t k;        // logical depth in elements
+    uint32_t n_tiles;  // ceil(n / 32)
+    uint32_t k_chunks; // padded depth in 16-byte chunks, multiple of 8
+    uint64_t data_offset;
+    uint64_t sums_offset; // u32 x (32 * n_tiles): 128 * sum(b') per column for u8, zeros otherwise
+    uint64_t total_bytes;
+    uint64_t norms_offset; // u32 or f32 x (32 * n_tiles): sum(b^2) per column (exact mod 2^32 for the integer types)
+};
+static_assert(sizeof(PackedHeader) == 64, "header must stay 64 bytes");
+
+struct Geometry {
+    uint32_t elem_bytes;   // bytes per element in the caller's A and B
+    uint32_t packed_bytes; // bytes per element in the image and in LDS (fp8 is widened to f16)
+    uint32_t n, k, n_tiles, k_chunks;
+    uint64_t k_bytes;      // bytes of one packed row: k * packed_bytes
+    uint64_t k_src_bytes;  // bytes of one source row: k * elem_bytes
+    uint64_t data_bytes, sums_bytes, norms_bytes, total_bytes;
+};
+
+inline int elem_bytes_of(int dtype) {
+    switch (dtype) {
+    case kI8:
+    case kU8:
+    case kE4M3:
+    case kE5M2: return 1;
+    case kF16:
+    case kBF16: return 2;
+    default: return 0;
+    }
+}
+
+/** The fp8 MFMA forms of gfx950 align the products inside one lane's k-group to the largest of them and
+ *  keep only about 14 bits (1 + 2^-14 comes back as 1), far from the f32 accumulation of the reference's
+ *  kernels (dot/serial.h:522-600). e4m3 and e5m2 are therefore widened, exactly, to f16 and run on the f16
+ *  MFMA, whose products and sums are kept to full f32 precision: B at pack time, A on its way into LDS. */
+inline int packed_bytes_of(int dtype) { return (dtype == kE4M3 || dtype == kE5M2) ? 2 : elem_bytes_of(dtype); }
+
+inline bool make_geometry(int dtype, size_t n, size_t k, Geometry &g) {
+    int const eb = elem_bytes_of(dtype);
+    if (!eb) return false;
+    if (n > 0x7FFFFFFFull || k > 0x3FFFFFFFull) return false;
+    g.elem_bytes = (uint32_t)eb, g.packed_bytes = (uint32_t)packed_bytes_of(dtype), g.n = (uint32_t)n, g.k = (uint32_t)k;
+    g.k_bytes = (uint64_t)k * g.packed_bytes;
+    g.k_src_bytes = (uint64_t)k * eb;
+    uint64_t const chunks = (g.k_bytes + kChunkBytes - 1) / kChunkBytes;
+    g.k_chunks = (uint32_t)((chunks + 2 * kStageChunks - 1) / (2 * kStageChunks) * (2 * kStageChunks)); // an even number of stages
+    g.n_tiles = (uint32_t)((n + kTileRows - 1) / kTileRows);
+    g.data_bytes = (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes;
+    g.sums_bytes = (uint64_t)g.n_tiles * kTileRows * sizeof(uint32_t);
+    g.norms_bytes = g.sums_bytes;
+    g.total_bytes = sizeof(PackedHeader) + g.data_bytes + g.sums_bytes + g.norms_bytes;
+    return true;
+}
+
+
+/**
+ *  Load one 16-byte chunk of which only the first `valid` bytes exist (valid may be <= 0 or >= 16),
+ *  with loads no wider than the pointer's known alignment `avec`. Missing bytes read as zero; `xr`
+ *  (0 or 0x80808080) is applied to existing bytes only, so zero padding stays zero for u8.
+ */
+__device__ __forceinline__ v4i load_chunk_guarded(uint8_t const *p, int valid, int avec, uint32_t xr) {
+    v4i out;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        int const rem = valid - 4 * w;
+        uint32_t x = 0;
+        if (rem >= 4 && avec >= 4) { x = *(uint32_t const *)(p + 4 * w) ^ xr; }
+        else if (rem > 0) {
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                if (b < rem) x |= (uint32_t)(uint8_t)(p[4 * w + b] ^ (uint8_t)xr) << (8 * b);
+        }
+        out[w] = (int)x;
+    }
+    return out;
+}
+
+__device__ __forceinline__ uint32_t sum_bytes_u8(v4i v) {
+    uint32_t s = __builtin_amdgcn_sad_u8((uint32_t)v[0], 0u, 0u);
+    s = __builtin_amdgcn_sad_u8((uint32_t)v[1], 0u, s);
+    s = __builtin_amdgcn_sad_u8((uint32_t)v[2], 0u, s);
+    s = __builtin_amdgcn_sad_u8((uint32_t)v[3], 0u, s);
+    return s;
+}
+
+/** Eight OCP fp8 values (two dwords) -> eight f16 values, exact for every code incl. subnormals, Inf, NaN. */
+template <bool E5M2>
+__device__ __forceinline__ v4i widen_fp8x8(uint32_t lo, uint32_t hi) {
+    typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+    v2h p0, p1, p2, p3;
+    if (E5M2) {
+        p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(lo, 1.0f, false);
+        p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(lo, 1.0f, true);
+        p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(hi, 1.0f, false);
+        p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(hi, 1.0f, true);
+    }
+    else {
+        p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false);
+        p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, true);
+        p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, false);
+        p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, true);
+    }
+    v4i out;
+    out[0] = __builtin_bit_cast(int, p0), out[1] = __builtin_bit_cast(int, p1);
+    out[2] = __builtin_bit_cast(int, p2), out[3] = __builtin_bit_cast(int, p3);
+    return out;
+}
+
+#pragma region Packing
+
+/**
+ *  One thread per 16-byte chunk of the image. A block of 256 threads covers 32 rows x 8 chunks: reads are
+ *  128 (64 for fp8) contiguous bytes per row, writes are eight 512-byte runs. WIDEN: 0 copies the
+ *  elements, 1 widens e4m3 to f16, 2 widens e5m2 to f16 (8 source bytes per chunk).
+ */
+template <int WIDEN>
+__global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
+                                                   uint64_t k_src_bytes, uint32_t k_chunks, uint8_t *__restrict__ data,
+                                                   int avec, uint32_t xr, PackedHeader header) {
+    constexpr int kSrcChunk = WIDEN ? 8 : 16;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *(PackedHeader *)(data - sizeof(PackedHeader)) = header; // (64 bytes in front of the tiles)
+    uint32_t const groups = k_chunks / kStageChunks;
+    uint32_t const tile = blockIdx.x / groups;
+    uint32_t const group = blockIdx.x % groups;
+    uint32_t const r = threadIdx.x >> 3;
+    uint32_t const c = group * kStageChunks + (threadIdx.x & 7);
+    uint64_t const row = (uint64_t)tile * kTileRows + r;
+    int64_t const left = (int64_t)k_src_bytes - (int64_t)c * kSrcChunk;
+    int const valid = row < n ? (int)(left > kSrcChunk ? kSrcChunk : (left < 0 ? 0 : left)) : 0;
+    v4i v = {0, 0, 0, 0};
+    if (valid > 0) {
+        uint8_t const *src = b + row * b_stride + (uint64_t)c * kSrcChunk;
+        if (!WIDEN && valid == 16 && avec >= 16) {
+            v = *(v4i const *)src;
+            v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
+        }
+        else { v = load_chunk_guarded(src, valid, avec, xr); }
+        if (WIDEN) v = widen_fp8x8<WIDEN == 2>((uint32_t)v[0], (uint32_t)v[1]);
+    }
+    *(v4i *)(data + (((uint64_t)tile * k_chunks + c) * kTileRows + r) * kChunkBytes) = v;
+}
+
+/** Sum of the squares of the 8 values of a 16-byte chunk of bf16 (f32 = bits << 16) or f16, in f64. */
+template <bool BF16_VALUES>
+__device__ __forceinline__ double chunk_sumsq_f64(v4i v) {
+    double sum = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        float lo, hi;
+        if (BF16_VALUES) {
+            lo = __builtin_bit_cast(float, (uint32_t)v[w] << 16), hi = __builtin_bit_cast(float, (uint32_t)v[w] & 0xFFFF0000u);
+        }
+        else {
+            typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+            int const word = v[w]; // a named copy: bit-casting the vector element expression itself reads element 0
+            v2h const pair = __builtin_bit_cast(v2h, word);
+            lo = (float)pair[0], hi = (float)pair[1];
+        }
+        sum = __builtin_fma((double)lo, (double)lo, sum);
+        sum = __builtin_fma((double)hi, (double)hi, sum);
+    }
+    return sum;
+}
+
+/**
+ *  Per-column terms, from the packed tiles: the u8 compensation term (128 * sum of the signed packed bytes of
+ *  the row, mod 2^32; zero for the other types) and the column's sum of squares, which the angular and
+ *  euclidean products need (reference: the norms behind the packed rows, dots/serial.h:326-332): exact mod
+ *  2^32 for the integer types, accumulated in f64 and rounded once to f32 for the float types.
+ *  Four wavefronts per tile: lane l of wavefront w owns row l % 32 and every eighth chunk starting at 2 w + l / 32.
+ *  KIND: 0 i8, 1 u8, 2 bf16, 3 f16 (and fp8, stored widened to f16).
+ */
+template <int KIND>
+__global__ __launch_bounds__(256) void column_terms_kernel(uint8_t const *__restrict__ data, uint32_t k_chunks, uint32_t k,
+                                                           uint32_t *__restrict__ sums, uint32_t *__restrict__ norms) {
+    __shared__ int part_sum[8][32];
+    __shared__ uint32_t part_squares[8][32];
+    __shared__ double part_f64[8][32];
+    uint32_t const tile = blockIdx.x;
+    uint32_t const first = threadIdx.x >> 5, row = threadIdx.x & 31; // chunk residue mod 8, row of the tile
+    uint8_t const *base = data + (uint64_t)tile * k_chunks * kTileChunkBytes + row * kChunkBytes;
+    int sum = 0;
+    uint32_t squares = 0;
+    double squares_f64 = 0;
+    for (uint32_t c = first; c < k_chunks; c += 8) {
+        v4i const v = *(v4i const *)(base + (uint64_t)c * kTileChunkBytes);
+        if (KIND == 0) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) squares = (uint32_t)__builtin_amdgcn_sdot4(v[w], v[w], (int)squares, false);
+        }
+        else if (KIND == 1) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                sum = __builtin_amdgcn_sdot4(v[w], 0x01010101, sum, false);
+                squares = (uint32_t)__builtin_amdgcn_sdot4(v[w], v[w], (int)squares, false);
+            }
+        }
+        else { squares_f64 += chunk_sumsq_f64<KIND == 2>(v); }
+    }
+    part_sum[first][row] = sum, part_squares[first][row] = squares, part_f64[first][row] = squares_f64;
+    __syncthreads();
+    if (threadIdx.x < 32) {
+        sum = 0, squares = 0, squares_f64 = 0;
+#pragma unroll
+        for (int part = 0; part < 8; ++part) sum += part_sum[part][row], squares += part_squares[part][row], squares_f64 += part_f64[part][row];
+        // u8 is stored as b - 128 (and its padding as 0): sum(b^2) = sum((b - 128)^2) + 256 * sum(b - 128) + 128^2 * k
+        if (KIND == 1) squares += 256u * (uint32_t)sum + 16384u * k;
+        sums[(uint64_t)tile * kTileRows + row] = (uint32_t)sum * 128u;
+        norms[(uint64_t)tile * kTileRows + row] = KIND < 2 ? squares : __builtin_bit_cast(uint32_t, (float)squares_f64);
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t *p, uint64_t count, uint32_t value) {
+    uint64_t const i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) p[i] = value;
+}
+
+__global__ __launch_bounds__(64) void write_header_kernel(PackedHeader *dst, PackedHeader h) {
+    if (threadIdx.x == 0) *dst = h;
+}
+
+/** `tri_mask` all ones: only the elements with col >= row + tri_shift (on or right of a diagonal); 0: all of them. */
+__global__ __launch_bounds__(256) void fill_rows_kernel(uint8_t *c, uint32_t m, uint32_t n, uint64_t c_stride,
+                                                        uint32_t value, uint32_t tri_shift, uint32_t tri_mask) {
+    uint64_t const i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    uint64_t const row = i / n, col = i % n;
+    if (row < m && (((uint32_t)row + tri_shift) & tri_mask) <= (uint32_t)col) *(uint32_t *)(c + row * c_stride + col * 4) = value;
+}
+
+#pragma endregion Packing
+
+#pragma region Element types
+
+/**
+ *  Float accumulation. One MFMA accumulator rounds once per 8 products at the magnitude of the whole running
+ *  sum; over a depth of thousands that is 1.4x the error of the reference's scalar kernel for bf16 (4 lanes,
+ *  dot/serial.h:406-439), 3x that of its 16-lane AVX-512 kernels (dot/genoa.h:237-256), and 4x the scalar
+ *  kernel's for fp8, whose products and short sums are exact in f32 (dot/serial.h:522-600). The float types
+ *  therefore fold the accumulator into a second one every `chunk_stages` stages (about an eighth of the depth,
+ *  at most 16 stages = 1024 values): the running sums stay short, and the error drops to that of the reference's
+ *  best kernels (measured ratios next to the tests). Two accumulator sets do not fit the 256 x 256 tile, so
+ *  these types stop at 128 x 256. NK_HALF_SINGLE_ACCUMULATOR builds bf16/f16 without the second set (faster,
+ *  less accurate; for comparison only).
+ */
+#ifdef NK_HALF_SINGLE_ACCUMULATOR
+constexpr bool kHalfChunked = false;
+#else
+constexpr bool kHalfChunked = true;
+#endif
+
+struct I8 {
+    static constexpr bool kChunked = false; // fold the accumulator into a second one every few stages
+    static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
+    static __device__ __forceinline__ v4i widen(v4i v) { return v; }
+    typedef v16i acc_t;
+    typedef uint32_t norm_t; // what a row's sum of squares accumulates in
+    static constexpr int kDtype = kI8;
+    static constexpr bool kUnsigned = false;
+    /** Sum of the squares of the source values behind one staged chunk (`raw`: as loaded, `wide`: as it goes to LDS). */
+    static __device__ __forceinline__ norm_t sumsq(v4i raw, v4i) {
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum = __builtin_amdgcn_sdot4(raw[w], raw[w], sum, false);
+        return (uint32_t)sum;
+    }
+    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
+    }
+};
+struct U8 : I8 {
+    static constexpr int kDtype = kU8;
+    static constexpr bool kUnsigned = true;
+    static __device__ __forceinline__ norm_t sumsq(v4i raw, v4i) {
+        uint32_t sum = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum = __builtin_amdgcn_udot4((uint32_t)raw[w], (uint32_t)raw[w], sum, false);
+        return sum;
+    }
+};
+struct BF16 {
+    static constexpr bool kChunked = kHalfChunked;
+    static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
+    static __device__ __forceinline__ v4i widen(v4i v) { return v; }
+    typedef v16f acc_t;
+    typedef double norm_t;
+    static constexpr int kDtype = kBF16;
+    static constexpr bool kUnsigned = false;
+    /** The 8 products are exact in f32; their short sum is rounded a few times, the long sum runs in f64. */
+    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) {
+        float sum = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            float const lo = __builtin_bit_cast(float, (uint32_t)wide[w] << 16);
+            float const hi = __builtin_bit_cast(float, (uint32_t)wide[w] & 0xFFFF0000u);
+            sum = __builtin_fmaf(lo, lo, sum), sum = __builtin_fmaf(hi, hi, sum);
+        }
+        return (double)sum;
+    }
+    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), acc, 0,
+                                                      0, 0);
+    }
+};
+struct F16 {
+    static constexpr bool kChunked = kHalfChunked;
+    static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
+    static __device__ __forceinline__ v4i widen(v4i v) { return v; }
+    typedef v16f acc_t;
+    typedef double norm_t;
+    static constexpr int kDtype = kF16;
+    static constexpr bool kUnsigned = false;
+    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { // also e4m3 / e5m2, which are f16 by then
+        typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+        float sum = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) { // (mixed-precision fused multiply-adds; the packed f16 dot instruction rounds too early)
+            int const word = wide[w]; // a named copy: bit-casting the vector element expression itself reads element 0
+            v2h const pair = __builtin_bit_cast(v2h, word);
+            float const lo = (float)pair[0], hi = (float)pair[1];
+            sum = __builtin_fmaf(lo, lo, sum), sum = __builtin_fmaf(hi, hi, sum);
+        }
+        return (double)sum;
+    }
+    static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), acc, 0, 0,
+                                                     0);
+    }
+};
+/** fp8 runs widened to f16 (exact), on the f16 MFMA; see widen_fp8x8. */
+struct E4M3 : F16 {
+    static constexpr bool kChunked = true;
+    static constexpr int kDtype = kE4M3;
+    static constexpr int kSrcChunk = 8;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<false>((uint32_t)v[0], (uint32_t)v[1]); }
+};
+struct E5M2 : F16 {
+    static constexpr bool kChunked = true;
+    static constexpr int kDtype = kE5M2;
+    static constexpr int kSrcChunk = 8;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<true>((uint32_t)v[0], (uint32_t)v[1]); }
+};
+
+/**
+ *  Distances from a dot product and two sums of squares, as the reference's scalar finalisers compute them
+ *  (spatial/serial.h:257-344): integer inputs are converted to f32 first (the i8 kernels read both norms as
+ *  signed 32-bit integers, the u8 kernels as unsigned); angular = max(1 - dot * rsqrt(qn * tn), 0), and 0 or
+ *  1 when the product of the norms is not positive; euclidean = sqrt(max(qn + tn - 2 * dot, 0)).
+ */
+template <class T>
+__device__ __forceinline__ float norm_as_f32(uint32_t bits) {
+    if (T::kDtype == kI8) return (float)(int)bits;
+    if (T::kDtype == kU8) return (float)bits;
+    return __builtin_bit_cast(float, bits);
+}
+
+/** METRIC: 1 angular, 2 euclidean. `query` and `target` are the row's and the column's sums of squares as f32
+ *  (converted once per row and once per column of a tile). The reciprocal square root is the hardware's estimate
+ *  (1 ulp) refined by one Newton step with fused residuals: identical rows must cancel to within a rounding or
+ *  two, as the reference's three Newton steps do (splitting it into a factor per row and a factor per column
+ *  would save half of the operations and lose exactly that). */
+template <class T, int METRIC>
+__device__ __forceinline__ uint32_t distance_from_dot(uint32_t dot_bits, float query, float target) {
+    float const dot = T::kDtype == kI8 ? (float)(int)dot_bits : (T::kDtype == kU8 ? (float)dot_bits : __builtin_bit_cast(float, dot_bits));
+    float result;
+    if (METRIC == 1) {
+        float const product = query * target;
+        float root = __builtin_amdgcn_rsqf(product);
+        float const residual = __builtin_fmaf(-(product * root), root, 1.0f);
+        root = __builtin_fmaf(root * 0.5f, residual, root);
+        float const unclipped = __builtin_fmaxf(__builtin_fmaf(-dot, root, 1.0f), 0.0f);
+        result = product > 0 ? unclipped : (dot == 0 ? 0.0f : 1.0f);
+    }
+    else {
+        // The hardware's reciprocal square root is good to about one unit in the last place; one Newton step on
+        // the root itself (residual by a fused multiply-add) leaves it correctly rounded but for rare ties, as
+        // the square roots of the reference's vector kernels are.
+        float const squared = __builtin_fmaf(-2.0f, dot, query + target);
+        float const inverse = __builtin_amdgcn_rsqf(squared);
+        float root = squared * inverse;
+        root = __builtin_fmaf(__builtin_fmaf(-root, root, squared), 0.5f * inverse, root);
+        result = squared > 0 ? root : 0.0f;
+    }
+    return __builtin_bit_cast(uint32_t, result);
+}
+
+#pragma endregion Element types
+
+#pragma region Packed product
+
+#ifdef NK_TUNE
+__device__ unsigned long long g_debug_clocks[8];
+#endif
+
+template <int V>
+struct slot_c {
+    static constexpr int value = V;
+};
+
+/** Second-level accumulators: real for the chunked types, empty (no registers) for the others. */
+template <class acc_t, int TM, int TN, bool kChunked>
+struct Totals {
+    acc_t value[TM][TN];
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) value[i][j][v] = 0;
+    }
+    __device__ __forceinline__ void fold(acc_t (&acc)[TM][TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                value[i][j] += acc[i][j];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+            }
+    }
+    __device__ __forceinline__ auto finish(acc_t const (&acc)[TM][TN], int i, int j, int v) const {
+        return acc[i][j][v] + value[i][j][v];
+    }
+};
+template <class acc_t, int TM, int TN>
+struct Totals<acc_t, TM, TN, false> {
+    __device__ __forceinline__ void clear() {}
+    __device__ __forceinline__ void fold(acc_t (&)[TM][TN]) {}
+    __device__ __forceinline__ auto finish(acc_t const (&acc)[TM][TN], int i, int j, int v) const { return acc[i][j][v]; }
+};
+
+
+/**
+ *  Workgroup index -> output tile. Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each
+ *  with a private L2, so ids are first regrouped into 8 contiguous ranges (one per XCD) and each range
+ *  walks the tile grid in column-major bands of 8 tile rows: tiles resident on one XCD at the same time
+ *  share A row blocks and B column tiles in that XCD's L2.
+ */
+__device__ __forceinline__ void tile_of_block(uint32_t pid, GemmArgs const &g, uint32_t &tm, uint32_t &tn) {
+    uint32_t const tiles_m = g.tiles_m, tiles_n = g.tiles_n;
+    uint32_t const total = g.tile_count;
+    uint32_t const per_xcd = total / 8;
+    uint32_t lid = pid;
+    if (pid < per_xcd * 8) lid = (pid % 8) * per_xcd + pid / 8;
+    if (g.tile_list) { // a triangular grid: the same walk with the tiles left of the diagonal left out, listed
+        typedef __attribute__((address_space(4))) uint32_t const constant_u32_t;
+        constant_u32_t *entry = (constant_u32_t *)g.tile_list + 2 * (uint64_t)lid;
+        tm = entry[0], tn = entry[1];
+        return;
+    }
+    constexpr uint32_t kBand = kTileBand;
+    uint32_t const width = kBand * tiles_n;
+    uint32_t const band = lid / width;
+    uint32_t const first = band * kBand;
+    uint32_t const rows = tiles_m - first < kBand ? tiles_m - first : kBand;
+    uint32_t const in_band = lid % width;
+    tm = first + in_band % rows;
+    tn = in_band / rows;
+}
+
+/** First tile column of tile row `t` that holds an element on or right of the diagonal col = row + shift; tiles
+ *  are 2^bm_log2 rows by 2^bn_log2 columns. */
+__host__ __device__ inline uint32_t first_live_tile(uint32_t t, uint32_t bm_log2, uint32_t bn_log2, uint32_t shift) {
+    return ((t << bm_log2) + shift) >> bn_log2;
+}
+
+/**
+ *  The tile list of a triangular grid, in the order of `tile_of_block`: bands of kTileBand tile rows, column
+ *  by column within a band, top to bottom within a column, and only tiles with something on or right of the
+ *  diagonal. One workgroup per list: the bands' sizes are scanned 256 at a time, then every band is filled by all
+ *  threads, a column each. A band's first columns form a staircase (row t joins at column first_live_tile(t)); the cells
+ *  left of column c number the sum over its rows of max(0, c - first_live_tile(t)).
+ */
+struct TriangleGrid {
+    uint32_t tiles_m, tiles_n, bm_log2, bn_log2, shift;
+    uint32_t *band_start, *list;
+};
+struct TriangleGrids {
+    TriangleGrid grid[2];
+};
+__global__ __launch_bounds__(256) void triangle_tiles_kernel(TriangleGrids grids) {
+    TriangleGrid const &mine = grids.grid[blockIdx.x]; // one workgroup per list
+    uint32_t const tiles_m = mine.tiles_m, tiles_n = mine.tiles_n, bm_log2 = mine.bm_log2, bn_log2 = mine.bn_log2,
+                   shift = mine.shift;
+    uint32_t *band_start = mine.band_start, *list = mine.list;
+    __shared__ uint32_t scan[256];
+    __shared__ uint32_t base;
+    uint32_t const tid = threadIdx.x;
+    uint32_t const bands = (tiles_m + kTileBand - 1) / kTileBand;
+    if (tid == 0) base = 0, band_start[0] = 0;
+    __syncthreads();
+    for (uint32_t chunk = 0; chunk < bands; chunk += 256) {
+        uint32_t const band = chunk + tid;
+        uint32_t count = 0;
+        if (band < bands) {
+            uint32_t const first = band * kTileBand, last = first + kTileBand < tiles_m ? first + kTileBand : tiles_m;
+            for (uint32_t t = first; t < last; ++t) {
+                uint32_t const from = first_live_tile(t, bm_log2, bn_log2, shift);
+                count += from < tiles_n ? tiles_n - from : 0;
+            }
+        }
+        scan[tid] = count;
+        __syncthreads();
+        for (uint32_t step = 1; step < 256; step *= 2) {
+            uint32_t const below = tid >= step ? scan[tid - step] : 0;
+            __syncthreads();
+            scan[tid] += below;
+            __syncthreads();
+        }
+        if (band < bands) band_start[band + 1] = base + scan[tid];
+        __syncthreads();
+        if (tid == 255) base += scan[255];
+        __syncthreads();
+    }
+    for (uint32_t band = 0; band < bands; ++band) {
+        uint32_t const first = band * kTileBand, last = first + kTileBand < tiles_m ? first + kTileBand : tiles_m;
+        uint32_t joins[kTileBand]; // where each row of the band joins (past the grid for rows that do not exist)
+#pragma unroll
+        for (uint32_t i = 0; i < kTileBand; ++i) joins[i] = first + i < last ? first_live_tile(first + i, bm_log2, bn_log2, shift) : 0xFFFFFFFFu;
+        uint32_t const start = band_start[band];
+        for (uint32_t column = joins[0] + tid; column < tiles_n; column += 256) {
+            uint32_t at = start;
+#pragma unroll
+            for (uint32_t i = 0; i < kTileBand; ++i) at += column > joins[i] ? column - joins[i] : 0;
+#pragma unroll
+            for (uint32_t i = 0; i < kTileBand; ++i)
+                if (joins[i] <= column) list[2 * (uint64_t)at] = first + i, list[2 * (uint64_t)at + 1] = column, ++at;
+        }
+    }
+}
+
+/**
+ *  A persistent workgroup of 4 wavefronts (one per SIMD) walks over (32*TM) x (128*TN) tiles of C. Every
+ *  wavefront owns all 32*TM rows of the tile and its own 32*TN columns: B fragments are loaded by exactly
+ *  one wavefront, straight from the packed image into registers; the shared A block goes through LDS.
+ *  Being persistent lets the stores of one tile drain while the next tile is already being computed.
+ *
+ *  A stage is 128 bytes of (packed-width) K per row = four MFMA k-steps. LDS holds two stages of A, rows
+ *  128 bytes apart, the 16-byte chunk `c` of row `r` stored at chunk position c ^ ((r >> 1) & 7): the 16
+ *  rows that one pass of a ds_read_b128 touches then fall into 16 different 16-byte bank groups (measured:
+ *  SQ_LDS_BANK_CONFLICT = 0).
+ *
+ *  The steady-state loop handles two stages per trip so that every register slot and LDS buffer has a
+ *  compile-time index, and its body is one basic block (no branches: prefetch indices are clamped instead),
+ *  which keeps the compiler's s_waitcnt counting exact. Everything is fetched two stages ahead:
+ *      k-step q MFMAs of (s, q) under the LDS reads of the A fragments of (s, q+1); then the B registers
+ *               just consumed are refilled with B(s+2, q)
+ *      k-step 2 also moves A(s+1), loaded two stages ago, from registers into the other LDS buffer and
+ *               refills those registers with A(s+3)
+ *      before the last k-step: one barrier; the first fragments of stage s+1 are read under its MFMAs
+ *  The packed image pads K with zeros to an even number of stages; on the A side, the bytes a stage reads
+ *  past the end of a row (the next row's, or nothing past the end of the matrix) are masked to zero on their
+ *  way into LDS, so ragged depths run through the same loop. Only A that is not even dword-aligned takes a
+ *  plain guarded loop instead.
+ *
+ *  A is the MFMA's first operand, so a lane ends up with one column and 16 rows of each 32x32 block and the
+ *  epilogue stores dwords that are contiguous across lanes: 128 bytes per row per instruction, any C
+ *  alignment. (The other orientation, one row and runs of 4 columns per lane stored as 128-bit vectors,
+ *  needs a quarter of the store instructions but writes 32-byte pieces of 32 different rows; it measured
+ *  12 % slower on the square shapes and 9 % slower on the retrieval shape.)
+ */
+template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, int DBG = 0>
+__global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChunked ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
+    typedef typename T::acc_t acc_t;
+    constexpr int BM = TM * 32;
+    constexpr int NT = 256;
+    constexpr int kStageLds = BM * kStageBytes;
+    constexpr int kLoads = BM * kStageChunks / NT; // 16-byte LDS chunks per thread per stage = TM
+    constexpr int kSrcStage = kStageChunks * T::kSrcChunk; // source bytes of A per row per stage
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStageLds];
+    __shared__ __attribute__((aligned(16))) uint32_t row_terms[T::kUnsigned ? BM : 4]; // u8 only: 128 * (sum of the bytes of each A row of the tile)
+    __shared__ uint32_t row_part[T::kUnsigned ? 2 * BM * kStageChunks : 1]; // u8 only: the partial sums behind them
+    typedef typename T::norm_t norm_t;
+    __shared__ __attribute__((aligned(16))) uint32_t row_norms[NORMS ? BM : 4]; // distances only: sum of squares of each A row
+    __shared__ norm_t norm_part[NORMS ? 2 * BM * kStageChunks : 1];              // ... and the partial sums behind them
+
+    uint32_t const tid = threadIdx.x, lane = tid & 63;
+    // The wavefront index is the same in all lanes; telling the compiler keeps B addressing in scalar registers.
+    uint32_t const wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // Trust, but verify: the image must have been packed for this dtype and these dimensions.
+    PackedHeader const *header = (PackedHeader const *)g.bp;
+    bool const image_ok = header->magic == kMagic && header->version == kVersion &&
+                          header->dtype == (uint32_t)T::kDtype && header->n == g.n && header->k == g.k &&
+                          header->k_chunks == g.k_chunks && header->n_tiles == g.n_tiles;
+    uint8_t const *data = g.bp + sizeof(PackedHeader);
+    uint32_t const *col_terms = (uint32_t const *)(data + (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes);
+    uint32_t const *col_norms = col_terms + (uint64_t)g.n_tiles * kTileRows;
+
+    uint32_t const stages = g.k_chunks / kStageChunks;
+    // Stages the pipelined loop takes: all of them when A is at least dword-aligned, which is all that
+    // multi-dword global loads need. (readfirstlane: the value is uniform, and it must stay in a scalar register
+    // because the stage offsets of the buffer loads derive from it.)
+    uint32_t const fast = __builtin_amdgcn_readfirstlane(g.avec >= 4 ? stages : 0);
+    uint32_t const xr = T::kUnsigned ? 0x80808080u : 0u;
+    uint32_t const a_pos = tid & 7;
+    // A fragment reads: lane l takes row l % 32 of each 32-row block and chunk 2q + l / 32.
+    uint32_t a_frag[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        uint32_t const r = lane & 31, c = 2 * q + (lane >> 5);
+        a_frag[q] = r * kStageBytes + ((c ^ ((r >> 1) & 7)) << 4);
+    }
+
+    // A staging: thread t fetches chunk t % 8 of rows i*32 + t/8 of a tile and stores it at its swizzled
+    // position. The offsets are the same for every tile: rows past the end of A are cut off by the size of
+    // the tile's buffer descriptor (such loads return zeros, and their outputs are never stored).
+    uint32_t a_off[kLoads]; // byte offset of the thread's source chunk from the tile's first row
+    uint32_t a_lds[kLoads]; // where it goes in an LDS stage
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+        uint32_t const r = i * 32 + (tid >> 3);
+        a_off[i] = r * (uint32_t)g.a_stride + a_pos * T::kSrcChunk;
+        a_lds[i] = r * kStageBytes + ((a_pos ^ ((r >> 1) & 7)) << 4);
+    }
+    uint32_t const b_lane = lane * kChunkBytes;
+
+    // Loads go through buffer descriptors: one scalar descriptor plus a 32-bit per-lane offset is the cheapest
+    // address form to issue (a single address register per lane, no 64-bit vector adds), and a descriptor is
+    // all that has to change from one tile to the next. B fragment streams of this wavefront: one descriptor
+    // per 32-column tile (tile index clamped to the last one), every lane at offset lane * 16.
+    struct TileView {
+        uint32_t row0, col0;
+        uint8_t const *a; // first row of the tile
+        uint32_t a_bytes; // up to the end of its last row that exists
+        uint8_t const *b; // first 32-column tile of this wavefront
+        uint32_t b_bytes; // up to the end of the packed tiles (or as far as 32 bits reach)
+        uint32_t b_tile[TN]; // offsets of the wavefront's tiles from `b`
+    };
+    auto view_of = [&](uint32_t tile) {
+        TileView view;
+        uint32_t tile_m, tile_n;
+        tile_of_block(tile, g, tile_m, tile_n);
+        view.row0 = tile_m * BM;
+        view.col0 = tile_n * (128 * TN) + wave * (32 * TN);
+        uint32_t const rows_here = g.m - view.row0 < (uint32_t)BM ? g.m - view.row0 : (uint32_t)BM;
+        view.a = g.a + (uint64_t)view.row0 * g.a_stride;
+        // (whole dwords: a dword-aligned A never ends in the middle of one that could fault)
+        view.a_bytes = (rows_here - 1) * (uint32_t)g.a_stride + (((uint32_t)g.k_src_bytes + 3u) & ~3u);
+        uint32_t const tile_bytes = g.k_chunks * kTileChunkBytes;
+        uint32_t const first = view.col0 / 32 < g.n_tiles ? view.col0 / 32 : g.n_tiles - 1;
+        view.b = data + (uint64_t)first * tile_bytes;
+        uint64_t const left = (uint64_t)(g.n_tiles - first) * tile_bytes;
+        view.b_bytes = left < 0xFFFFFFFFull ? (uint32_t)left : 0xFFFFFFFFu;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) view.b_tile[j] = (first + j < g.n_tiles ? j : g.n_tiles - 1 - first) * tile_bytes;
+        return view;
+    };
+    auto a_rsrc_of = [](TileView const &view) {
+        return __builtin_amdgcn_make_buffer_rsrc((void *)view.a, 0, (int)view.a_bytes, 0x00020000);
+    };
+    auto b_rsrc_of = [](TileView const &view) {
+        return __builtin_amdgcn_make_buffer_rsrc((void *)view.b, 0, (int)view.b_bytes, 0x00020000);
+    };
+
+    // When every stage of a tile goes through the pipelined loop, the prefetches of a tile's last stages
+    // fetch the first stages of the workgroup's next tile instead of running dry: the pipeline is primed once
+    // and then runs across tile boundaries, and the stores of one tile drain under the next tile's MFMAs.
+    constexpr bool across = ACROSS; // the host checks that it holds: fast == stages and stages >= 4
+    uint32_t const tile_count = g.tile_count;
+    // u8 only: every thread sums the unsigned bytes it stages, per staged row, in LDS slots of its own (slot
+    // i * 256 + tid: fire-and-forget LDS adds instead of 2 x kLoads registers held through the loop). Two sets:
+    // what is staged ahead for the next tile goes to the other one, and the sets swap roles with every tile.
+    uint32_t sums_here = 0; // offset of the set of the tile being computed
+    if (T::kUnsigned) {
+#pragma unroll
+        for (int i = 0; i < 2 * kLoads; ++i) row_part[i * NT + tid] = 0;
+    }
+    auto add_row_sum = [&](int i, uint32_t value, uint32_t set) {
+        __hip_atomic_fetch_add(&row_part[set + i * NT + tid], value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    // Distances: the same bookkeeping for the sums of squares of the rows (u32, or f64 for the float types).
+    if (NORMS) {
+#pragma unroll
+        for (int i = 0; i < 2 * kLoads; ++i) norm_part[i * NT + tid] = 0;
+    }
+    auto add_row_norm = [&](int i, norm_t value, uint32_t set) {
+        __hip_atomic_fetch_add(&norm_part[set + i * NT + tid], value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    v4i a_reg[2][kLoads];
+    v4i b_reg[2][TN][4];
+    v4i af[2][TM];
+
+    typedef __attribute__((address_space(1))) uint8_t global_u8_t;
+    typedef __attribute__((address_space(1))) uint32_t global_u32_t;
+    if (!image_ok) { // the image was not packed for this call: the reference's error convention, all bits set
+        for (uint32_t tile = blockIdx.x; tile < g.tile_count; tile += gridDim.x) {
+            uint32_t tile_m, tile_n;
+            tile_of_block(tile, g, tile_m, tile_n);
+            for (uint32_t at = tid; at < (uint32_t)BM * 128 * TN; at += NT) {
+                uint32_t const row = tile_m * BM + at / (128 * TN), col = tile_n * (128 * TN) + at % (128 * TN);
+                if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col) *(global_u32_t *)((global_u8_t *)g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 4) = 0xFFFFFFFFu;
+            }
+        }
+        return;
+    }
+    TileView cur, nxt;
+    acc_t acc[TM][TN];
+    constexpr bool kChunked = T::kChunked;
+    Totals<acc_t, TM, TN, kChunked> total; // second-level accumulators of the chunked types (see E4M3)
+
+    // A(s) -> registers, in four parts so that the loads can be spread over four k-steps.
+    auto load_a = [&](TileView const &view, uint32_t s, auto slot_tag, auto part_tag) {
+        constexpr int slot = decltype(slot_tag)::value, part = decltype(part_tag)::value;
+        __amdgpu_buffer_rsrc_t const rsrc = a_rsrc_of(view);
+        uint32_t const stage_offset = s * kSrcStage;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            if (i * 4 / kLoads != part) continue;
+            v4i v = {0, 0, 0, 0};
+            if (T::kSrcChunk == 16) {
+                v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, a_off[i], stage_offset, 0));
+            }
+            else {
+                typedef unsigned v2u __attribute__((ext_vector_type(2)));
+                v2u const narrow = __builtin_amdgcn_raw_buffer_load_b64(rsrc, a_off[i], stage_offset, 0);
+                v[0] = (int)narrow[0], v[1] = (int)narrow[1];
+            }
+            a_reg[slot][i] = v;
+        }
+    };
+    auto load_a_all = [&](TileView const &view, uint32_t s, auto slot_tag) {
+        load_a(view, s, slot_tag, slot_c<0>()), load_a(view, s, slot_tag, slot_c<1>());
+        load_a(view, s, slot_tag, slot_c<2>()), load_a(view, s, slot_tag, slot_c<3>());
+    };
+    // Element-wise work on the staged chunks happens here, after the loads have had time to land.
+    // `mine` is 1 for a stage of this tile and 0 for one staged ahead for the next tile.
+    // `s` is the stage the registers hold: the bytes of its chunk that lie past the end of the row are cleared
+    // (for whole stages the masks come out as all ones; no branch either way).
+    int const a_tail = (int)(uint32_t)g.k_src_bytes - (int)(a_pos * T::kSrcChunk); // bytes of the row from this thread's chunk on, stage 0
+    auto store_a = [&](auto buffer_tag, auto slot_tag, uint32_t s, uint32_t mine) {
+        constexpr int buffer = decltype(buffer_tag)::value, slot = decltype(slot_tag)::value;
+        uint8_t *dst = lds + buffer * kStageLds;
+        int const left = a_tail - (int)(s * kSrcStage);
+        uint32_t keep[T::kSrcChunk / 4];
+#pragma unroll
+        for (int w = 0; w < T::kSrcChunk / 4; ++w) {
+            int const over = left - 4 * w, bytes = over < 0 ? 0 : (over > 4 ? 4 : over);
+            keep[w] = bytes == 4 ? 0xFFFFFFFFu : ((1u << (8 * bytes)) - 1u);
+        }
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            v4i v = a_reg[slot][i];
+#pragma unroll
+            for (int w = 0; w < T::kSrcChunk / 4; ++w) v[w] &= (int)keep[w];
+            // (without a next tile to stage for, what is staged past the end is dropped)
+            uint32_t const set = across && !mine ? sums_here ^ (uint32_t)(kLoads * NT) : sums_here;
+            v4i const raw = v;
+            if (T::kUnsigned) {
+                uint32_t const sum = sum_bytes_u8(v);
+                add_row_sum(i, across ? sum : sum * mine, set);
+                v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
+            }
+            v4i const wide = T::widen(v);
+            if (NORMS) {
+                norm_t const squares = T::sumsq(raw, wide);
+                add_row_norm(i, across || mine ? squares : (norm_t)0, set);
+            }
+            *(v4i *)(dst + a_lds[i]) = wide;
+        }
+    };
+    auto load_b = [&](TileView const &view, uint32_t s, auto slot_tag, auto q_tag) {
+        constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
+        __amdgpu_buffer_rsrc_t const rsrc = b_rsrc_of(view);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            b_reg[slot][j][q] = __builtin_bit_cast(
+                v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_lane + q * 2 * kTileChunkBytes,
+                                                           view.b_tile[j] + s * (kStageChunks * kTileChunkBytes), 0));
+    };
+    auto read_frags = [&](auto buffer_tag, auto q_tag, auto parity_tag) {
+        constexpr int buffer = decltype(buffer_tag)::value, q = decltype(q_tag)::value,
+                      parity = decltype(parity_tag)::value;
+        uint8_t const *src = lds + buffer * kStageLds + a_frag[q];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[parity][i] = *(v4i const *)(src + i * 32 * kStageBytes);
+    };
+    auto multiply = [&](auto slot_tag, auto q_tag) {
+        constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[q & 1][i], b_reg[slot][j][q]);
+    };
+    // Scheduling hints for one k-step. Masks: 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write.
+    // Fragment reads go one-to-one with the first TM MFMAs; the global loads of the k-step (TN of B
+    // and a quarter of A) are spread over the remaining MFMAs; k-step 2 also carries the LDS writes.
+    auto schedule_k_step = [&](auto writes_tag) {
+        constexpr bool writes = decltype(writes_tag)::value != 0;
+        constexpr int loads = TN + (kLoads >= 4 ? kLoads / 4 : 1);
+        constexpr int rest = TM * (TN - 1);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        if constexpr (rest == 0) {
+            if (writes) __builtin_amdgcn_sched_group_barrier(0x200, kLoads, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, loads, 0);
+        }
+        else {
+#pragma unroll
+            for (int i = 0; i < rest; ++i) {
+                if (writes && i < kLoads) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                if (i * loads / rest != (i + 1) * loads / rest || (loads > rest && i == 0))
+                    __builtin_amdgcn_sched_group_barrier(0x020, loads > rest ? loads : 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+            if (writes && kLoads > rest) __builtin_amdgcn_sched_group_barrier(0x200, kLoads - rest, 0);
+        }
+    };
+    // One stage of the steady state; `P` = stage parity = LDS buffer = register slot. Stages s+2 and
+    // s+3 are fetched here; past the tile's end they are the first stages of `nxt` (the next tile, or
+    // this one again when nothing follows: loads of valid memory that nobody uses).
+    auto stage = [&](auto parity_tag, uint32_t s) {
+        constexpr int P = decltype(parity_tag)::value;
+        bool const wrap2 = s + 2 >= fast, wrap3 = s + 3 >= fast;
+        uint32_t const s2 = wrap2 ? s + 2 - fast : s + 2, s3 = wrap3 ? s + 3 - fast : s + 3;
+        TileView const &a2 = wrap2 ? nxt : cur, &a3 = wrap3 ? nxt : cur, &b2 = a2;
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
+        multiply(slot_c<P>(), slot_c<0>());
+        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<0>()), load_a(a2, s2, slot_c<P>(), slot_c<2>());
+        schedule_k_step(slot_c<0>());
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
+        multiply(slot_c<P>(), slot_c<1>());
+        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<1>()), load_a(a2, s2, slot_c<P>(), slot_c<3>());
+        schedule_k_step(slot_c<0>());
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
+        multiply(slot_c<P>(), slot_c<2>());
+        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<2>());
+        // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
+        // at the previous barrier); then its registers start being refilled with A(s+3).
+        if (!(DBG & 8)) store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, s + 1 < fast ? 1u : 0u);
+        if (!(DBG & 1)) load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
+        schedule_k_step(slot_c<1>());
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 4)) __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(DBG & 2)) read_frags(slot_c<P ^ 1>(), slot_c<0>(), slot_c<0>());
+        multiply(slot_c<P>(), slot_c<3>());
+        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<3>()), load_a(a3, s3, slot_c<P ^ 1>(), slot_c<1>());
+        schedule_k_step(slot_c<0>());
+    };
+
+    // Fills the pipeline for a tile: stages 0 and 1 on their way, A(0) in LDS, its first fragments read.
+    auto prime = [&]() {
+        __syncthreads(); // the previous tile's last fragment reads are done
+        load_a_all(cur, 0, slot_c<0>());
+        load_b(cur, 0, slot_c<0>(), slot_c<0>()), load_b(cur, 0, slot_c<0>(), slot_c<1>());
+        load_b(cur, 0, slot_c<0>(), slot_c<2>()), load_b(cur, 0, slot_c<0>(), slot_c<3>());
+        load_a_all(cur, 1, slot_c<1>());
+        load_b(cur, 1, slot_c<1>(), slot_c<0>()), load_b(cur, 1, slot_c<1>(), slot_c<1>());
+        load_b(cur, 1, slot_c<1>(), slot_c<2>()), load_b(cur, 1, slot_c<1>(), slot_c<3>());
+        store_a(slot_c<0>(), slot_c<0>(), 0u, 1u);
+        // the first half of A(2), as k-steps 2 and 3 of a stage "-1" would have issued it
+        // (with two stages in all it is A(0) again, which nobody uses)
+        uint32_t const third = fast > 2 ? 2 : 0;
+        load_a(cur, third, slot_c<0>(), slot_c<0>()), load_a(cur, third, slot_c<0>(), slot_c<1>());
+        __syncthreads();
+        read_frags(slot_c<0>(), slot_c<0>(), slot_c<0>());
+    };
+    if constexpr (across) {
+        cur = view_of(blockIdx.x);
+        prime();
+    }
+
+    for (uint32_t tile = blockIdx.x; tile < tile_count; tile += gridDim.x) {
+#ifdef NK_TUNE
+        unsigned long long const debug_t0 = clock64(), debug_tw0 = wall_clock64();
+        unsigned long long debug_t1 = 0, debug_t2 = 0;
+#endif
+        cur = view_of(tile);
+        bool const has_next = across && tile + gridDim.x < tile_count;
+        nxt = view_of(has_next ? tile + gridDim.x : tile);
+        uint32_t const row0 = cur.row0, col0 = cur.col0;
+
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+        // u8: the column terms of this tile are fetched now and used in the epilogue, so that nothing has to
+        // wait for them (a wait for a load is a wait for every store issued before it).
+        uint32_t col_term[TN], col_norm[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            col_term[j] = 0, col_norm[j] = 0;
+            uint32_t const t = col0 / 32 + j < g.n_tiles ? col0 / 32 + j : g.n_tiles - 1;
+            if constexpr (T::kUnsigned) col_term[j] = col_terms[(uint64_t)t * kTileRows + (lane & 31)];
+            if constexpr (NORMS) col_norm[j] = col_norms[(uint64_t)t * kTileRows + (lane & 31)];
+        }
+        total.clear();
+
+        {
+#ifdef NK_TUNE
+            unsigned long long const debug_c0 = clock64(), debug_w0 = wall_clock64();
+#endif
+            if (across || fast > 0) { // (always, when the pipeline runs across tiles: the host checked)
+                if constexpr (!across) prime();
+#ifdef NK_TUNE
+                debug_t1 = clock64();
+#endif
+                uint32_t until_fold = g.chunk_stages;
+                for (uint32_t s = 0; s < fast; s += 2) {
+                    stage(slot_c<0>(), s);
+                    stage(slot_c<1>(), s + 1);
+                    if constexpr (kChunked) {
+                        until_fold -= 2;
+                        if (until_fold == 0) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            total.fold(acc);
+                            until_fold = g.chunk_stages;
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#ifdef NK_TUNE
+            if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + (tile_count > 45 * gridDim.x ? 40 : 1) * gridDim.x) {
+                g_debug_clocks[0] = clock64() - debug_c0, g_debug_clocks[1] = wall_clock64() - debug_w0;
+                g_debug_clocks[2] = fast;
+                g_debug_clocks[3] = debug_c0 - debug_t0, g_debug_clocks[4] = debug_t1 - debug_c0;
+            }
+            debug_t2 = clock64();
+#endif
+
+            // Remaining stages: the ragged end of K, or everything when A cannot be read with vector loads.
+            if (!across && fast < stages) {
+                uint8_t const *a_tile = g.a + (uint64_t)row0 * g.a_stride;
+                uint32_t a_slow[kLoads]; // rows clamped to the last one: plain loads have no descriptor to stop them
+#pragma unroll
+                for (int i = 0; i < kLoads; ++i) {
+                    uint32_t const r = i * 32 + (tid >> 3);
+                    uint32_t const row = row0 + r < g.m ? r : g.m - 1 - row0;
+                    a_slow[i] = row * (uint32_t)g.a_stride + a_pos * T::kSrcChunk;
+                }
+                uint32_t until_fold = g.chunk_stages;
+                for (uint32_t s = fast; s < stages; ++s) {
+                    __syncthreads();
+                    int64_t const left = (int64_t)g.k_src_bytes - (int64_t)s * kSrcStage - (int64_t)a_pos * T::kSrcChunk;
+                    int const valid = (int)(left > T::kSrcChunk ? T::kSrcChunk : (left < 0 ? 0 : left));
+#pragma unroll
+                    for (int i = 0; i < kLoads; ++i) {
+                        v4i v = load_chunk_guarded(a_tile + (uint64_t)s * kSrcStage + a_slow[i], valid, g.avec, 0u);
+                        v4i const raw = v;
+                        if (T::kUnsigned) {
+                            add_row_sum(i, sum_bytes_u8(v), sums_here);
+#pragma unroll
+                            for (int w = 0; w < 4; ++w) { // flip only bytes that exist: the zero padding stays zero
+                                int const rem = valid - 4 * w;
+                                uint32_t const mask = rem >= 4 ? 0x80808080u : (rem <= 0 ? 0u : (0x80808080u >> (8 * (4 - rem))));
+                                v[w] ^= (int)mask;
+                            }
+                        }
+                        v4i const wide = T::widen(v);
+                        if (NORMS) add_row_norm(i, T::sumsq(raw, wide), sums_here);
+                        *(v4i *)(lds + a_lds[i]) = wide;
+                    }
+                    load_b(cur, s, slot_c<0>(), slot_c<0>()), load_b(cur, s, slot_c<0>(), slot_c<1>());
+                    load_b(cur, s, slot_c<0>(), slot_c<2>()), load_b(cur, s, slot_c<0>(), slot_c<3>());
+                    __syncthreads();
+                    read_frags(slot_c<0>(), slot_c<0>(), slot_c<0>());
+                    read_frags(slot_c<0>(), slot_c<1>(), slot_c<1>());
+                    multiply(slot_c<0>(), slot_c<0>());
+                    read_frags(slot_c<0>(), slot_c<2>(), slot_c<0>());
+                    multiply(slot_c<0>(), slot_c<1>());
+                    read_frags(slot_c<0>(), slot_c<3>(), slot_c<1>());
+                    multiply(slot_c<0>(), slot_c<2>());
+                    multiply(slot_c<0>(), slot_c<3>());
+                    if constexpr (kChunked) { // the same two-level accumulation as the pipelined loop
+                        if (--until_fold == 0) {
+                            total.fold(acc);
+                            until_fold = g.chunk_stages;
+                        }
+                    }
+                }
+            }
+        }
+
+        // Epilogue. Accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.
+        uint32_t const half = lane >> 5, col_in_tile = lane & 31;
+        if (T::kUnsigned || NORMS) {
+            __syncthreads();
+            // The 8 threads that staged a row left its partial sums in 8 adjacent slots.
+            if (tid < BM) {
+                if (T::kUnsigned) {
+                    uint32_t const *parts = &row_part[sums_here + tid * 8];
+                    uint32_t sum = 0;
+#pragma unroll
+                    for (int part = 0; part < 8; ++part) sum += parts[part];
+                    row_terms[tid] = sum * 128u;
+                }
+                if (NORMS) {
+                    norm_t const *parts = &norm_part[sums_here + tid * 8];
+                    norm_t sum = 0;
+#pragma unroll
+                    for (int part = 0; part < 8; ++part) sum += parts[part];
+                    uint32_t bits;
+                    if constexpr (sizeof(norm_t) == 8) bits = __builtin_bit_cast(uint32_t, (float)sum); // f64 -> f32, once
+                    else bits = (uint32_t)sum;
+                    row_norms[tid] = __builtin_bit_cast(uint32_t, norm_as_f32<T>(bits));
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i) { // own slots: ready for the tile after next
+                if (T::kUnsigned) row_part[sums_here + i * NT + tid] = 0;
+                if (NORMS) norm_part[sums_here + i * NT + tid] = 0;
+            }
+            sums_here ^= (uint32_t)(kLoads * NT);
+        }
+        // Stores: a scalar base plus one 32-bit per-lane offset, through an explicitly global pointer. (A store
+        // through a generic pointer counts as an LDS operation as well, and with such stores in flight the
+        // loads prefetched for the next tile could only be waited for all at once.) Tiles that touch the
+        // matrix edge take the masked copy of the loop.
+        // Of a triangular grid, a wavefront's part of a tile is stored whole (all of it right of the diagonal), not
+        // at all (all of it left), or through the masked copy.
+        // What only the stores need is read from the kernel's arguments again, here, rather than held in a dozen
+        // scalar registers through the loop (the empty asm hides from the compiler that it is the same memory).
+        typedef __attribute__((address_space(4))) GemmArgs const late_args_t;
+        late_args_t *late = (late_args_t *)__builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("" : "+s"(late));
+        bool const interior = row0 + BM <= late->m && col0 + 32 * TN <= late->n &&
+                              (((row0 + (BM - 1) + late->tri_shift) & late->tri_mask) <= col0);
+        bool const nothing = ((row0 + late->tri_shift) & late->tri_mask) > col0 + (32 * TN - 1);
+        global_u8_t *c_tile = (global_u8_t *)late->c + (uint64_t)row0 * late->c_stride + (uint64_t)col0 * 4;
+        auto store_all = [&](auto masked_tag, auto metric_tag) {
+            constexpr bool masked = decltype(masked_tag)::value != 0;
+            constexpr int metric = decltype(metric_tag)::value;
+            uint64_t const row_step = late->c_stride;
+            // Lane l holds column l % 32; register v holds row 8 * (v / 4) + 4 * (l / 32) + v % 4.
+            uint32_t const lane_offset = 4 * half * (uint32_t)late->c_stride + col_in_tile * 4;
+            // Masked tiles: rows of the matrix from this lane's first one on, and how far right of the diagonal
+            // col = row + tri_shift its first element lies (element (r, 32 j) from there is stored when
+            // r - 32 j <= that distance; without a triangle everything is).
+            int const rows_left = (int)(late->m - row0 - 4 * half);
+            int const diagonal = late->tri_mask ? (int)(col0 + col_in_tile) - (int)(row0 + 4 * half + late->tri_shift) : 0x7FFFFFFF;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                bool const col_ok = col0 + j * 32 + col_in_tile < late->n;
+                // Rows come in runs of 4 that start 8 apart: the base advances by one row or by five. The
+                // empty asm keeps it a running scalar (otherwise every row's base is precomputed and the
+                // scalar registers overflow).
+                global_u8_t *row_base = c_tile + j * 128;
+                v4i row_term4 = {0, 0, 0, 0}, row_norm4 = {0, 0, 0, 0};
+                float const col_value = metric != 0 ? norm_as_f32<T>(col_norm[j]) : 0.0f;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        int const r_fixed = i * 32 + 8 * (v / 4) + (v % 4); // row of lanes 0..31; lanes 32..63 are 4 rows below
+                        // a named copy: bit-casting the vector element expression itself reads lane 0
+                        auto const element = total.finish(acc, i, j, v);
+                        uint32_t bits = __builtin_bit_cast(uint32_t, element);
+                        if (T::kUnsigned) {
+                            // the terms of 4 consecutive rows in one LDS read
+                            if (v % 4 == 0) row_term4 = *(v4i const *)&row_terms[i * 32 + 8 * (v / 4) + 4 * half];
+                            bits += (uint32_t)row_term4[v % 4] + col_term[j];
+                        }
+                        if (metric != 0) {
+                            if (v % 4 == 0) row_norm4 = *(v4i const *)&row_norms[i * 32 + 8 * (v / 4) + 4 * half];
+                            int const row_bits = row_norm4[v % 4];
+                            bits = distance_from_dot<T, metric == 2 ? 2 : 1>(bits, __builtin_bit_cast(float, row_bits), col_value);
+                        }
+                        bool keep = true;
+                        if (masked) {
+                            keep = col_ok && r_fixed < rows_left && r_fixed - j * 32 <= diagonal;
+                            // a vector's distance from itself is exactly 0 (dots/serial.h:2871-2876)
+                            if (metric != 0 && r_fixed - j * 32 == diagonal) bits = 0;
+                        }
+                        if ((!(DBG & 16) || bits == 0x12345678u) && keep) // (timing experiment: almost no stores)
+                            *(global_u32_t *)(row_base + lane_offset) = bits;
+                        row_base += (v % 4 == 3 ? 5 : 1) * row_step;
+                        asm volatile("" : "+s"(row_base));
+                    }
+                    // u8 reads a row term per element: keep those reads from being hoisted by the hundred
+                    // (registers are what the prefetched tile is short of here).
+                    if (T::kUnsigned || metric != 0) __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        if (nothing) {}
+        else if constexpr (NORMS) { // which distance is a run-time choice: one kernel serves both
+            if (late->metric == 2) {
+                if (interior) store_all(slot_c<0>(), slot_c<2>());
+                else store_all(slot_c<1>(), slot_c<2>());
+            }
+            else {
+                if (interior) store_all(slot_c<0>(), slot_c<1>());
+                else store_all(slot_c<1>(), slot_c<1>());
+            }
+        }
+        else {
+            if (interior) store_all(slot_c<0>(), slot_c<0>());
+            else store_all(slot_c<1>(), slot_c<0>());
+        }
+#ifdef NK_TUNE
+        if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + (g.tile_count > 45 * gridDim.x ? 40 : 1) * gridDim.x) {
+            g_debug_clocks[5] = clock64() - debug_t2, g_debug_clocks[6] = clock64() - debug_t0;
+            g_debug_clocks[7] = wall_clock64() - debug_tw0;
+        }
+#endif
+    }
+}
+
+struct TileConfig {
+    int tm, tn;
+};
+// Index 0 is "choose for me"; 1.. are explicit.
+constexpr TileConfig kConfigs[] = {{0, 0}, {8, 2}, {4, 2}, {4, 1}, {2, 1}};
+constexpr int kConfigCount = sizeof(kConfigs) / sizeof(kConfigs[0]);
+
+
+/** Tiles of a bm x bn grid over m x n outputs with something on or right of the diagonal col = row + shift. */
+inline uint32_t log2_of(uint32_t power_of_two) { return (uint32_t)__builtin_ctz(power_of_two); }
+inline uint64_t live_tiles(uint64_t m, uint64_t n, uint32_t bm, uint32_t bn, uint32_t shift) {
+    uint32_t const tiles_m = (uint32_t)((m + bm - 1) / bm), tiles_n = (uint32_t)((n + bn - 1) / bn);
+    uint64_t count = 0;
+    for (uint32_t t = 0; t < tiles_m; ++t) {
+        uint32_t const from = first_live_tile(t, log2_of(bm), log2_of(bn), shift);
+        count += from < tiles_n ? tiles_n - from : 0;
+    }
+    return count;
+}
+inline size_t triangle_scratch_bytes(uint64_t m, uint64_t n, uint32_t bm, uint32_t bn, uint32_t shift) {
+    uint64_t const bands = ((m + bm - 1) / bm + kTileBand - 1) / kTileBand;
+    return (size_t)(((bands + 1 + 1) & ~1ull) * 4 + live_tiles(m, n, bm, bn, shift) * 8);
+}
+
+/** `slots_only`: do not launch, only report how many workgroups of the kernel this call would use are resident on
+ *  the device at once. */
+template <class T, int TM, int TN>
+hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle, int *slots_only = nullptr) {
+    constexpr int BM = TM * 32, BN = TN * 128;
+    g.tiles_m = (g.m + BM - 1) / BM;
+    g.tiles_n = (g.n + BN - 1) / BN;
+    uint64_t tiles = (uint64_t)g.tiles_m * g.tiles_n;
+    if (tiles > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    g.tile_list = nullptr;
+    if (triangle) {
+        tiles = live_tiles(g.m, g.n, BM, BN, g.tri_shift);
+        if (!tiles) return hipSuccess;
+        if (triangle_scratch_bytes(g.m, g.n, BM, BN, g.tri_shift) > triangle->bytes) return hipErrorInvalidValue;
+        uint32_t const bands = (g.tiles_m + kTileBand - 1) / kTileBand;
+        g.tile_list = triangle->words + ((bands + 1 + 1) & ~1u); // (written by the caller's triangle_tiles_kernel)
+    }
+    g.tile_count = (uint32_t)tiles;
+    // The tile's A offsets are 32-bit: (rows of a tile) * stride must stay below 4 GiB.
+    if ((uint64_t)BM * g.a_stride > 0xFFFFFFFFull) return hipErrorInvalidValue;
+    // So are the per-lane C offsets: 4 rows plus the tile's width.
+    if (4 * (uint64_t)g.c_stride + BN * 4 > 0xFFFFFFFFull) return hipErrorInvalidValue;
+    // The offsets into a wavefront's B tiles are 32-bit as well.
+    if ((uint64_t)(TN + 1) * g.k_chunks * kTileChunkBytes > 0xFFFFFFFFull) return hipErrorInvalidValue;
+    // The pipeline runs across tile boundaries when the pipelined loop takes the stages of a tile (A readable
+    // with dword loads) and there are enough of them to prefetch three ahead.
+    uint32_t const stages = g.k_chunks / kStageChunks;
+    bool const across = g.avec >= 4 && stages >= 4 && !(g_variant & 1);
+    bool const norms = g.metric != 0;
+    void (*kernel)(GemmArgs) = norms ? (across ? dots_packed_kernel<T, TM, TN, true, true> : dots_packed_kernel<T, TM, TN, false, true>)
+                                     : (across ? dots_packed_kernel<T, TM, TN, true, false> : dots_packed_kernel<T, TM, TN, false, false>);
+#ifdef NK_TUNE // timing experiments that leave parts of the loop out (results are wrong on purpose)
+    if constexpr (TM == 8 && TN == 2 && T::kDtype == kI8) {
+        switch (g_variant >> 2) {
+        case 1: kernel = dots_packed_kernel<T, TM, TN, false, false, 1>; break;
+        case 2: kernel = dots_packed_kernel<T, TM, TN, false, false, 2>; break;
+        case 3: kernel = dots_packed_kernel<T, TM, TN, false, false, 4>; break;
+        case 4: kernel = dots_packed_kernel<T, TM, TN, false, false, 16>; break;
+        case 5: kernel = dots_packed_kernel<T, TM, TN, false, false, 17>; break;
+        default: break;
+        }
+    }
+#endif
+    // Persistent grid: as many workgroups as fit on the device at once (queried once per kernel).
+    static int resident_of[4] = {0, 0, 0, 0};
+    int &resident = resident_of[(across ? 1 : 0) + (norms ? 2 : 0)];
+    if (!resident) {
+        int per_cu = 0, device = 0;
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (void const *)kernel, 256, 0);
+        if (e != hipSuccess) return e;
+        if (!g_cu_count) {
+            hipDeviceProp_t properties;
+            if ((e = hipGetDevice(&device)) != hipSuccess) return e;
+            if ((e = hipGetDeviceProperties(&properties, device)) != hipSuccess) return e;
+            g_cu_count = properties.multiProcessorCount;
+        }
+        resident = (per_cu > 0 ? per_cu : 1) * (g_cu_count > 0 ? g_cu_count : 256);
+    }
+    if (slots_only) {
+        *slots_only = resident;
+        return hipSuccess;
+    }
+    uint32_t const blocks = (uint32_t)(tiles < (uint64_t)resident ? tiles : (uint64_t)resident);
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, g);
+    return hipGetLastError();
+}
+
+template <class T>
+hipError_t launch_config(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle, int config,
+                         int *slots_only = nullptr) {
+    switch (config) {
+    case 1:
+        if constexpr (T::kChunked) return hipErrorInvalidValue;
+        else return launch_one<T, 8, 2>(g, stream, triangle, slots_only);
+    case 2: return launch_one<T, 4, 2>(g, stream, triangle, slots_only);
+    case 3: return launch_one<T, 4, 1>(g, stream, triangle, slots_only);
+    default: return launch_one<T, 2, 1>(g, stream, triangle, slots_only);
+    }
+}
+
+template <class T>
+hipError_t launch_typed(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle) {
+    int config = g_forced_config & 0x7F;
+    bool const chosen_here = config <= 0 || config >= kConfigCount;
+    auto tiles_of = [&](GemmArgs const &args, int c) {
+        uint64_t const bm = kConfigs[c].tm * 32, bn = (uint64_t)kConfigs[c].tn * 128;
+        if (triangle) return live_tiles(args.m, args.n, (uint32_t)bm, (uint32_t)bn, args.tri_shift);
+        return ((args.m + bm - 1) / bm) * ((args.n + bn - 1) / bn);
+    };
+    // Largest tile that still gives every one of the 256 CUs at least one workgroup.
+    auto choose = [&](GemmArgs const &args, int first) {
+        int best = 4;
+        for (int c = first; c <= 4; ++c)
+            if (tiles_of(args, c) >= 256) {
+                best = c;
+                break;
+            }
+        // Distances over a shallow depth are bound by the epilogue (a finaliser and a store per output): two
+        // workgroups per CU of 128 x 128 tiles overlap it with the other's loop better than one large tile does
+        // (measured on 1024 x 1,048,576 x 768: 2.17 against 2.33 ms angular, 1.98 against 2.07 ms euclidean).
+        if (args.metric != 0 && best < 3 && args.k_chunks / kStageChunks <= 8 && tiles_of(args, 3) >= 256) best = 3;
+        if (T::kChunked && best == 1) best = 2; // two accumulator sets do not fit the 256 x 256 tile
+        return best;
+    };
+    if (chosen_here) config = choose(g, 1);
+    if (T::kChunked && config == 1) config = 2;
+    // Where the tile list of a launch goes (the same arithmetic as launch_one's) and what it holds.
+    auto grid_of = [](GemmArgs const &args, int c, TriangleScratch const &scratch) {
+        uint32_t const bm = kConfigs[c].tm * 32, bn = kConfigs[c].tn * 128;
+        TriangleGrid grid;
+        grid.tiles_m = (args.m + bm - 1) / bm, grid.tiles_n = (args.n + bn - 1) / bn;
+        grid.bm_log2 = log2_of(bm), grid.bn_log2 = log2_of(bn), grid.shift = args.tri_shift;
+        uint32_t const bands = (grid.tiles_m + kTileBand - 1) / kTileBand;
+        grid.band_start = scratch.words, grid.list = scratch.words + ((bands + 1 + 1) & ~1u);
+        return grid;
+    };
+
+    // A triangular grid rarely fills a whole number of rounds of the persistent workgroups, and a last round that
+    // is mostly empty costs as much as a full one. When that last round would be less than half full, the tile rows
+    // from the top that fill whole rounds go to this tile shape and the rows below them, the narrow end of the
+    // triangle, to a second launch with small tiles that spreads them over the whole device.
+    if (triangle && (chosen_here || (g_forced_config & 0x80)) && config < 4) {
+        int slots = 0;
+        GemmArgs probe = g;
+        hipError_t e = launch_config<T>(probe, stream, triangle, config, &slots);
+        if (e != hipSuccess) return e;
+        uint64_t const live = tiles_of(g, config);
+        uint64_t const rounds = slots > 0 ? live / (uint64_t)slots : 0, rest = slots > 0 ? live % (uint64_t)slots : 0;
+        if (rounds >= 1 && rest > 0 && rest * 2 <= (uint64_t)slots) {
+            uint32_t const bm = kConfigs[config].tm * 32, bn = kConfigs[config].tn * 128;
+            uint32_t const tiles_m = (g.m + bm - 1) / bm, tiles_n = (g.n + bn - 1) / bn;
+            uint64_t count = 0;
+            uint32_t keep = 0; // tile rows that stay with the large tiles
+            for (; keep < tiles_m; ++keep) {
+                uint32_t const from = first_live_tile(keep, log2_of(bm), log2_of(bn), g.tri_shift);
+                uint64_t const here = from < tiles_n ? tiles_n - from : 0;
+                if (count + here > rounds * (uint64_t)slots) break;
+                count += here;
+            }
+            if (keep > 0 && keep < tiles_m) {
+                GemmArgs top = g, bottom = g;
+                top.m = keep * bm;
+                bottom.m = g.m - top.m;
+                bottom.a += (uint64_t)top.m * g.a_stride, bottom.c += (uint64_t)top.m * g.c_stride;
+                bottom.tri_shift = g.tri_shift + top.m;
+                // each launch builds its tile list in its own half of the scratch memory
+                size_t const half = triangle->bytes / 2 / 8 * 8;
+                TriangleScratch const first_half = {triangle->words, half}, second_half = {triangle->words + half / 4, half};
+                int const small = choose(bottom, config + 1);
+                TriangleGrids grids;
+                grids.grid[0] = grid_of(top, config, first_half), grids.grid[1] = grid_of(bottom, small, second_half);
+                hipLaunchKernelGGL(triangle_tiles_kernel, dim3(2), dim3(256), 0, stream, grids);
+                if ((e = hipGetLastError()) != hipSuccess) return e;
+                if ((e = launch_config<T>(top, stream, &first_half, config)) != hipSuccess) return e;
+                return launch_config<T>(bottom, stream, &second_half, small);
+            }
+        }
+    }
+    if (triangle && tiles_of(g, config) > 0) {
+        TriangleGrids grids;
+        grids.grid[0] = grids.grid[1] = grid_of(g, config, *triangle);
+        hipLaunchKernelGGL(triangle_tiles_kernel, dim3(1), dim3(256), 0, stream, grids);
+        hipError_t const e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return launch_config<T>(g, stream, triangle, config);
+}
+
+inline int widest_load(void const *p, size_t stride) {
+    uintptr_t const bits = (uintptr_t)p | (uintptr_t)stride;
+    if (!(bits & 15)) return 16;
+    if (!(bits & 7)) return 8;
+    if (!(bits & 3)) return 4;
+    if (!(bits & 1)) return 2;
+    return 1;
+}
+
+#pragma endregion Packed product
+
+} // namespace
+
+#endif // NUMKONG_AMD_DOTS_GFX950_HPP

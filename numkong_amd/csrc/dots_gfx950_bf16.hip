@@ -1,0 +1,11 @@
+/**
+ *  @brief The bf16 product kernels of the gfx950 backend, every tile shape.
+ *  @file numkong_amd/csrc/dots_gfx950_bf16.hip
+ */
+#include "dots_gfx950.hpp"
+
+namespace nk_gfx950 {
+hipError_t launch_bf16(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle) {
+    return launch_typed<BF16>(g, stream, triangle);
+}
+} // namespace nk_gfx950
