@@ -29,8 +29,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 # MI355X published dense peaks, in T(FL)OP/s, for the MFMA the dtype runs on; HBM3E in GB/s.
-MFMA_PEAK = {"i8": 5000.0, "u8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "e4m3": 2500.0, "e5m2": 2500.0}
-MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2": "widened to f16, priced against the f16 MFMA peak"}
+MFMA_PEAK = {"i8": 5000.0, "u8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "e4m3": 2500.0, "e5m2": 2500.0,
+             "e2m3": 2500.0, "e3m2": 2500.0, "i4": 5000.0, "u4": 5000.0}
+MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2": "widened to f16, priced against the f16 MFMA peak",
+             "e2m3": "widened to f16, priced against the f16 MFMA peak", "e3m2": "widened to f16, priced against the f16 MFMA peak",
+             "i4": "widened to i8, priced against the i8 MFMA peak", "u4": "widened to i8, priced against the i8 MFMA peak"}
 HBM_PEAK = 8000.0
 # HBM-side bytes per launch (L2 <-> fabric) from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --probe`,
 # each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
@@ -46,7 +49,8 @@ MEASURED_TRAFFIC = {
 }
 HEADLINE = ("i8", 8192, 8192, 8192)
 OTHERS = [("bf16", 8192, 8192, 8192, "dots"), ("e4m3", 8192, 8192, 8192, "dots"), ("i8", 1024, 1 << 20, 768, "dots"),
-          ("i8", 1024, 1 << 20, 768, "angular"), ("i8", 8192, 8192, 8192, "symmetric"), ("bf16", 8192, 8192, 8192, "symmetric")]
+          ("i8", 1024, 1 << 20, 768, "angular"), ("i8", 8192, 8192, 8192, "symmetric"), ("bf16", 8192, 8192, 8192, "symmetric"),
+          ("i4", 8192, 8192, 8192, "dots"), ("e2m3", 8192, 8192, 8192, "dots")]
 KINDS = {"angular": ord("N"), "euclidean": ord("E")}  # nk_kernel_angulars_packed_k, nk_kernel_euclideans_packed_k
 # nk_kernel_dots_symmetric_k, nk_kernel_angulars_symmetric_k, nk_kernel_euclideans_symmetric_k
 SYMMETRIC_KINDS = {"symmetric": ord("y"), "symmetric-angular": ord("n"), "symmetric-euclidean": ord("D")}
@@ -59,6 +63,10 @@ def make_operands(dtype, m, n, k, seed=42):
 
     g = torch.Generator(device="cuda:0").manual_seed(seed)
     def one(rows):
+        if dtype in ("i4", "u4"):  # two 4-bit values per byte, every byte value
+            return torch.randint(0, 256, (rows, (k + 1) // 2), dtype=torch.uint8, device="cuda:0", generator=g)
+        if dtype in ("e2m3", "e3m2"):  # every 6-bit code is a finite number
+            return torch.randint(0, 64, (rows, k), dtype=torch.uint8, device="cuda:0", generator=g)
         if dtype == "i8":
             return torch.randint(-128, 128, (rows, k), dtype=torch.int8, device="cuda:0", generator=g)
         if dtype == "u8":
@@ -84,7 +92,7 @@ def time_symmetric(dtype, n, k, steps, warmup, metric):
 
     lib = nk.library()
     vectors, _ = make_operands(dtype, n, 1, k)
-    code, width = api.DTYPES[dtype][0], api.DTYPES[dtype][1]
+    code, row_bytes = api.DTYPES[dtype][0], vectors.shape[1] * vectors.element_size()
     result = torch.zeros((n, n), dtype=torch.int32 if dtype in ("i8", "u8") and metric == "symmetric" else torch.float32,
                          device="cuda:0")
     workspace_bytes = lib.nk_amd_symmetric_workspace_size(code, n, k, 0, n)
@@ -92,7 +100,7 @@ def time_symmetric(dtype, n, k, steps, warmup, metric):
     stream = torch.cuda.current_stream().cuda_stream
 
     def step():
-        status = lib.nk_amd_symmetric_async(SYMMETRIC_KINDS[metric], code, vectors.data_ptr(), n, k, k * width,
+        status = lib.nk_amd_symmetric_async(SYMMETRIC_KINDS[metric], code, vectors.data_ptr(), n, k, row_bytes,
                                             result.data_ptr(), n * 4, 0, n, workspace.data_ptr(), workspace_bytes, stream)
         if status:
             raise RuntimeError(lib.nk_hip_last_error().decode())
@@ -133,16 +141,16 @@ def time_gpu(dtype, m, n, k, steps, warmup, metric="dots"):
     packed = nk.dots_pack(b, dtype)
     del b
     c = torch.empty((m, n), dtype=torch.int32 if dtype in ("i8", "u8") and metric == "dots" else torch.float32, device="cuda:0")
-    code, width = api.DTYPES[dtype][0], api.DTYPES[dtype][1]
+    code, row_bytes = api.DTYPES[dtype][0], a.shape[1] * a.element_size()
     stream = torch.cuda.current_stream().cuda_stream  # the kernel is launched on this stream, so torch events see it
 
     def step():
         if metric == "dots":
             status = lib.nk_amd_dots_packed_async(code, a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(), m, n, k,
-                                                  k * width, n * 4, stream)
+                                                  row_bytes, n * 4, stream)
         else:  # the same product with the distance finaliser fused into its epilogue
             status = lib.nk_amd_spatials_packed_async(KINDS[metric], code, a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(),
-                                                      m, n, k, k * width, n * 4, stream)
+                                                      m, n, k, row_bytes, n * 4, stream)
         if status:
             raise RuntimeError(lib.nk_hip_last_error().decode())
 
@@ -161,7 +169,7 @@ def time_gpu(dtype, m, n, k, steps, warmup, metric="dots"):
     ops = 2.0 * m * n * k
     result = {"ms_per_step": wall, "kernel_ms": device_ms, "gso_per_s": ops / (wall * 1e-3) / 1e9}
     if m * n >= 64 * k * 8 and dtype in ("i8", "u8") and n >= 1 << 18:  # retrieval shape: HBM-bound on C and the packed stream
-        algorithmic = (m * k + n * k) * width + m * n * 4
+        algorithmic = (m + n) * row_bytes + m * n * 4
         result["roofline"] = {"bound": "hbm", "achieved": algorithmic / (device_ms * 1e-3) / 1e9, "peak": HBM_PEAK,
                               "unit": "GB/s", "frac": algorithmic / (device_ms * 1e-3) / 1e9 / HBM_PEAK,
                               "traffic": MEASURED_TRAFFIC.get((dtype, m, n, k) if metric == "dots" else (dtype, m, n, k, metric))}

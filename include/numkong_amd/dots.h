@@ -49,6 +49,10 @@ typedef unsigned short nk_f16_t;
 typedef unsigned short nk_bf16_t;
 typedef unsigned char nk_e4m3_t;
 typedef unsigned char nk_e5m2_t;
+typedef unsigned char nk_e2m3_t; /* one 6-bit float per byte */
+typedef unsigned char nk_e3m2_t;
+typedef unsigned char nk_i4x2_t; /* two 4-bit integers per byte, the even dimension in the low nibble */
+typedef unsigned char nk_u4x2_t;
 typedef nk_u64_t nk_size_t;
 
 /** Element types (reference: include/numkong/types.h:923-952; same numeric codes). */
@@ -63,6 +67,10 @@ typedef enum {
     nk_bf16_k = 1 << 13,
     nk_e4m3_k = 1 << 14,
     nk_e5m2_k = 1 << 15,
+    nk_i4_k = 1 << 16,
+    nk_u4_k = 1 << 17,
+    nk_e2m3_k = 1 << 18,
+    nk_e3m2_k = 1 << 19,
 } nk_dtype_t;
 
 /** Kernel kinds (reference: include/numkong/capabilities.h:178-253; same codes). The three dots kinds and the
@@ -107,6 +115,10 @@ NK_DYNAMIC nk_size_t nk_dots_packed_size_bf16(nk_size_t width, nk_size_t depth);
 NK_DYNAMIC nk_size_t nk_dots_packed_size_f16(nk_size_t width, nk_size_t depth);
 NK_DYNAMIC nk_size_t nk_dots_packed_size_e4m3(nk_size_t width, nk_size_t depth);
 NK_DYNAMIC nk_size_t nk_dots_packed_size_e5m2(nk_size_t width, nk_size_t depth);
+NK_DYNAMIC nk_size_t nk_dots_packed_size_e2m3(nk_size_t width, nk_size_t depth);
+NK_DYNAMIC nk_size_t nk_dots_packed_size_e3m2(nk_size_t width, nk_size_t depth);
+NK_DYNAMIC nk_size_t nk_dots_packed_size_i4(nk_size_t width, nk_size_t depth); /* depth in 4-bit values */
+NK_DYNAMIC nk_size_t nk_dots_packed_size_u4(nk_size_t width, nk_size_t depth);
 
 /* Pack row-major B (width rows of depth elements, b_stride bytes apart). Reference: include/numkong/dots.h:203-237. */
 NK_DYNAMIC void nk_dots_pack_i8(nk_i8_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride, void *b_packed);
@@ -119,6 +131,14 @@ NK_DYNAMIC void nk_dots_pack_e4m3(nk_e4m3_t const *b, nk_size_t width, nk_size_t
                                   void *b_packed);
 NK_DYNAMIC void nk_dots_pack_e5m2(nk_e5m2_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
                                   void *b_packed);
+NK_DYNAMIC void nk_dots_pack_e2m3(nk_e2m3_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
+                                  void *b_packed);
+NK_DYNAMIC void nk_dots_pack_e3m2(nk_e3m2_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
+                                  void *b_packed);
+NK_DYNAMIC void nk_dots_pack_i4(nk_i4x2_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
+                                void *b_packed);
+NK_DYNAMIC void nk_dots_pack_u4(nk_u4x2_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
+                                void *b_packed);
 
 /* C = A * B^T with widened accumulators, C overwritten. Reference: include/numkong/dots.h:248-287. */
 NK_DYNAMIC void nk_dots_packed_i8(nk_i8_t const *a, void const *b_packed, nk_i32_t *c, nk_size_t height,
@@ -133,6 +153,14 @@ NK_DYNAMIC void nk_dots_packed_e4m3(nk_e4m3_t const *a, void const *b_packed, nk
                                     nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
 NK_DYNAMIC void nk_dots_packed_e5m2(nk_e5m2_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,
                                     nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
+NK_DYNAMIC void nk_dots_packed_e2m3(nk_e2m3_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,
+                                    nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
+NK_DYNAMIC void nk_dots_packed_e3m2(nk_e3m2_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,
+                                    nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
+NK_DYNAMIC void nk_dots_packed_i4(nk_i4x2_t const *a, void const *b_packed, nk_i32_t *c, nk_size_t height,
+                                  nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
+NK_DYNAMIC void nk_dots_packed_u4(nk_u4x2_t const *a, void const *b_packed, nk_u32_t *c, nk_size_t height,
+                                  nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
 
 /* Distances over the same packed B, in one pass: result[i][j] = angular (1 - cosine) or euclidean distance between
  * row i of A and row j of B, f32 for all six types. Reference: include/numkong/spatials.h:139-266. */
@@ -172,6 +200,27 @@ NK_AMD_DECLARE_SYMMETRIC_(f16, nk_f16_t, nk_f32_t)
 NK_AMD_DECLARE_SYMMETRIC_(e4m3, nk_e4m3_t, nk_f32_t)
 NK_AMD_DECLARE_SYMMETRIC_(e5m2, nk_e5m2_t, nk_f32_t)
 #undef NK_AMD_DECLARE_SYMMETRIC_
+
+/* The 6-bit floats and the 4-bit integers have the dot-product kinds only (packed above, symmetric here), with their
+ * backend-suffixed names; their distance kinds resolve to the error stubs. */
+#define NK_AMD_DECLARE_DOTS_ONLY_(T, in_t, out_t)                                                                      \
+    NK_DYNAMIC void nk_dots_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,              \
+                                          nk_size_t stride, out_t *result, nk_size_t result_stride,                   \
+                                          nk_size_t row_start, nk_size_t row_count);                                  \
+    NK_DYNAMIC nk_size_t nk_dots_packed_size_##T##_gfx950(nk_size_t width, nk_size_t depth);                          \
+    NK_DYNAMIC void nk_dots_pack_##T##_gfx950(in_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,    \
+                                              void *b_packed);                                                        \
+    NK_DYNAMIC void nk_dots_packed_##T##_gfx950(in_t const *a, void const *b_packed, out_t *c, nk_size_t height,      \
+                                                nk_size_t width, nk_size_t depth, nk_size_t a_stride,                 \
+                                                nk_size_t c_stride);                                                  \
+    NK_DYNAMIC void nk_dots_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,     \
+                                                   nk_size_t stride, out_t *result, nk_size_t result_stride,          \
+                                                   nk_size_t row_start, nk_size_t row_count);
+NK_AMD_DECLARE_DOTS_ONLY_(e2m3, nk_e2m3_t, nk_f32_t)
+NK_AMD_DECLARE_DOTS_ONLY_(e3m2, nk_e3m2_t, nk_f32_t)
+NK_AMD_DECLARE_DOTS_ONLY_(i4, nk_i4x2_t, nk_i32_t)
+NK_AMD_DECLARE_DOTS_ONLY_(u4, nk_u4x2_t, nk_u32_t)
+#undef NK_AMD_DECLARE_DOTS_ONLY_
 
 /* Capability and lookup API. Reference: c/numkong.c:767-768, 831-913. */
 NK_DYNAMIC int nk_uses_dynamic_dispatch(void);

@@ -7,6 +7,7 @@ reference's Python entry points ``dots_pack`` / ``dots_packed`` / ``dots_symmetr
 (reference: python/matrix.c:151-227, 324-622) for tensors that already live on the GPU, using PyTorch only to own device memory.
 """
 from .api import (  # noqa: F401
+    DISTANCE_DTYPES,
     DTYPES,
     NumKongAmdError,
     PackedMatrix,

@@ -23,16 +23,25 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # nk_dtype_t codes (reference: include/numkong/types.h:923-952)
 NK_I8, NK_I32, NK_U8, NK_U32 = 1 << 2, 1 << 4, 1 << 6, 1 << 8
 NK_F32, NK_F16, NK_BF16, NK_E4M3, NK_E5M2 = 1 << 11, 1 << 12, 1 << 13, 1 << 14, 1 << 15
+NK_I4, NK_U4, NK_E2M3, NK_E3M2 = 1 << 16, 1 << 17, 1 << 18, 1 << 19
 
-# name -> (nk code, element bytes, output torch dtype name)
+# name -> (nk code, bytes per stored value, output torch dtype name, dimensions per stored value)
 DTYPES = {
-    "i8": (NK_I8, 1, "int32"),
-    "u8": (NK_U8, 1, "int32"),  # u32 results are returned as their int32 bit patterns
-    "bf16": (NK_BF16, 2, "float32"),
-    "f16": (NK_F16, 2, "float32"),
-    "e4m3": (NK_E4M3, 1, "float32"),
-    "e5m2": (NK_E5M2, 1, "float32"),
+    "i8": (NK_I8, 1, "int32", 1),
+    "u8": (NK_U8, 1, "int32", 1),  # u32 results are returned as their int32 bit patterns
+    "bf16": (NK_BF16, 2, "float32", 1),
+    "f16": (NK_F16, 2, "float32", 1),
+    "e4m3": (NK_E4M3, 1, "float32", 1),
+    "e5m2": (NK_E5M2, 1, "float32", 1),
+    "e2m3": (NK_E2M3, 1, "float32", 1),  # 6-bit floats, one per byte
+    "e3m2": (NK_E3M2, 1, "float32", 1),
+    "i4": (NK_I4, 1, "int32", 2),  # two 4-bit values per byte: a (rows, depth / 2) byte tensor, as the reference's
+    "u4": (NK_U4, 1, "int32", 2),  # bindings take them (python/matrix.c:603: depth *= dimensions per value)
 }
+
+
+# the types that also have the distance kinds (the 6-bit floats and 4-bit integers have dot products only)
+DISTANCE_DTYPES = ("i8", "u8", "bf16", "f16", "e4m3", "e5m2")
 
 
 class NumKongAmdError(RuntimeError):
@@ -70,10 +79,11 @@ def library() -> ctypes.CDLL:
         getattr(lib, f"nk_dots_pack_{name}").argtypes = [vp, sz, sz, sz, vp]
         getattr(lib, f"nk_dots_packed_{name}").restype = None
         getattr(lib, f"nk_dots_packed_{name}").argtypes = [vp, vp, vp, sz, sz, sz, sz, sz]
-        for stem in ("nk_angulars_packed_", "nk_euclideans_packed_"):
+        for stem in ("nk_angulars_packed_", "nk_euclideans_packed_") if name in DISTANCE_DTYPES else ():
             getattr(lib, stem + name).restype = None
             getattr(lib, stem + name).argtypes = [vp, vp, vp, sz, sz, sz, sz, sz]
-        for stem in ("nk_dots_symmetric_", "nk_angulars_symmetric_", "nk_euclideans_symmetric_"):
+        stems = ("nk_dots_symmetric_", "nk_angulars_symmetric_", "nk_euclideans_symmetric_")
+        for stem in stems if name in DISTANCE_DTYPES else stems[:1]:
             getattr(lib, stem + name).restype = None
             getattr(lib, stem + name).argtypes = [vp, sz, sz, sz, vp, sz, sz, sz]
     lib.nk_amd_symmetric_workspace_size.restype = sz
@@ -153,12 +163,12 @@ def dots_pack(b, dtype: str) -> PackedMatrix:
     import torch
 
     b = _as_matrix(b, dtype, "b")
-    width, depth = int(b.shape[0]), int(b.shape[1])
+    width, depth = int(b.shape[0]), int(b.shape[1]) * DTYPES[dtype][3]
     size = dots_packed_size(dtype, width, depth)
     if size == 0:
         raise NumKongAmdError("nk_dots_packed_size returned 0 (unsupported dtype or dimensions)")
     buffer = torch.empty(size, dtype=torch.uint8, device=b.device)
-    stride = int(b.stride(0)) * b.element_size() if width > 1 else depth * b.element_size()
+    stride = int(b.stride(0)) * b.element_size() if width > 1 else int(b.shape[1]) * b.element_size()
     getattr(library(), f"nk_dots_pack_{dtype}")(b.data_ptr(), width, depth, stride, buffer.data_ptr())
     _check("nk_dots_pack_" + dtype)
     return PackedMatrix(dtype, width, depth, buffer)
@@ -170,7 +180,7 @@ def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out):
     if not isinstance(packed, PackedMatrix):
         raise TypeError("packed must be a PackedMatrix from dots_pack()")
     a = _as_matrix(a, packed.dtype, "a")
-    height, depth = int(a.shape[0]), int(a.shape[1])
+    height, depth = int(a.shape[0]), int(a.shape[1]) * DTYPES[packed.dtype][3]
     if depth != packed.depth:
         raise ValueError(f"depth mismatch: a has {depth} columns, packed matrix has depth {packed.depth}")
     out_dtype = getattr(torch, out_dtype_name)
@@ -185,7 +195,7 @@ def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out):
             raise TypeError(f"out must have dtype {out_dtype}")
         if packed.width > 1 and out.stride(1) != 1:
             raise ValueError("out rows must be contiguous")
-    a_stride = int(a.stride(0)) * a.element_size() if height > 1 else depth * a.element_size()
+    a_stride = int(a.stride(0)) * a.element_size() if height > 1 else int(a.shape[1]) * a.element_size()
     c_stride = int(out.stride(0)) * 4 if height > 1 else packed.width * 4
     getattr(library(), stem + packed.dtype)(
         a.data_ptr(), packed.buffer.data_ptr(), out.data_ptr(), height, packed.width, depth, a_stride, c_stride
@@ -200,13 +210,22 @@ def dots_packed(a, packed: PackedMatrix, out=None):
                            a, packed, out)
 
 
+def _needs_distances(dtype: str) -> None:
+    if dtype not in DISTANCE_DTYPES:
+        raise TypeError(f"dtype {dtype!r} has the dot-product kinds only; distances need one of {DISTANCE_DTYPES}")
+
+
 def angulars_packed(a, packed: PackedMatrix, out=None):
     """Angular distances ``1 - cos(a_i, b_j)`` as float32 (reference: ``nk_angulars_packed_<dtype>``)."""
+    if isinstance(packed, PackedMatrix):
+        _needs_distances(packed.dtype)
     return _packed_product("nk_angulars_packed_", "float32", a, packed, out)
 
 
 def euclideans_packed(a, packed: PackedMatrix, out=None):
     """Euclidean distances ``|a_i - b_j|`` as float32 (reference: ``nk_euclideans_packed_<dtype>``)."""
+    if isinstance(packed, PackedMatrix):
+        _needs_distances(packed.dtype)
     return _packed_product("nk_euclideans_packed_", "float32", a, packed, out)
 
 
@@ -214,7 +233,7 @@ def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_r
     import torch
 
     vectors = _as_matrix(vectors, dtype, "vectors")
-    count, depth = int(vectors.shape[0]), int(vectors.shape[1])
+    count, depth = int(vectors.shape[0]), int(vectors.shape[1]) * DTYPES[dtype][3]
     out_dtype = getattr(torch, out_dtype_name)
     if out is None:
         # (the reference leaves what it does not write uninitialised; zeros are easier on the eye)
@@ -232,7 +251,7 @@ def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_r
     last = count if end_row is None else int(end_row)
     if first < 0 or last < 0 or first > count or last > count or first > last:
         raise ValueError(f"Invalid row range [{first}, {last}) for {count} vectors")
-    stride = int(vectors.stride(0)) * vectors.element_size() if count > 1 else depth * vectors.element_size()
+    stride = int(vectors.stride(0)) * vectors.element_size() if count > 1 else int(vectors.shape[1]) * vectors.element_size()
     out_stride = int(out.stride(0)) * 4 if count > 1 else count * 4
     getattr(library(), stem + dtype)(vectors.data_ptr(), count, depth, stride, out.data_ptr(), out_stride, first, last - first)
     _check(stem + dtype)
@@ -249,9 +268,11 @@ def dots_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
 
 def angulars_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
     """Upper triangle of the pairwise angular distances as float32; the diagonal is exactly 0."""
+    _needs_distances(dtype)
     return _symmetric("nk_angulars_symmetric_", "float32", vectors, dtype, out, start_row, end_row)
 
 
 def euclideans_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
     """Upper triangle of the pairwise euclidean distances as float32; the diagonal is exactly 0."""
+    _needs_distances(dtype)
     return _symmetric("nk_euclideans_symmetric_", "float32", vectors, dtype, out, start_row, end_row)

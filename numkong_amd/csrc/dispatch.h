@@ -3,7 +3,7 @@
  *  @file numkong_amd/csrc/dispatch.h
  *
  *  Mirrors the role of the reference's c/dispatch.h:37-506, reduced to the packed-dots, packed-distance and symmetric slots
- *  (reference slots: c/dispatch.h:279-336, 353-380) for i8, u8, bf16, f16, e4m3, e5m2.
+ *  (reference slots: c/dispatch.h:279-336, 353-380) for i8, u8, bf16, f16, e4m3, e5m2, e2m3, e3m2, i4, u4.
  */
 #ifndef NUMKONG_AMD_DISPATCH_H
 #define NUMKONG_AMD_DISPATCH_H
@@ -16,16 +16,20 @@ extern "C" {
 
 typedef struct {
     nk_dots_packed_size_punned_t dots_packed_size_i8, dots_packed_size_u8, dots_packed_size_bf16,
-        dots_packed_size_f16, dots_packed_size_e4m3, dots_packed_size_e5m2;
-    nk_dots_pack_punned_t dots_pack_i8, dots_pack_u8, dots_pack_bf16, dots_pack_f16, dots_pack_e4m3, dots_pack_e5m2;
+        dots_packed_size_f16, dots_packed_size_e4m3, dots_packed_size_e5m2, dots_packed_size_e2m3, dots_packed_size_e3m2,
+        dots_packed_size_i4, dots_packed_size_u4;
+    nk_dots_pack_punned_t dots_pack_i8, dots_pack_u8, dots_pack_bf16, dots_pack_f16, dots_pack_e4m3, dots_pack_e5m2, dots_pack_e2m3, dots_pack_e3m2,
+        dots_pack_i4, dots_pack_u4;
     nk_dots_packed_punned_t dots_packed_i8, dots_packed_u8, dots_packed_bf16, dots_packed_f16, dots_packed_e4m3,
-        dots_packed_e5m2;
+        dots_packed_e5m2, dots_packed_e2m3, dots_packed_e3m2,
+        dots_packed_i4, dots_packed_u4;
     nk_dots_packed_punned_t angulars_packed_i8, angulars_packed_u8, angulars_packed_bf16, angulars_packed_f16,
         angulars_packed_e4m3, angulars_packed_e5m2;
     nk_dots_packed_punned_t euclideans_packed_i8, euclideans_packed_u8, euclideans_packed_bf16, euclideans_packed_f16,
         euclideans_packed_e4m3, euclideans_packed_e5m2;
     nk_dots_symmetric_punned_t dots_symmetric_i8, dots_symmetric_u8, dots_symmetric_bf16, dots_symmetric_f16,
-        dots_symmetric_e4m3, dots_symmetric_e5m2;
+        dots_symmetric_e4m3, dots_symmetric_e5m2, dots_symmetric_e2m3, dots_symmetric_e3m2,
+        dots_symmetric_i4, dots_symmetric_u4;
     nk_dots_symmetric_punned_t angulars_symmetric_i8, angulars_symmetric_u8, angulars_symmetric_bf16,
         angulars_symmetric_f16, angulars_symmetric_e4m3, angulars_symmetric_e5m2;
     nk_dots_symmetric_punned_t euclideans_symmetric_i8, euclideans_symmetric_u8, euclideans_symmetric_bf16,
@@ -54,6 +58,10 @@ NK_AMD_DECLARE_DISPATCH_(bf16)
 NK_AMD_DECLARE_DISPATCH_(f16)
 NK_AMD_DECLARE_DISPATCH_(e4m3)
 NK_AMD_DECLARE_DISPATCH_(e5m2)
+NK_AMD_DECLARE_DISPATCH_(e2m3)
+NK_AMD_DECLARE_DISPATCH_(e3m2)
+NK_AMD_DECLARE_DISPATCH_(i4)
+NK_AMD_DECLARE_DISPATCH_(u4)
 #undef NK_AMD_DECLARE_DISPATCH_
 
 /**
@@ -112,6 +120,42 @@ NK_AMD_DECLARE_DISPATCH_(e5m2)
                                 (nk_kernel_punned_t *)&t->angulars_symmetric_##T, &used);                             \
         nk_dispatch_##T##_find_(caps, nk_kernel_euclideans_symmetric_k,                                               \
                                 (nk_kernel_punned_t *)&t->euclideans_symmetric_##T, &used);                           \
+    }
+
+/** The same for the types that have the dot-product kinds only (the 6-bit floats, the 4-bit integers). */
+#define NK_AMD_DEFINE_DISPATCH_DOTS_(T)                                                                               \
+    void nk_dispatch_##T##_find_(nk_capability_t v, nk_kernel_kind_t k, nk_kernel_punned_t *m, nk_capability_t *c) { \
+        typedef nk_kernel_punned_t m_t;                                                                               \
+        if (v & nk_cap_gfx950_k) switch (k) {                                                                         \
+            case nk_kernel_dots_packed_size_k:                                                                        \
+                *m = (m_t)&nk_dots_packed_size_##T##_gfx950, *c = nk_cap_gfx950_k;                                    \
+                return;                                                                                               \
+            case nk_kernel_dots_pack_k: *m = (m_t)&nk_dots_pack_##T##_gfx950, *c = nk_cap_gfx950_k; return;          \
+            case nk_kernel_dots_packed_k: *m = (m_t)&nk_dots_packed_##T##_gfx950, *c = nk_cap_gfx950_k; return;      \
+            case nk_kernel_dots_symmetric_k: *m = (m_t)&nk_dots_symmetric_##T##_gfx950, *c = nk_cap_gfx950_k; return; \
+            default: break;                                                                                           \
+            }                                                                                                         \
+        switch (k) {                                                                                                  \
+        case nk_kernel_dots_packed_size_k: *m = (m_t)nk_error_packed_size_, *c = 0; return;                          \
+        case nk_kernel_dots_pack_k: *m = (m_t)nk_error_pack_, *c = 0; return;                                        \
+        case nk_kernel_dots_packed_k:                                                                                 \
+        case nk_kernel_angulars_packed_k:                                                                             \
+        case nk_kernel_euclideans_packed_k: *m = (m_t)nk_error_dots_, *c = 0; return;                                \
+        case nk_kernel_dots_symmetric_k:                                                                              \
+        case nk_kernel_angulars_symmetric_k:                                                                          \
+        case nk_kernel_euclideans_symmetric_k: *m = (m_t)nk_error_dots_symmetric_, *c = 0; return;                   \
+        default: *m = (m_t)nk_error_dense_, *c = 0; return;                                                          \
+        }                                                                                                             \
+    }                                                                                                                 \
+    void nk_dispatch_##T##_init_(nk_capability_t caps) {                                                              \
+        nk_implementations_t *t = &nk_dispatch_table;                                                                 \
+        nk_capability_t used;                                                                                         \
+        nk_dispatch_##T##_find_(caps, nk_kernel_dots_packed_size_k, (nk_kernel_punned_t *)&t->dots_packed_size_##T,  \
+                                &used);                                                                               \
+        nk_dispatch_##T##_find_(caps, nk_kernel_dots_pack_k, (nk_kernel_punned_t *)&t->dots_pack_##T, &used);         \
+        nk_dispatch_##T##_find_(caps, nk_kernel_dots_packed_k, (nk_kernel_punned_t *)&t->dots_packed_##T, &used);     \
+        nk_dispatch_##T##_find_(caps, nk_kernel_dots_symmetric_k, (nk_kernel_punned_t *)&t->dots_symmetric_##T,      \
+                                &used);                                                                               \
     }
 
 #ifdef __cplusplus

@@ -1,9 +1,9 @@
 /**
- *  @brief Dispatch for F16 packed dots: binds the table slots and `nk_find_kernel_punned` to gfx950.
+ *  @brief Dispatch for the F16 kinds: binds the table slots and `nk_find_kernel_punned` to gfx950.
  *  @file numkong_amd/csrc/dispatch_f16.c
  *
- *  Counterpart of the reference's c/dispatch_f16.c (`nk_dispatch_f16_find_`, `nk_dispatch_f16_init_`),
- *  for the kinds nk_kernel_dots_packed_size_k, nk_kernel_dots_pack_k, nk_kernel_dots_packed_k only.
+ *  Counterpart of the reference's c/dispatch_f16.c (`nk_dispatch_f16_find_`, `nk_dispatch_f16_init_`), for the kinds
+ *  this backend serves: the packed dots (size, pack, product), the packed distances and the symmetric kinds.
  */
 #include "dispatch.h"
 

@@ -108,7 +108,7 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
     if (!make_geometry(dtype, n, k, g)) return fail_msg("nk_hip_dots_pack: unsupported dtype or dimensions");
     if (!b_packed || ((uintptr_t)b_packed & 15)) return fail_msg("nk_hip_dots_pack: b_packed must be 16-byte aligned");
     if (n && k && !b) return fail_msg("nk_hip_dots_pack: b is NULL");
-    if (g.elem_bytes == 2 && (((uintptr_t)b | b_stride) & 1)) return fail_msg("nk_hip_dots_pack: 16-bit B is misaligned");
+    if (elem_bits_of(dtype) == 16 && (((uintptr_t)b | b_stride) & 1)) return fail_msg("nk_hip_dots_pack: 16-bit B is misaligned");
 
     PackedHeader h;
     memset(&h, 0, sizeof(h));
@@ -132,7 +132,16 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
         uint64_t const blocks = (uint64_t)g.n_tiles * (g.k_chunks / kStageChunks);
         if (blocks > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_pack: matrix too large");
         uint32_t const xr = dtype == kU8 ? 0x80808080u : 0u;
-        auto kernel = dtype == kE4M3 ? pack_kernel<1> : (dtype == kE5M2 ? pack_kernel<2> : pack_kernel<0>);
+        void (*kernel)(uint8_t const *, uint64_t, uint32_t, uint64_t, uint32_t, uint8_t *, int, uint32_t, PackedHeader) = pack_kernel<0>;
+        switch (widen_kind_of(dtype)) {
+        case 1: kernel = pack_kernel<1>; break;
+        case 2: kernel = pack_kernel<2>; break;
+        case 3: kernel = pack_kernel<3>; break;
+        case 4: kernel = pack_kernel<4>; break;
+        case 5: kernel = pack_kernel<5>; break;
+        case 6: kernel = pack_kernel<6>; break;
+        default: break;
+        }
         hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride,
                            g.n, g.k_src_bytes, g.k_chunks, data, widest_load(b, b_stride), xr, h);
         e = hipGetLastError();
@@ -140,8 +149,10 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
     }
     if (g.n_tiles && terms) {
         if (g.k_chunks) {
-            auto kernel = dtype == kI8 ? column_terms_kernel<0>
-                          : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
+            // by what the image holds: signed bytes (i8 and the widened 4-bit types), offset u8, bf16, f16 (and what is widened to it)
+            auto kernel = dtype == kI8 || dtype == kI4 || dtype == kU4
+                              ? column_terms_kernel<0>
+                              : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
             hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(256), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);
         }
         else {
@@ -194,7 +205,7 @@ static int product_async(int dtype, int metric, void const *a, void const *b_pac
         return e == hipSuccess ? 0 : fail(e, "fill_rows_kernel");
     }
     if (!a) return fail_msg("nk_hip_dots_packed: a is NULL");
-    if (geo.elem_bytes == 2 && (((uintptr_t)a | a_stride) & 1)) return fail_msg("nk_hip_dots_packed: 16-bit A is misaligned");
+    if (elem_bits_of(dtype) == 16 && (((uintptr_t)a | a_stride) & 1)) return fail_msg("nk_hip_dots_packed: 16-bit A is misaligned");
 
     GemmArgs g;
     memset(&g, 0, sizeof(g));
@@ -218,6 +229,10 @@ static int product_async(int dtype, int metric, void const *a, void const *b_pac
     case kF16: e = launch_f16(g, stream, triangle); break;
     case kE4M3: e = launch_e4m3(g, stream, triangle); break;
     case kE5M2: e = launch_e5m2(g, stream, triangle); break;
+    case kE2M3: e = launch_e2m3(g, stream, triangle); break;
+    case kE3M2: e = launch_e3m2(g, stream, triangle); break;
+    case kI4: e = launch_i4(g, stream, triangle); break;
+    case kU4: e = launch_u4(g, stream, triangle); break;
     default: return fail_msg("nk_hip_dots_packed: unsupported dtype");
     }
     return e == hipSuccess ? 0 : fail(e, "dots_packed_kernel");

@@ -80,6 +80,10 @@ hipError_t launch_bf16(GemmArgs &g, hipStream_t stream, TriangleScratch const *t
 hipError_t launch_f16(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
 hipError_t launch_e4m3(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
 hipError_t launch_e5m2(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_e2m3(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_e3m2(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_i4(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_u4(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
 
 extern int g_forced_config; // 0: the heuristic picks the tile shape; see nk_hip_set_tile_config
 extern int g_variant;       // timing experiments of tuning builds
@@ -107,6 +111,10 @@ enum : int {
     kBF16 = 1 << 13,
     kE4M3 = 1 << 14,
     kE5M2 = 1 << 15,
+    kI4 = 1 << 16, // two 4-bit integers per byte, the even dimension in the low nibble
+    kU4 = 1 << 17,
+    kE2M3 = 1 << 18, // 6-bit floats, one per byte (bits 6 and 7 ignored)
+    kE3M2 = 1 << 19,
 };
 
 constexpr uint32_t kMagic = 0x35394B4Eu; // "NK95"
@@ -134,22 +142,27 @@ struct PackedHeader {
 static_assert(sizeof(PackedHeader) == 64, "header must stay 64 bytes");
 
 struct Geometry {
-    uint32_t elem_bytes;   // bytes per element in the caller's A and B
+    uint32_t elem_bytes;   // bytes per element in the caller's A and B (1 for the 4-bit types, two to a byte)
     uint32_t packed_bytes; // bytes per element in the image and in LDS (fp8 is widened to f16)
     uint32_t n, k, n_tiles, k_chunks;
     uint64_t k_bytes;      // bytes of one packed row: k * packed_bytes
-    uint64_t k_src_bytes;  // bytes of one source row: k * elem_bytes
+    uint64_t k_src_bytes;  // bytes of one source row
     uint64_t data_bytes, sums_bytes, norms_bytes, total_bytes;
 };
 
-inline int elem_bytes_of(int dtype) {
+/** Bits per element in the caller's A and B (0: not a type of this backend). */
+inline int elem_bits_of(int dtype) {
     switch (dtype) {
+    case kI4:
+    case kU4: return 4;
     case kI8:
     case kU8:
     case kE4M3:
-    case kE5M2: return 1;
+    case kE5M2:
+    case kE2M3:
+    case kE3M2: return 8;
     case kF16:
-    case kBF16: return 2;
+    case kBF16: return 16;
     default: return 0;
     }
 }
@@ -157,16 +170,28 @@ inline int elem_bytes_of(int dtype) {
 /** The fp8 MFMA forms of gfx950 align the products inside one lane's k-group to the largest of them and
  *  keep only about 14 bits (1 + 2^-14 comes back as 1), far from the f32 accumulation of the reference's
  *  kernels (dot/serial.h:522-600). e4m3 and e5m2 are therefore widened, exactly, to f16 and run on the f16
- *  MFMA, whose products and sums are kept to full f32 precision: B at pack time, A on its way into LDS. */
-inline int packed_bytes_of(int dtype) { return (dtype == kE4M3 || dtype == kE5M2) ? 2 : elem_bytes_of(dtype); }
+ *  MFMA, whose products and sums are kept to full f32 precision: B at pack time, A on its way into LDS.
+ *  The 6-bit floats go the same way (every e2m3 / e3m2 value is an f16 value), and the 4-bit integers are
+ *  widened to i8 for the i8 MFMA. */
+inline int packed_bytes_of(int dtype) {
+    switch (dtype) {
+    case kE4M3:
+    case kE5M2:
+    case kE2M3:
+    case kE3M2: return 2;
+    case kI4:
+    case kU4: return 1;
+    default: return elem_bits_of(dtype) / 8;
+    }
+}
 
 inline bool make_geometry(int dtype, size_t n, size_t k, Geometry &g) {
-    int const eb = elem_bytes_of(dtype);
-    if (!eb) return false;
+    int const bits = elem_bits_of(dtype);
+    if (!bits) return false;
     if (n > 0x7FFFFFFFull || k > 0x3FFFFFFFull) return false;
-    g.elem_bytes = (uint32_t)eb, g.packed_bytes = (uint32_t)packed_bytes_of(dtype), g.n = (uint32_t)n, g.k = (uint32_t)k;
+    g.elem_bytes = (uint32_t)(bits + 7) / 8, g.packed_bytes = (uint32_t)packed_bytes_of(dtype), g.n = (uint32_t)n, g.k = (uint32_t)k;
     g.k_bytes = (uint64_t)k * g.packed_bytes;
-    g.k_src_bytes = (uint64_t)k * eb;
+    g.k_src_bytes = ((uint64_t)k * bits + 7) / 8; // (4-bit types: whole bytes, as the reference loads them, cast/serial.h:533-538)
     uint64_t const chunks = (g.k_bytes + kChunkBytes - 1) / kChunkBytes;
     g.k_chunks = (uint32_t)((chunks + 2 * kStageChunks - 1) / (2 * kStageChunks) * (2 * kStageChunks)); // an even number of stages
     g.n_tiles = (uint32_t)((n + kTileRows - 1) / kTileRows);
@@ -231,12 +256,76 @@ __device__ __forceinline__ v4i widen_fp8x8(uint32_t lo, uint32_t hi) {
     return out;
 }
 
+/**
+ *  Eight 6-bit floats, one per byte (two dwords) -> eight f16 values, exact. Both formats are IEEE-like with
+ *  subnormals and no Inf/NaN (e2m3: 2 exponent bits, bias 1; e3m2: 3 exponent bits, bias 3; reference decoders:
+ *  cast/serial.h:1318-1330, 1455-1470), so the exponent and mantissa bits, moved under an f16's sign bit, read as the
+ *  value scaled by a power of two, subnormals included: one packed multiply by 2^14 (e2m3) or 2^12 (e3m2) finishes
+ *  two values at a time. Bits 6 and 7 of a byte are ignored, as the reference does.
+ */
+template <bool E3M2>
+__device__ __forceinline__ v4i widen_fp6x8(uint32_t lo, uint32_t hi) {
+    typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+    constexpr int kShift = E3M2 ? 8 : 7; // exponent field up to bit 10 of the f16
+    v2h const scale = E3M2 ? v2h {(_Float16)4096.0f, (_Float16)4096.0f} : v2h {(_Float16)16384.0f, (_Float16)16384.0f};
+    v4i out;
+#pragma unroll
+    for (int pair = 0; pair < 4; ++pair) {
+        uint32_t const word = pair < 2 ? lo : hi;
+        // bytes 2 * (pair % 2) and 2 * (pair % 2) + 1 of the word, each in a 16-bit lane of its own
+        uint32_t const codes = __builtin_amdgcn_perm(0u, word, pair % 2 ? 0x0C030C02u : 0x0C010C00u);
+        uint32_t const bits = ((codes << 10) & 0x80008000u) | ((codes & 0x001F001Fu) << kShift);
+        v2h const value = __builtin_bit_cast(v2h, bits) * scale;
+        out[pair] = __builtin_bit_cast(int, value);
+    }
+    return out;
+}
+
+/** Sixteen 4-bit integers (two dwords; the even dimension in the low nibble) -> sixteen i8 values: the low nibbles
+ *  of a dword's four bytes, then its high nibbles (any order serves as long as A and B use the same one).
+ *  Signed: a nibble n with bit 3 set becomes n | 0xF0, the byte-wise (n ^ 8) - 8 of dot/serial.h:781-785. */
+template <bool SIGNED>
+__device__ __forceinline__ v4i widen_i4x16(uint32_t lo, uint32_t hi) {
+    auto extend = [](uint32_t nibbles) {
+        if (!SIGNED) return nibbles;
+        uint32_t const top = nibbles & 0x08080808u;
+        return nibbles | ((top << 5) - (top << 1)); // 0xF0 where bit 3 is set (the last byte's carry leaves the word)
+    };
+    v4i out;
+    out[0] = (int)extend(lo & 0x0F0F0F0Fu), out[1] = (int)extend((lo >> 4) & 0x0F0F0F0Fu);
+    out[2] = (int)extend(hi & 0x0F0F0F0Fu), out[3] = (int)extend((hi >> 4) & 0x0F0F0F0Fu);
+    return out;
+}
+
+/** Widening of 8 source bytes to one 16-byte chunk, by kind: 1 e4m3, 2 e5m2, 3 e2m3, 4 e3m2 (to f16); 5 i4, 6 u4
+ *  (to i8). */
+template <int WIDEN>
+__device__ __forceinline__ v4i widen_chunk(uint32_t lo, uint32_t hi) {
+    if constexpr (WIDEN == 1) return widen_fp8x8<false>(lo, hi);
+    else if constexpr (WIDEN == 2) return widen_fp8x8<true>(lo, hi);
+    else if constexpr (WIDEN == 3) return widen_fp6x8<false>(lo, hi);
+    else if constexpr (WIDEN == 4) return widen_fp6x8<true>(lo, hi);
+    else if constexpr (WIDEN == 5) return widen_i4x16<true>(lo, hi);
+    else return widen_i4x16<false>(lo, hi);
+}
+inline int widen_kind_of(int dtype) {
+    switch (dtype) {
+    case kE4M3: return 1;
+    case kE5M2: return 2;
+    case kE2M3: return 3;
+    case kE3M2: return 4;
+    case kI4: return 5;
+    case kU4: return 6;
+    default: return 0;
+    }
+}
+
 #pragma region Packing
 
 /**
  *  One thread per 16-byte chunk of the image. A block of 256 threads covers 32 rows x 8 chunks: reads are
- *  128 (64 for fp8) contiguous bytes per row, writes are eight 512-byte runs. WIDEN: 0 copies the
- *  elements, 1 widens e4m3 to f16, 2 widens e5m2 to f16 (8 source bytes per chunk).
+ *  128 (64 for the widened types) contiguous bytes per row, writes are eight 512-byte runs. WIDEN: 0 copies the
+ *  elements, otherwise the kind of widen_chunk (8 source bytes per chunk).
  */
 template <int WIDEN>
 __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
@@ -260,7 +349,7 @@ __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b
             v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
         }
         else { v = load_chunk_guarded(src, valid, avec, xr); }
-        if (WIDEN) v = widen_fp8x8<WIDEN == 2>((uint32_t)v[0], (uint32_t)v[1]);
+        if constexpr (WIDEN != 0) v = widen_chunk<WIDEN>((uint32_t)v[0], (uint32_t)v[1]);
     }
     *(v4i *)(data + (((uint64_t)tile * k_chunks + c) * kTileRows + r) * kChunkBytes) = v;
 }
@@ -381,6 +470,7 @@ struct I8 {
     typedef uint32_t norm_t; // what a row's sum of squares accumulates in
     static constexpr int kDtype = kI8;
     static constexpr bool kUnsigned = false;
+    static constexpr bool kDistances = true; // the distance kinds are built for this type (NORMS kernels)
     /** Sum of the squares of the source values behind one staged chunk (`raw`: as loaded, `wide`: as it goes to LDS). */
     static __device__ __forceinline__ norm_t sumsq(v4i raw, v4i) {
         int sum = 0;
@@ -410,6 +500,7 @@ struct BF16 {
     typedef double norm_t;
     static constexpr int kDtype = kBF16;
     static constexpr bool kUnsigned = false;
+    static constexpr bool kDistances = true;
     /** The 8 products are exact in f32; their short sum is rounded a few times, the long sum runs in f64. */
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) {
         float sum = 0;
@@ -434,6 +525,7 @@ struct F16 {
     typedef double norm_t;
     static constexpr int kDtype = kF16;
     static constexpr bool kUnsigned = false;
+    static constexpr bool kDistances = true;
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { // also e4m3 / e5m2, which are f16 by then
         typedef _Float16 v2h __attribute__((ext_vector_type(2)));
         float sum = 0;
@@ -464,6 +556,37 @@ struct E5M2 : F16 {
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<true>((uint32_t)v[0], (uint32_t)v[1]); }
 };
+/** The 6-bit floats run widened to f16 as well; see widen_fp6x8. */
+struct E2M3 : F16 {
+    static constexpr bool kChunked = true;
+    static constexpr int kDtype = kE2M3;
+    static constexpr bool kDistances = false; // dot products only
+    static constexpr int kSrcChunk = 8;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp6x8<false>((uint32_t)v[0], (uint32_t)v[1]); }
+};
+struct E3M2 : F16 {
+    static constexpr bool kChunked = true;
+    static constexpr int kDtype = kE3M2;
+    static constexpr bool kDistances = false; // dot products only
+    static constexpr int kSrcChunk = 8;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp6x8<true>((uint32_t)v[0], (uint32_t)v[1]); }
+};
+/** The 4-bit integers run widened to i8 on the i8 MFMA; see widen_i4x16. Unsigned nibbles are non-negative i8 values
+ *  as they are: none of u8's offset arithmetic. */
+struct I4 : I8 {
+    static constexpr int kDtype = kI4;
+    static constexpr bool kDistances = false; // dot products only
+    static constexpr int kSrcChunk = 8;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_i4x16<true>((uint32_t)v[0], (uint32_t)v[1]); }
+    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); }
+};
+struct U4 : I8 {
+    static constexpr int kDtype = kU4;
+    static constexpr bool kDistances = false; // dot products only
+    static constexpr int kSrcChunk = 8;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_i4x16<false>((uint32_t)v[0], (uint32_t)v[1]); }
+    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); }
+};
 
 /**
  *  Distances from a dot product and two sums of squares, as the reference's scalar finalisers compute them
@@ -473,8 +596,8 @@ struct E5M2 : F16 {
  */
 template <class T>
 __device__ __forceinline__ float norm_as_f32(uint32_t bits) {
-    if (T::kDtype == kI8) return (float)(int)bits;
-    if (T::kDtype == kU8) return (float)bits;
+    if (T::kDtype == kI8 || T::kDtype == kI4) return (float)(int)bits;
+    if (T::kDtype == kU8 || T::kDtype == kU4) return (float)bits;
     return __builtin_bit_cast(float, bits);
 }
 
@@ -485,7 +608,9 @@ __device__ __forceinline__ float norm_as_f32(uint32_t bits) {
  *  would save half of the operations and lose exactly that). */
 template <class T, int METRIC>
 __device__ __forceinline__ uint32_t distance_from_dot(uint32_t dot_bits, float query, float target) {
-    float const dot = T::kDtype == kI8 ? (float)(int)dot_bits : (T::kDtype == kU8 ? (float)dot_bits : __builtin_bit_cast(float, dot_bits));
+    float const dot = T::kDtype == kI8 || T::kDtype == kI4
+                          ? (float)(int)dot_bits
+                          : (T::kDtype == kU8 || T::kDtype == kU4 ? (float)dot_bits : __builtin_bit_cast(float, dot_bits));
     float result;
     if (METRIC == 1) {
         float const product = query * target;
@@ -1285,8 +1410,11 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
     uint32_t const stages = g.k_chunks / kStageChunks;
     bool const across = g.avec >= 4 && stages >= 4 && !(g_variant & 1);
     bool const norms = g.metric != 0;
-    void (*kernel)(GemmArgs) = norms ? (across ? dots_packed_kernel<T, TM, TN, true, true> : dots_packed_kernel<T, TM, TN, false, true>)
-                                     : (across ? dots_packed_kernel<T, TM, TN, true, false> : dots_packed_kernel<T, TM, TN, false, false>);
+    void (*kernel)(GemmArgs) = across ? dots_packed_kernel<T, TM, TN, true, false> : dots_packed_kernel<T, TM, TN, false, false>;
+    if constexpr (T::kDistances) {
+        if (norms) kernel = across ? dots_packed_kernel<T, TM, TN, true, true> : dots_packed_kernel<T, TM, TN, false, true>;
+    }
+    else if (norms) return hipErrorInvalidValue;
 #ifdef NK_TUNE // timing experiments that leave parts of the loop out (results are wrong on purpose)
     if constexpr (TM == 8 && TN == 2 && T::kDtype == kI8) {
         switch (g_variant >> 2) {

@@ -28,14 +28,19 @@ static void nk_amd_set_error_(char const *where) {
 
 char const *nk_amd_last_error(void) { return nk_amd_error_; }
 
-static size_t nk_amd_element_bytes_(nk_dtype_t dtype) {
+/** Bytes of one row of `k` elements: two 4-bit values to a byte, whole bytes (cast/serial.h:533-538). */
+static size_t nk_amd_row_bytes_(nk_dtype_t dtype, size_t k) {
     switch (dtype) {
+    case nk_i4_k:
+    case nk_u4_k: return (k + 1) / 2;
     case nk_i8_k:
     case nk_u8_k:
     case nk_e4m3_k:
-    case nk_e5m2_k: return 1;
+    case nk_e5m2_k:
+    case nk_e2m3_k:
+    case nk_e3m2_k: return k;
     case nk_f16_k:
-    case nk_bf16_k: return 2;
+    case nk_bf16_k: return k * 2;
     default: return 0;
     }
 }
@@ -77,7 +82,6 @@ static nk_size_t nk_amd_packed_size_(nk_dtype_t dtype, nk_size_t n, nk_size_t k)
 static void nk_amd_pack_(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t k, nk_size_t b_stride,
                          void *b_packed) {
     nk_amd_error_[0] = 0;
-    size_t const element_bytes = nk_amd_element_bytes_(dtype);
     size_t const total = nk_hip_dots_packed_size((int)dtype, n, k);
     if (!total || !b_packed) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_pack: unsupported dtype or dimensions");
@@ -96,7 +100,7 @@ static void nk_amd_pack_(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t
     int status = 0;
 
     if (b_kind == 0) {
-        size_t const row_bytes = k * element_bytes;
+        size_t const row_bytes = nk_amd_row_bytes_(dtype, k);
         device_b_stride = nk_amd_round_up_(row_bytes, 16);
         status = nk_hip_malloc(&staged_b, n * device_b_stride);
         if (!status) status = nk_hip_memcpy2d_h2d(staged_b, device_b_stride, b, b_stride, row_bytes, n, NULL);
@@ -119,7 +123,6 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
                            nk_size_t n, nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {
     nk_amd_error_[0] = 0;
     if (!m || !n) return;
-    size_t const element_bytes = nk_amd_element_bytes_(dtype);
     size_t const total = nk_hip_dots_packed_size((int)dtype, n, k);
     if (nk_hip_device_count() <= 0) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_packed: no HIP device");
@@ -141,7 +144,7 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
     int status = 0;
 
     if (a_kind == 0) {
-        size_t const row_bytes = k * element_bytes;
+        size_t const row_bytes = nk_amd_row_bytes_(dtype, k);
         device_a_stride = nk_amd_round_up_(row_bytes, 16);
         status = nk_hip_malloc(&staged_a, m * device_a_stride);
         if (!status) status = nk_hip_memcpy2d_h2d(staged_a, device_a_stride, a, a_stride, row_bytes, m, NULL);
@@ -210,7 +213,6 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
                               nk_size_t row_count) {
     nk_amd_error_[0] = 0;
     if (!n || !row_count || row_start >= n) return;
-    size_t const element_bytes = nk_amd_element_bytes_(dtype);
     if (nk_hip_device_count() <= 0) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_symmetric: no HIP device");
         nk_amd_fill_symmetric_error_(result, 0, n, result_stride);
@@ -234,7 +236,7 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
     int status = nk_hip_malloc(&workspace, workspace_bytes);
 
     if (!status && v_kind == 0) {
-        size_t const row_bytes = k * element_bytes;
+        size_t const row_bytes = nk_amd_row_bytes_(dtype, k);
         device_stride = nk_amd_round_up_(row_bytes, 16);
         status = nk_hip_malloc(&staged_v, (n - first) * device_stride);
         if (!status)
@@ -268,7 +270,7 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
     if (workspace) nk_hip_free(workspace);
 }
 
-#define NK_AMD_DEFINE_BACKEND_(T, in_t, out_t)                                                                     \
+#define NK_AMD_DEFINE_BACKEND_DOTS_(T, in_t, out_t)                                                                     \
     nk_size_t nk_dots_packed_size_##T##_gfx950(nk_size_t width, nk_size_t depth) {                                 \
         return nk_amd_packed_size_(nk_##T##_k, width, depth);                                                      \
     }                                                                                                              \
@@ -280,6 +282,14 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
                                      nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride) {   \
         nk_amd_packed_(nk_##T##_k, 0, a, b_packed, c, height, width, depth, a_stride, c_stride);                   \
     }                                                                                                              \
+    void nk_dots_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,             \
+                                        nk_size_t stride, out_t *result, nk_size_t result_stride,                  \
+                                        nk_size_t row_start, nk_size_t row_count) {                                \
+        nk_amd_symmetric_(nk_##T##_k, 0, vectors, vectors_count, depth, stride, result, result_stride, row_start,  \
+                          row_count);                                                                              \
+    }
+
+#define NK_AMD_DEFINE_BACKEND_DISTANCES_(T, in_t)                                                                   \
     void nk_angulars_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,       \
                                          nk_size_t width, nk_size_t depth, nk_size_t a_stride,                     \
                                          nk_size_t c_stride) {                                                     \
@@ -289,12 +299,6 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
                                            nk_size_t width, nk_size_t depth, nk_size_t a_stride,                   \
                                            nk_size_t c_stride) {                                                   \
         nk_amd_packed_(nk_##T##_k, 2, a, b_packed, c, height, width, depth, a_stride, c_stride);                   \
-    }                                                                                                              \
-    void nk_dots_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,             \
-                                        nk_size_t stride, out_t *result, nk_size_t result_stride,                  \
-                                        nk_size_t row_start, nk_size_t row_count) {                                \
-        nk_amd_symmetric_(nk_##T##_k, 0, vectors, vectors_count, depth, stride, result, result_stride, row_start,  \
-                          row_count);                                                                              \
     }                                                                                                              \
     void nk_angulars_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,         \
                                             nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,           \
@@ -309,9 +313,19 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
                           row_count);                                                                              \
     }
 
-NK_AMD_DEFINE_BACKEND_(i8, nk_i8_t, nk_i32_t)
-NK_AMD_DEFINE_BACKEND_(u8, nk_u8_t, nk_u32_t)
-NK_AMD_DEFINE_BACKEND_(bf16, nk_bf16_t, nk_f32_t)
-NK_AMD_DEFINE_BACKEND_(f16, nk_f16_t, nk_f32_t)
-NK_AMD_DEFINE_BACKEND_(e4m3, nk_e4m3_t, nk_f32_t)
-NK_AMD_DEFINE_BACKEND_(e5m2, nk_e5m2_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(i8, nk_i8_t, nk_i32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(i8, nk_i8_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(u8, nk_u8_t, nk_u32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(u8, nk_u8_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(bf16, nk_bf16_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(bf16, nk_bf16_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(f16, nk_f16_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(f16, nk_f16_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(e4m3, nk_e4m3_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(e4m3, nk_e4m3_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(e5m2, nk_e5m2_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(e5m2, nk_e5m2_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(e2m3, nk_e2m3_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(i4, nk_i4x2_t, nk_i32_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(u4, nk_u4x2_t, nk_u32_t)

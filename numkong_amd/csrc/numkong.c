@@ -50,7 +50,7 @@ void nk_error_dots_symmetric_(void const *vectors, nk_size_t n_vectors, nk_size_
     nk_error_dots_(vectors, 0, result, n_vectors, n_vectors, depth, stride, result_stride);
 }
 
-#define NK_AMD_DISPATCH_CROSS_(T, in_t, out_t)                                                                  \
+#define NK_AMD_DISPATCH_DOTS_(T, in_t, out_t)                                                                   \
     NK_DYNAMIC nk_size_t nk_dots_packed_size_##T(nk_size_t n, nk_size_t k) {                                    \
         return nk_dispatch_table.dots_packed_size_##T(n, k);                                                    \
     }                                                                                                           \
@@ -62,19 +62,21 @@ void nk_error_dots_symmetric_(void const *vectors, nk_size_t n_vectors, nk_size_
                                        nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {                   \
         nk_dispatch_table.dots_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                         \
     }                                                                                                           \
-    NK_DYNAMIC void nk_angulars_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t m,      \
-                                           nk_size_t n, nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) { \
-        nk_dispatch_table.angulars_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                     \
-    }                                                                                                           \
-    NK_DYNAMIC void nk_euclideans_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t m,    \
-                                             nk_size_t n, nk_size_t k, nk_size_t a_stride,                      \
-                                             nk_size_t c_stride) {                                              \
-        nk_dispatch_table.euclideans_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                   \
-    }                                                                                                           \
     NK_DYNAMIC void nk_dots_symmetric_##T(in_t const *vectors, nk_size_t n, nk_size_t k, nk_size_t stride,      \
                                           out_t *result, nk_size_t result_stride, nk_size_t row_start,          \
                                           nk_size_t row_count) {                                                \
         nk_dispatch_table.dots_symmetric_##T(vectors, n, k, stride, result, result_stride, row_start, row_count); \
+    }
+
+#define NK_AMD_DISPATCH_DISTANCES_(T, in_t)                                                                     \
+    NK_DYNAMIC void nk_angulars_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t m,       \
+                                           nk_size_t n, nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {  \
+        nk_dispatch_table.angulars_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                     \
+    }                                                                                                           \
+    NK_DYNAMIC void nk_euclideans_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t m,     \
+                                             nk_size_t n, nk_size_t k, nk_size_t a_stride,                      \
+                                             nk_size_t c_stride) {                                              \
+        nk_dispatch_table.euclideans_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                   \
     }                                                                                                           \
     NK_DYNAMIC void nk_angulars_symmetric_##T(in_t const *vectors, nk_size_t n, nk_size_t k, nk_size_t stride,  \
                                               nk_f32_t *result, nk_size_t result_stride, nk_size_t row_start,   \
@@ -89,12 +91,22 @@ void nk_error_dots_symmetric_(void const *vectors, nk_size_t n_vectors, nk_size_
                                                    row_count);                                                  \
     }
 
-NK_AMD_DISPATCH_CROSS_(i8, nk_i8_t, nk_i32_t)
-NK_AMD_DISPATCH_CROSS_(u8, nk_u8_t, nk_u32_t)
-NK_AMD_DISPATCH_CROSS_(bf16, nk_bf16_t, nk_f32_t)
-NK_AMD_DISPATCH_CROSS_(f16, nk_f16_t, nk_f32_t)
-NK_AMD_DISPATCH_CROSS_(e4m3, nk_e4m3_t, nk_f32_t)
-NK_AMD_DISPATCH_CROSS_(e5m2, nk_e5m2_t, nk_f32_t)
+NK_AMD_DISPATCH_DOTS_(i8, nk_i8_t, nk_i32_t)
+NK_AMD_DISPATCH_DISTANCES_(i8, nk_i8_t)
+NK_AMD_DISPATCH_DOTS_(u8, nk_u8_t, nk_u32_t)
+NK_AMD_DISPATCH_DISTANCES_(u8, nk_u8_t)
+NK_AMD_DISPATCH_DOTS_(bf16, nk_bf16_t, nk_f32_t)
+NK_AMD_DISPATCH_DISTANCES_(bf16, nk_bf16_t)
+NK_AMD_DISPATCH_DOTS_(f16, nk_f16_t, nk_f32_t)
+NK_AMD_DISPATCH_DISTANCES_(f16, nk_f16_t)
+NK_AMD_DISPATCH_DOTS_(e4m3, nk_e4m3_t, nk_f32_t)
+NK_AMD_DISPATCH_DISTANCES_(e4m3, nk_e4m3_t)
+NK_AMD_DISPATCH_DOTS_(e5m2, nk_e5m2_t, nk_f32_t)
+NK_AMD_DISPATCH_DISTANCES_(e5m2, nk_e5m2_t)
+NK_AMD_DISPATCH_DOTS_(e2m3, nk_e2m3_t, nk_f32_t)
+NK_AMD_DISPATCH_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
+NK_AMD_DISPATCH_DOTS_(i4, nk_i4x2_t, nk_i32_t)
+NK_AMD_DISPATCH_DOTS_(u4, nk_u4x2_t, nk_u32_t)
 
 NK_DYNAMIC int nk_uses_dynamic_dispatch(void) { return 1; }
 
@@ -124,6 +136,10 @@ NK_DYNAMIC void nk_dispatch_table_update(nk_capability_t caps) {
     nk_dispatch_f16_init_(caps);
     nk_dispatch_e4m3_init_(caps);
     nk_dispatch_e5m2_init_(caps);
+    nk_dispatch_e2m3_init_(caps);
+    nk_dispatch_e3m2_init_(caps);
+    nk_dispatch_i4_init_(caps);
+    nk_dispatch_u4_init_(caps);
 }
 
 NK_DYNAMIC void nk_find_kernel_punned(nk_kernel_kind_t kind, nk_dtype_t dtype, nk_capability_t viable,
@@ -137,6 +153,10 @@ NK_DYNAMIC void nk_find_kernel_punned(nk_kernel_kind_t kind, nk_dtype_t dtype, n
     case nk_f16_k: nk_dispatch_f16_find_(viable, kind, m, c); return;
     case nk_e4m3_k: nk_dispatch_e4m3_find_(viable, kind, m, c); return;
     case nk_e5m2_k: nk_dispatch_e5m2_find_(viable, kind, m, c); return;
+    case nk_e2m3_k: nk_dispatch_e2m3_find_(viable, kind, m, c); return;
+    case nk_e3m2_k: nk_dispatch_e3m2_find_(viable, kind, m, c); return;
+    case nk_i4_k: nk_dispatch_i4_find_(viable, kind, m, c); return;
+    case nk_u4_k: nk_dispatch_u4_find_(viable, kind, m, c); return;
     default: break;
     }
     *m = (nk_kernel_punned_t)0;
@@ -153,17 +173,21 @@ NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t i
         case nk_f16_k:
         case nk_e4m3_k:
         case nk_e5m2_k: return nk_f32_k;
-        default: return nk_dtype_unknown_k;
+        default: return nk_dtype_unknown_k; /* (the 6-bit floats and 4-bit integers have the dot-product kinds only) */
         }
     }
     if (kind != nk_kernel_dots_packed_k && kind != nk_kernel_dots_symmetric_k) return nk_dtype_unknown_k;
     switch (input) {
-    case nk_i8_k: return nk_i32_k;
-    case nk_u8_k: return nk_u32_k;
+    case nk_i8_k:
+    case nk_i4_k: return nk_i32_k;
+    case nk_u8_k:
+    case nk_u4_k: return nk_u32_k;
     case nk_bf16_k:
     case nk_f16_k:
     case nk_e4m3_k:
-    case nk_e5m2_k: return nk_f32_k;
+    case nk_e5m2_k:
+    case nk_e2m3_k:
+    case nk_e3m2_k: return nk_f32_k;
     default: return nk_dtype_unknown_k;
     }
 }

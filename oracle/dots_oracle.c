@@ -44,6 +44,14 @@
  *      nk_{angulars,euclideans}_symmetric_<T>_serial (bit for bit for i8/u8, float types as above), over windows that
  *      start and end off the reference's 32- and 128-row blocks, and against the packed restatement with B = A.
  *
+ *    - the remaining narrow types of the dots family, products only (packed and symmetric): e2m3 and e3m2 (decoded by
+ *      the formats' definition, 4 f32 lane sums like the other float types), i4 and u4 (two nibbles per byte, the even
+ *      dimension in the low one, whole bytes even for an odd depth; exact)
+ *          include/numkong/cast/serial.h:533-538, 1280-1330, 1418-1470, include/numkong/dot/serial.h:602-800
+ *      Pinned bit for bit against nk_cast_serial (all 256 byte values decode; encoder on finite probes incl. every
+ *      tie) and nk_dots_packed_<T>_serial / nk_dots_symmetric_<T>_serial; their distance kinds are not restated
+ *      (and not built).
+ *
  *  Parity unpinned: the per-column norms of FLOAT types in the serial packed image as stored bytes (the
  *  reference computes them with the host-dispatched nk_reduce_moments_*, whose summation order is not restated
  *  here). They are not read by dots_packed; nko_serial_pack writes zeros there and the tests compare header +
@@ -61,6 +69,10 @@ enum {
     NKO_BF16 = 1 << 13,
     NKO_E4M3 = 1 << 14,
     NKO_E5M2 = 1 << 15,
+    NKO_I4 = 1 << 16,   /* two 4-bit integers per byte, the even dimension in the low nibble */
+    NKO_U4 = 1 << 17,
+    NKO_E2M3 = 1 << 18, /* 6-bit floats, one per byte, bits 6 and 7 ignored */
+    NKO_E3M2 = 1 << 19,
 };
 
 #define NKO_API __attribute__((visibility("default")))
@@ -88,6 +100,10 @@ typedef struct {
 static small_format_t const k_f16 = {5, 10, 15, 1, 0, 0, 0x7E00};
 static small_format_t const k_e4m3 = {4, 3, 7, 0, 1, 1, 0x7F};
 static small_format_t const k_e5m2 = {5, 2, 15, 1, 0, 0, 0x7D};
+/* FP6: no Inf, no NaN, overflow saturates (cast/serial.h:1280-1330, 1333-1339, 1418-1470); a NaN input has no
+ * defined image here and is not used. */
+static small_format_t const k_e2m3 = {2, 3, 1, 0, 0, 1, 0x1F};
+static small_format_t const k_e3m2 = {3, 2, 3, 0, 0, 1, 0x1F};
 
 static float small_decode(small_format_t const *fmt, uint32_t code) {
     int const total = 1 + fmt->ebits + fmt->mbits;
@@ -120,7 +136,8 @@ static uint32_t small_encode(small_format_t const *fmt, float x) {
     uint32_t const magnitude_bits = bits & 0x7FFFFFFFu;
     uint32_t const e_max = (1u << fmt->ebits) - 1;
     uint32_t const max_finite = fmt->has_inf ? ((e_max << fmt->mbits) - 1)        /* largest below Inf   */
-                                             : ((e_max << fmt->mbits) | ((1u << fmt->mbits) - 2)); /* E4M3FN: 0x7E */
+                                : fmt->nan_is_all_ones ? ((e_max << fmt->mbits) | ((1u << fmt->mbits) - 2)) /* E4M3FN: 0x7E */
+                                                       : ((e_max << fmt->mbits) | ((1u << fmt->mbits) - 1)); /* FP6: every code is a number */
     uint32_t const inf_code = e_max << fmt->mbits;
     if (magnitude_bits > 0x7F800000u) {
         if (fmt->mbits == 10) { /* f16 keeps the truncated payload, never letting it become zero */
@@ -167,6 +184,10 @@ NKO_API float nko_e4m3_to_f32(uint8_t x) { return small_decode(&k_e4m3, x); }
 NKO_API uint8_t nko_f32_to_e4m3(float x) { return (uint8_t)small_encode(&k_e4m3, x); }
 NKO_API float nko_e5m2_to_f32(uint8_t x) { return small_decode(&k_e5m2, x); }
 NKO_API uint8_t nko_f32_to_e5m2(float x) { return (uint8_t)small_encode(&k_e5m2, x); }
+NKO_API float nko_e2m3_to_f32(uint8_t x) { return small_decode(&k_e2m3, x & 0x3Fu); }
+NKO_API uint8_t nko_f32_to_e2m3(float x) { return (uint8_t)small_encode(&k_e2m3, x); }
+NKO_API float nko_e3m2_to_f32(uint8_t x) { return small_decode(&k_e3m2, x & 0x3Fu); }
+NKO_API uint8_t nko_f32_to_e3m2(float x) { return (uint8_t)small_encode(&k_e3m2, x); }
 
 /* bf16 is the top half of an f32; the reference rounds by adding 0x7FFF plus the kept LSB and does not
  * special-case NaN or overflow (cast/serial.h:768-784), which is restated literally because it defines
@@ -190,9 +211,22 @@ static int element_bytes(int dtype) {
     }
 }
 
+/* 4-bit types: a row of `depth` dimensions is read as whole bytes, both nibbles of the last one included when the
+ * depth is odd, exactly as the reference's loads do (cast/serial.h:533-538, dot/serial.h:705-718, 777-790). */
+static size_t effective_depth(int dtype, size_t depth) {
+    return dtype == NKO_I4 || dtype == NKO_U4 ? (depth + 1) / 2 * 2 : depth;
+}
+
 /* Value of element `i` of a row as f32 (integers are exact in f32 too: |x| <= 255). */
 static float element_f32(int dtype, void const *row, size_t i) {
     switch (dtype) {
+    case NKO_U4: return (float)((((uint8_t const *)row)[i / 2] >> (4 * (i & 1))) & 0xF);
+    case NKO_I4: {
+        int const nibble = (((uint8_t const *)row)[i / 2] >> (4 * (i & 1))) & 0xF;
+        return (float)((nibble ^ 8) - 8); /* dot/serial.h:781-785 */
+    }
+    case NKO_E2M3: return nko_e2m3_to_f32(((uint8_t const *)row)[i]);
+    case NKO_E3M2: return nko_e3m2_to_f32(((uint8_t const *)row)[i]);
     case NKO_I8: return (float)((int8_t const *)row)[i];
     case NKO_U8: return (float)((uint8_t const *)row)[i];
     case NKO_F16: return nko_f16_to_f32(((uint16_t const *)row)[i]);
@@ -213,6 +247,8 @@ NKO_API void nko_encode(int dtype, float const *src, size_t count, void *dst) {
         case NKO_BF16: ((uint16_t *)dst)[i] = nko_f32_to_bf16(src[i]); break;
         case NKO_E4M3: ((uint8_t *)dst)[i] = nko_f32_to_e4m3(src[i]); break;
         case NKO_E5M2: ((uint8_t *)dst)[i] = nko_f32_to_e5m2(src[i]); break;
+        case NKO_E2M3: ((uint8_t *)dst)[i] = nko_f32_to_e2m3(src[i]); break;
+        case NKO_E3M2: ((uint8_t *)dst)[i] = nko_f32_to_e3m2(src[i]); break;
         default: break;
         }
 }
@@ -321,6 +357,7 @@ NKO_API void nko_serial_packed(int dtype, void const *a, void const *packed, voi
  *  when `magnitude` is not NULL, sum |a * b| per element, the scale of the normwise error. */
 NKO_API void nko_dots_f64(int dtype, void const *a, void const *b, double *c, double *magnitude, size_t rows,
                           size_t columns, size_t depth, size_t a_stride, size_t b_stride) {
+    depth = effective_depth(dtype, depth);
     for (size_t i = 0; i < rows; ++i) {
         unsigned char const *a_row = (unsigned char const *)a + i * a_stride;
         for (size_t j = 0; j < columns; ++j) {
@@ -473,15 +510,12 @@ NKO_API void nko_spatials_f64(int dtype, int metric, void const *a, void const *
  *  same init/update/finalize functions for both; f16 goes through nk_dot_f16x8_*_serial, dot/serial.h:345-374,
  *  which keeps the same four lane sums, lane = k mod 4, as the f32x4 path of its packed kernel). */
 static uint32_t serial_dot_bits(int dtype, void const *a_row, void const *b_row, size_t depth) {
-    if (dtype == NKO_I8) {
+    depth = effective_depth(dtype, depth);
+    if (dtype == NKO_I8 || dtype == NKO_U8 || dtype == NKO_I4 || dtype == NKO_U4) {
+        /* exact in 64 bits, truncated to 32: i64 for the signed types, u64 for the unsigned, the same bits either way */
         int64_t sum = 0;
-        for (size_t l = 0; l < depth; ++l) sum += (int64_t)((int8_t const *)a_row)[l] * ((int8_t const *)b_row)[l];
-        return (uint32_t)(int32_t)sum;
-    }
-    if (dtype == NKO_U8) {
-        uint64_t sum = 0;
-        for (size_t l = 0; l < depth; ++l) sum += (uint64_t)((uint8_t const *)a_row)[l] * ((uint8_t const *)b_row)[l];
-        return (uint32_t)sum;
+        for (size_t l = 0; l < depth; ++l) sum += (int64_t)element_f32(dtype, a_row, l) * (int64_t)element_f32(dtype, b_row, l);
+        return (uint32_t)(uint64_t)sum;
     }
     float lanes[4] = {0, 0, 0, 0};
     for (size_t l = 0; l < depth; ++l) {
@@ -489,6 +523,18 @@ static uint32_t serial_dot_bits(int dtype, void const *a_row, void const *b_row,
         lanes[l & 3] += product;
     }
     return f32_to_bits(((lanes[0] + lanes[1]) + lanes[2]) + lanes[3]);
+}
+
+/** C = A * B^T with the serial backend's rounding from UNPACKED operands: what nk_dots_packed_<T>_serial returns for
+ *  any of the ten types (for the six older ones it equals nko_serial_pack + nko_serial_packed, which also restate
+ *  the serial image; for e2m3, e3m2, i4, u4 only the arithmetic is restated: dot/serial.h:602-800). */
+NKO_API void nko_serial_dots(int dtype, void const *a, void const *b, void *c, size_t rows, size_t columns, size_t depth,
+                             size_t a_stride, size_t b_stride, size_t c_stride) {
+    for (size_t i = 0; i < rows; ++i) {
+        uint32_t *out = (uint32_t *)((unsigned char *)c + i * c_stride);
+        for (size_t j = 0; j < columns; ++j)
+            out[j] = serial_dot_bits(dtype, (unsigned char const *)a + i * a_stride, (unsigned char const *)b + j * b_stride, depth);
+    }
 }
 
 /** nk_dots_symmetric_<T>_serial (metric 0), nk_angulars_symmetric_<T>_serial (1), nk_euclideans_symmetric_<T>_serial

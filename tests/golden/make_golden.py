@@ -20,7 +20,7 @@ def main():
         raise SystemExit("build oracle/_ref first: make -C oracle")
     out = support.GOLDEN_DIR
     rng = np.random.default_rng(2024)
-    only = sys.argv[1] if len(sys.argv) > 1 else ""  # e.g. "spatials" or "symmetric": rewrite only that family's files
+    only = sys.argv[1] if len(sys.argv) > 1 else ""  # e.g. "spatials", "symmetric" or "narrow": rewrite only that family's files
     for dtype in support.FLOAT_DTYPES if only in ("", "cast", "dots") else []:
         codes = np.arange(256 if support.STORAGE[dtype] == np.uint8 else 65536).astype(support.STORAGE[dtype])
         if len(codes) > 256:
@@ -83,6 +83,22 @@ def main():
                             row_count=row_count, dots_serial=results["dots"].astype(support.OUTPUT[dtype]),
                             angulars_serial=results["angular"].astype(np.float32),
                             euclideans_serial=results["euclidean"].astype(np.float32))
+    # The narrow types (dot-product kinds only): a ragged packed product with an odd depth, all 256 decodings of the
+    # 6-bit floats, and a symmetric window; owned elements only, zeros elsewhere.
+    rng = np.random.default_rng(2027)
+    for dtype in support.NARROW_DTYPES if only in ("", "narrow") else []:
+        a = np.ascontiguousarray(support.random_matrix(oracle, dtype, 13, 77, rng, pad=3))
+        b = np.ascontiguousarray(support.random_matrix(oracle, dtype, 21, 77, rng, pad=1))
+        count, depth, row_start, row_count = 45, 202, 5, 34
+        vectors = np.ascontiguousarray(support.random_matrix(oracle, dtype, count, depth, rng))
+        i, j = np.arange(count)[:, None], np.arange(count)[None, :]
+        own = (i >= row_start) & (i < row_start + row_count) & (j >= i)
+        extra = {"decoded": reference.cast(np.arange(256, dtype=np.uint8), dtype, "f32")} if dtype in support.NARROW_FLOAT_DTYPES else {}
+        np.savez_compressed(os.path.join(out, f"narrow_{dtype}.npz"), dtype=dtype, a=a, b=b,
+                            c_serial=reference.dots_packed(dtype, a, b), vectors=vectors, row_start=row_start,
+                            row_count=row_count,
+                            symmetric_serial=np.where(own, reference.symmetric("dots", dtype, vectors, row_start, row_count), 0)
+                            .astype(support.OUTPUT[dtype]), **extra)
     print("wrote", len(os.listdir(out)) - 1, "fixtures to", out)
 
 

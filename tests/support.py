@@ -17,11 +17,23 @@ REFERENCE_PATH = os.path.join(ROOT, "oracle", "_ref", "libnumkong.so")
 GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
 
 # nk_dtype_t codes (reference: include/numkong/types.h:923-952)
-CODES = {"i8": 1 << 2, "u8": 1 << 6, "f32": 1 << 11, "f16": 1 << 12, "bf16": 1 << 13, "e4m3": 1 << 14, "e5m2": 1 << 15}
-STORAGE = {"i8": np.int8, "u8": np.uint8, "f16": np.uint16, "bf16": np.uint16, "e4m3": np.uint8, "e5m2": np.uint8}
-OUTPUT = {"i8": np.int32, "u8": np.uint32, "f16": np.float32, "bf16": np.float32, "e4m3": np.float32, "e5m2": np.float32}
+CODES = {"i8": 1 << 2, "u8": 1 << 6, "f32": 1 << 11, "f16": 1 << 12, "bf16": 1 << 13, "e4m3": 1 << 14, "e5m2": 1 << 15,
+         "i4": 1 << 16, "u4": 1 << 17, "e2m3": 1 << 18, "e3m2": 1 << 19}
+STORAGE = {"i8": np.int8, "u8": np.uint8, "f16": np.uint16, "bf16": np.uint16, "e4m3": np.uint8, "e5m2": np.uint8,
+           "i4": np.uint8, "u4": np.uint8, "e2m3": np.uint8, "e3m2": np.uint8}
+OUTPUT = {"i8": np.int32, "u8": np.uint32, "f16": np.float32, "bf16": np.float32, "e4m3": np.float32, "e5m2": np.float32,
+          "i4": np.int32, "u4": np.uint32, "e2m3": np.float32, "e3m2": np.float32}
 FLOAT_DTYPES = ("bf16", "f16", "e4m3", "e5m2")
-ALL_DTYPES = ("i8", "u8") + FLOAT_DTYPES
+ALL_DTYPES = ("i8", "u8") + FLOAT_DTYPES  # the types with every kind: packed dots, packed distances, symmetric
+# the types with the dot-product kinds only: 6-bit floats (one per byte), 4-bit integers (two per byte)
+NARROW_FLOAT_DTYPES = ("e2m3", "e3m2")
+NARROW_DTYPES = NARROW_FLOAT_DTYPES + ("i4", "u4")
+DIMENSIONS_PER_VALUE = {"i4": 2, "u4": 2}
+
+
+def depth_of(dtype: str, matrix: np.ndarray) -> int:
+    """Dimensions of a row: the stored values times the dimensions each holds (two for the 4-bit types)."""
+    return matrix.shape[1] * DIMENSIONS_PER_VALUE.get(dtype, 1)
 KIND_SIZE, KIND_PACK, KIND_PACKED = ord("P"), ord("Q"), ord("G")
 KIND_ANGULARS, KIND_EUCLIDEANS = ord("N"), ord("E")  # packed distances: same prototype as the packed product
 # symmetric kinds (vectors, count, depth, stride, result, result_stride, row_start, row_count), by metric
@@ -54,11 +66,13 @@ class Oracle:
         lib.nko_serial_spatials.argtypes = [_i32, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz]
         lib.nko_spatials_f64.argtypes = [_i32, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
         lib.nko_serial_symmetric.argtypes = [_i32, _i32, _vp, _sz, _sz, _sz, _vp, _sz, _sz, _sz]
+        lib.nko_serial_dots.argtypes = [_i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz]
 
     def decode(self, dtype: str, codes: np.ndarray) -> np.ndarray:
         codes = np.ascontiguousarray(codes, dtype=STORAGE[dtype])
-        out = np.empty(codes.shape, dtype=np.float32)
-        self.lib.nko_decode(CODES[dtype], _ptr(codes), codes.size, _ptr(out))
+        per = DIMENSIONS_PER_VALUE.get(dtype, 1)
+        out = np.empty(codes.shape[:-1] + (codes.shape[-1] * per,), dtype=np.float32)
+        self.lib.nko_decode(CODES[dtype], _ptr(codes), out.size, _ptr(out))
         return out
 
     def encode(self, dtype: str, values: np.ndarray) -> np.ndarray:
@@ -77,11 +91,15 @@ class Oracle:
         return packed
 
     def dots_packed(self, dtype: str, a: np.ndarray, b: np.ndarray) -> np.ndarray:
-        """C = A @ B.T with the serial backend's rounding (pack + packed product)."""
-        m, k = a.shape
+        """C = A @ B.T with the serial backend's rounding (pack + packed product; the narrow types, whose serial image
+        is not restated, straight from the unpacked rows)."""
+        m, k = a.shape[0], depth_of(dtype, a)
         n = b.shape[0]
-        packed = self.pack(dtype, b)
         c = np.empty((m, n), dtype=OUTPUT[dtype])
+        if dtype in NARROW_DTYPES:
+            self.lib.nko_serial_dots(CODES[dtype], _ptr(a), _ptr(b), _ptr(c), m, n, k, a.strides[0], b.strides[0], c.strides[0])
+            return c
+        packed = self.pack(dtype, b)
         self.lib.nko_serial_packed(CODES[dtype], _ptr(a), _ptr(packed), _ptr(c), m, n, k, a.strides[0], c.strides[0])
         return c
 
@@ -113,7 +131,7 @@ class Oracle:
                   out: np.ndarray = None) -> np.ndarray:
         """`nk_{dots,angulars,euclideans}_symmetric_<dtype>_serial` into `out` (count x count; fresh and zeroed when
         not given): only result[i][j], i in the row window, j >= i, is written."""
-        count, depth = vectors.shape
+        count, depth = vectors.shape[0], depth_of(dtype, vectors)
         if out is None:
             out = np.zeros((count, count), dtype=OUTPUT[dtype] if metric == "dots" else np.float32)
         rows = count - row_start if row_count is None else row_count
@@ -123,7 +141,7 @@ class Oracle:
 
     def truth(self, dtype: str, a: np.ndarray, b: np.ndarray):
         """(f64 ground truth, sum |a*b|) as the reference's own tests compute it."""
-        m, k = a.shape
+        m, k = a.shape[0], depth_of(dtype, a)
         n = b.shape[0]
         c = np.empty((m, n), dtype=np.float64)
         mag = np.empty((m, n), dtype=np.float64)
@@ -178,13 +196,13 @@ class Reference:
         return int(self.kernel(KIND_SIZE, dtype, viable)[0](n, k))
 
     def pack(self, dtype: str, b: np.ndarray, viable: int = CAP_SERIAL) -> np.ndarray:
-        n, k = b.shape
+        n, k = b.shape[0], depth_of(dtype, b)
         packed = np.zeros(self.packed_size(dtype, n, k, viable) + 64, dtype=np.uint8)
         self.kernel(KIND_PACK, dtype, viable)[0](_ptr(b), n, k, b.strides[0], _ptr(packed))
         return packed
 
     def dots_packed(self, dtype: str, a: np.ndarray, b: np.ndarray, viable: int = CAP_SERIAL) -> np.ndarray:
-        m, k = a.shape
+        m, k = a.shape[0], depth_of(dtype, a)
         n = b.shape[0]
         packed = self.pack(dtype, b, viable)
         c = np.empty((m, n), dtype=OUTPUT[dtype])
@@ -203,7 +221,7 @@ class Reference:
     def symmetric(self, metric: str, dtype: str, vectors: np.ndarray, row_start: int = 0, row_count=None,
                   out: np.ndarray = None, viable: int = CAP_SERIAL) -> np.ndarray:
         """The chosen backend's symmetric kernel into `out` (count x count; fresh and zeroed when not given)."""
-        count, depth = vectors.shape
+        count, depth = vectors.shape[0], depth_of(dtype, vectors)
         if out is None:
             out = np.zeros((count, count), dtype=OUTPUT[dtype] if metric == "dots" else np.float32)
         rows = count - row_start if row_count is None else row_count
@@ -233,6 +251,12 @@ def random_matrix(oracle: Oracle, dtype: str, rows: int, cols: int, rng: np.rand
            "fp8"       N(0,1) scaled to half of the largest finite value, 1 % exact zeros
     """
     shape = (rows, cols + pad)
+    if dtype in ("i4", "u4"):  # `cols` dimensions, two to a byte: every byte value, both nibbles random
+        packed = rng.integers(0, 256, size=(rows, (cols + 1) // 2 + pad), dtype=np.uint8)
+        return packed[:, : (cols + 1) // 2] if pad else packed
+    if dtype in NARROW_FLOAT_DTYPES and kind == "default":  # every 6-bit code is a finite number; the top two bits are ignored
+        full = rng.integers(0, 256, size=shape, dtype=np.uint8)
+        return full[:, :cols] if pad else full
     if dtype == "i8":
         full = rng.integers(-128, 128, size=shape, dtype=np.int8)
     elif dtype == "u8":

@@ -161,7 +161,7 @@ def test_python_mirror_validates_arguments():
     with pytest.raises(ValueError):
         nk.dots_pack(cpu, "i8")  # must live on the GPU
     with pytest.raises(TypeError):
-        nk.dots_pack(cpu, "i4")
+        nk.dots_pack(cpu, "u1")
     with pytest.raises(TypeError):
         nk.dots_pack([[1, 2]], "i8")
     with pytest.raises(TypeError):
@@ -170,3 +170,5 @@ def test_python_mirror_validates_arguments():
         nk.dots_symmetric(cpu, "i8")  # must live on the GPU
     with pytest.raises(TypeError):
         nk.angulars_symmetric(cpu, "f64")
+    with pytest.raises(TypeError):
+        nk.euclideans_symmetric(cpu, "i4")  # the 4-bit integers have the dot-product kinds only

@@ -16,7 +16,7 @@ import numpy as np
 import pytest
 
 from tests import support
-from tests.support import ALL_DTYPES, FLOAT_DTYPES, STORAGE
+from tests.support import ALL_DTYPES, FLOAT_DTYPES, NARROW_DTYPES, NARROW_FLOAT_DTYPES, STORAGE
 
 
 def same_floats(x, y):
@@ -319,6 +319,72 @@ def test_symmetric_equals_packed_with_both_sides_the_same(oracle, dtype):
         assert not np.diag(got).any()
 
 
+@pytest.mark.parametrize("dtype", NARROW_FLOAT_DTYPES)
+def test_six_bit_floats_match_reference_and_definition(oracle, reference, dtype):
+    """All 256 byte values decode as the format defines them (sign, `e` exponent bits with bias, `m` mantissa bits,
+    subnormals, no Inf or NaN, bits 6 and 7 ignored), and as nk_cast_serial decodes them; the encoder agrees with it on
+    finite probes including every tie between neighbours of the grid."""
+    ebits, mbits, bias = {"e2m3": (2, 3, 1), "e3m2": (3, 2, 3)}[dtype]
+    codes = np.arange(256, dtype=np.uint8)
+    got = oracle.decode(dtype, codes[None, :])[0]
+    for code in range(256):
+        sign, e, m = (code >> 5) & 1, (code >> mbits) & ((1 << ebits) - 1), code & ((1 << mbits) - 1)
+        expected = m * 2.0 ** (1 - bias - mbits) if e == 0 else (1 + m / 2.0 ** mbits) * 2.0 ** (e - bias)
+        assert float(got[code]) == (-expected if sign else expected), hex(code)
+    assert float(got.max()) == {"e2m3": 7.5, "e3m2": 28.0}[dtype]
+    if reference is None:
+        pytest.skip("reference build not present")
+    assert same_floats(got, reference.cast(codes, dtype, "f32"))
+    rng = np.random.default_rng(3)
+    grid = np.unique(np.abs(got))
+    mids = ((grid[:-1].astype(np.float64) + grid[1:]) / 2).astype(np.float32)
+    probes = np.concatenate([grid, mids, np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf)),
+                             np.array([30, 100, 1e6, 1e-3, 1e-8], np.float32)]
+                            + [rng.standard_normal(20000).astype(np.float32) * np.float32(scale) for scale in (0.01, 0.3, 2, 10, 100)])
+    probes = np.concatenate([probes, -probes])
+    assert np.array_equal(oracle.encode(dtype, probes), reference.cast(probes, "f32", dtype))
+
+
+@pytest.mark.parametrize("dtype", NARROW_DTYPES)
+def test_narrow_products_match_reference_serial(oracle, reference, dtype):
+    """nk_dots_packed_<T>_serial and nk_dots_symmetric_<T>_serial for e2m3, e3m2, i4, u4, bit for bit, odd depths
+    (whole bytes for the 4-bit types, both nibbles of the last one) included."""
+    if reference is None:
+        pytest.skip("reference build not present")
+    rng = np.random.default_rng(64)
+    for m, n, k in [(1, 1, 1), (3, 5, 16), (7, 9, 100), (4, 4, 33), (13, 21, 77), (5, 6, 2050)]:
+        a, b = support.random_matrix(oracle, dtype, m, k, rng), support.random_matrix(oracle, dtype, n, k, rng)
+        assert np.array_equal(oracle.dots_packed(dtype, a, b).view(np.uint32), reference.dots_packed(dtype, a, b).view(np.uint32)), (dtype, m, n, k)
+    for count, depth, row_start, row_count in SYMMETRIC_CASES[:6]:
+        vectors = support.random_matrix(oracle, dtype, count, depth, rng)
+        own = upper_window(count, row_start, row_count)
+        mine = oracle.symmetric("dots", dtype, vectors, row_start, row_count)
+        ref = reference.symmetric("dots", dtype, vectors, row_start, row_count)
+        assert np.array_equal(mine.view(np.uint32)[own], ref.view(np.uint32)[own]), (dtype, count, depth, row_start)
+
+
+@pytest.mark.parametrize("dtype", NARROW_DTYPES)
+def test_narrow_products_closed_forms(oracle, dtype):
+    """Needs no reference. 4-bit integers: the exact product of the unpacked nibbles (low nibble first, i4 sign-extended)
+    in numpy int64. 6-bit floats: every value is a multiple of 1/8 (e2m3) or 1/16 (e3m2) below 2^5, so short dots are
+    exact in f32 and must equal the f64 product of the decoded values."""
+    rng = np.random.default_rng(65)
+    a, b = support.random_matrix(oracle, dtype, 9, 64, rng), support.random_matrix(oracle, dtype, 11, 64, rng)
+    got = oracle.dots_packed(dtype, a, b)
+    if dtype in ("i4", "u4"):
+        def unpack(x):
+            nibbles = np.stack([x & 0xF, x >> 4], axis=-1).reshape(x.shape[0], -1).astype(np.int64)
+            return np.where(nibbles >= 8, nibbles - 16, nibbles) if dtype == "i4" else nibbles
+        exact = unpack(a) @ unpack(b).T
+        assert np.array_equal(got.astype(np.int64) & 0xFFFFFFFF, exact & 0xFFFFFFFF)
+        assert np.array_equal(oracle.decode(dtype, a).astype(np.int64), unpack(a))
+    else:
+        decoded_a, decoded_b = oracle.decode(dtype, a).astype(np.float64), oracle.decode(dtype, b).astype(np.float64)
+        assert np.array_equal(got.astype(np.float64), decoded_a @ decoded_b.T)
+        truth, _ = oracle.truth(dtype, a, b)
+        assert np.array_equal(truth, decoded_a @ decoded_b.T)
+
+
 @pytest.mark.parametrize("dtype", ["i8", "u8"])
 def test_integer_product_closed_form(oracle, dtype):
     rng = np.random.default_rng(11)
@@ -372,6 +438,13 @@ def test_golden_vectors(oracle, name):
         dtype = str(data["dtype"])
         assert same_floats(oracle.decode(dtype, data["codes"]), data["decoded"])
         assert np.array_equal(oracle.encode(dtype, data["values"]), data["encoded"])
+    elif name.startswith("narrow_"):
+        dtype, a, b, vectors = str(data["dtype"]), data["a"], data["b"], data["vectors"]
+        assert same_floats(oracle.dots_packed(dtype, a, b).view(np.float32), data["c_serial"].view(np.float32))
+        if dtype in NARROW_FLOAT_DTYPES:
+            assert same_floats(oracle.decode(dtype, np.arange(256, dtype=np.uint8)[None, :])[0], data["decoded"])
+        mine = oracle.symmetric("dots", dtype, vectors, int(data["row_start"]), int(data["row_count"]))
+        assert same_floats(mine.view(np.float32), data["symmetric_serial"].view(np.float32))
     elif name.startswith("symmetric_"):
         dtype, vectors = str(data["dtype"]), data["vectors"]
         row_start, row_count = int(data["row_start"]), int(data["row_count"])

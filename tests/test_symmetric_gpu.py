@@ -49,7 +49,7 @@ def owned(count, row_start, row_count):
 def gpu_symmetric(metric, dtype, vectors, row_start=0, row_count=None, config=0):
     """The call on a poisoned result; returns the raw 32-bit patterns."""
     count = vectors.shape[0]
-    out_dtype = torch.float32 if metric != "dots" or dtype in FLOAT_DTYPES else torch.int32
+    out_dtype = torch.float32 if metric != "dots" or OUTPUT[dtype] == np.float32 else torch.int32
     out = torch.full((count, count), POISON, dtype=torch.int32, device=DEV).view(out_dtype)
     end = count if row_count is None else min(count, row_start + row_count)
     nk.library().nk_hip_set_tile_config(config)
