@@ -139,14 +139,25 @@ class PackedMatrix:
     def nbytes(self) -> int:
         return int(self.buffer.numel())
 
+    @property
+    def shape(self):
+        """(width, depth), as the reference's PackedMatrix reports it."""
+        return (self.width, self.depth)
+
+    def __rmatmul__(self, a):
+        """``a @ packed`` is ``dots_packed(a, packed)``: the reference's ``Tensor @ PackedMatrix`` (python/matrix.c:324-490)."""
+        return dots_packed(a, self)
+
 
 def _as_matrix(t, dtype: str, what: str):
     import torch
 
     if dtype not in DTYPES:
         raise TypeError(f"unsupported dtype {dtype!r}; expected one of {sorted(DTYPES)}")
+    if not isinstance(t, torch.Tensor) and hasattr(t, "__dlpack__"):
+        t = torch.from_dlpack(t)  # any DLPack exporter of device memory (reference: python/dlpack_interop.c)
     if not isinstance(t, torch.Tensor):
-        raise TypeError(f"{what} must be a torch.Tensor")
+        raise TypeError(f"{what} must be a torch.Tensor or export DLPack")
     if t.dim() != 2:
         raise ValueError(f"{what} must be 2-dimensional, got {t.dim()} dimensions")
     if not t.is_cuda:

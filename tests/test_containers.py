@@ -1,0 +1,61 @@
+"""The containers over the C ABI: include/numkong_amd/matrix.hpp (C++: typed entry points, owning packed_matrix) through
+the program tests/cpp/test_matrix.cpp, and the Python PackedMatrix (`a @ packed`, DLPack operands).
+
+Reference counterparts: include/numkong/matrix.hpp:170-253, include/numkong/dots.hpp:94-150, python/matrix.c:151-227,
+324-490, python/dlpack_interop.c."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import numkong_amd as nk
+from tests import support
+
+PROGRAM = os.path.join(support.ROOT, "numkong_amd", "lib", "test_matrix")
+
+
+def run_program():
+    if not os.path.exists(PROGRAM):
+        pytest.fail(f"{PROGRAM} is missing: build it with `make -C numkong_amd/csrc`")
+    done = subprocess.run([PROGRAM], capture_output=True, text=True, timeout=300)
+    return done.returncode, done.stdout + done.stderr
+
+
+def test_cpp_containers_without_a_gpu_refuse_cleanly():
+    if nk.library().nk_hip_device_count() > 0:
+        pytest.skip("a GPU is present: covered by the GPU test")
+    code, text = run_program()
+    assert code == 0 and "FAILED" not in text and "containers refuse cleanly" in text, text
+
+
+@pytest.mark.gpu
+def test_cpp_containers_on_the_gpu():
+    code, text = run_program()
+    assert code == 0 and "FAILED" not in text and "all container checks passed" in text, text
+    assert text.count("ok:") >= 9
+
+
+@pytest.mark.gpu
+def test_python_packed_matrix_operator_and_dlpack(oracle):
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(91)
+    a, b = support.random_matrix(oracle, "i8", 33, 100, rng), support.random_matrix(oracle, "i8", 21, 100, rng)
+    ga, gb = torch.from_numpy(a).to("cuda:0"), torch.from_numpy(b).to("cuda:0")
+    packed = nk.dots_pack(gb, "i8")
+    assert packed.shape == (21, 100) and packed.nbytes == nk.dots_packed_size("i8", 21, 100)
+    expected = a.astype(np.int64) @ b.astype(np.int64).T
+    assert np.array_equal((ga @ packed).cpu().numpy(), expected)
+
+    class Exporter:  # any object that exports DLPack, not a torch.Tensor
+        def __init__(self, tensor):
+            self.tensor = tensor
+
+        def __dlpack__(self, **kwargs):
+            return self.tensor.__dlpack__(**kwargs)
+
+        def __dlpack_device__(self):
+            return self.tensor.__dlpack_device__()
+
+    again = nk.dots_packed(Exporter(ga), nk.dots_pack(Exporter(gb), "i8"))
+    assert np.array_equal(again.cpu().numpy(), expected)
