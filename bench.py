@@ -30,10 +30,11 @@ if ROOT not in sys.path:
 
 # MI355X published dense peaks, in T(FL)OP/s, for the MFMA the dtype runs on; HBM3E in GB/s.
 MFMA_PEAK = {"i8": 5000.0, "u8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "e4m3": 2500.0, "e5m2": 2500.0,
-             "e2m3": 2500.0, "e3m2": 2500.0, "i4": 5000.0, "u4": 5000.0}
+             "e2m3": 2500.0, "e3m2": 2500.0, "i4": 5000.0, "u4": 5000.0, "u1": 5000.0}
 MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2": "widened to f16, priced against the f16 MFMA peak",
              "e2m3": "widened to f16, priced against the f16 MFMA peak", "e3m2": "widened to f16, priced against the f16 MFMA peak",
-             "i4": "widened to i8, priced against the i8 MFMA peak", "u4": "widened to i8, priced against the i8 MFMA peak"}
+             "i4": "widened to i8, priced against the i8 MFMA peak", "u4": "widened to i8, priced against the i8 MFMA peak",
+             "u1": "bits widened to i8 zeros and ones, priced against the i8 MFMA peak"}
 HBM_PEAK = 8000.0
 # HBM-side bytes per launch (L2 <-> fabric) from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --probe`,
 # each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
@@ -50,7 +51,7 @@ MEASURED_TRAFFIC = {
 HEADLINE = ("i8", 8192, 8192, 8192)
 OTHERS = [("bf16", 8192, 8192, 8192, "dots"), ("e4m3", 8192, 8192, 8192, "dots"), ("i8", 1024, 1 << 20, 768, "dots"),
           ("i8", 1024, 1 << 20, 768, "angular"), ("i8", 8192, 8192, 8192, "symmetric"), ("bf16", 8192, 8192, 8192, "symmetric"),
-          ("i4", 8192, 8192, 8192, "dots"), ("e2m3", 8192, 8192, 8192, "dots")]
+          ("i4", 8192, 8192, 8192, "dots"), ("e2m3", 8192, 8192, 8192, "dots"), ("u1", 8192, 8192, 8192, "dots")]
 KINDS = {"angular": ord("N"), "euclidean": ord("E")}  # nk_kernel_angulars_packed_k, nk_kernel_euclideans_packed_k
 # nk_kernel_dots_symmetric_k, nk_kernel_angulars_symmetric_k, nk_kernel_euclideans_symmetric_k
 SYMMETRIC_KINDS = {"symmetric": ord("y"), "symmetric-angular": ord("n"), "symmetric-euclidean": ord("D")}
@@ -65,6 +66,8 @@ def make_operands(dtype, m, n, k, seed=42):
     def one(rows):
         if dtype in ("i4", "u4"):  # two 4-bit values per byte, every byte value
             return torch.randint(0, 256, (rows, (k + 1) // 2), dtype=torch.uint8, device="cuda:0", generator=g)
+        if dtype == "u1":  # eight bits per byte
+            return torch.randint(0, 256, (rows, (k + 7) // 8), dtype=torch.uint8, device="cuda:0", generator=g)
         if dtype in ("e2m3", "e3m2"):  # every 6-bit code is a finite number
             return torch.randint(0, 64, (rows, k), dtype=torch.uint8, device="cuda:0", generator=g)
         if dtype == "i8":

@@ -53,11 +53,13 @@ typedef unsigned char nk_e2m3_t; /* one 6-bit float per byte */
 typedef unsigned char nk_e3m2_t;
 typedef unsigned char nk_i4x2_t; /* two 4-bit integers per byte, the even dimension in the low nibble */
 typedef unsigned char nk_u4x2_t;
+typedef unsigned char nk_u1x8_t; /* eight 1-bit values per byte */
 typedef nk_u64_t nk_size_t;
 
 /** Element types (reference: include/numkong/types.h:923-952; same numeric codes). */
 typedef enum {
     nk_dtype_unknown_k = 0,
+    nk_u1_k = 1 << 1,
     nk_i8_k = 1 << 2,
     nk_i32_k = 1 << 4,
     nk_u8_k = 1 << 6,
@@ -119,6 +121,7 @@ NK_DYNAMIC nk_size_t nk_dots_packed_size_e2m3(nk_size_t width, nk_size_t depth);
 NK_DYNAMIC nk_size_t nk_dots_packed_size_e3m2(nk_size_t width, nk_size_t depth);
 NK_DYNAMIC nk_size_t nk_dots_packed_size_i4(nk_size_t width, nk_size_t depth); /* depth in 4-bit values */
 NK_DYNAMIC nk_size_t nk_dots_packed_size_u4(nk_size_t width, nk_size_t depth);
+NK_DYNAMIC nk_size_t nk_dots_packed_size_u1(nk_size_t width, nk_size_t depth); /* depth in bits */
 
 /* Pack row-major B (width rows of depth elements, b_stride bytes apart). Reference: include/numkong/dots.h:203-237. */
 NK_DYNAMIC void nk_dots_pack_i8(nk_i8_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride, void *b_packed);
@@ -138,6 +141,8 @@ NK_DYNAMIC void nk_dots_pack_e3m2(nk_e3m2_t const *b, nk_size_t width, nk_size_t
 NK_DYNAMIC void nk_dots_pack_i4(nk_i4x2_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
                                 void *b_packed);
 NK_DYNAMIC void nk_dots_pack_u4(nk_u4x2_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
+                                void *b_packed);
+NK_DYNAMIC void nk_dots_pack_u1(nk_u1x8_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
                                 void *b_packed);
 
 /* C = A * B^T with widened accumulators, C overwritten. Reference: include/numkong/dots.h:248-287. */
@@ -160,6 +165,9 @@ NK_DYNAMIC void nk_dots_packed_e3m2(nk_e3m2_t const *a, void const *b_packed, nk
 NK_DYNAMIC void nk_dots_packed_i4(nk_i4x2_t const *a, void const *b_packed, nk_i32_t *c, nk_size_t height,
                                   nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
 NK_DYNAMIC void nk_dots_packed_u4(nk_u4x2_t const *a, void const *b_packed, nk_u32_t *c, nk_size_t height,
+                                  nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
+/* 1-bit values: c[i][j] = popcount(a_i AND b_j). Reference: include/numkong/dots.h:289-296. */
+NK_DYNAMIC void nk_dots_packed_u1(nk_u1x8_t const *a, void const *b_packed, nk_u32_t *c, nk_size_t height,
                                   nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
 
 /* Distances over the same packed B, in one pass: result[i][j] = angular (1 - cosine) or euclidean distance between
@@ -201,7 +209,7 @@ NK_AMD_DECLARE_SYMMETRIC_(e4m3, nk_e4m3_t, nk_f32_t)
 NK_AMD_DECLARE_SYMMETRIC_(e5m2, nk_e5m2_t, nk_f32_t)
 #undef NK_AMD_DECLARE_SYMMETRIC_
 
-/* The 6-bit floats and the 4-bit integers have the dot-product kinds only (packed above, symmetric here), with their
+/* The 6-bit floats, the 4-bit integers and the 1-bit type have the dot-product kinds only (packed above, symmetric here), with their
  * backend-suffixed names; their distance kinds resolve to the error stubs. */
 #define NK_AMD_DECLARE_DOTS_ONLY_(T, in_t, out_t)                                                                      \
     NK_DYNAMIC void nk_dots_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,              \
@@ -220,6 +228,7 @@ NK_AMD_DECLARE_DOTS_ONLY_(e2m3, nk_e2m3_t, nk_f32_t)
 NK_AMD_DECLARE_DOTS_ONLY_(e3m2, nk_e3m2_t, nk_f32_t)
 NK_AMD_DECLARE_DOTS_ONLY_(i4, nk_i4x2_t, nk_i32_t)
 NK_AMD_DECLARE_DOTS_ONLY_(u4, nk_u4x2_t, nk_u32_t)
+NK_AMD_DECLARE_DOTS_ONLY_(u1, nk_u1x8_t, nk_u32_t)
 #undef NK_AMD_DECLARE_DOTS_ONLY_
 
 /* Capability and lookup API. Reference: c/numkong.c:767-768, 831-913. */

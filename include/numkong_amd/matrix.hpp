@@ -56,7 +56,7 @@ NK_AMD_DEFINE_TYPE_(e5m2, nk_e5m2_t, nk_f32_t, 1)
 NK_AMD_DEFINE_TYPE_(e2m3, nk_e2m3_t, nk_f32_t, 1)
 NK_AMD_DEFINE_TYPE_(e3m2, nk_e3m2_t, nk_f32_t, 1)
 #undef NK_AMD_DEFINE_TYPE_
-/* the 4-bit types are named after their two-to-a-byte storage in the C ABI */
+/* the sub-byte types are named after their storage in the C ABI: two 4-bit or eight 1-bit values to a byte */
 struct i4x2_t {
     using raw_t = nk_i4x2_t;
     using dot_result_t = nk_i32_t;
@@ -91,6 +91,25 @@ struct u4x2_t {
     static void symmetric(raw_t const *v, nk_size_t n, nk_size_t k, nk_size_t stride, dot_result_t *out,
                           nk_size_t out_stride, nk_size_t row_start, nk_size_t row_count) noexcept {
         nk_dots_symmetric_u4(v, n, k, stride, out, out_stride, row_start, row_count);
+    }
+};
+
+struct u1x8_t {
+    using raw_t = nk_u1x8_t;
+    using dot_result_t = nk_u32_t;
+    static constexpr nk_dtype_t dtype = nk_u1_k;
+    static constexpr std::size_t dimensions_per_value = 8;
+    static nk_size_t packed_size(nk_size_t n, nk_size_t k) noexcept { return nk_dots_packed_size_u1(n, k); }
+    static void pack(raw_t const *b, nk_size_t n, nk_size_t k, nk_size_t stride, void *packed) noexcept {
+        nk_dots_pack_u1(b, n, k, stride, packed);
+    }
+    static void packed(raw_t const *a, void const *b, dot_result_t *c, nk_size_t m, nk_size_t n, nk_size_t k,
+                       nk_size_t a_stride, nk_size_t c_stride) noexcept {
+        nk_dots_packed_u1(a, b, c, m, n, k, a_stride, c_stride);
+    }
+    static void symmetric(raw_t const *v, nk_size_t n, nk_size_t k, nk_size_t stride, dot_result_t *out,
+                          nk_size_t out_stride, nk_size_t row_start, nk_size_t row_count) noexcept {
+        nk_dots_symmetric_u1(v, n, k, stride, out, out_stride, row_start, row_count);
     }
 };
 

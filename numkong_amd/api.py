@@ -23,7 +23,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # nk_dtype_t codes (reference: include/numkong/types.h:923-952)
 NK_I8, NK_I32, NK_U8, NK_U32 = 1 << 2, 1 << 4, 1 << 6, 1 << 8
 NK_F32, NK_F16, NK_BF16, NK_E4M3, NK_E5M2 = 1 << 11, 1 << 12, 1 << 13, 1 << 14, 1 << 15
-NK_I4, NK_U4, NK_E2M3, NK_E3M2 = 1 << 16, 1 << 17, 1 << 18, 1 << 19
+NK_I4, NK_U4, NK_E2M3, NK_E3M2, NK_U1 = 1 << 16, 1 << 17, 1 << 18, 1 << 19, 1 << 1
 
 # name -> (nk code, bytes per stored value, output torch dtype name, dimensions per stored value)
 DTYPES = {
@@ -37,6 +37,7 @@ DTYPES = {
     "e3m2": (NK_E3M2, 1, "float32", 1),
     "i4": (NK_I4, 1, "int32", 2),  # two 4-bit values per byte: a (rows, depth / 2) byte tensor, as the reference's
     "u4": (NK_U4, 1, "int32", 2),  # bindings take them (python/matrix.c:603: depth *= dimensions per value)
+    "u1": (NK_U1, 1, "int32", 8),  # eight bits per byte; the dot product is popcount(a & b)
 }
 
 

@@ -3,7 +3,7 @@
  *  @file numkong_amd/csrc/dispatch.h
  *
  *  Mirrors the role of the reference's c/dispatch.h:37-506, reduced to the packed-dots, packed-distance and symmetric slots
- *  (reference slots: c/dispatch.h:279-336, 353-380) for i8, u8, bf16, f16, e4m3, e5m2, e2m3, e3m2, i4, u4.
+ *  (reference slots: c/dispatch.h:279-336, 353-380) for i8, u8, bf16, f16, e4m3, e5m2, e2m3, e3m2, i4, u4, u1.
  */
 #ifndef NUMKONG_AMD_DISPATCH_H
 #define NUMKONG_AMD_DISPATCH_H
@@ -17,19 +17,19 @@ extern "C" {
 typedef struct {
     nk_dots_packed_size_punned_t dots_packed_size_i8, dots_packed_size_u8, dots_packed_size_bf16,
         dots_packed_size_f16, dots_packed_size_e4m3, dots_packed_size_e5m2, dots_packed_size_e2m3, dots_packed_size_e3m2,
-        dots_packed_size_i4, dots_packed_size_u4;
+        dots_packed_size_i4, dots_packed_size_u4, dots_packed_size_u1;
     nk_dots_pack_punned_t dots_pack_i8, dots_pack_u8, dots_pack_bf16, dots_pack_f16, dots_pack_e4m3, dots_pack_e5m2, dots_pack_e2m3, dots_pack_e3m2,
-        dots_pack_i4, dots_pack_u4;
+        dots_pack_i4, dots_pack_u4, dots_pack_u1;
     nk_dots_packed_punned_t dots_packed_i8, dots_packed_u8, dots_packed_bf16, dots_packed_f16, dots_packed_e4m3,
         dots_packed_e5m2, dots_packed_e2m3, dots_packed_e3m2,
-        dots_packed_i4, dots_packed_u4;
+        dots_packed_i4, dots_packed_u4, dots_packed_u1;
     nk_dots_packed_punned_t angulars_packed_i8, angulars_packed_u8, angulars_packed_bf16, angulars_packed_f16,
         angulars_packed_e4m3, angulars_packed_e5m2;
     nk_dots_packed_punned_t euclideans_packed_i8, euclideans_packed_u8, euclideans_packed_bf16, euclideans_packed_f16,
         euclideans_packed_e4m3, euclideans_packed_e5m2;
     nk_dots_symmetric_punned_t dots_symmetric_i8, dots_symmetric_u8, dots_symmetric_bf16, dots_symmetric_f16,
         dots_symmetric_e4m3, dots_symmetric_e5m2, dots_symmetric_e2m3, dots_symmetric_e3m2,
-        dots_symmetric_i4, dots_symmetric_u4;
+        dots_symmetric_i4, dots_symmetric_u4, dots_symmetric_u1;
     nk_dots_symmetric_punned_t angulars_symmetric_i8, angulars_symmetric_u8, angulars_symmetric_bf16,
         angulars_symmetric_f16, angulars_symmetric_e4m3, angulars_symmetric_e5m2;
     nk_dots_symmetric_punned_t euclideans_symmetric_i8, euclideans_symmetric_u8, euclideans_symmetric_bf16,
@@ -62,6 +62,7 @@ NK_AMD_DECLARE_DISPATCH_(e2m3)
 NK_AMD_DECLARE_DISPATCH_(e3m2)
 NK_AMD_DECLARE_DISPATCH_(i4)
 NK_AMD_DECLARE_DISPATCH_(u4)
+NK_AMD_DECLARE_DISPATCH_(u1)
 #undef NK_AMD_DECLARE_DISPATCH_
 
 /**

@@ -140,6 +140,7 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
         case 4: kernel = pack_kernel<4>; break;
         case 5: kernel = pack_kernel<5>; break;
         case 6: kernel = pack_kernel<6>; break;
+        case 7: kernel = pack_kernel<7>; break;
         default: break;
         }
         hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride,
@@ -150,7 +151,7 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
     if (g.n_tiles && terms) {
         if (g.k_chunks) {
             // by what the image holds: signed bytes (i8 and the widened 4-bit types), offset u8, bf16, f16 (and what is widened to it)
-            auto kernel = dtype == kI8 || dtype == kI4 || dtype == kU4
+            auto kernel = dtype == kI8 || dtype == kI4 || dtype == kU4 || dtype == kU1
                               ? column_terms_kernel<0>
                               : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
             hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(256), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);
@@ -233,6 +234,7 @@ static int product_async(int dtype, int metric, void const *a, void const *b_pac
     case kE3M2: e = launch_e3m2(g, stream, triangle); break;
     case kI4: e = launch_i4(g, stream, triangle); break;
     case kU4: e = launch_u4(g, stream, triangle); break;
+    case kU1: e = launch_u1(g, stream, triangle); break;
     default: return fail_msg("nk_hip_dots_packed: unsupported dtype");
     }
     return e == hipSuccess ? 0 : fail(e, "dots_packed_kernel");

@@ -84,6 +84,7 @@ hipError_t launch_e2m3(GemmArgs &g, hipStream_t stream, TriangleScratch const *t
 hipError_t launch_e3m2(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
 hipError_t launch_i4(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
 hipError_t launch_u4(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
+hipError_t launch_u1(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
 
 extern int g_forced_config; // 0: the heuristic picks the tile shape; see nk_hip_set_tile_config
 extern int g_variant;       // timing experiments of tuning builds
@@ -115,6 +116,7 @@ enum : int {
     kU4 = 1 << 17,
     kE2M3 = 1 << 18, // 6-bit floats, one per byte (bits 6 and 7 ignored)
     kE3M2 = 1 << 19,
+    kU1 = 1 << 1, // eight 1-bit values per byte
 };
 
 constexpr uint32_t kMagic = 0x35394B4Eu; // "NK95"
@@ -153,6 +155,7 @@ struct Geometry {
 /** Bits per element in the caller's A and B (0: not a type of this backend). */
 inline int elem_bits_of(int dtype) {
     switch (dtype) {
+    case kU1: return 1;
     case kI4:
     case kU4: return 4;
     case kI8:
@@ -172,7 +175,7 @@ inline int elem_bits_of(int dtype) {
  *  kernels (dot/serial.h:522-600). e4m3 and e5m2 are therefore widened, exactly, to f16 and run on the f16
  *  MFMA, whose products and sums are kept to full f32 precision: B at pack time, A on its way into LDS.
  *  The 6-bit floats go the same way (every e2m3 / e3m2 value is an f16 value), and the 4-bit integers are
- *  widened to i8 for the i8 MFMA. */
+ *  widened to i8 for the i8 MFMA, and so are single bits (0 or 1: their dot product is the popcount of the AND). */
 inline int packed_bytes_of(int dtype) {
     switch (dtype) {
     case kE4M3:
@@ -180,7 +183,8 @@ inline int packed_bytes_of(int dtype) {
     case kE2M3:
     case kE3M2: return 2;
     case kI4:
-    case kU4: return 1;
+    case kU4:
+    case kU1: return 1;
     default: return elem_bits_of(dtype) / 8;
     }
 }
@@ -190,8 +194,8 @@ inline bool make_geometry(int dtype, size_t n, size_t k, Geometry &g) {
     if (!bits) return false;
     if (n > 0x7FFFFFFFull || k > 0x3FFFFFFFull) return false;
     g.elem_bytes = (uint32_t)(bits + 7) / 8, g.packed_bytes = (uint32_t)packed_bytes_of(dtype), g.n = (uint32_t)n, g.k = (uint32_t)k;
-    g.k_bytes = (uint64_t)k * g.packed_bytes;
-    g.k_src_bytes = ((uint64_t)k * bits + 7) / 8; // (4-bit types: whole bytes, as the reference loads them, cast/serial.h:533-538)
+    g.k_src_bytes = ((uint64_t)k * bits + 7) / 8; // (sub-byte types: whole bytes, as the reference loads them, cast/serial.h:519-538)
+    g.k_bytes = bits < 8 ? g.k_src_bytes * (8 / bits) * g.packed_bytes : (uint64_t)k * g.packed_bytes;
     uint64_t const chunks = (g.k_bytes + kChunkBytes - 1) / kChunkBytes;
     g.k_chunks = (uint32_t)((chunks + 2 * kStageChunks - 1) / (2 * kStageChunks) * (2 * kStageChunks)); // an even number of stages
     g.n_tiles = (uint32_t)((n + kTileRows - 1) / kTileRows);
@@ -297,8 +301,17 @@ __device__ __forceinline__ v4i widen_i4x16(uint32_t lo, uint32_t hi) {
     return out;
 }
 
-/** Widening of 8 source bytes to one 16-byte chunk, by kind: 1 e4m3, 2 e5m2, 3 e2m3, 4 e3m2 (to f16); 5 i4, 6 u4
- *  (to i8). */
+/** Sixteen bits (the low half of `bits`, the first dimension in bit 0) -> sixteen i8 values 0 or 1. Four bits times
+ *  0x00204081 land in bit 0 of four different bytes. */
+__device__ __forceinline__ v4i widen_u1x16(uint32_t bits) {
+    v4i out;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) out[w] = (int)((((bits >> (4 * w)) & 0xFu) * 0x00204081u) & 0x01010101u);
+    return out;
+}
+
+/** Widening of the source bytes behind one 16-byte chunk, by kind: 1 e4m3, 2 e5m2, 3 e2m3, 4 e3m2 (8 bytes to f16);
+ *  5 i4, 6 u4 (8 bytes to i8); 7 u1 (2 bytes to i8). */
 template <int WIDEN>
 __device__ __forceinline__ v4i widen_chunk(uint32_t lo, uint32_t hi) {
     if constexpr (WIDEN == 1) return widen_fp8x8<false>(lo, hi);
@@ -306,7 +319,8 @@ __device__ __forceinline__ v4i widen_chunk(uint32_t lo, uint32_t hi) {
     else if constexpr (WIDEN == 3) return widen_fp6x8<false>(lo, hi);
     else if constexpr (WIDEN == 4) return widen_fp6x8<true>(lo, hi);
     else if constexpr (WIDEN == 5) return widen_i4x16<true>(lo, hi);
-    else return widen_i4x16<false>(lo, hi);
+    else if constexpr (WIDEN == 6) return widen_i4x16<false>(lo, hi);
+    else return widen_u1x16(lo);
 }
 inline int widen_kind_of(int dtype) {
     switch (dtype) {
@@ -316,6 +330,7 @@ inline int widen_kind_of(int dtype) {
     case kE3M2: return 4;
     case kI4: return 5;
     case kU4: return 6;
+    case kU1: return 7;
     default: return 0;
     }
 }
@@ -331,7 +346,7 @@ template <int WIDEN>
 __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
                                                    uint64_t k_src_bytes, uint32_t k_chunks, uint8_t *__restrict__ data,
                                                    int avec, uint32_t xr, PackedHeader header) {
-    constexpr int kSrcChunk = WIDEN ? 8 : 16;
+    constexpr int kSrcChunk = WIDEN == 0 ? 16 : (WIDEN == 7 ? 2 : 8);
     if (blockIdx.x == 0 && threadIdx.x == 0) *(PackedHeader *)(data - sizeof(PackedHeader)) = header; // (64 bytes in front of the tiles)
     uint32_t const groups = k_chunks / kStageChunks;
     uint32_t const tile = blockIdx.x / groups;
@@ -578,6 +593,14 @@ struct I4 : I8 {
     static constexpr bool kDistances = false; // dot products only
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_i4x16<true>((uint32_t)v[0], (uint32_t)v[1]); }
+    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); }
+};
+/** Single bits run as i8 values 0 and 1: sixteen of them behind two source bytes. */
+struct U1 : I8 {
+    static constexpr int kDtype = kU1;
+    static constexpr bool kDistances = false; // dot products only
+    static constexpr int kSrcChunk = 2;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_u1x16((uint32_t)v[0]); }
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); }
 };
 struct U4 : I8 {
@@ -841,7 +864,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // Stages the pipelined loop takes: all of them when A is at least dword-aligned, which is all that
     // multi-dword global loads need. (readfirstlane: the value is uniform, and it must stay in a scalar register
     // because the stage offsets of the buffer loads derive from it.)
-    uint32_t const fast = __builtin_amdgcn_readfirstlane(g.avec >= 4 ? stages : 0);
+    uint32_t const fast = __builtin_amdgcn_readfirstlane(g.avec >= (T::kSrcChunk < 4 ? T::kSrcChunk : 4) ? stages : 0);
     uint32_t const xr = T::kUnsigned ? 0x80808080u : 0u;
     uint32_t const a_pos = tid & 7;
     // A fragment reads: lane l takes row l % 32 of each 32-row block and chunk 2q + l / 32.
@@ -885,8 +908,9 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         view.col0 = tile_n * (128 * TN) + wave * (32 * TN);
         uint32_t const rows_here = g.m - view.row0 < (uint32_t)BM ? g.m - view.row0 : (uint32_t)BM;
         view.a = g.a + (uint64_t)view.row0 * g.a_stride;
-        // (whole dwords: a dword-aligned A never ends in the middle of one that could fault)
-        view.a_bytes = (rows_here - 1) * (uint32_t)g.a_stride + (((uint32_t)g.k_src_bytes + 3u) & ~3u);
+        // (whole aligned loads: an aligned A never ends in the middle of one that could fault)
+        constexpr uint32_t kLoadAlign = T::kSrcChunk < 4 ? T::kSrcChunk : 4; // (2-byte loads for the 1-bit type)
+        view.a_bytes = (rows_here - 1) * (uint32_t)g.a_stride + (((uint32_t)g.k_src_bytes + kLoadAlign - 1) & ~(kLoadAlign - 1));
         uint32_t const tile_bytes = g.k_chunks * kTileChunkBytes;
         uint32_t const first = view.col0 / 32 < g.n_tiles ? view.col0 / 32 : g.n_tiles - 1;
         view.b = data + (uint64_t)first * tile_bytes;
@@ -961,6 +985,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             if (T::kSrcChunk == 16) {
                 v = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, a_off[i], stage_offset, 0));
             }
+            else if (T::kSrcChunk == 2) { v[0] = (int)(uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, a_off[i], stage_offset, 0); }
             else {
                 typedef unsigned v2u __attribute__((ext_vector_type(2)));
                 v2u const narrow = __builtin_amdgcn_raw_buffer_load_b64(rsrc, a_off[i], stage_offset, 0);
@@ -982,9 +1007,10 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         constexpr int buffer = decltype(buffer_tag)::value, slot = decltype(slot_tag)::value;
         uint8_t *dst = lds + buffer * kStageLds;
         int const left = a_tail - (int)(s * kSrcStage);
-        uint32_t keep[T::kSrcChunk / 4];
+        constexpr int kSrcWords = (T::kSrcChunk + 3) / 4;
+        uint32_t keep[kSrcWords];
 #pragma unroll
-        for (int w = 0; w < T::kSrcChunk / 4; ++w) {
+        for (int w = 0; w < kSrcWords; ++w) {
             int const over = left - 4 * w, bytes = over < 0 ? 0 : (over > 4 ? 4 : over);
             keep[w] = bytes == 4 ? 0xFFFFFFFFu : ((1u << (8 * bytes)) - 1u);
         }
@@ -992,7 +1018,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         for (int i = 0; i < kLoads; ++i) {
             v4i v = a_reg[slot][i];
 #pragma unroll
-            for (int w = 0; w < T::kSrcChunk / 4; ++w) v[w] &= (int)keep[w];
+            for (int w = 0; w < kSrcWords; ++w) v[w] &= (int)keep[w];
             // (without a next tile to stage for, what is staged past the end is dropped)
             uint32_t const set = across && !mine ? sums_here ^ (uint32_t)(kLoads * NT) : sums_here;
             v4i const raw = v;
@@ -1408,7 +1434,7 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
     // The pipeline runs across tile boundaries when the pipelined loop takes the stages of a tile (A readable
     // with dword loads) and there are enough of them to prefetch three ahead.
     uint32_t const stages = g.k_chunks / kStageChunks;
-    bool const across = g.avec >= 4 && stages >= 4 && !(g_variant & 1);
+    bool const across = g.avec >= (T::kSrcChunk < 4 ? T::kSrcChunk : 4) && stages >= 4 && !(g_variant & 1);
     bool const norms = g.metric != 0;
     void (*kernel)(GemmArgs) = across ? dots_packed_kernel<T, TM, TN, true, false> : dots_packed_kernel<T, TM, TN, false, false>;
     if constexpr (T::kDistances) {

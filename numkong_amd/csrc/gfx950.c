@@ -28,9 +28,10 @@ static void nk_amd_set_error_(char const *where) {
 
 char const *nk_amd_last_error(void) { return nk_amd_error_; }
 
-/** Bytes of one row of `k` elements: two 4-bit values to a byte, whole bytes (cast/serial.h:533-538). */
+/** Bytes of one row of `k` elements: eight 1-bit or two 4-bit values to a byte, whole bytes (cast/serial.h:519-538). */
 static size_t nk_amd_row_bytes_(nk_dtype_t dtype, size_t k) {
     switch (dtype) {
+    case nk_u1_k: return (k + 7) / 8;
     case nk_i4_k:
     case nk_u4_k: return (k + 1) / 2;
     case nk_i8_k:
@@ -329,3 +330,4 @@ NK_AMD_DEFINE_BACKEND_DOTS_(e2m3, nk_e2m3_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(i4, nk_i4x2_t, nk_i32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(u4, nk_u4x2_t, nk_u32_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(u1, nk_u1x8_t, nk_u32_t)

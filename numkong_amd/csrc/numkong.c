@@ -107,6 +107,7 @@ NK_AMD_DISPATCH_DOTS_(e2m3, nk_e2m3_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(i4, nk_i4x2_t, nk_i32_t)
 NK_AMD_DISPATCH_DOTS_(u4, nk_u4x2_t, nk_u32_t)
+NK_AMD_DISPATCH_DOTS_(u1, nk_u1x8_t, nk_u32_t)
 
 NK_DYNAMIC int nk_uses_dynamic_dispatch(void) { return 1; }
 
@@ -140,6 +141,7 @@ NK_DYNAMIC void nk_dispatch_table_update(nk_capability_t caps) {
     nk_dispatch_e3m2_init_(caps);
     nk_dispatch_i4_init_(caps);
     nk_dispatch_u4_init_(caps);
+    nk_dispatch_u1_init_(caps);
 }
 
 NK_DYNAMIC void nk_find_kernel_punned(nk_kernel_kind_t kind, nk_dtype_t dtype, nk_capability_t viable,
@@ -157,6 +159,7 @@ NK_DYNAMIC void nk_find_kernel_punned(nk_kernel_kind_t kind, nk_dtype_t dtype, n
     case nk_e3m2_k: nk_dispatch_e3m2_find_(viable, kind, m, c); return;
     case nk_i4_k: nk_dispatch_i4_find_(viable, kind, m, c); return;
     case nk_u4_k: nk_dispatch_u4_find_(viable, kind, m, c); return;
+    case nk_u1_k: nk_dispatch_u1_find_(viable, kind, m, c); return;
     default: break;
     }
     *m = (nk_kernel_punned_t)0;
@@ -181,7 +184,8 @@ NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t i
     case nk_i8_k:
     case nk_i4_k: return nk_i32_k;
     case nk_u8_k:
-    case nk_u4_k: return nk_u32_k;
+    case nk_u4_k:
+    case nk_u1_k: return nk_u32_k;
     case nk_bf16_k:
     case nk_f16_k:
     case nk_e4m3_k:

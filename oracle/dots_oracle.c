@@ -46,7 +46,8 @@
  *
  *    - the remaining narrow types of the dots family, products only (packed and symmetric): e2m3 and e3m2 (decoded by
  *      the formats' definition, 4 f32 lane sums like the other float types), i4 and u4 (two nibbles per byte, the even
- *      dimension in the low one, whole bytes even for an odd depth; exact)
+ *      dimension in the low one, whole bytes even for an odd depth; exact) and u1 (eight bits per byte, popcount of
+ *      the AND over whole bytes)
  *          include/numkong/cast/serial.h:533-538, 1280-1330, 1418-1470, include/numkong/dot/serial.h:602-800
  *      Pinned bit for bit against nk_cast_serial (all 256 byte values decode; encoder on finite probes incl. every
  *      tie) and nk_dots_packed_<T>_serial / nk_dots_symmetric_<T>_serial; their distance kinds are not restated
@@ -73,6 +74,7 @@ enum {
     NKO_U4 = 1 << 17,
     NKO_E2M3 = 1 << 18, /* 6-bit floats, one per byte, bits 6 and 7 ignored */
     NKO_E3M2 = 1 << 19,
+    NKO_U1 = 1 << 1, /* eight 1-bit values per byte; their dot product is the popcount of the AND */
 };
 
 #define NKO_API __attribute__((visibility("default")))
@@ -211,15 +213,17 @@ static int element_bytes(int dtype) {
     }
 }
 
-/* 4-bit types: a row of `depth` dimensions is read as whole bytes, both nibbles of the last one included when the
- * depth is odd, exactly as the reference's loads do (cast/serial.h:533-538, dot/serial.h:705-718, 777-790). */
+/* Sub-byte types: a row of `depth` dimensions is read as whole bytes, all of the last one included when the depth
+ * does not fill it, exactly as the reference's loads do (cast/serial.h:519-538, dot/serial.h:705-718, 777-790, 824-832). */
 static size_t effective_depth(int dtype, size_t depth) {
+    if (dtype == NKO_U1) return (depth + 7) / 8 * 8; /* cast/serial.h:519-524 */
     return dtype == NKO_I4 || dtype == NKO_U4 ? (depth + 1) / 2 * 2 : depth;
 }
 
 /* Value of element `i` of a row as f32 (integers are exact in f32 too: |x| <= 255). */
 static float element_f32(int dtype, void const *row, size_t i) {
     switch (dtype) {
+    case NKO_U1: return (float)((((uint8_t const *)row)[i / 8] >> (i & 7)) & 1);
     case NKO_U4: return (float)((((uint8_t const *)row)[i / 2] >> (4 * (i & 1))) & 0xF);
     case NKO_I4: {
         int const nibble = (((uint8_t const *)row)[i / 2] >> (4 * (i & 1))) & 0xF;
@@ -511,7 +515,7 @@ NKO_API void nko_spatials_f64(int dtype, int metric, void const *a, void const *
  *  which keeps the same four lane sums, lane = k mod 4, as the f32x4 path of its packed kernel). */
 static uint32_t serial_dot_bits(int dtype, void const *a_row, void const *b_row, size_t depth) {
     depth = effective_depth(dtype, depth);
-    if (dtype == NKO_I8 || dtype == NKO_U8 || dtype == NKO_I4 || dtype == NKO_U4) {
+    if (dtype == NKO_I8 || dtype == NKO_U8 || dtype == NKO_I4 || dtype == NKO_U4 || dtype == NKO_U1) {
         /* exact in 64 bits, truncated to 32: i64 for the signed types, u64 for the unsigned, the same bits either way */
         int64_t sum = 0;
         for (size_t l = 0; l < depth; ++l) sum += (int64_t)element_f32(dtype, a_row, l) * (int64_t)element_f32(dtype, b_row, l);
@@ -527,7 +531,7 @@ static uint32_t serial_dot_bits(int dtype, void const *a_row, void const *b_row,
 
 /** C = A * B^T with the serial backend's rounding from UNPACKED operands: what nk_dots_packed_<T>_serial returns for
  *  any of the ten types (for the six older ones it equals nko_serial_pack + nko_serial_packed, which also restate
- *  the serial image; for e2m3, e3m2, i4, u4 only the arithmetic is restated: dot/serial.h:602-800). */
+ *  the serial image; for e2m3, e3m2, i4, u4, u1 only the arithmetic is restated: dot/serial.h:602-832). */
 NKO_API void nko_serial_dots(int dtype, void const *a, void const *b, void *c, size_t rows, size_t columns, size_t depth,
                              size_t a_stride, size_t b_stride, size_t c_stride) {
     for (size_t i = 0; i < rows; ++i) {

@@ -18,17 +18,18 @@ GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
 
 # nk_dtype_t codes (reference: include/numkong/types.h:923-952)
 CODES = {"i8": 1 << 2, "u8": 1 << 6, "f32": 1 << 11, "f16": 1 << 12, "bf16": 1 << 13, "e4m3": 1 << 14, "e5m2": 1 << 15,
-         "i4": 1 << 16, "u4": 1 << 17, "e2m3": 1 << 18, "e3m2": 1 << 19}
+         "i4": 1 << 16, "u4": 1 << 17, "e2m3": 1 << 18, "e3m2": 1 << 19, "u1": 1 << 1}
 STORAGE = {"i8": np.int8, "u8": np.uint8, "f16": np.uint16, "bf16": np.uint16, "e4m3": np.uint8, "e5m2": np.uint8,
-           "i4": np.uint8, "u4": np.uint8, "e2m3": np.uint8, "e3m2": np.uint8}
+           "i4": np.uint8, "u4": np.uint8, "e2m3": np.uint8, "e3m2": np.uint8, "u1": np.uint8}
 OUTPUT = {"i8": np.int32, "u8": np.uint32, "f16": np.float32, "bf16": np.float32, "e4m3": np.float32, "e5m2": np.float32,
-          "i4": np.int32, "u4": np.uint32, "e2m3": np.float32, "e3m2": np.float32}
+          "i4": np.int32, "u4": np.uint32, "e2m3": np.float32, "e3m2": np.float32, "u1": np.uint32}
 FLOAT_DTYPES = ("bf16", "f16", "e4m3", "e5m2")
 ALL_DTYPES = ("i8", "u8") + FLOAT_DTYPES  # the types with every kind: packed dots, packed distances, symmetric
-# the types with the dot-product kinds only: 6-bit floats (one per byte), 4-bit integers (two per byte)
+# the types with the dot-product kinds only: 6-bit floats (one per byte), 4-bit integers (two per byte), bits (eight)
 NARROW_FLOAT_DTYPES = ("e2m3", "e3m2")
-NARROW_DTYPES = NARROW_FLOAT_DTYPES + ("i4", "u4")
-DIMENSIONS_PER_VALUE = {"i4": 2, "u4": 2}
+NARROW_INT_DTYPES = ("i4", "u4", "u1")
+NARROW_DTYPES = NARROW_FLOAT_DTYPES + NARROW_INT_DTYPES
+DIMENSIONS_PER_VALUE = {"i4": 2, "u4": 2, "u1": 8}
 
 
 def depth_of(dtype: str, matrix: np.ndarray) -> int:
@@ -251,9 +252,10 @@ def random_matrix(oracle: Oracle, dtype: str, rows: int, cols: int, rng: np.rand
            "fp8"       N(0,1) scaled to half of the largest finite value, 1 % exact zeros
     """
     shape = (rows, cols + pad)
-    if dtype in ("i4", "u4"):  # `cols` dimensions, two to a byte: every byte value, both nibbles random
-        packed = rng.integers(0, 256, size=(rows, (cols + 1) // 2 + pad), dtype=np.uint8)
-        return packed[:, : (cols + 1) // 2] if pad else packed
+    if dtype in DIMENSIONS_PER_VALUE:  # `cols` dimensions, two or eight to a byte: every byte value, all of it random
+        per = DIMENSIONS_PER_VALUE[dtype]
+        packed = rng.integers(0, 256, size=(rows, (cols + per - 1) // per + pad), dtype=np.uint8)
+        return packed[:, : (cols + per - 1) // per] if pad else packed
     if dtype in NARROW_FLOAT_DTYPES and kind == "default":  # every 6-bit code is a finite number; the top two bits are ignored
         full = rng.integers(0, 256, size=shape, dtype=np.uint8)
         return full[:, :cols] if pad else full

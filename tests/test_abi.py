@@ -161,7 +161,7 @@ def test_python_mirror_validates_arguments():
     with pytest.raises(ValueError):
         nk.dots_pack(cpu, "i8")  # must live on the GPU
     with pytest.raises(TypeError):
-        nk.dots_pack(cpu, "u1")
+        nk.dots_pack(cpu, "f64")
     with pytest.raises(TypeError):
         nk.dots_pack([[1, 2]], "i8")
     with pytest.raises(TypeError):

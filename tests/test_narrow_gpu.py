@@ -1,11 +1,12 @@
-"""Parity of the narrow types of the dots family (e2m3, e3m2, i4, u4) with the reference, through the C ABI, on a real MI355X.
+"""Parity of the narrow types of the dots family (e2m3, e3m2, i4, u4, u1) with the reference, through the C ABI, on a real MI355X.
 
 `nk_dots_packed_size_<T>`, `nk_dots_pack_<T>`, `nk_dots_packed_<T>`, `nk_dots_symmetric_<T>` for the 6-bit floats (one
-per byte) and the 4-bit integers (two per byte, depth counted in 4-bit values): reference
-include/numkong/dots/serial.h:2601-2678, arithmetic in include/numkong/dot/serial.h:602-800. On the GPU the 6-bit floats
-are widened, exactly, to f16 and the 4-bit integers to i8, B at pack time and A on its way into LDS.
+per byte), the 4-bit integers (two per byte, depth counted in 4-bit values) and single bits (eight per byte, depth in
+bits, the product is the popcount of the AND): reference include/numkong/dots/serial.h:2601-2695, arithmetic in
+include/numkong/dot/serial.h:602-832. On the GPU the 6-bit floats are widened, exactly, to f16 and the 4-bit integers
+and the bits to i8, B at pack time and A on its way into LDS.
 
-  * i4 / u4: bit-exact against the oracle's restatement of the serial kernels and against numpy int64 products of the
+  * i4 / u4 / u1: bit-exact against the oracle's restatement of the serial kernels and against numpy int64 products of the
     unpacked nibbles;
   * e2m3 / e3m2: the float gate of tests/test_dots_gpu.py against the serial restatement and the host-dispatched kernel;
     where every partial sum is exact in f32 (short depths: all values are multiples of 1/16 below 32) bit-exact as well;
@@ -20,7 +21,7 @@ torch = pytest.importorskip("torch")
 
 import numkong_amd as nk  # noqa: E402
 from tests import support  # noqa: E402
-from tests.support import NARROW_DTYPES, NARROW_FLOAT_DTYPES  # noqa: E402
+from tests.support import NARROW_DTYPES, NARROW_FLOAT_DTYPES, NARROW_INT_DTYPES  # noqa: E402
 from tests.test_dots_gpu import DEV, assert_float_gate, best_dispatch, gpu_dots, to_gpu  # noqa: E402
 from tests.test_symmetric_gpu import POISON, gpu_symmetric, owned, reference_library  # noqa: E402
 
@@ -28,6 +29,9 @@ pytestmark = pytest.mark.gpu
 
 
 def unpack_nibbles(dtype, x):
+    """The integer values behind the bytes of a sub-byte type, low bits first."""
+    if dtype == "u1":
+        return np.unpackbits(x, axis=1, bitorder="little").astype(np.int64)
     nibbles = np.stack([x & 0xF, x >> 4], axis=-1).reshape(x.shape[0], -1).astype(np.int64)
     return np.where(nibbles >= 8, nibbles - 16, nibbles) if dtype == "i4" else nibbles
 
@@ -35,7 +39,7 @@ def unpack_nibbles(dtype, x):
 def check(oracle, dtype, a, b, config=0, where=""):
     got = gpu_dots(dtype, a, b, config)
     serial = oracle.dots_packed(dtype, a, b)
-    if dtype in ("i4", "u4"):
+    if dtype in NARROW_INT_DTYPES:
         exact = (unpack_nibbles(dtype, a) @ unpack_nibbles(dtype, b).T) & 0xFFFFFFFF
         assert np.array_equal(got.view(np.uint32).astype(np.int64), exact), where
         assert np.array_equal(got.view(np.uint32), serial.view(np.uint32)), where
@@ -66,12 +70,12 @@ def test_every_byte_value_widens_exactly(oracle, dtype):
     stored = depth // support.DIMENSIONS_PER_VALUE.get(dtype, 1)
     every = np.zeros((256, stored), np.uint8)
     every[:, 0] = np.arange(256)
-    one = {"e2m3": 0x08, "e3m2": 0x0C, "i4": 0x01, "u4": 0x01}[dtype]
+    one = {"e2m3": 0x08, "e3m2": 0x0C, "i4": 0x01, "u4": 0x01, "u1": 0x01}[dtype]
     units = np.zeros((2, stored), np.uint8)
     units[0, 0] = one                                      # picks dimension 0
-    units[1, 0] = one << 4 if dtype in ("i4", "u4") else 0  # picks dimension 1 (the high nibble)
+    units[1, 0] = {"i4": 0x10, "u4": 0x10, "u1": 0x02}.get(dtype, 0)  # picks dimension 1 (the high nibble, the second bit)
     decoded = oracle.decode(dtype, every)
-    expected = decoded[:, :2] if dtype in ("i4", "u4") else np.stack([decoded[:, 0], np.zeros(256, np.float32)], axis=1)
+    expected = decoded[:, :2] if dtype in NARROW_INT_DTYPES else np.stack([decoded[:, 0], np.zeros(256, np.float32)], axis=1)
     as_a = gpu_dots(dtype, every, units)
     as_b = gpu_dots(dtype, units, every)
     assert np.array_equal(as_a.astype(np.float64), expected.astype(np.float64))
@@ -113,7 +117,7 @@ def test_deep_and_strided(oracle, dtype):
     assert (c[:, n:] == 0x5A5A5A5A).all()
     serial = oracle.dots_packed(dtype, a_full, b_full)
     got = np.ascontiguousarray(c[:, :n])
-    if dtype in ("i4", "u4"):
+    if dtype in NARROW_INT_DTYPES:
         assert np.array_equal(got, serial.view(np.uint32))
     else:
         truth, magnitude = oracle.truth(dtype, a_full, b_full)
@@ -131,7 +135,7 @@ def test_golden_vectors(oracle, name):
     bits = gpu_symmetric("dots", dtype, vectors, row_start, row_count)
     own = owned(vectors.shape[0], row_start, row_count)
     assert (bits[~own] == POISON).all()
-    if dtype in ("i4", "u4"):
+    if dtype in NARROW_INT_DTYPES:
         assert np.array_equal(got.view(np.uint32), data["c_serial"].view(np.uint32))
         assert np.array_equal(bits[own], data["symmetric_serial"].view(np.uint32)[own])
     else:
@@ -149,7 +153,7 @@ def test_symmetric_windows(oracle, dtype):
         bits = gpu_symmetric("dots", dtype, vectors, row_start, row_count)
         assert (bits[~own] == POISON).all()
         serial = oracle.symmetric("dots", dtype, vectors, row_start, row_count)
-        if dtype in ("i4", "u4"):
+        if dtype in NARROW_INT_DTYPES:
             assert np.array_equal(bits[own], serial.view(np.uint32)[own])
         else:
             truth, magnitude = oracle.truth(dtype, vectors, vectors)
@@ -177,7 +181,7 @@ def test_full_size_properties(oracle, dtype):
     rows = np.array([0, 1001, 4095])
     sample = rectangle[torch.from_numpy(rows).to(DEV)].cpu().numpy()
     serial = oracle.dots_packed(dtype, vectors[rows], vectors)
-    if dtype in ("i4", "u4"):
+    if dtype in NARROW_INT_DTYPES:
         assert np.array_equal(sample.view(np.uint32), serial.view(np.uint32))
     else:
         truth, magnitude = oracle.truth(dtype, vectors[rows], vectors)

@@ -347,8 +347,8 @@ def test_six_bit_floats_match_reference_and_definition(oracle, reference, dtype)
 
 @pytest.mark.parametrize("dtype", NARROW_DTYPES)
 def test_narrow_products_match_reference_serial(oracle, reference, dtype):
-    """nk_dots_packed_<T>_serial and nk_dots_symmetric_<T>_serial for e2m3, e3m2, i4, u4, bit for bit, odd depths
-    (whole bytes for the 4-bit types, both nibbles of the last one) included."""
+    """nk_dots_packed_<T>_serial and nk_dots_symmetric_<T>_serial for e2m3, e3m2, i4, u4, u1, bit for bit, depths that
+    do not fill the last byte of a sub-byte type (whole bytes are read) included."""
     if reference is None:
         pytest.skip("reference build not present")
     rng = np.random.default_rng(64)
@@ -365,14 +365,16 @@ def test_narrow_products_match_reference_serial(oracle, reference, dtype):
 
 @pytest.mark.parametrize("dtype", NARROW_DTYPES)
 def test_narrow_products_closed_forms(oracle, dtype):
-    """Needs no reference. 4-bit integers: the exact product of the unpacked nibbles (low nibble first, i4 sign-extended)
-    in numpy int64. 6-bit floats: every value is a multiple of 1/8 (e2m3) or 1/16 (e3m2) below 2^5, so short dots are
+    """Needs no reference. 4-bit integers and bits: the exact product of the unpacked values (low bits first, i4
+    sign-extended) in numpy int64. 6-bit floats: every value is a multiple of 1/8 (e2m3) or 1/16 (e3m2) below 2^5, so short dots are
     exact in f32 and must equal the f64 product of the decoded values."""
     rng = np.random.default_rng(65)
     a, b = support.random_matrix(oracle, dtype, 9, 64, rng), support.random_matrix(oracle, dtype, 11, 64, rng)
     got = oracle.dots_packed(dtype, a, b)
-    if dtype in ("i4", "u4"):
+    if dtype in ("i4", "u4", "u1"):
         def unpack(x):
+            if dtype == "u1":
+                return np.unpackbits(x, axis=1, bitorder="little").astype(np.int64)
             nibbles = np.stack([x & 0xF, x >> 4], axis=-1).reshape(x.shape[0], -1).astype(np.int64)
             return np.where(nibbles >= 8, nibbles - 16, nibbles) if dtype == "i4" else nibbles
         exact = unpack(a) @ unpack(b).T
