@@ -30,11 +30,13 @@ if ROOT not in sys.path:
 
 # MI355X published dense peaks, in T(FL)OP/s, for the MFMA the dtype runs on; HBM3E in GB/s.
 MFMA_PEAK = {"i8": 5000.0, "u8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "e4m3": 2500.0, "e5m2": 2500.0,
-             "e2m3": 2500.0, "e3m2": 2500.0, "i4": 5000.0, "u4": 5000.0, "u1": 5000.0}
+             "e2m3": 2500.0, "e3m2": 2500.0, "i4": 5000.0, "u4": 5000.0, "u1": 5000.0, "f32": 78.6, "f64": 78.6}
 MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2": "widened to f16, priced against the f16 MFMA peak",
              "e2m3": "widened to f16, priced against the f16 MFMA peak", "e3m2": "widened to f16, priced against the f16 MFMA peak",
              "i4": "widened to i8, priced against the i8 MFMA peak", "u4": "widened to i8, priced against the i8 MFMA peak",
-             "u1": "bits widened to i8 zeros and ones, priced against the i8 MFMA peak"}
+             "u1": "bits widened to i8 zeros and ones, priced against the i8 MFMA peak",
+             "f32": "f64 accumulation on the vector units (same 78.6 TFLOP/s as the f64 MFMA)",
+             "f64": "compensated f64 sums on the vector units: about 17 f64 operations per multiply-add, priced as 2"}
 HBM_PEAK = 8000.0
 # HBM-side bytes per launch (L2 <-> fabric) from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --probe`,
 # each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
@@ -51,7 +53,8 @@ MEASURED_TRAFFIC = {
 HEADLINE = ("i8", 8192, 8192, 8192)
 OTHERS = [("bf16", 8192, 8192, 8192, "dots"), ("e4m3", 8192, 8192, 8192, "dots"), ("i8", 1024, 1 << 20, 768, "dots"),
           ("i8", 1024, 1 << 20, 768, "angular"), ("i8", 8192, 8192, 8192, "symmetric"), ("bf16", 8192, 8192, 8192, "symmetric"),
-          ("i4", 8192, 8192, 8192, "dots"), ("e2m3", 8192, 8192, 8192, "dots"), ("u1", 8192, 8192, 8192, "dots")]
+          ("i4", 8192, 8192, 8192, "dots"), ("e2m3", 8192, 8192, 8192, "dots"), ("u1", 8192, 8192, 8192, "dots"),
+          ("f32", 4096, 4096, 4096, "dots"), ("f64", 4096, 4096, 4096, "dots")]
 KINDS = {"angular": ord("N"), "euclidean": ord("E")}  # nk_kernel_angulars_packed_k, nk_kernel_euclideans_packed_k
 # nk_kernel_dots_symmetric_k, nk_kernel_angulars_symmetric_k, nk_kernel_euclideans_symmetric_k
 SYMMETRIC_KINDS = {"symmetric": ord("y"), "symmetric-angular": ord("n"), "symmetric-euclidean": ord("D")}
@@ -66,6 +69,8 @@ def make_operands(dtype, m, n, k, seed=42):
     def one(rows):
         if dtype in ("i4", "u4"):  # two 4-bit values per byte, every byte value
             return torch.randint(0, 256, (rows, (k + 1) // 2), dtype=torch.uint8, device="cuda:0", generator=g)
+        if dtype in ("f32", "f64"):
+            return torch.randn((rows, k), device="cuda:0", generator=g, dtype=torch.float32 if dtype == "f32" else torch.float64)
         if dtype == "u1":  # eight bits per byte
             return torch.randint(0, 256, (rows, (k + 7) // 8), dtype=torch.uint8, device="cuda:0", generator=g)
         if dtype in ("e2m3", "e3m2"):  # every 6-bit code is a finite number
@@ -143,14 +148,16 @@ def time_gpu(dtype, m, n, k, steps, warmup, metric="dots"):
     a, b = make_operands(dtype, m, n, k)
     packed = nk.dots_pack(b, dtype)
     del b
-    c = torch.empty((m, n), dtype=torch.int32 if dtype in ("i8", "u8") and metric == "dots" else torch.float32, device="cuda:0")
+    wide = dtype in ("f32", "f64")  # f64 results
+    c = torch.empty((m, n), dtype=torch.float64 if wide else (torch.int32 if dtype in ("i8", "u8") and metric == "dots" else torch.float32),
+                    device="cuda:0")
     code, row_bytes = api.DTYPES[dtype][0], a.shape[1] * a.element_size()
     stream = torch.cuda.current_stream().cuda_stream  # the kernel is launched on this stream, so torch events see it
 
     def step():
         if metric == "dots":
             status = lib.nk_amd_dots_packed_async(code, a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(), m, n, k,
-                                                  row_bytes, n * 4, stream)
+                                                  row_bytes, n * c.element_size(), stream)
         else:  # the same product with the distance finaliser fused into its epilogue
             status = lib.nk_amd_spatials_packed_async(KINDS[metric], code, a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(),
                                                       m, n, k, row_bytes, n * 4, stream)

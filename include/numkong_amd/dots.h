@@ -64,6 +64,7 @@ typedef enum {
     nk_i32_k = 1 << 4,
     nk_u8_k = 1 << 6,
     nk_u32_k = 1 << 8,
+    nk_f64_k = 1 << 10,
     nk_f32_k = 1 << 11,
     nk_f16_k = 1 << 12,
     nk_bf16_k = 1 << 13,
@@ -122,6 +123,8 @@ NK_DYNAMIC nk_size_t nk_dots_packed_size_e3m2(nk_size_t width, nk_size_t depth);
 NK_DYNAMIC nk_size_t nk_dots_packed_size_i4(nk_size_t width, nk_size_t depth); /* depth in 4-bit values */
 NK_DYNAMIC nk_size_t nk_dots_packed_size_u4(nk_size_t width, nk_size_t depth);
 NK_DYNAMIC nk_size_t nk_dots_packed_size_u1(nk_size_t width, nk_size_t depth); /* depth in bits */
+NK_DYNAMIC nk_size_t nk_dots_packed_size_f32(nk_size_t width, nk_size_t depth);
+NK_DYNAMIC nk_size_t nk_dots_packed_size_f64(nk_size_t width, nk_size_t depth);
 
 /* Pack row-major B (width rows of depth elements, b_stride bytes apart). Reference: include/numkong/dots.h:203-237. */
 NK_DYNAMIC void nk_dots_pack_i8(nk_i8_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride, void *b_packed);
@@ -144,6 +147,10 @@ NK_DYNAMIC void nk_dots_pack_u4(nk_u4x2_t const *b, nk_size_t width, nk_size_t d
                                 void *b_packed);
 NK_DYNAMIC void nk_dots_pack_u1(nk_u1x8_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
                                 void *b_packed);
+NK_DYNAMIC void nk_dots_pack_f32(nk_f32_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
+                                 void *b_packed);
+NK_DYNAMIC void nk_dots_pack_f64(nk_f64_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,
+                                 void *b_packed);
 
 /* C = A * B^T with widened accumulators, C overwritten. Reference: include/numkong/dots.h:248-287. */
 NK_DYNAMIC void nk_dots_packed_i8(nk_i8_t const *a, void const *b_packed, nk_i32_t *c, nk_size_t height,
@@ -169,6 +176,13 @@ NK_DYNAMIC void nk_dots_packed_u4(nk_u4x2_t const *a, void const *b_packed, nk_u
 /* 1-bit values: c[i][j] = popcount(a_i AND b_j). Reference: include/numkong/dots.h:289-296. */
 NK_DYNAMIC void nk_dots_packed_u1(nk_u1x8_t const *a, void const *b_packed, nk_u32_t *c, nk_size_t height,
                                   nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
+
+/* The two wide types: f64 results. f32 products are exact in f64 and summed in f64; f64 uses the reference's
+ * compensated sum, and both reproduce its serial kernels bit for bit (include/numkong/dot/serial.h:262-335). */
+NK_DYNAMIC void nk_dots_packed_f32(nk_f32_t const *a, void const *b_packed, nk_f64_t *c, nk_size_t height,
+                                   nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
+NK_DYNAMIC void nk_dots_packed_f64(nk_f64_t const *a, void const *b_packed, nk_f64_t *c, nk_size_t height,
+                                   nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
 
 /* Distances over the same packed B, in one pass: result[i][j] = angular (1 - cosine) or euclidean distance between
  * row i of A and row j of B, f32 for all six types. Reference: include/numkong/spatials.h:139-266. */
@@ -209,7 +223,7 @@ NK_AMD_DECLARE_SYMMETRIC_(e4m3, nk_e4m3_t, nk_f32_t)
 NK_AMD_DECLARE_SYMMETRIC_(e5m2, nk_e5m2_t, nk_f32_t)
 #undef NK_AMD_DECLARE_SYMMETRIC_
 
-/* The 6-bit floats, the 4-bit integers and the 1-bit type have the dot-product kinds only (packed above, symmetric here), with their
+/* The 6-bit floats, the 4-bit integers, the 1-bit type and the two wide types (f32, f64) have the dot-product kinds only (packed above, symmetric here), with their
  * backend-suffixed names; their distance kinds resolve to the error stubs. */
 #define NK_AMD_DECLARE_DOTS_ONLY_(T, in_t, out_t)                                                                      \
     NK_DYNAMIC void nk_dots_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,              \
@@ -229,6 +243,8 @@ NK_AMD_DECLARE_DOTS_ONLY_(e3m2, nk_e3m2_t, nk_f32_t)
 NK_AMD_DECLARE_DOTS_ONLY_(i4, nk_i4x2_t, nk_i32_t)
 NK_AMD_DECLARE_DOTS_ONLY_(u4, nk_u4x2_t, nk_u32_t)
 NK_AMD_DECLARE_DOTS_ONLY_(u1, nk_u1x8_t, nk_u32_t)
+NK_AMD_DECLARE_DOTS_ONLY_(f32, nk_f32_t, nk_f64_t)
+NK_AMD_DECLARE_DOTS_ONLY_(f64, nk_f64_t, nk_f64_t)
 #undef NK_AMD_DECLARE_DOTS_ONLY_
 
 /* Capability and lookup API. Reference: c/numkong.c:767-768, 831-913. */

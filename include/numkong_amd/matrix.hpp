@@ -55,6 +55,8 @@ NK_AMD_DEFINE_TYPE_(e4m3, nk_e4m3_t, nk_f32_t, 1)
 NK_AMD_DEFINE_TYPE_(e5m2, nk_e5m2_t, nk_f32_t, 1)
 NK_AMD_DEFINE_TYPE_(e2m3, nk_e2m3_t, nk_f32_t, 1)
 NK_AMD_DEFINE_TYPE_(e3m2, nk_e3m2_t, nk_f32_t, 1)
+NK_AMD_DEFINE_TYPE_(f32, nk_f32_t, nk_f64_t, 1)
+NK_AMD_DEFINE_TYPE_(f64, nk_f64_t, nk_f64_t, 1)
 #undef NK_AMD_DEFINE_TYPE_
 /* the sub-byte types are named after their storage in the C ABI: two 4-bit or eight 1-bit values to a byte */
 struct i4x2_t {

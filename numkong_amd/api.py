@@ -22,7 +22,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 
 # nk_dtype_t codes (reference: include/numkong/types.h:923-952)
 NK_I8, NK_I32, NK_U8, NK_U32 = 1 << 2, 1 << 4, 1 << 6, 1 << 8
-NK_F32, NK_F16, NK_BF16, NK_E4M3, NK_E5M2 = 1 << 11, 1 << 12, 1 << 13, 1 << 14, 1 << 15
+NK_F64, NK_F32, NK_F16, NK_BF16, NK_E4M3, NK_E5M2 = 1 << 10, 1 << 11, 1 << 12, 1 << 13, 1 << 14, 1 << 15
 NK_I4, NK_U4, NK_E2M3, NK_E3M2, NK_U1 = 1 << 16, 1 << 17, 1 << 18, 1 << 19, 1 << 1
 
 # name -> (nk code, bytes per stored value, output torch dtype name, dimensions per stored value)
@@ -38,6 +38,8 @@ DTYPES = {
     "i4": (NK_I4, 1, "int32", 2),  # two 4-bit values per byte: a (rows, depth / 2) byte tensor, as the reference's
     "u4": (NK_U4, 1, "int32", 2),  # bindings take them (python/matrix.c:603: depth *= dimensions per value)
     "u1": (NK_U1, 1, "int32", 8),  # eight bits per byte; the dot product is popcount(a & b)
+    "f32": (NK_F32, 4, "float64", 1),  # the two wide types give f64 results
+    "f64": (NK_F64, 8, "float64", 1),
 }
 
 
@@ -208,7 +210,7 @@ def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out):
         if packed.width > 1 and out.stride(1) != 1:
             raise ValueError("out rows must be contiguous")
     a_stride = int(a.stride(0)) * a.element_size() if height > 1 else int(a.shape[1]) * a.element_size()
-    c_stride = int(out.stride(0)) * 4 if height > 1 else packed.width * 4
+    c_stride = int(out.stride(0)) * out.element_size() if height > 1 else packed.width * out.element_size()
     getattr(library(), stem + packed.dtype)(
         a.data_ptr(), packed.buffer.data_ptr(), out.data_ptr(), height, packed.width, depth, a_stride, c_stride
     )
@@ -264,7 +266,7 @@ def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_r
     if first < 0 or last < 0 or first > count or last > count or first > last:
         raise ValueError(f"Invalid row range [{first}, {last}) for {count} vectors")
     stride = int(vectors.stride(0)) * vectors.element_size() if count > 1 else int(vectors.shape[1]) * vectors.element_size()
-    out_stride = int(out.stride(0)) * 4 if count > 1 else count * 4
+    out_stride = int(out.stride(0)) * out.element_size() if count > 1 else count * out.element_size()
     getattr(library(), stem + dtype)(vectors.data_ptr(), count, depth, stride, out.data_ptr(), out_stride, first, last - first)
     _check(stem + dtype)
     return out

@@ -3,7 +3,7 @@
  *  @file numkong_amd/csrc/dispatch.h
  *
  *  Mirrors the role of the reference's c/dispatch.h:37-506, reduced to the packed-dots, packed-distance and symmetric slots
- *  (reference slots: c/dispatch.h:279-336, 353-380) for i8, u8, bf16, f16, e4m3, e5m2, e2m3, e3m2, i4, u4, u1.
+ *  (reference slots: c/dispatch.h:279-336, 353-380) for i8, u8, bf16, f16, e4m3, e5m2, e2m3, e3m2, i4, u4, u1, f32, f64.
  */
 #ifndef NUMKONG_AMD_DISPATCH_H
 #define NUMKONG_AMD_DISPATCH_H
@@ -17,19 +17,19 @@ extern "C" {
 typedef struct {
     nk_dots_packed_size_punned_t dots_packed_size_i8, dots_packed_size_u8, dots_packed_size_bf16,
         dots_packed_size_f16, dots_packed_size_e4m3, dots_packed_size_e5m2, dots_packed_size_e2m3, dots_packed_size_e3m2,
-        dots_packed_size_i4, dots_packed_size_u4, dots_packed_size_u1;
+        dots_packed_size_i4, dots_packed_size_u4, dots_packed_size_u1, dots_packed_size_f32, dots_packed_size_f64;
     nk_dots_pack_punned_t dots_pack_i8, dots_pack_u8, dots_pack_bf16, dots_pack_f16, dots_pack_e4m3, dots_pack_e5m2, dots_pack_e2m3, dots_pack_e3m2,
-        dots_pack_i4, dots_pack_u4, dots_pack_u1;
+        dots_pack_i4, dots_pack_u4, dots_pack_u1, dots_pack_f32, dots_pack_f64;
     nk_dots_packed_punned_t dots_packed_i8, dots_packed_u8, dots_packed_bf16, dots_packed_f16, dots_packed_e4m3,
         dots_packed_e5m2, dots_packed_e2m3, dots_packed_e3m2,
-        dots_packed_i4, dots_packed_u4, dots_packed_u1;
+        dots_packed_i4, dots_packed_u4, dots_packed_u1, dots_packed_f32, dots_packed_f64;
     nk_dots_packed_punned_t angulars_packed_i8, angulars_packed_u8, angulars_packed_bf16, angulars_packed_f16,
         angulars_packed_e4m3, angulars_packed_e5m2;
     nk_dots_packed_punned_t euclideans_packed_i8, euclideans_packed_u8, euclideans_packed_bf16, euclideans_packed_f16,
         euclideans_packed_e4m3, euclideans_packed_e5m2;
     nk_dots_symmetric_punned_t dots_symmetric_i8, dots_symmetric_u8, dots_symmetric_bf16, dots_symmetric_f16,
         dots_symmetric_e4m3, dots_symmetric_e5m2, dots_symmetric_e2m3, dots_symmetric_e3m2,
-        dots_symmetric_i4, dots_symmetric_u4, dots_symmetric_u1;
+        dots_symmetric_i4, dots_symmetric_u4, dots_symmetric_u1, dots_symmetric_f32, dots_symmetric_f64;
     nk_dots_symmetric_punned_t angulars_symmetric_i8, angulars_symmetric_u8, angulars_symmetric_bf16,
         angulars_symmetric_f16, angulars_symmetric_e4m3, angulars_symmetric_e5m2;
     nk_dots_symmetric_punned_t euclideans_symmetric_i8, euclideans_symmetric_u8, euclideans_symmetric_bf16,
@@ -46,6 +46,11 @@ void nk_error_dots_(void const *a, void const *b_packed, void *c, nk_size_t m, n
                     nk_size_t a_stride, nk_size_t c_stride);
 void nk_error_dots_symmetric_(void const *vectors, nk_size_t n_vectors, nk_size_t depth, nk_size_t stride, void *result,
                               nk_size_t result_stride, nk_size_t row_start, nk_size_t row_count);
+/* the same two for the types with 8-byte outputs (f32, f64) */
+void nk_error_dots_wide_(void const *a, void const *b_packed, void *c, nk_size_t m, nk_size_t n, nk_size_t k,
+                         nk_size_t a_stride, nk_size_t c_stride);
+void nk_error_dots_symmetric_wide_(void const *vectors, nk_size_t n_vectors, nk_size_t depth, nk_size_t stride,
+                                   void *result, nk_size_t result_stride, nk_size_t row_start, nk_size_t row_count);
 
 /* Per-dtype lookup and table initialisation (reference: c/dispatch.h:483-506). */
 #define NK_AMD_DECLARE_DISPATCH_(T)                                                                              \
@@ -63,6 +68,8 @@ NK_AMD_DECLARE_DISPATCH_(e3m2)
 NK_AMD_DECLARE_DISPATCH_(i4)
 NK_AMD_DECLARE_DISPATCH_(u4)
 NK_AMD_DECLARE_DISPATCH_(u1)
+NK_AMD_DECLARE_DISPATCH_(f32)
+NK_AMD_DECLARE_DISPATCH_(f64)
 #undef NK_AMD_DECLARE_DISPATCH_
 
 /**
@@ -124,7 +131,7 @@ NK_AMD_DECLARE_DISPATCH_(u1)
     }
 
 /** The same for the types that have the dot-product kinds only (the 6-bit floats, the 4-bit integers). */
-#define NK_AMD_DEFINE_DISPATCH_DOTS_(T)                                                                               \
+#define NK_AMD_DEFINE_DISPATCH_DOTS_WITH_(T, dots_stub, symmetric_stub)                                               \
     void nk_dispatch_##T##_find_(nk_capability_t v, nk_kernel_kind_t k, nk_kernel_punned_t *m, nk_capability_t *c) { \
         typedef nk_kernel_punned_t m_t;                                                                               \
         if (v & nk_cap_gfx950_k) switch (k) {                                                                         \
@@ -141,10 +148,10 @@ NK_AMD_DECLARE_DISPATCH_(u1)
         case nk_kernel_dots_pack_k: *m = (m_t)nk_error_pack_, *c = 0; return;                                        \
         case nk_kernel_dots_packed_k:                                                                                 \
         case nk_kernel_angulars_packed_k:                                                                             \
-        case nk_kernel_euclideans_packed_k: *m = (m_t)nk_error_dots_, *c = 0; return;                                \
+        case nk_kernel_euclideans_packed_k: *m = (m_t)dots_stub, *c = 0; return;                                \
         case nk_kernel_dots_symmetric_k:                                                                              \
         case nk_kernel_angulars_symmetric_k:                                                                          \
-        case nk_kernel_euclideans_symmetric_k: *m = (m_t)nk_error_dots_symmetric_, *c = 0; return;                   \
+        case nk_kernel_euclideans_symmetric_k: *m = (m_t)symmetric_stub, *c = 0; return;                   \
         default: *m = (m_t)nk_error_dense_, *c = 0; return;                                                          \
         }                                                                                                             \
     }                                                                                                                 \
@@ -158,6 +165,11 @@ NK_AMD_DECLARE_DISPATCH_(u1)
         nk_dispatch_##T##_find_(caps, nk_kernel_dots_symmetric_k, (nk_kernel_punned_t *)&t->dots_symmetric_##T,      \
                                 &used);                                                                               \
     }
+
+#define NK_AMD_DEFINE_DISPATCH_DOTS_(T) NK_AMD_DEFINE_DISPATCH_DOTS_WITH_(T, nk_error_dots_, nk_error_dots_symmetric_)
+/** ... and for the two types whose outputs are 8 bytes wide. */
+#define NK_AMD_DEFINE_DISPATCH_WIDE_(T) \
+    NK_AMD_DEFINE_DISPATCH_DOTS_WITH_(T, nk_error_dots_wide_, nk_error_dots_symmetric_wide_)
 
 #ifdef __cplusplus
 }

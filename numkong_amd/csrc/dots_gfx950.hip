@@ -95,6 +95,8 @@ int nk_hip_stream_synchronize(void *stream) {
 }
 
 size_t nk_hip_dots_packed_size(int dtype, size_t n, size_t k) {
+    WideGeometry wide;
+    if (wide_geometry(dtype, n, k, wide)) return (size_t)wide.total_bytes;
     Geometry g;
     if (!make_geometry(dtype, n, k, g)) return 0;
     return (size_t)g.total_bytes;
@@ -105,9 +107,14 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
                       bool terms) {
     hipStream_t stream = (hipStream_t)stream_;
     Geometry g;
-    if (!make_geometry(dtype, n, k, g)) return fail_msg("nk_hip_dots_pack: unsupported dtype or dimensions");
+    bool const wide = dtype == kF32 || dtype == kF64;
+    if (!wide && !make_geometry(dtype, n, k, g)) return fail_msg("nk_hip_dots_pack: unsupported dtype or dimensions");
     if (!b_packed || ((uintptr_t)b_packed & 15)) return fail_msg("nk_hip_dots_pack: b_packed must be 16-byte aligned");
     if (n && k && !b) return fail_msg("nk_hip_dots_pack: b is NULL");
+    if (wide) {
+        hipError_t const status = wide_pack(dtype, b, n, k, b_stride, b_packed, stream);
+        return status == hipSuccess ? 0 : fail(status, "nk_hip_dots_pack (f32 / f64)");
+    }
     if (elem_bits_of(dtype) == 16 && (((uintptr_t)b | b_stride) & 1)) return fail_msg("nk_hip_dots_pack: 16-bit B is misaligned");
 
     PackedHeader h;
@@ -191,6 +198,12 @@ static int product_async(int dtype, int metric, void const *a, void const *b_pac
                          TriangleScratch const *triangle = nullptr, uint32_t shift = 0) {
     hipStream_t stream = (hipStream_t)stream_;
     if (!m || !n) return 0;
+    if (dtype == kF32 || dtype == kF64) { // f64 results, a kernel of their own
+        if (metric != 0) return fail_msg("nk_hip_dots_packed: f32 and f64 have the dot-product kinds only");
+        if (!c || !b_packed || (k && !a)) return fail_msg("nk_hip_dots_packed: NULL operand");
+        hipError_t const status = wide_product(dtype, a, b_packed, c, m, n, k, a_stride, c_stride, stream, triangle != nullptr, shift);
+        return status == hipSuccess ? 0 : fail(status, "nk_hip_dots_packed (f32 / f64)");
+    }
     Geometry geo;
     if (!make_geometry(dtype, n, k, geo)) return fail_msg("nk_hip_dots_packed: unsupported dtype or dimensions");
     if (m > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_packed: too many rows");
@@ -260,10 +273,15 @@ static bool symmetric_window(int dtype, size_t n, size_t k, size_t row_start, si
     w.row_end = row_count < n - row_start ? row_start + row_count : n;
     w.col_begin = row_start / kTileRows * kTileRows;
     w.columns = n - w.col_begin;
+    w.scratch_bytes = 0;
+    WideGeometry wide;
+    if (wide_geometry(dtype, w.columns, k, wide)) { // (no tile lists: that kernel walks the full grid and skips tiles)
+        w.image_bytes = (size_t)((wide.total_bytes + 255) & ~255ull);
+        return true;
+    }
     Geometry geo;
     if (!make_geometry(dtype, w.columns, k, geo)) return false;
     w.image_bytes = (size_t)((geo.total_bytes + 255) & ~255ull);
-    w.scratch_bytes = 0;
     uint32_t const shift = (uint32_t)(row_start - w.col_begin);
     for (int c = 1; c < kConfigCount; ++c) {
         size_t const bytes = triangle_scratch_bytes(w.row_end - row_start, w.columns, kConfigs[c].tm * 32,
@@ -290,7 +308,8 @@ int nk_hip_symmetric_async(int dtype, int metric, void const *vectors, size_t n,
     if (!symmetric_window(dtype, n, k, row_start, row_count, w)) return fail_msg("nk_hip_symmetric: unsupported dtype or dimensions");
     if (!workspace || ((uintptr_t)workspace & 255)) return fail_msg("nk_hip_symmetric: workspace must be 256-byte aligned");
     if (workspace_bytes < w.image_bytes + w.scratch_bytes) return fail_msg("nk_hip_symmetric: workspace too small");
-    if (!result || ((uintptr_t)result & 3) || (result_stride & 3)) return fail_msg("nk_hip_symmetric: result must be 4-byte aligned");
+    size_t const out_bytes = dtype == kF32 || dtype == kF64 ? 8 : 4;
+    if (!result || (((uintptr_t)result | result_stride) & (out_bytes - 1))) return fail_msg("nk_hip_symmetric: result is misaligned");
     if (k && !vectors) return fail_msg("nk_hip_symmetric: vectors is NULL");
     // The columns of the window, packed as the B of an ordinary product; the rows of the window are its A.
     uint8_t const *rows = (uint8_t const *)vectors;
@@ -298,7 +317,7 @@ int nk_hip_symmetric_async(int dtype, int metric, void const *vectors, size_t n,
                             metric != 0 || dtype == kU8);
     if (status) return status;
     TriangleScratch const scratch = {(uint32_t *)((uint8_t *)workspace + w.image_bytes), w.scratch_bytes};
-    uint8_t *c = (uint8_t *)result + row_start * result_stride + w.col_begin * 4;
+    uint8_t *c = (uint8_t *)result + row_start * result_stride + w.col_begin * out_bytes;
     return product_async(dtype, metric, rows + row_start * stride, workspace, c, w.row_end - row_start, w.columns, k, stride,
                          result_stride, stream, &scratch, (uint32_t)(row_start - w.col_begin));
 }

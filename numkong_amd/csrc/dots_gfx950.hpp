@@ -86,6 +86,17 @@ hipError_t launch_i4(GemmArgs &g, hipStream_t stream, TriangleScratch const *tri
 hipError_t launch_u4(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
 hipError_t launch_u1(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle);
 
+/** The wide types (f32, f64; f64 results), dots_gfx950_wide.hip: image = header + k-major f64 with zero padding. */
+struct WideGeometry {
+    uint32_t elem_bytes, n, k, n_padded, k_padded;
+    uint64_t total_bytes;
+};
+bool wide_geometry(int dtype, size_t n, size_t k, WideGeometry &g);
+hipError_t wide_pack(int dtype, void const *b, size_t n, size_t k, size_t b_stride, void *b_packed, hipStream_t stream);
+/** `triangle`: only the outputs with col >= row + shift (the symmetric kinds). */
+hipError_t wide_product(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n, size_t k,
+                        size_t a_stride, size_t c_stride, hipStream_t stream, bool triangle, uint32_t shift);
+
 extern int g_forced_config; // 0: the heuristic picks the tile shape; see nk_hip_set_tile_config
 extern int g_variant;       // timing experiments of tuning builds
 extern int g_cu_count;      // compute units of the device, asked once
@@ -117,6 +128,8 @@ enum : int {
     kE2M3 = 1 << 18, // 6-bit floats, one per byte (bits 6 and 7 ignored)
     kE3M2 = 1 << 19,
     kU1 = 1 << 1, // eight 1-bit values per byte
+    kF64 = 1 << 10, // the two wide types: f64 results, a vector kernel of their own (dots_gfx950_wide.hip)
+    kF32 = 1 << 11,
 };
 
 constexpr uint32_t kMagic = 0x35394B4Eu; // "NK95"

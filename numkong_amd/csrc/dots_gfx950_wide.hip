@@ -1,0 +1,270 @@
+/**
+ *  @brief The f32 and f64 members of the packed-dots family on gfx950: f64 results, vector units.
+ *  @file numkong_amd/csrc/dots_gfx950_wide.hip
+ *
+ *  Replaces `nk_dots_{packed_size,pack,packed,symmetric}_{f32,f64}_<isa>` (reference instantiations:
+ *  include/numkong/dots/serial.h:2458-2491; arithmetic: include/numkong/dot/serial.h:262-335,
+ *  include/numkong/scalar/serial.h:128-136, include/numkong/reduce/serial.h:33-48). Both produce f64:
+ *
+ *    f32  every product is exact in f64; four running f64 sums take the products by k mod 4 and are combined as
+ *         ((s0 + s1) + s2) + s3;
+ *    f64  compensated ("dot2"): two lanes by k mod 2, each a running sum plus the accumulated rounding errors of its
+ *         products (by FMA) and of its additions (TwoSum); the four numbers are folded by one more chain of TwoSums.
+ *
+ *  MI355X runs f64 on the vector units at the rate of its f64 matrix instructions (78.6 TFLOP/s either way), and the
+ *  compensated sum has no matrix form at all, so this is a register-tiled vector kernel, not an MFMA one: 256 threads
+ *  compute a 64 x 64 tile of C, 4 x 4 outputs each with the reference's own four accumulators per output, in the
+ *  reference's own order along k, so the results are those of its serial kernels bit for bit. A goes through LDS
+ *  transposed (k-major), B comes from an image that is already k-major f64: [64-byte header][k padded to 8][n padded
+ *  to 64] doubles, zeros in the padding (x * 0 adds nothing to either kind of sum).
+ */
+#include "dots_gfx950.hpp"
+
+namespace {
+
+constexpr int kWideTile = 64;  // rows and columns of C per workgroup
+constexpr int kWideDepth = 8;  // k per step through LDS
+
+struct WideArgs {
+    uint8_t const *a;
+    double const *b; // the image's doubles, right behind its header: element (k, column) at b[k * n_padded + column]
+    int dtype;
+    uint8_t *c;
+    uint64_t a_stride, c_stride;
+    uint32_t m, n, k, n_padded, k_padded;
+    uint32_t tri_shift, tri_mask; // symmetric form: store only col >= row + tri_shift (mask all ones), see GemmArgs
+};
+
+/** B (n rows of k elements, row-major, f32 or f64) -> k-major f64 with zero padding; 32 x 32 blocks through LDS so
+ *  that both sides are touched in runs. */
+template <bool F64>
+__global__ __launch_bounds__(256) void pack_wide_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
+                                                        uint32_t k, uint32_t n_padded, double *__restrict__ out,
+                                                        PackedHeader header) {
+    __shared__ double block[32][33];
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *(PackedHeader *)((uint8_t *)out - sizeof(PackedHeader)) = header;
+    uint32_t const row0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+    uint32_t const tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 32 x 8
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t const row = row0 + ty + 8 * i, at = k0 + tx;
+        double value = 0;
+        if (row < n && at < k) {
+            uint8_t const *source = b + (uint64_t)row * b_stride;
+            value = F64 ? ((double const *)source)[at] : (double)((float const *)source)[at];
+        }
+        block[ty + 8 * i][tx] = value;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t const at = k0 + ty + 8 * i, row = row0 + tx; // (padding rows and depths are written too, as zeros)
+        out[(uint64_t)at * n_padded + row] = block[tx][ty + 8 * i];
+    }
+}
+
+/** One step of the reference's compensated dot product (scalar/serial.h:128-136), contraction off: every operation
+ *  below rounds on its own, which is what makes the recovered errors exact. */
+__device__ __forceinline__ void dot2_step(double &sum, double &compensation, double a, double b) {
+#pragma clang fp contract(off)
+    double const product = a * b;
+    double const product_error = __builtin_fma(a, b, -product);
+    double const running = sum + product;
+    double const recovered = running - sum;
+    double const sum_error = (sum - (running - recovered)) + (product - recovered);
+    sum = running;
+    compensation += sum_error + product_error;
+}
+
+/** reduce/serial.h:33-48 over (s0, c0, s1, c1). */
+__device__ __forceinline__ double fold_compensated(double const (&lane)[4]) {
+#pragma clang fp contract(off)
+    double running = 0, error = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { // order: sum of lane 0, its compensation, sum of lane 1, its compensation
+        double const value = lane[i];
+        double const tentative = running + value;
+        double const recovered = tentative - running;
+        error += (running - (tentative - recovered)) + (value - recovered);
+        running = tentative;
+    }
+    return running + error;
+}
+
+template <bool F64>
+__global__ __launch_bounds__(256) void dots_wide_kernel(WideArgs g) {
+    __shared__ double a_lds[2][kWideDepth][kWideTile + 1];
+    __shared__ double b_lds[2][kWideDepth][kWideTile];
+    uint32_t const tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    uint32_t const row0 = blockIdx.y * kWideTile, col0 = blockIdx.x * kWideTile;
+    // symmetric form: a tile wholly left of the diagonal has nothing to store
+    if (((row0 + g.tri_shift) & g.tri_mask) > col0 + (kWideTile - 1)) return;
+    typedef __attribute__((address_space(1))) double global_f64_t;
+    typedef __attribute__((address_space(1))) uint64_t global_u64_t;
+    // Trust, but verify: an image packed for another type or other dimensions poisons the outputs (all bits set),
+    // the reference's error convention, instead of being read with this call's geometry.
+    PackedHeader const *header = (PackedHeader const *)((uint8_t const *)g.b - sizeof(PackedHeader));
+    if (!(header->magic == kMagic && header->version == kVersion && header->dtype == (uint32_t)g.dtype && header->n == g.n &&
+          header->k == g.k)) {
+        for (uint32_t at = tid; at < kWideTile * kWideTile; at += 256) {
+            uint32_t const row = row0 + at / kWideTile, col = col0 + at % kWideTile;
+            if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col)
+                *(global_u64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8) = ~0ull;
+        }
+        return;
+    }
+
+    // accumulators: per output, four numbers: f32 inputs: sums of k = 0, 1, 2, 3 mod 4; f64 inputs: (s0, c0, s1, c1)
+    double acc[4][4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[i][j][v] = 0;
+
+    // staging: A: thread t brings 2 consecutive k of row t / 4 ... (64 rows x 8 k = 512 values, 2 per thread);
+    //          B: thread t brings 2 consecutive columns of depth t / 32 (8 x 64 = 512 values, 2 per thread)
+    uint32_t const a_row = tid >> 2, a_k = (tid & 3) * 2;
+    uint32_t const b_k = tid >> 5, b_col = (tid & 31) * 2;
+    uint8_t const *a_source = g.a + (uint64_t)(row0 + a_row < g.m ? row0 + a_row : 0) * g.a_stride;
+    bool const a_exists = row0 + a_row < g.m;
+    double a_next[2], b_next[2];
+    auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            uint32_t const at = k0 + a_k + e;
+            double value = 0;
+            if (a_exists && at < g.k) value = F64 ? ((double const *)a_source)[at] : (double)((float const *)a_source)[at];
+            a_next[e] = value;
+        }
+        double const *b_source = g.b + (uint64_t)(k0 + b_k) * g.n_padded + col0 + b_col; // (inside the padded image)
+        b_next[0] = b_source[0], b_next[1] = b_source[1];
+    };
+    auto stash = [&](int buffer) {
+        a_lds[buffer][a_k][a_row] = a_next[0], a_lds[buffer][a_k + 1][a_row] = a_next[1];
+        b_lds[buffer][b_k][b_col] = b_next[0], b_lds[buffer][b_k][b_col + 1] = b_next[1];
+    };
+
+    // The reference pads a row with zeros to its step (4 values for f32, 2 for f64) and runs them through the sums
+    // like any other (which can turn a -0 sum into +0); so does this, and no further.
+    uint32_t const depth = F64 ? (g.k + 1) & ~1u : (g.k + 3) & ~3u;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    int buffer = 0;
+    for (uint32_t k0 = 0; k0 < depth; k0 += kWideDepth) {
+        bool const more = k0 + kWideDepth < depth;
+        if (more) fetch(k0 + kWideDepth);
+#pragma unroll
+        for (int kk = 0; kk < kWideDepth; ++kk) {
+            if (k0 + kk >= depth) break; // (uniform; only the last step can be short)
+            double a_value[4], b_value[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a_value[i] = a_lds[buffer][kk][ty + 16 * i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b_value[j] = b_lds[buffer][kk][tx + 16 * j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (F64) dot2_step(acc[i][j][2 * (kk & 1)], acc[i][j][2 * (kk & 1) + 1], a_value[i], b_value[j]);
+                    else acc[i][j][kk & 3] = __builtin_fma(a_value[i], b_value[j], acc[i][j][kk & 3]); // exact product, one rounding
+                }
+        }
+        if (more) stash(buffer ^ 1);
+        __syncthreads();
+        buffer ^= 1;
+    }
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t const row = row0 + ty + 16 * i;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t const col = col0 + tx + 16 * j;
+            double result;
+            if (F64) result = fold_compensated(acc[i][j]);
+            else {
+#pragma clang fp contract(off)
+                result = ((acc[i][j][0] + acc[i][j][1]) + acc[i][j][2]) + acc[i][j][3];
+            }
+            if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col)
+                *(global_f64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8) = result;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_wide_kernel(uint8_t *c, uint32_t m, uint32_t n, uint64_t c_stride, uint64_t bits,
+                                                        uint32_t tri_shift, uint32_t tri_mask) {
+    uint64_t const i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    uint64_t const row = i / n, col = i % n;
+    if (row < m && (((uint32_t)row + tri_shift) & tri_mask) <= (uint32_t)col) *(uint64_t *)(c + row * c_stride + col * 8) = bits;
+}
+
+} // namespace
+
+namespace nk_gfx950 {
+
+bool wide_geometry(int dtype, size_t n, size_t k, WideGeometry &g) {
+    if (dtype != kF32 && dtype != kF64) return false;
+    if (n > 0x7FFFFFFFull || k > 65535ull * 32) return false; // (one workgroup row of the pack grid per 32 depths)
+    g.elem_bytes = dtype == kF64 ? 8 : 4;
+    g.n = (uint32_t)n, g.k = (uint32_t)k;
+    g.n_padded = (uint32_t)((n + kWideTile - 1) / kWideTile * kWideTile);
+    g.k_padded = (uint32_t)((k + 31) / 32 * 32); // the pack kernel writes whole 32 x 32 blocks
+    g.total_bytes = sizeof(PackedHeader) + (uint64_t)g.n_padded * g.k_padded * 8;
+    return true;
+}
+
+hipError_t wide_pack(int dtype, void const *b, size_t n, size_t k, size_t b_stride, void *b_packed, hipStream_t stream) {
+    WideGeometry g;
+    if (!wide_geometry(dtype, n, k, g)) return hipErrorInvalidValue;
+    if (((uintptr_t)b | b_stride) & (g.elem_bytes - 1)) return hipErrorInvalidValue; // elements must be aligned
+    PackedHeader h;
+    memset(&h, 0, sizeof(h));
+    h.magic = kMagic, h.version = kVersion, h.dtype = (uint32_t)dtype, h.elem_bytes = 8;
+    h.n = g.n, h.k = g.k, h.n_tiles = g.n_padded / kWideTile, h.k_chunks = g.k_padded;
+    h.data_offset = sizeof(PackedHeader), h.sums_offset = h.norms_offset = h.total_bytes = g.total_bytes;
+    double *out = (double *)((uint8_t *)b_packed + sizeof(PackedHeader));
+    if (!g.n_padded || !g.k_padded) {
+        hipLaunchKernelGGL(write_header_kernel, dim3(1), dim3(64), 0, stream, (PackedHeader *)b_packed, h);
+        return hipGetLastError();
+    }
+    dim3 const grid(g.n_padded / 32, g.k_padded / 32);
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    if (dtype == kF64) hipLaunchKernelGGL(pack_wide_kernel<true>, grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, out, h);
+    else hipLaunchKernelGGL(pack_wide_kernel<false>, grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, out, h);
+    return hipGetLastError();
+}
+
+hipError_t wide_product(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n, size_t k,
+                        size_t a_stride, size_t c_stride, hipStream_t stream, bool triangle, uint32_t shift) {
+    WideGeometry geo;
+    if (!wide_geometry(dtype, n, k, geo)) return hipErrorInvalidValue;
+    if (m > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    if (((uintptr_t)c | c_stride) & 7) return hipErrorInvalidValue;
+    uint32_t const tri_mask = triangle ? 0xFFFFFFFFu : 0u;
+    if (k == 0) {
+        uint64_t const blocks = ((uint64_t)m * n + 255) / 256;
+        if (blocks > 0x7FFFFFFFull) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(fill_wide_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t *)c, (uint32_t)m, (uint32_t)n,
+                           (uint64_t)c_stride, 0ull, shift, tri_mask);
+        return hipGetLastError();
+    }
+    if (((uintptr_t)a | a_stride) & (geo.elem_bytes - 1)) return hipErrorInvalidValue;
+    WideArgs g;
+    memset(&g, 0, sizeof(g));
+    g.dtype = dtype;
+    g.a = (uint8_t const *)a, g.b = (double const *)((uint8_t const *)b_packed + sizeof(PackedHeader)), g.c = (uint8_t *)c;
+    g.a_stride = a_stride, g.c_stride = c_stride;
+    g.m = (uint32_t)m, g.n = geo.n, g.k = geo.k, g.n_padded = geo.n_padded, g.k_padded = geo.k_padded;
+    g.tri_shift = shift, g.tri_mask = tri_mask;
+    dim3 const grid(geo.n_padded / kWideTile, (uint32_t)((m + kWideTile - 1) / kWideTile));
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    if (dtype == kF64) hipLaunchKernelGGL(dots_wide_kernel<true>, grid, dim3(256), 0, stream, g);
+    else hipLaunchKernelGGL(dots_wide_kernel<false>, grid, dim3(256), 0, stream, g);
+    return hipGetLastError();
+}
+
+} // namespace nk_gfx950

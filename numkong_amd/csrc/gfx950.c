@@ -42,21 +42,26 @@ static size_t nk_amd_row_bytes_(nk_dtype_t dtype, size_t k) {
     case nk_e3m2_k: return k;
     case nk_f16_k:
     case nk_bf16_k: return k * 2;
+    case nk_f32_k: return k * 4;
+    case nk_f64_k: return k * 8;
     default: return 0;
     }
 }
 
+/** Bytes of one output: f64 for the two wide types, 32 bits for everything else on this path. */
+static size_t nk_amd_output_bytes_(nk_dtype_t dtype) { return dtype == nk_f32_k || dtype == nk_f64_k ? 8 : 4; }
+
 static size_t nk_amd_round_up_(size_t x, size_t to) { return (x + to - 1) / to * to; }
 
 /** 0xFF over the m x n outputs only: the reference stub writes n * 8 bytes per row (c/numkong.c:209-216),
- *  which overruns 4-byte outputs; the convention is kept, the overrun is not. */
-static void nk_amd_fill_error_(void *c, int c_kind, size_t m, size_t n, size_t c_stride) {
+ *  which overruns 4-byte outputs; the convention is kept, the overrun is not (`out_bytes` per output). */
+static void nk_amd_fill_error_(void *c, int c_kind, size_t m, size_t n, size_t c_stride, size_t out_bytes) {
     if (!c || !m || !n) return;
-    if (c_kind == 1) {
-        if (nk_hip_fill_rows_async(c, m, n, c_stride, 0xFFFFFFFFu, NULL) == 0) nk_hip_stream_synchronize(NULL);
+    if (c_kind == 1) { /* (as 32-bit words: two per f64 output) */
+        if (nk_hip_fill_rows_async(c, m, n * out_bytes / 4, c_stride, 0xFFFFFFFFu, NULL) == 0) nk_hip_stream_synchronize(NULL);
         return;
     }
-    for (size_t row = 0; row < m; ++row) memset((char *)c + row * c_stride, 0xFF, n * 4);
+    for (size_t row = 0; row < m; ++row) memset((char *)c + row * c_stride, 0xFF, n * out_bytes);
 }
 
 int nk_amd_dots_pack_async(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t k, nk_size_t b_stride,
@@ -124,16 +129,17 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
                            nk_size_t n, nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {
     nk_amd_error_[0] = 0;
     if (!m || !n) return;
+    size_t const out_bytes = nk_amd_output_bytes_(dtype);
     size_t const total = nk_hip_dots_packed_size((int)dtype, n, k);
     if (nk_hip_device_count() <= 0) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_packed: no HIP device");
-        nk_amd_fill_error_(c, 0, m, n, c_stride);
+        nk_amd_fill_error_(c, 0, m, n, c_stride, out_bytes);
         return;
     }
     int const c_kind = nk_hip_pointer_kind(c);
     if (!total || !b_packed || !c) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_packed: unsupported dtype or dimensions");
-        nk_amd_fill_error_(c, c_kind, m, n, c_stride);
+        nk_amd_fill_error_(c, c_kind, m, n, c_stride, out_bytes);
         return;
     }
     int const a_kind = k ? nk_hip_pointer_kind(a) : 1;
@@ -157,7 +163,7 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
         device_p = staged_p;
     }
     if (!status && c_kind == 0) {
-        device_c_stride = nk_amd_round_up_(n * 4, 16);
+        device_c_stride = nk_amd_round_up_(n * out_bytes, 16);
         status = nk_hip_malloc(&staged_c, m * device_c_stride);
         device_c = staged_c;
     }
@@ -167,11 +173,11 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
     if (!status && metric != 0)
         status = nk_hip_spatials_packed_async((int)dtype, metric, device_a, device_p, device_c, m, n, k, device_a_stride,
                                               device_c_stride, NULL);
-    if (!status && staged_c) status = nk_hip_memcpy2d_d2h(c, c_stride, staged_c, device_c_stride, n * 4, m, NULL);
+    if (!status && staged_c) status = nk_hip_memcpy2d_d2h(c, c_stride, staged_c, device_c_stride, n * out_bytes, m, NULL);
     if (!status) status = nk_hip_stream_synchronize(NULL);
     if (status) {
         nk_amd_set_error_("nk_dots_packed");
-        nk_amd_fill_error_(c, c_kind, m, n, c_stride);
+        nk_amd_fill_error_(c, c_kind, m, n, c_stride, out_bytes);
     }
     if (staged_a) nk_hip_free(staged_a);
     if (staged_p) nk_hip_free(staged_p);
@@ -200,8 +206,8 @@ int nk_amd_symmetric_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void const *
 }
 
 /** 0xFF over the whole n x n result, as the reference's stub does (c/numkong.c:218-227), 4 bytes per output. */
-static void nk_amd_fill_symmetric_error_(void *result, int kind, size_t n, size_t result_stride) {
-    nk_amd_fill_error_(result, kind, n, n, result_stride);
+static void nk_amd_fill_symmetric_error_(void *result, int kind, size_t n, size_t result_stride, size_t out_bytes) {
+    nk_amd_fill_error_(result, kind, n, n, result_stride, out_bytes);
 }
 
 /**
@@ -214,16 +220,17 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
                               nk_size_t row_count) {
     nk_amd_error_[0] = 0;
     if (!n || !row_count || row_start >= n) return;
+    size_t const out_bytes = nk_amd_output_bytes_(dtype);
     if (nk_hip_device_count() <= 0) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_symmetric: no HIP device");
-        nk_amd_fill_symmetric_error_(result, 0, n, result_stride);
+        nk_amd_fill_symmetric_error_(result, 0, n, result_stride, out_bytes);
         return;
     }
     int const r_kind = nk_hip_pointer_kind(result);
     size_t const workspace_bytes = nk_hip_symmetric_workspace_size((int)dtype, n, k, row_start, row_count);
     if (!workspace_bytes || !result) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_symmetric: unsupported dtype or dimensions");
-        nk_amd_fill_symmetric_error_(result, r_kind, n, result_stride);
+        nk_amd_fill_symmetric_error_(result, r_kind, n, result_stride, out_bytes);
         return;
     }
     size_t const row_end = row_count < n - row_start ? row_start + row_count : n;
@@ -245,26 +252,26 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
                                          row_bytes, n - first, NULL);
         device_v = (char const *)staged_v - first * device_stride;
     }
-    char *host_window = (char *)result + row_start * result_stride + first * 4;
+    char *host_window = (char *)result + row_start * result_stride + first * out_bytes;
     if (!status && r_kind == 0) {
-        device_r_stride = nk_amd_round_up_((n - first) * 4, 16);
+        device_r_stride = nk_amd_round_up_((n - first) * out_bytes, 16);
         status = nk_hip_malloc(&staged_r, (row_end - row_start) * device_r_stride);
         if (!status)
-            status = nk_hip_memcpy2d_h2d(staged_r, device_r_stride, host_window, result_stride, (n - first) * 4,
+            status = nk_hip_memcpy2d_h2d(staged_r, device_r_stride, host_window, result_stride, (n - first) * out_bytes,
                                          row_end - row_start, NULL);
-        device_r = (char *)staged_r - row_start * device_r_stride - first * 4;
+        device_r = (char *)staged_r - row_start * device_r_stride - first * out_bytes;
     }
     if (!status)
         status = nk_hip_symmetric_async((int)dtype, metric, device_v, n, k, device_stride, device_r, device_r_stride,
                                         row_start, row_count, workspace, workspace_bytes, NULL);
     if (!status && staged_r)
-        status = nk_hip_memcpy2d_d2h(host_window, result_stride, staged_r, device_r_stride, (n - first) * 4,
+        status = nk_hip_memcpy2d_d2h(host_window, result_stride, staged_r, device_r_stride, (n - first) * out_bytes,
                                      row_end - row_start, NULL);
     if (!status) status = nk_hip_stream_synchronize(NULL);
     else (void)nk_hip_stream_synchronize(NULL);
     if (status) {
         nk_amd_set_error_("nk_dots_symmetric");
-        nk_amd_fill_symmetric_error_(result, r_kind, n, result_stride);
+        nk_amd_fill_symmetric_error_(result, r_kind, n, result_stride, out_bytes);
     }
     if (staged_v) nk_hip_free(staged_v);
     if (staged_r) nk_hip_free(staged_r);
@@ -331,3 +338,5 @@ NK_AMD_DEFINE_BACKEND_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(i4, nk_i4x2_t, nk_i32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(u4, nk_u4x2_t, nk_u32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(u1, nk_u1x8_t, nk_u32_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(f32, nk_f32_t, nk_f64_t)
+NK_AMD_DEFINE_BACKEND_DOTS_(f64, nk_f64_t, nk_f64_t)

@@ -43,11 +43,23 @@ void nk_error_dots_(void const *a, void const *b_packed, void *c, nk_size_t m, n
     for (nk_size_t row = 0; row < m; ++row) nk_fill_error_((char *)c + row * c_stride, n * 4);
 }
 
+/** The same for the types with f64 outputs: n * 8 bytes per row, what the reference's stub writes for every type. */
+void nk_error_dots_wide_(void const *a, void const *b_packed, void *c, nk_size_t m, nk_size_t n, nk_size_t k,
+                         nk_size_t a_stride, nk_size_t c_stride) {
+    nk_error_dots_(a, b_packed, c, m, 2 * n, k, a_stride, c_stride);
+}
+
 /** The reference's stub poisons the whole n x n result, whatever the window (c/numkong.c:218-227). */
 void nk_error_dots_symmetric_(void const *vectors, nk_size_t n_vectors, nk_size_t depth, nk_size_t stride, void *result,
                               nk_size_t result_stride, nk_size_t row_start, nk_size_t row_count) {
     (void)row_start, (void)row_count;
     nk_error_dots_(vectors, 0, result, n_vectors, n_vectors, depth, stride, result_stride);
+}
+
+void nk_error_dots_symmetric_wide_(void const *vectors, nk_size_t n_vectors, nk_size_t depth, nk_size_t stride,
+                                   void *result, nk_size_t result_stride, nk_size_t row_start, nk_size_t row_count) {
+    (void)row_start, (void)row_count;
+    nk_error_dots_(vectors, 0, result, n_vectors, 2 * n_vectors, depth, stride, result_stride);
 }
 
 #define NK_AMD_DISPATCH_DOTS_(T, in_t, out_t)                                                                   \
@@ -108,6 +120,8 @@ NK_AMD_DISPATCH_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(i4, nk_i4x2_t, nk_i32_t)
 NK_AMD_DISPATCH_DOTS_(u4, nk_u4x2_t, nk_u32_t)
 NK_AMD_DISPATCH_DOTS_(u1, nk_u1x8_t, nk_u32_t)
+NK_AMD_DISPATCH_DOTS_(f32, nk_f32_t, nk_f64_t)
+NK_AMD_DISPATCH_DOTS_(f64, nk_f64_t, nk_f64_t)
 
 NK_DYNAMIC int nk_uses_dynamic_dispatch(void) { return 1; }
 
@@ -142,6 +156,8 @@ NK_DYNAMIC void nk_dispatch_table_update(nk_capability_t caps) {
     nk_dispatch_i4_init_(caps);
     nk_dispatch_u4_init_(caps);
     nk_dispatch_u1_init_(caps);
+    nk_dispatch_f32_init_(caps);
+    nk_dispatch_f64_init_(caps);
 }
 
 NK_DYNAMIC void nk_find_kernel_punned(nk_kernel_kind_t kind, nk_dtype_t dtype, nk_capability_t viable,
@@ -160,6 +176,8 @@ NK_DYNAMIC void nk_find_kernel_punned(nk_kernel_kind_t kind, nk_dtype_t dtype, n
     case nk_i4_k: nk_dispatch_i4_find_(viable, kind, m, c); return;
     case nk_u4_k: nk_dispatch_u4_find_(viable, kind, m, c); return;
     case nk_u1_k: nk_dispatch_u1_find_(viable, kind, m, c); return;
+    case nk_f32_k: nk_dispatch_f32_find_(viable, kind, m, c); return;
+    case nk_f64_k: nk_dispatch_f64_find_(viable, kind, m, c); return;
     default: break;
     }
     *m = (nk_kernel_punned_t)0;
@@ -192,6 +210,8 @@ NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t i
     case nk_e5m2_k:
     case nk_e2m3_k:
     case nk_e3m2_k: return nk_f32_k;
+    case nk_f32_k:
+    case nk_f64_k: return nk_f64_k;
     default: return nk_dtype_unknown_k;
     }
 }

@@ -53,6 +53,13 @@
  *      tie) and nk_dots_packed_<T>_serial / nk_dots_symmetric_<T>_serial; their distance kinds are not restated
  *      (and not built).
  *
+ *    - the two wide types, products only (packed and symmetric), f64 results: f32 by four f64 lane sums, f64 by the
+ *      compensated two-lane sum with its compensated fold
+ *          include/numkong/dot/serial.h:262-335, include/numkong/scalar/serial.h:128-136, include/numkong/reduce/serial.h:33-48
+ *      Pinned bit for bit against nk_dots_packed_{f32,f64}_serial / nk_dots_symmetric_{f32,f64}_serial, and by what
+ *      the arithmetic fixes: integer-valued inputs (exact), and for f64 a sum that cancels catastrophically in plain
+ *      f64 and comes out right only if the compensation works.
+ *
  *  Parity unpinned: the per-column norms of FLOAT types in the serial packed image as stored bytes (the
  *  reference computes them with the host-dispatched nk_reduce_moments_*, whose summation order is not restated
  *  here). They are not read by dots_packed; nko_serial_pack writes zeros there and the tests compare header +
@@ -75,6 +82,8 @@ enum {
     NKO_E2M3 = 1 << 18, /* 6-bit floats, one per byte, bits 6 and 7 ignored */
     NKO_E3M2 = 1 << 19,
     NKO_U1 = 1 << 1, /* eight 1-bit values per byte; their dot product is the popcount of the AND */
+    NKO_F64 = 1 << 10, /* the two wide types: 8-byte (f64) results */
+    NKO_F32 = 1 << 11,
 };
 
 #define NKO_API __attribute__((visibility("default")))
@@ -529,6 +538,47 @@ static uint32_t serial_dot_bits(int dtype, void const *a_row, void const *b_row,
     return f32_to_bits(((lanes[0] + lanes[1]) + lanes[2]) + lanes[3]);
 }
 
+/** The wide types. f32 (dot/serial.h:305-335): products, exact in f64, go to four f64 sums by k mod 4 (rows are padded
+ *  with zeros to a multiple of 4, and the zeros are added like any other term), combined ((s0 + s1) + s2) + s3.
+ *  f64 (dot/serial.h:262-303, scalar/serial.h:128-136, reduce/serial.h:33-48): two lanes by k mod 2 (padded to a multiple
+ *  of 2), each a running sum and a compensation fed by the exact error of every product (by fma) and of every addition
+ *  (TwoSum); the four numbers are folded in the order s0, c0, s1, c1 by one more compensated chain. This file is compiled
+ *  with contraction off, so every operation written here rounds on its own. */
+static double serial_dot_wide(int dtype, void const *a_row, void const *b_row, size_t depth) {
+    if (dtype == NKO_F32) {
+        float const *a = (float const *)a_row, *b = (float const *)b_row;
+        double lanes[4] = {0, 0, 0, 0};
+        size_t const padded = (depth + 3) / 4 * 4;
+        for (size_t l = 0; l < padded; ++l) {
+            double const x = l < depth ? (double)a[l] : 0.0, y = l < depth ? (double)b[l] : 0.0;
+            lanes[l & 3] += x * y;
+        }
+        return ((lanes[0] + lanes[1]) + lanes[2]) + lanes[3];
+    }
+    double const *a = (double const *)a_row, *b = (double const *)b_row;
+    double sums[2] = {0, 0}, compensations[2] = {0, 0};
+    size_t const padded = (depth + 1) / 2 * 2;
+    for (size_t l = 0; l < padded; ++l) {
+        double const x = l < depth ? a[l] : 0.0, y = l < depth ? b[l] : 0.0;
+        double const product = x * y;
+        double const product_error = fma(x, y, -product);
+        double const running = sums[l & 1] + product;
+        double const recovered = running - sums[l & 1];
+        double const sum_error = (sums[l & 1] - (running - recovered)) + (product - recovered);
+        sums[l & 1] = running;
+        compensations[l & 1] += sum_error + product_error;
+    }
+    double const values[4] = {sums[0], compensations[0], sums[1], compensations[1]};
+    double running = 0, error = 0;
+    for (int i = 0; i < 4; ++i) {
+        double const tentative = running + values[i];
+        double const recovered = tentative - running;
+        error += (running - (tentative - recovered)) + (values[i] - recovered);
+        running = tentative;
+    }
+    return running + error;
+}
+
 /** C = A * B^T with the serial backend's rounding from UNPACKED operands: what nk_dots_packed_<T>_serial returns for
  *  any of the ten types (for the six older ones it equals nko_serial_pack + nko_serial_packed, which also restate
  *  the serial image; for e2m3, e3m2, i4, u4, u1 only the arithmetic is restated: dot/serial.h:602-832). */
@@ -536,8 +586,11 @@ NKO_API void nko_serial_dots(int dtype, void const *a, void const *b, void *c, s
                              size_t a_stride, size_t b_stride, size_t c_stride) {
     for (size_t i = 0; i < rows; ++i) {
         uint32_t *out = (uint32_t *)((unsigned char *)c + i * c_stride);
-        for (size_t j = 0; j < columns; ++j)
-            out[j] = serial_dot_bits(dtype, (unsigned char const *)a + i * a_stride, (unsigned char const *)b + j * b_stride, depth);
+        for (size_t j = 0; j < columns; ++j) {
+            void const *a_row = (unsigned char const *)a + i * a_stride, *b_row = (unsigned char const *)b + j * b_stride;
+            if (dtype == NKO_F32 || dtype == NKO_F64) ((double *)out)[j] = serial_dot_wide(dtype, a_row, b_row, depth);
+            else out[j] = serial_dot_bits(dtype, a_row, b_row, depth);
+        }
     }
 }
 
@@ -558,6 +611,10 @@ NKO_API void nko_serial_symmetric(int dtype, int metric, void const *vectors, si
         unsigned char const *a_row = (unsigned char const *)vectors + i * stride;
         uint32_t *out = (uint32_t *)((unsigned char *)result + i * result_stride);
         for (size_t j = i; j < count; ++j) {
+            if (dtype == NKO_F32 || dtype == NKO_F64) { /* (dot-product kind only, 8-byte outputs) */
+                ((double *)out)[j] = serial_dot_wide(dtype, a_row, (unsigned char const *)vectors + j * stride, depth);
+                continue;
+            }
             uint32_t const dot = serial_dot_bits(dtype, a_row, (unsigned char const *)vectors + j * stride, depth);
             if (!metric) out[j] = dot;
             else out[j] = i == j ? 0u : f32_to_bits(serial_from_dot(dtype, metric, dot, norms[i], norms[j]));

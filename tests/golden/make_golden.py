@@ -20,7 +20,7 @@ def main():
         raise SystemExit("build oracle/_ref first: make -C oracle")
     out = support.GOLDEN_DIR
     rng = np.random.default_rng(2024)
-    only = sys.argv[1] if len(sys.argv) > 1 else ""  # e.g. "spatials", "symmetric" or "narrow": rewrite only that family's files
+    only = sys.argv[1] if len(sys.argv) > 1 else ""  # e.g. "spatials", "symmetric", "narrow" or "wide": rewrite only that family's files
     for dtype in support.FLOAT_DTYPES if only in ("", "cast", "dots") else []:
         codes = np.arange(256 if support.STORAGE[dtype] == np.uint8 else 65536).astype(support.STORAGE[dtype])
         if len(codes) > 256:
@@ -99,6 +99,19 @@ def main():
                             row_count=row_count,
                             symmetric_serial=np.where(own, reference.symmetric("dots", dtype, vectors, row_start, row_count), 0)
                             .astype(support.OUTPUT[dtype]), **extra)
+    # The wide types (f64 results): a ragged packed product with an odd depth and a symmetric window, lognormal inputs.
+    rng = np.random.default_rng(2028)
+    for dtype in support.WIDE_DTYPES if only in ("", "wide") else []:
+        a = np.ascontiguousarray(support.random_matrix(oracle, dtype, 13, 77, rng, "lognormal", pad=3))
+        b = np.ascontiguousarray(support.random_matrix(oracle, dtype, 21, 77, rng, "lognormal", pad=1))
+        count, depth, row_start, row_count = 45, 203, 5, 34
+        vectors = np.ascontiguousarray(support.random_matrix(oracle, dtype, count, depth, rng, "lognormal"))
+        i, j = np.arange(count)[:, None], np.arange(count)[None, :]
+        own = (i >= row_start) & (i < row_start + row_count) & (j >= i)
+        np.savez_compressed(os.path.join(out, f"wide_{dtype}.npz"), dtype=dtype, a=a, b=b,
+                            c_serial=reference.dots_packed(dtype, a, b), vectors=vectors, row_start=row_start,
+                            row_count=row_count,
+                            symmetric_serial=np.where(own, reference.symmetric("dots", dtype, vectors, row_start, row_count), 0.0))
     print("wrote", len(os.listdir(out)) - 1, "fixtures to", out)
 
 

@@ -18,11 +18,13 @@ GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
 
 # nk_dtype_t codes (reference: include/numkong/types.h:923-952)
 CODES = {"i8": 1 << 2, "u8": 1 << 6, "f32": 1 << 11, "f16": 1 << 12, "bf16": 1 << 13, "e4m3": 1 << 14, "e5m2": 1 << 15,
-         "i4": 1 << 16, "u4": 1 << 17, "e2m3": 1 << 18, "e3m2": 1 << 19, "u1": 1 << 1}
+         "i4": 1 << 16, "u4": 1 << 17, "e2m3": 1 << 18, "e3m2": 1 << 19, "u1": 1 << 1, "f64": 1 << 10}
 STORAGE = {"i8": np.int8, "u8": np.uint8, "f16": np.uint16, "bf16": np.uint16, "e4m3": np.uint8, "e5m2": np.uint8,
-           "i4": np.uint8, "u4": np.uint8, "e2m3": np.uint8, "e3m2": np.uint8, "u1": np.uint8}
+           "i4": np.uint8, "u4": np.uint8, "e2m3": np.uint8, "e3m2": np.uint8, "u1": np.uint8,
+           "f32": np.float32, "f64": np.float64}
 OUTPUT = {"i8": np.int32, "u8": np.uint32, "f16": np.float32, "bf16": np.float32, "e4m3": np.float32, "e5m2": np.float32,
-          "i4": np.int32, "u4": np.uint32, "e2m3": np.float32, "e3m2": np.float32, "u1": np.uint32}
+          "i4": np.int32, "u4": np.uint32, "e2m3": np.float32, "e3m2": np.float32, "u1": np.uint32,
+          "f32": np.float64, "f64": np.float64}
 FLOAT_DTYPES = ("bf16", "f16", "e4m3", "e5m2")
 ALL_DTYPES = ("i8", "u8") + FLOAT_DTYPES  # the types with every kind: packed dots, packed distances, symmetric
 # the types with the dot-product kinds only: 6-bit floats (one per byte), 4-bit integers (two per byte), bits (eight)
@@ -30,6 +32,7 @@ NARROW_FLOAT_DTYPES = ("e2m3", "e3m2")
 NARROW_INT_DTYPES = ("i4", "u4", "u1")
 NARROW_DTYPES = NARROW_FLOAT_DTYPES + NARROW_INT_DTYPES
 DIMENSIONS_PER_VALUE = {"i4": 2, "u4": 2, "u1": 8}
+WIDE_DTYPES = ("f32", "f64")  # f64 results; the dot-product kinds only
 
 
 def depth_of(dtype: str, matrix: np.ndarray) -> int:
@@ -97,7 +100,7 @@ class Oracle:
         m, k = a.shape[0], depth_of(dtype, a)
         n = b.shape[0]
         c = np.empty((m, n), dtype=OUTPUT[dtype])
-        if dtype in NARROW_DTYPES:
+        if dtype in NARROW_DTYPES or dtype in WIDE_DTYPES:
             self.lib.nko_serial_dots(CODES[dtype], _ptr(a), _ptr(b), _ptr(c), m, n, k, a.strides[0], b.strides[0], c.strides[0])
             return c
         packed = self.pack(dtype, b)
@@ -258,6 +261,12 @@ def random_matrix(oracle: Oracle, dtype: str, rows: int, cols: int, rng: np.rand
         return packed[:, : (cols + per - 1) // per] if pad else packed
     if dtype in NARROW_FLOAT_DTYPES and kind == "default":  # every 6-bit code is a finite number; the top two bits are ignored
         full = rng.integers(0, 256, size=shape, dtype=np.uint8)
+        return full[:, :cols] if pad else full
+    if dtype in WIDE_DTYPES:  # N(0,1), or the reference tests' lognormal family with random signs
+        z = rng.standard_normal(shape)
+        if kind == "lognormal":
+            z = np.exp(z) * rng.choice(np.array([-1.0, 1.0]), size=shape)
+        full = z.astype(STORAGE[dtype])
         return full[:, :cols] if pad else full
     if dtype == "i8":
         full = rng.integers(-128, 128, size=shape, dtype=np.int8)

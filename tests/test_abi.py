@@ -53,8 +53,10 @@ def test_packed_size_formula():
             assert nk.dots_packed_size(t, n, k) == 64 + tiles * chunks * 512 + tiles * 256, (t, n, k)
         assert nk.dots_packed_size(t, 0, 0) == 64
         assert nk.dots_packed_size(t, 1 << 40, 8) == 0  # dimensions beyond 32 bits are refused, as the error stub does
+    # the two wide types keep f64 values k-major: header + 8 bytes x (n padded to 64) x (k padded to 32)
+    assert nk.dots_packed_size("f32", 100, 70) == nk.dots_packed_size("f64", 100, 70) == 64 + 8 * 128 * 96
     with pytest.raises(TypeError):
-        nk.dots_packed_size("f64", 4, 4)
+        nk.dots_packed_size("f16c", 4, 4)
 
 
 def find(lib, kind, dtype_code, viable):
@@ -86,7 +88,19 @@ def test_lookup_and_capabilities():
             assert fn and cap == 0
         fn, cap = find(lib, ord("Y"), code, CAP_GFX950)  # symmetric hamming distances: not on this path
         assert fn and cap == 0
-    assert find(lib, ord("G"), 1 << 10, CAP_GFX950) == (None, 0)  # f64: unknown dtype -> null kernel
+    assert find(lib, ord("G"), 1 << 20, CAP_GFX950) == (None, 0)  # f64c: unknown dtype -> null kernel
+    for name in ("e2m3", "e3m2", "i4", "u4", "u1", "f32", "f64"):  # the dot-product kinds only
+        code = api.DTYPES[name][0]
+        for kind, stem in ((ord("P"), "nk_dots_packed_size_"), (ord("Q"), "nk_dots_pack_"), (ord("G"), "nk_dots_packed_"),
+                           (ord("y"), "nk_dots_symmetric_")):
+            fn, cap = find(lib, kind, code, CAP_GFX950 | 1)
+            assert fn == ctypes.cast(getattr(lib, f"{stem}{name}_gfx950"), ctypes.c_void_p).value and cap == CAP_GFX950
+        for kind in (ord("N"), ord("E"), ord("n"), ord("D")):
+            fn, cap = find(lib, kind, code, CAP_GFX950)
+            assert fn and cap == 0
+        expected = {"i4": 1 << 4, "u4": 1 << 8, "u1": 1 << 8, "f32": 1 << 10, "f64": 1 << 10}.get(name, 1 << 11)
+        assert lib.nk_kernel_output_dtype(ord("G"), code) == lib.nk_kernel_output_dtype(ord("y"), code) == expected
+        assert lib.nk_kernel_output_dtype(ord("N"), code) == 0
     out = {"i8": 1 << 4, "u8": 1 << 8, "bf16": 1 << 11, "f16": 1 << 11, "e4m3": 1 << 11, "e5m2": 1 << 11}
     for t, expected in out.items():
         assert lib.nk_kernel_output_dtype(ord("G"), api.DTYPES[t][0]) == expected
@@ -118,6 +132,10 @@ def test_error_convention_without_backend():
         g = np.zeros((5, 6), np.int32)
         lib.nk_dots_symmetric_i8(b.ctypes.data, 5, 7, 7, g.ctypes.data, 24, 1, 2)
         assert (g[:, :5] == -1).all() and (g[:, 5] == 0).all()
+        # the wide types' stubs poison 8 bytes per output
+        d = np.zeros((3, 6), np.float64)
+        lib.nk_dots_packed_f64(d.ctypes.data, packed.ctypes.data, d.ctypes.data, 3, 5, 6, 48, 48)
+        assert np.isnan(d[:, :5]).all() and (d[:, 5] == 0).all()
     finally:
         lib.nk_dispatch_table_update(lib.nk_capabilities_compiled())
     assert lib.nk_dots_packed_size_i8(5, 7) == 64 + 16 * 512 + 256
@@ -161,7 +179,7 @@ def test_python_mirror_validates_arguments():
     with pytest.raises(ValueError):
         nk.dots_pack(cpu, "i8")  # must live on the GPU
     with pytest.raises(TypeError):
-        nk.dots_pack(cpu, "f64")
+        nk.dots_pack(cpu, "f16c")
     with pytest.raises(TypeError):
         nk.dots_pack([[1, 2]], "i8")
     with pytest.raises(TypeError):
@@ -169,6 +187,6 @@ def test_python_mirror_validates_arguments():
     with pytest.raises(ValueError):
         nk.dots_symmetric(cpu, "i8")  # must live on the GPU
     with pytest.raises(TypeError):
-        nk.angulars_symmetric(cpu, "f64")
+        nk.angulars_symmetric(cpu, "f16c")
     with pytest.raises(TypeError):
         nk.euclideans_symmetric(cpu, "i4")  # the 4-bit integers have the dot-product kinds only

@@ -16,7 +16,7 @@ import numpy as np
 import pytest
 
 from tests import support
-from tests.support import ALL_DTYPES, FLOAT_DTYPES, NARROW_DTYPES, NARROW_FLOAT_DTYPES, STORAGE
+from tests.support import ALL_DTYPES, FLOAT_DTYPES, NARROW_DTYPES, NARROW_FLOAT_DTYPES, STORAGE, WIDE_DTYPES
 
 
 def same_floats(x, y):
@@ -387,6 +387,51 @@ def test_narrow_products_closed_forms(oracle, dtype):
         assert np.array_equal(truth, decoded_a @ decoded_b.T)
 
 
+@pytest.mark.parametrize("dtype", WIDE_DTYPES)
+def test_wide_products_match_reference_serial(oracle, reference, dtype):
+    """nk_dots_packed_{f32,f64}_serial and nk_dots_symmetric_{f32,f64}_serial (f64 results), bit for bit: N(0,1) and
+    lognormal inputs with random signs, depths off the 4- and 2-value steps."""
+    if reference is None:
+        pytest.skip("reference build not present")
+    rng = np.random.default_rng(66)
+    for kind in ("default", "lognormal"):
+        for m, n, k in [(1, 1, 1), (3, 5, 16), (7, 9, 101), (4, 4, 33), (13, 21, 77), (5, 6, 2050)]:
+            a, b = support.random_matrix(oracle, dtype, m, k, rng, kind), support.random_matrix(oracle, dtype, n, k, rng, kind)
+            assert np.array_equal(oracle.dots_packed(dtype, a, b).view(np.uint64), reference.dots_packed(dtype, a, b).view(np.uint64)), (dtype, kind, m, n, k)
+    for count, depth, row_start, row_count in SYMMETRIC_CASES[:6]:
+        vectors = support.random_matrix(oracle, dtype, count, depth, rng)
+        own = upper_window(count, row_start, row_count)
+        mine = oracle.symmetric("dots", dtype, vectors, row_start, row_count)
+        ref = reference.symmetric("dots", dtype, vectors, row_start, row_count)
+        assert np.array_equal(mine.view(np.uint64)[own], ref.view(np.uint64)[own]), (dtype, count, depth, row_start)
+        assert not mine[~own].any()
+
+
+def test_wide_products_closed_forms(oracle):
+    """Needs no reference. Small integers: every sum is exact in f64, so both kinds equal the int64 product. f64 only:
+    sums that plain f64 gets wrong and a sum in twice the working precision gets right: 1e100 + 1 - 1e100 = 1, and a
+    long alternating series whose large terms cancel, checked against exact rational arithmetic."""
+    from fractions import Fraction
+
+    rng = np.random.default_rng(67)
+    ints_a, ints_b = rng.integers(-1000, 1000, (9, 130)), rng.integers(-1000, 1000, (11, 130))
+    for dtype in WIDE_DTYPES:
+        got = oracle.dots_packed(dtype, ints_a.astype(support.STORAGE[dtype]), ints_b.astype(support.STORAGE[dtype]))
+        assert np.array_equal(got, (ints_a @ ints_b.T).astype(np.float64))
+    a = np.array([[1e100, 1.0, -1e100, 3.0]])
+    b = np.array([[1.0, 1.0, 1.0, 0.5]])
+    assert oracle.dots_packed("f64", a, b)[0, 0] == 2.5 and float(a[0] @ b[0]) != 2.5  # (numpy's plain sum loses the 1)
+    x = (rng.standard_normal((4, 257)) * 10.0 ** rng.integers(-8, 9, (4, 257)))
+    y = (rng.standard_normal((3, 257)) * 10.0 ** rng.integers(-8, 9, (3, 257)))
+    got = oracle.dots_packed("f64", x, y)
+    for i in range(4):
+        for j in range(3):
+            exact = sum(Fraction(float(p)) * Fraction(float(q)) for p, q in zip(x[i], y[j]))
+            scale = sum(abs(Fraction(float(p)) * Fraction(float(q))) for p, q in zip(x[i], y[j]))
+            # within one rounding of the exact value plus the second-order term of a doubled precision
+            assert abs(Fraction(float(got[i, j])) - exact) <= abs(exact) * Fraction(1, 2 ** 52) + scale * Fraction(257 ** 2, 2 ** 104)
+
+
 @pytest.mark.parametrize("dtype", ["i8", "u8"])
 def test_integer_product_closed_form(oracle, dtype):
     rng = np.random.default_rng(11)
@@ -440,6 +485,11 @@ def test_golden_vectors(oracle, name):
         dtype = str(data["dtype"])
         assert same_floats(oracle.decode(dtype, data["codes"]), data["decoded"])
         assert np.array_equal(oracle.encode(dtype, data["values"]), data["encoded"])
+    elif name.startswith("wide_"):
+        dtype, a, b, vectors = str(data["dtype"]), data["a"], data["b"], data["vectors"]
+        assert np.array_equal(oracle.dots_packed(dtype, a, b).view(np.uint64), data["c_serial"].view(np.uint64))
+        mine = oracle.symmetric("dots", dtype, vectors, int(data["row_start"]), int(data["row_count"]))
+        assert np.array_equal(mine.view(np.uint64), data["symmetric_serial"].view(np.uint64))
     elif name.startswith("narrow_"):
         dtype, a, b, vectors = str(data["dtype"]), data["a"], data["b"], data["vectors"]
         assert same_floats(oracle.dots_packed(dtype, a, b).view(np.float32), data["c_serial"].view(np.float32))
