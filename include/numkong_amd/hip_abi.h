@@ -11,7 +11,9 @@
  *  non-zero HIP error code; `nk_hip_last_error()` returns a thread-local description of the last failure.
  *
  *  `dtype` arguments take the `nk_dtype_t` codes of <numkong_amd/dots.h> (reference:
- *  include/numkong/types.h:923-952): nk_i8_k, nk_u8_k, nk_bf16_k, nk_f16_k, nk_e4m3_k, nk_e5m2_k.
+ *  include/numkong/types.h:923-952): nk_i8_k, nk_u8_k, nk_bf16_k, nk_f16_k, nk_e4m3_k, nk_e5m2_k (every kind), and
+ *  nk_e2m3_k, nk_e3m2_k, nk_i4_k, nk_u4_k, nk_u1_k, nk_f32_k, nk_f64_k (the dot-product kinds; depth counts
+ *  dimensions, so 4-bit values or bits for the sub-byte types; f32 and f64 write 8-byte f64 outputs).
  */
 #ifndef NUMKONG_AMD_HIP_ABI_H
 #define NUMKONG_AMD_HIP_ABI_H
@@ -44,7 +46,7 @@ int nk_hip_stream_synchronize(void *stream);
 
 /**
  *  Bytes of the gfx950 packed image of an (n x k) B matrix: 64-byte header, MFMA-fragment tiles,
- *  per-column compensation terms, per-column sums of squares. Replaces `nk_dots_packed_size_<T>_<isa>`
+ *  per-column compensation terms, per-column sums of squares (f32 / f64: header and k-major f64 values). Replaces `nk_dots_packed_size_<T>_<isa>`
  *  (reference: include/numkong/dots/serial.h:245-271). Returns 0 for an unsupported dtype or when
  *  n or k do not fit 32 bits.
  */
@@ -58,9 +60,9 @@ int nk_hip_dots_pack_async(int dtype, void const *b, size_t n, size_t k, size_t 
                            void *stream);
 
 /**
- *  C[m x n] = A[m x k] * B^T with widened accumulators (i32 / u32 / f32), C overwritten.
+ *  C[m x n] = A[m x k] * B^T with widened accumulators (i32 / u32 / f32; f64 for f32 and f64 inputs), C overwritten.
  *  Replaces `nk_dots_packed_<T>_<isa>` (reference: include/numkong/dots/serial.h:520-1072).
- *  A packed image whose header does not match (dtype, n, k) makes every C element 0xFFFFFFFF.
+ *  A packed image whose header does not match (dtype, n, k) makes every C element all ones (0xFF bytes).
  */
 int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n,
                              size_t k, size_t a_stride, size_t c_stride, void *stream);

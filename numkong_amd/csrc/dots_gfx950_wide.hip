@@ -15,8 +15,8 @@
  *  compensated sum has no matrix form at all, so this is a register-tiled vector kernel, not an MFMA one: 256 threads
  *  compute a 64 x 64 tile of C, 4 x 4 outputs each with the reference's own four accumulators per output, in the
  *  reference's own order along k, so the results are those of its serial kernels bit for bit. A goes through LDS
- *  transposed (k-major), B comes from an image that is already k-major f64: [64-byte header][k padded to 8][n padded
- *  to 64] doubles, zeros in the padding (x * 0 adds nothing to either kind of sum).
+ *  transposed (k-major), B comes from an image that is already k-major f64: [64-byte header][k padded to 32][n padded
+ *  to 64] doubles, zeros in the padding.
  */
 #include "dots_gfx950.hpp"
 
