@@ -35,7 +35,7 @@ MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2":
              "e2m3": "widened to f16, priced against the f16 MFMA peak", "e3m2": "widened to f16, priced against the f16 MFMA peak",
              "i4": "widened to i8, priced against the i8 MFMA peak", "u4": "widened to i8, priced against the i8 MFMA peak",
              "u1": "bits widened to i8 zeros and ones, priced against the i8 MFMA peak",
-             "f32": "f64 accumulation on the vector units (same 78.6 TFLOP/s as the f64 MFMA)",
+             "f32": "exact f32 products summed in f64 on the f64 MFMA (78.6 TFLOP/s), four sums per output as in the reference",
              "f64": "compensated f64 sums on the vector units: about 17 f64 operations per multiply-add, priced as 2"}
 HBM_PEAK = 8000.0
 # HBM-side bytes per launch (L2 <-> fabric) from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --probe`,

@@ -1,5 +1,5 @@
 /**
- *  @brief The f32 and f64 members of the packed-dots family on gfx950: f64 results, vector units.
+ *  @brief The f32 and f64 members of the packed-dots family on gfx950: f64 results.
  *  @file numkong_amd/csrc/dots_gfx950_wide.hip
  *
  *  Replaces `nk_dots_{packed_size,pack,packed,symmetric}_{f32,f64}_<isa>` (reference instantiations:
@@ -7,16 +7,17 @@
  *  include/numkong/scalar/serial.h:128-136, include/numkong/reduce/serial.h:33-48). Both produce f64:
  *
  *    f32  every product is exact in f64; four running f64 sums take the products by k mod 4 and are combined as
- *         ((s0 + s1) + s2) + s3;
+ *         ((s0 + s1) + s2) + s3. Runs on the f64 matrix cores (`dots_f32_matrix_kernel`): one MFMA is a chain of
+ *         fused multiply-adds along its depth, which is exactly how the reference advances one of its four sums.
  *    f64  compensated ("dot2"): two lanes by k mod 2, each a running sum plus the accumulated rounding errors of its
  *         products (by FMA) and of its additions (TwoSum); the four numbers are folded by one more chain of TwoSums.
+ *         No matrix form exists for that, so it is a register-tiled kernel on the vector units, which on MI355X run
+ *         f64 at the rate of the f64 matrix instructions (78.6 TFLOP/s either way): 256 threads compute a 64 x 64
+ *         tile of C, 4 x 4 outputs each, A through LDS transposed (k-major).
  *
- *  MI355X runs f64 on the vector units at the rate of its f64 matrix instructions (78.6 TFLOP/s either way), and the
- *  compensated sum has no matrix form at all, so this is a register-tiled vector kernel, not an MFMA one: 256 threads
- *  compute a 64 x 64 tile of C, 4 x 4 outputs each with the reference's own four accumulators per output, in the
- *  reference's own order along k, so the results are those of its serial kernels bit for bit. A goes through LDS
- *  transposed (k-major), B comes from an image that is already k-major f64: [64-byte header][k padded to 32][n padded
- *  to 64] doubles, zeros in the padding.
+ *  Either way every output keeps the reference's own accumulators and takes its terms in the reference's own order
+ *  along k, so the results are those of its serial kernels bit for bit. B comes from an image that is already k-major
+ *  f64: [64-byte header][k padded to 32][n padded to 64] doubles, zeros in the padding.
  */
 #include "dots_gfx950.hpp"
 
@@ -91,8 +92,7 @@ __device__ __forceinline__ double fold_compensated(double const (&lane)[4]) {
     return running + error;
 }
 
-template <bool F64>
-__global__ __launch_bounds__(256) void dots_wide_kernel(WideArgs g) {
+__global__ __launch_bounds__(256) void dots_f64_compensated_kernel(WideArgs g) {
     __shared__ double a_lds[2][kWideDepth][kWideTile + 1];
     __shared__ double b_lds[2][kWideDepth][kWideTile];
     uint32_t const tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void dots_wide_kernel(WideArgs g) {
         return;
     }
 
-    // accumulators: per output, four numbers: f32 inputs: sums of k = 0, 1, 2, 3 mod 4; f64 inputs: (s0, c0, s1, c1)
+    // accumulators: per output, four numbers: (s0, c0, s1, c1)
     double acc[4][4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void dots_wide_kernel(WideArgs g) {
         for (int e = 0; e < 2; ++e) {
             uint32_t const at = k0 + a_k + e;
             double value = 0;
-            if (a_exists && at < g.k) value = F64 ? ((double const *)a_source)[at] : (double)((float const *)a_source)[at];
+            if (a_exists && at < g.k) value = ((double const *)a_source)[at];
             a_next[e] = value;
         }
         double const *b_source = g.b + (uint64_t)(k0 + b_k) * g.n_padded + col0 + b_col; // (inside the padded image)
@@ -146,9 +146,9 @@ __global__ __launch_bounds__(256) void dots_wide_kernel(WideArgs g) {
         b_lds[buffer][b_k][b_col] = b_next[0], b_lds[buffer][b_k][b_col + 1] = b_next[1];
     };
 
-    // The reference pads a row with zeros to its step (4 values for f32, 2 for f64) and runs them through the sums
-    // like any other (which can turn a -0 sum into +0); so does this, and no further.
-    uint32_t const depth = F64 ? (g.k + 1) & ~1u : (g.k + 3) & ~3u;
+    // The reference pads a row with zeros to its step of 2 values and runs them through the sums like any other;
+    // so does this, and no further.
+    uint32_t const depth = (g.k + 1) & ~1u;
     fetch(0);
     stash(0);
     __syncthreads();
@@ -168,8 +168,7 @@ __global__ __launch_bounds__(256) void dots_wide_kernel(WideArgs g) {
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    if (F64) dot2_step(acc[i][j][2 * (kk & 1)], acc[i][j][2 * (kk & 1) + 1], a_value[i], b_value[j]);
-                    else acc[i][j][kk & 3] = __builtin_fma(a_value[i], b_value[j], acc[i][j][kk & 3]); // exact product, one rounding
+                    dot2_step(acc[i][j][2 * (kk & 1)], acc[i][j][2 * (kk & 1) + 1], a_value[i], b_value[j]);
                 }
         }
         if (more) stash(buffer ^ 1);
@@ -183,16 +182,135 @@ __global__ __launch_bounds__(256) void dots_wide_kernel(WideArgs g) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             uint32_t const col = col0 + tx + 16 * j;
-            double result;
-            if (F64) result = fold_compensated(acc[i][j]);
-            else {
-#pragma clang fp contract(off)
-                result = ((acc[i][j][0] + acc[i][j][1]) + acc[i][j][2]) + acc[i][j][3];
-            }
+            double const result = fold_compensated(acc[i][j]);
             if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col)
                 *(global_f64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8) = result;
         }
     }
+}
+
+constexpr int kMatrixRows = 128, kMatrixCols = 64; // rows and columns of C per workgroup of the f32 matrix kernel
+constexpr int kMatrixDepth = 16;                     // k per step: four MFMA depths for each of the four sums
+constexpr int kMatrixAStride = kMatrixDepth + 4;     // floats per staged row of A: 16-byte reads of 16 rows spread over all banks
+constexpr int kMatrixBStride = kMatrixCols + 4;      // doubles per staged depth of B
+
+/**
+ *  f32 inputs on the f64 matrix cores. `v_mfma_f64_16x16x4_f64` is, per output, a chain of four fused multiply-adds in
+ *  ascending order of its depth index, each rounded to f64 (checked on the part against a host chain, bit for bit,
+ *  51,200 outputs with full-range f64 operands and accumulators). The reference keeps four f64 sums per output, sum r
+ *  taking the products of k = r, r + 4, r + 8, ... in that order (dot/serial.h:262-296), and a product of two f32 values
+ *  is exact in f64, so a fused multiply-add is the reference's multiply-then-add. Feeding one instruction the depths
+ *  k0 + r, k0 + r + 4, k0 + r + 8, k0 + r + 12 therefore advances sum r of a 16 x 16 block of outputs exactly as the
+ *  reference does, and four instructions (r = 0..3) consume 16 depths. Zero padding past the last depth adds products
+ *  of +0, which leave a sum that started at +0 unchanged (such a sum is never -0).
+ *
+ *  512 threads, 8 wavefronts as 4 x 2, each 32 x 32 outputs = 2 x 2 blocks x 4 sums = 128 accumulator registers; two
+ *  wavefronts per SIMD cover each other's LDS waits. A is staged as f32, [row][k] so that one 16-byte read gives a
+ *  lane the four operands (r = 0..3) of its row and depth group; B comes from the k-major f64 image into [k][column].
+ */
+__global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
+    typedef double __attribute__((ext_vector_type(4))) f64x4_t;
+    typedef double __attribute__((ext_vector_type(2))) f64x2_t;
+    typedef float __attribute__((ext_vector_type(4))) f32x4_t;
+    typedef __attribute__((address_space(1))) double global_f64_t;
+    typedef __attribute__((address_space(1))) uint64_t global_u64_t;
+    __shared__ __attribute__((aligned(16))) float a_lds[2][kMatrixRows][kMatrixAStride];
+    __shared__ __attribute__((aligned(16))) double b_lds[2][kMatrixDepth][kMatrixBStride];
+    uint32_t const tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t const row0 = blockIdx.y * kMatrixRows, col0 = blockIdx.x * kMatrixCols;
+    // symmetric form: a tile wholly left of the diagonal has nothing to store
+    if (((row0 + g.tri_shift) & g.tri_mask) > col0 + (kMatrixCols - 1)) return;
+    PackedHeader const *header = (PackedHeader const *)((uint8_t const *)g.b - sizeof(PackedHeader));
+    if (!(header->magic == kMagic && header->version == kVersion && header->dtype == (uint32_t)g.dtype && header->n == g.n &&
+          header->k == g.k)) { // (an image of another type or shape: poison, as the f64 kernel does)
+        for (uint32_t at = tid; at < kMatrixRows * kMatrixCols; at += 512) {
+            uint32_t const row = row0 + at / kMatrixCols, col = col0 + at % kMatrixCols;
+            if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col)
+                *(global_u64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8) = ~0ull;
+        }
+        return;
+    }
+
+    uint32_t const wave_row = (wave >> 1) * 32, wave_col = (wave & 1) * 32;
+    uint32_t const in_block = lane & 15, depth_group = lane >> 4;
+    f64x4_t acc[2][2][4]; // [row block][column block][sum r]; element v: row 4 v + lane / 16, column lane % 16
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = f64x4_t {0, 0, 0, 0};
+
+    // staging: A: thread t brings 4 consecutive k of row t / 4; B: 2 consecutive columns of depth t / 32
+    uint32_t const a_row = tid >> 2, a_k = (tid & 3) * 4;
+    uint32_t const b_k = tid >> 5, b_col = (tid & 31) * 2;
+    uint32_t const a_from = row0 + a_row < g.m ? row0 + a_row : g.m - 1; // (rows past the end repeat the last; never stored)
+    uint8_t const *a_source = g.a + (uint64_t)a_from * g.a_stride;
+    bool const aligned = ((((uint64_t)g.a) | g.a_stride) & 15) == 0;
+    f32x4_t a_next;
+    f64x2_t b_next;
+    auto fetch = [&](uint32_t k0) {
+        uint32_t const at = k0 + a_k;
+        if (aligned && at + 4 <= g.k) a_next = *(f32x4_t const *)(a_source + (uint64_t)at * 4);
+        else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a_next[e] = at + e < g.k ? ((float const *)a_source)[at + e] : 0.f;
+        }
+        b_next = *(f64x2_t const *)(g.b + (uint64_t)(k0 + b_k) * g.n_padded + col0 + b_col); // (inside the padded image)
+    };
+    auto stash = [&](int buffer) {
+        *(f32x4_t *)&a_lds[buffer][a_row][a_k] = a_next;
+        *(f64x2_t *)&b_lds[buffer][b_k][b_col] = b_next;
+    };
+
+    uint32_t const depth = (g.k + kMatrixDepth - 1) & ~(uint32_t)(kMatrixDepth - 1); // (the image is padded to 32)
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    int buffer = 0;
+    for (uint32_t k0 = 0; k0 < depth; k0 += kMatrixDepth) {
+        bool const more = k0 + kMatrixDepth < depth;
+        if (more) fetch(k0 + kMatrixDepth);
+        double a_operand[2][4], b_operand[2][4];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            f32x4_t const quad = *(f32x4_t const *)&a_lds[buffer][wave_row + 16 * i + in_block][4 * depth_group];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) a_operand[i][r] = (double)quad[r];
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) b_operand[j][r] = b_lds[buffer][r + 4 * depth_group][wave_col + 16 * j + in_block];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j][r] = __builtin_amdgcn_mfma_f64_16x16x4f64(a_operand[i][r], b_operand[j][r], acc[i][j][r], 0, 0, 0);
+        if (more) stash(buffer ^ 1);
+        __syncthreads();
+        buffer ^= 1;
+    }
+
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            uint32_t const row = row0 + wave_row + 16 * i + 4 * v + depth_group;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint32_t const col = col0 + wave_col + 16 * j + in_block;
+                double result;
+                {
+#pragma clang fp contract(off)
+                    result = ((acc[i][j][0][v] + acc[i][j][1][v]) + acc[i][j][2][v]) + acc[i][j][3][v];
+                }
+                if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col)
+                    *(global_f64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8) = result;
+            }
+        }
 }
 
 __global__ __launch_bounds__(256) void fill_wide_kernel(uint8_t *c, uint32_t m, uint32_t n, uint64_t c_stride, uint64_t bits,
@@ -244,6 +362,7 @@ hipError_t wide_product(int dtype, void const *a, void const *b_packed, void *c,
     if (!wide_geometry(dtype, n, k, geo)) return hipErrorInvalidValue;
     if (m > 0x7FFFFFFFull) return hipErrorInvalidValue;
     if (((uintptr_t)c | c_stride) & 7) return hipErrorInvalidValue;
+    if ((uintptr_t)b_packed & 15) return hipErrorInvalidValue; // (the kernels read the image 16 bytes at a time)
     uint32_t const tri_mask = triangle ? 0xFFFFFFFFu : 0u;
     if (k == 0) {
         uint64_t const blocks = ((uint64_t)m * n + 255) / 256;
@@ -262,8 +381,11 @@ hipError_t wide_product(int dtype, void const *a, void const *b_packed, void *c,
     g.tri_shift = shift, g.tri_mask = tri_mask;
     dim3 const grid(geo.n_padded / kWideTile, (uint32_t)((m + kWideTile - 1) / kWideTile));
     if (grid.y > 65535) return hipErrorInvalidValue;
-    if (dtype == kF64) hipLaunchKernelGGL(dots_wide_kernel<true>, grid, dim3(256), 0, stream, g);
-    else hipLaunchKernelGGL(dots_wide_kernel<false>, grid, dim3(256), 0, stream, g);
+    if (dtype == kF64) hipLaunchKernelGGL(dots_f64_compensated_kernel, grid, dim3(256), 0, stream, g);
+    else {
+        dim3 const matrix_grid(geo.n_padded / kMatrixCols, (uint32_t)((m + kMatrixRows - 1) / kMatrixRows));
+        hipLaunchKernelGGL(dots_f32_matrix_kernel, matrix_grid, dim3(512), 0, stream, g);
+    }
     return hipGetLastError();
 }
 

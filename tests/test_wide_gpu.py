@@ -4,7 +4,8 @@ on a real MI355X.
 `nk_dots_packed_size_<T>`, `nk_dots_pack_<T>`, `nk_dots_packed_<T>`, `nk_dots_symmetric_<T>` for f32 and f64: reference
 include/numkong/dots/serial.h:2458-2491, arithmetic include/numkong/dot/serial.h:262-335 (f32: exact products into four
 f64 lane sums; f64: the compensated two-lane sum of scalar/serial.h:128-136 folded by reduce/serial.h:33-48). The GPU
-kernel keeps the reference's own accumulators per output in the reference's own order along k, so the bar here is the
+kernels (f32: the f64 MFMA, whose chain of fused multiply-adds along its depth advances one lane sum; f64: vector units)
+keep the reference's own accumulators per output in the reference's own order along k, so the bar here is the
 integer one: BIT-EXACT against the oracle's restatement of the serial kernels (which tests/test_oracle.py pins bit for
 bit against the reference library), not a tolerance.
 """
