@@ -395,10 +395,11 @@ NKO_API void nko_dots_f64(int dtype, void const *a, void const *b, double *c, do
  *  (reduce/serial.h:223-300); integers: exact in 64 bits, truncated to 32 (dots/serial.h:154-164). Returned as
  *  the bits of the f32 or of the u32. */
 static uint32_t row_sumsq_bits(int dtype, void const *row, size_t depth) {
-    if (dtype == NKO_I8 || dtype == NKO_U8) {
+    depth = effective_depth(dtype, depth); /* (the 4-bit types count both halves of the last byte: reduce/serial.h:373-404) */
+    if (dtype == NKO_I8 || dtype == NKO_U8 || dtype == NKO_I4 || dtype == NKO_U4) {
         uint64_t sum = 0;
         for (size_t l = 0; l < depth; ++l) {
-            int64_t const v = dtype == NKO_I8 ? (int64_t)((int8_t const *)row)[l] : (int64_t)((uint8_t const *)row)[l];
+            int64_t const v = (int64_t)element_f32(dtype, row, l); /* small integers: exact */
             sum += (uint64_t)(v * v);
         }
         return (uint32_t)sum;
@@ -441,11 +442,12 @@ static float serial_rsqrt(float number) {
 }
 
 /** spatial/serial.h:257-344. `dot`, `query` and `target` arrive as 32-bit patterns: f32 for the float types,
- *  i32 for i8 (the i8 finalisers read both norms as signed), u32 for u8. */
+ *  i32 for i8 and i4 (their finalisers read both norms as signed), u32 for u8 and u4. */
 static float serial_from_dot(int dtype, int metric, uint32_t dot_bits, uint32_t query_bits, uint32_t target_bits) {
     float dot, query, target;
-    if (dtype == NKO_I8) dot = (float)(int32_t)dot_bits, query = (float)(int32_t)query_bits, target = (float)(int32_t)target_bits;
-    else if (dtype == NKO_U8) dot = (float)dot_bits, query = (float)query_bits, target = (float)target_bits;
+    if (dtype == NKO_I8 || dtype == NKO_I4)
+        dot = (float)(int32_t)dot_bits, query = (float)(int32_t)query_bits, target = (float)(int32_t)target_bits;
+    else if (dtype == NKO_U8 || dtype == NKO_U4) dot = (float)dot_bits, query = (float)query_bits, target = (float)target_bits;
     else dot = bits_to_f32(dot_bits), query = bits_to_f32(query_bits), target = bits_to_f32(target_bits);
     if (metric == 1) {
         volatile float product = query * target;
@@ -464,23 +466,22 @@ static float serial_from_dot(int dtype, int metric, uint32_t dot_bits, uint32_t 
     return root;
 }
 
+NKO_API void nko_serial_dots(int dtype, void const *a, void const *b, void *c, size_t rows, size_t columns, size_t depth,
+                             size_t a_stride, size_t b_stride, size_t c_stride);
+
 /** nk_angulars_packed_<T>_serial (metric 1) / nk_euclideans_packed_<T>_serial (metric 2) from unpacked B:
  *  the serial product, then the finaliser per element with the row's and the column's sum of squares. */
 NKO_API void nko_serial_spatials(int dtype, int metric, void const *a, void const *b, float *c, size_t rows,
                                  size_t columns, size_t depth, size_t a_stride, size_t b_stride, size_t c_stride) {
-    size_t const image_bytes = nko_serial_packed_size(dtype, columns, depth) + 64;
-    unsigned char *image = (unsigned char *)__builtin_malloc(image_bytes);
     uint32_t *target_norms = (uint32_t *)__builtin_malloc(columns * sizeof(uint32_t) + 4);
-    nko_serial_pack(dtype, b, columns, depth, b_stride, image);
     nko_row_sumsq(dtype, b, columns, depth, b_stride, target_norms);
-    nko_serial_packed(dtype, a, image, c, rows, columns, depth, a_stride, c_stride);
+    nko_serial_dots(dtype, a, b, c, rows, columns, depth, a_stride, b_stride, c_stride); /* (= pack + packed, per pair) */
     for (size_t i = 0; i < rows; ++i) {
         uint32_t const query_norm = row_sumsq_bits(dtype, (unsigned char const *)a + i * a_stride, depth);
         uint32_t *row = (uint32_t *)((unsigned char *)c + i * c_stride);
         for (size_t j = 0; j < columns; ++j)
             row[j] = f32_to_bits(serial_from_dot(dtype, metric, row[j], query_norm, target_norms[j]));
     }
-    __builtin_free(image);
     __builtin_free(target_norms);
 }
 
@@ -488,6 +489,7 @@ NKO_API void nko_serial_spatials(int dtype, int metric, void const *a, void cons
  *  references the same way: f64 dot and norms, then the formula). */
 NKO_API void nko_spatials_f64(int dtype, int metric, void const *a, void const *b, double *c, size_t rows, size_t columns,
                               size_t depth, size_t a_stride, size_t b_stride) {
+    depth = effective_depth(dtype, depth);
     for (size_t i = 0; i < rows; ++i) {
         unsigned char const *a_row = (unsigned char const *)a + i * a_stride;
         double query = 0;
