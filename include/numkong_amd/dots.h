@@ -185,7 +185,7 @@ NK_DYNAMIC void nk_dots_packed_f64(nk_f64_t const *a, void const *b_packed, nk_f
                                    nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
 
 /* Distances over the same packed B, in one pass: result[i][j] = angular (1 - cosine) or euclidean distance between
- * row i of A and row j of B, f32 for all six types. Reference: include/numkong/spatials.h:139-266. */
+ * row i of A and row j of B, f32 results for these ten types. Reference: include/numkong/spatials.h:139-300. */
 #define NK_AMD_DECLARE_SPATIALS_(T, in_t)                                                                              \
     NK_DYNAMIC void nk_angulars_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *result, nk_size_t rows,     \
                                            nk_size_t cols, nk_size_t depth, nk_size_t a_stride, nk_size_t r_stride);  \
@@ -197,6 +197,10 @@ NK_AMD_DECLARE_SPATIALS_(bf16, nk_bf16_t)
 NK_AMD_DECLARE_SPATIALS_(f16, nk_f16_t)
 NK_AMD_DECLARE_SPATIALS_(e4m3, nk_e4m3_t)
 NK_AMD_DECLARE_SPATIALS_(e5m2, nk_e5m2_t)
+NK_AMD_DECLARE_SPATIALS_(e2m3, nk_e2m3_t)
+NK_AMD_DECLARE_SPATIALS_(e3m2, nk_e3m2_t)
+NK_AMD_DECLARE_SPATIALS_(i4, nk_i4x2_t)
+NK_AMD_DECLARE_SPATIALS_(u4, nk_u4x2_t)
 #undef NK_AMD_DECLARE_SPATIALS_
 
 /* All pairs of one set of vectors: result[i][j] for i in [row_start, row_start + row_count), j >= i, is the dot
@@ -221,10 +225,14 @@ NK_AMD_DECLARE_SYMMETRIC_(bf16, nk_bf16_t, nk_f32_t)
 NK_AMD_DECLARE_SYMMETRIC_(f16, nk_f16_t, nk_f32_t)
 NK_AMD_DECLARE_SYMMETRIC_(e4m3, nk_e4m3_t, nk_f32_t)
 NK_AMD_DECLARE_SYMMETRIC_(e5m2, nk_e5m2_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(e2m3, nk_e2m3_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(e3m2, nk_e3m2_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(i4, nk_i4x2_t, nk_i32_t)
+NK_AMD_DECLARE_SYMMETRIC_(u4, nk_u4x2_t, nk_u32_t)
 #undef NK_AMD_DECLARE_SYMMETRIC_
 
-/* The 6-bit floats, the 4-bit integers, the 1-bit type and the two wide types (f32, f64) have the dot-product kinds only (packed above, symmetric here), with their
- * backend-suffixed names; their distance kinds resolve to the error stubs. */
+/* The 1-bit type and the two wide types (f32, f64) have the dot-product kinds only (packed above, symmetric here),
+ * with their backend-suffixed names; their distance kinds resolve to the error stubs. */
 #define NK_AMD_DECLARE_DOTS_ONLY_(T, in_t, out_t)                                                                      \
     NK_DYNAMIC void nk_dots_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,              \
                                           nk_size_t stride, out_t *result, nk_size_t result_stride,                   \
@@ -238,10 +246,6 @@ NK_AMD_DECLARE_SYMMETRIC_(e5m2, nk_e5m2_t, nk_f32_t)
     NK_DYNAMIC void nk_dots_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,     \
                                                    nk_size_t stride, out_t *result, nk_size_t result_stride,          \
                                                    nk_size_t row_start, nk_size_t row_count);
-NK_AMD_DECLARE_DOTS_ONLY_(e2m3, nk_e2m3_t, nk_f32_t)
-NK_AMD_DECLARE_DOTS_ONLY_(e3m2, nk_e3m2_t, nk_f32_t)
-NK_AMD_DECLARE_DOTS_ONLY_(i4, nk_i4x2_t, nk_i32_t)
-NK_AMD_DECLARE_DOTS_ONLY_(u4, nk_u4x2_t, nk_u32_t)
 NK_AMD_DECLARE_DOTS_ONLY_(u1, nk_u1x8_t, nk_u32_t)
 NK_AMD_DECLARE_DOTS_ONLY_(f32, nk_f32_t, nk_f64_t)
 NK_AMD_DECLARE_DOTS_ONLY_(f64, nk_f64_t, nk_f64_t)
@@ -290,6 +294,10 @@ NK_AMD_DECLARE_BACKEND_(bf16, nk_bf16_t, nk_f32_t)
 NK_AMD_DECLARE_BACKEND_(f16, nk_f16_t, nk_f32_t)
 NK_AMD_DECLARE_BACKEND_(e4m3, nk_e4m3_t, nk_f32_t)
 NK_AMD_DECLARE_BACKEND_(e5m2, nk_e5m2_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(e2m3, nk_e2m3_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(e3m2, nk_e3m2_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(i4, nk_i4x2_t, nk_i32_t)
+NK_AMD_DECLARE_BACKEND_(u4, nk_u4x2_t, nk_u32_t)
 #undef NK_AMD_DECLARE_BACKEND_
 
 /* Additions without a counterpart in the reference. */

@@ -11,9 +11,9 @@
  *  non-zero HIP error code; `nk_hip_last_error()` returns a thread-local description of the last failure.
  *
  *  `dtype` arguments take the `nk_dtype_t` codes of <numkong_amd/dots.h> (reference:
- *  include/numkong/types.h:923-952): nk_i8_k, nk_u8_k, nk_bf16_k, nk_f16_k, nk_e4m3_k, nk_e5m2_k (every kind), and
- *  nk_e2m3_k, nk_e3m2_k, nk_i4_k, nk_u4_k, nk_u1_k, nk_f32_k, nk_f64_k (the dot-product kinds; depth counts
- *  dimensions, so 4-bit values or bits for the sub-byte types; f32 and f64 write 8-byte f64 outputs).
+ *  include/numkong/types.h:923-952): nk_i8_k, nk_u8_k, nk_bf16_k, nk_f16_k, nk_e4m3_k, nk_e5m2_k, nk_e2m3_k, nk_e3m2_k,
+ *  nk_i4_k, nk_u4_k (every kind), and nk_u1_k, nk_f32_k, nk_f64_k (the dot-product kinds). Depth counts dimensions, so
+ *  4-bit values or bits for the sub-byte types; f32 and f64 write 8-byte f64 outputs.
  */
 #ifndef NUMKONG_AMD_HIP_ABI_H
 #define NUMKONG_AMD_HIP_ABI_H

@@ -115,13 +115,13 @@ struct u1x8_t {
     }
 };
 
-/** The distance kinds exist for the six wider types; `distances<T>` names their entry points. */
+/** The distance kinds exist for every type but u1, f32 and f64; `distances<T>` names their entry points. */
 template <typename value_type_>
 struct distances;
-#define NK_AMD_DEFINE_DISTANCES_(name)                                                                            \
+#define NK_AMD_DEFINE_DISTANCES_(tag, name)                                                                           \
     template <>                                                                                                   \
-    struct distances<name##_t> {                                                                                  \
-        using raw_t = name##_t::raw_t;                                                                            \
+    struct distances<tag> {                                                                               \
+        using raw_t = tag::raw_t;                                                                         \
         static void angulars_packed(raw_t const *a, void const *b, nk_f32_t *c, nk_size_t m, nk_size_t n,         \
                                     nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) noexcept {               \
             nk_angulars_packed_##name(a, b, c, m, n, k, a_stride, c_stride);                                      \
@@ -140,12 +140,16 @@ struct distances;
             nk_euclideans_symmetric_##name(v, n, k, stride, out, out_stride, row_start, row_count);               \
         }                                                                                                         \
     };
-NK_AMD_DEFINE_DISTANCES_(i8)
-NK_AMD_DEFINE_DISTANCES_(u8)
-NK_AMD_DEFINE_DISTANCES_(bf16)
-NK_AMD_DEFINE_DISTANCES_(f16)
-NK_AMD_DEFINE_DISTANCES_(e4m3)
-NK_AMD_DEFINE_DISTANCES_(e5m2)
+NK_AMD_DEFINE_DISTANCES_(i8_t, i8)
+NK_AMD_DEFINE_DISTANCES_(u8_t, u8)
+NK_AMD_DEFINE_DISTANCES_(bf16_t, bf16)
+NK_AMD_DEFINE_DISTANCES_(f16_t, f16)
+NK_AMD_DEFINE_DISTANCES_(e4m3_t, e4m3)
+NK_AMD_DEFINE_DISTANCES_(e5m2_t, e5m2)
+NK_AMD_DEFINE_DISTANCES_(e2m3_t, e2m3)
+NK_AMD_DEFINE_DISTANCES_(e3m2_t, e3m2)
+NK_AMD_DEFINE_DISTANCES_(i4x2_t, i4)
+NK_AMD_DEFINE_DISTANCES_(u4x2_t, u4)
 #undef NK_AMD_DEFINE_DISTANCES_
 
 /** Bytes of device memory; what `packed_matrix` keeps its image in unless told otherwise. */

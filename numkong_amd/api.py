@@ -44,7 +44,7 @@ DTYPES = {
 
 
 # the types that also have the distance kinds (the 6-bit floats and 4-bit integers have dot products only)
-DISTANCE_DTYPES = ("i8", "u8", "bf16", "f16", "e4m3", "e5m2")
+DISTANCE_DTYPES = ("i8", "u8", "bf16", "f16", "e4m3", "e5m2", "e2m3", "e3m2", "i4", "u4")
 
 
 class NumKongAmdError(RuntimeError):

@@ -7,4 +7,4 @@
  */
 #include "dispatch.h"
 
-NK_AMD_DEFINE_DISPATCH_DOTS_(e2m3)
+NK_AMD_DEFINE_DISPATCH_(e2m3)

@@ -7,4 +7,4 @@
  */
 #include "dispatch.h"
 
-NK_AMD_DEFINE_DISPATCH_DOTS_(e3m2)
+NK_AMD_DEFINE_DISPATCH_(e3m2)

@@ -7,4 +7,4 @@
  */
 #include "dispatch.h"
 
-NK_AMD_DEFINE_DISPATCH_DOTS_(i4)
+NK_AMD_DEFINE_DISPATCH_(i4)

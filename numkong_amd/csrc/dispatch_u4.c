@@ -7,4 +7,4 @@
  */
 #include "dispatch.h"
 
-NK_AMD_DEFINE_DISPATCH_DOTS_(u4)
+NK_AMD_DEFINE_DISPATCH_(u4)

@@ -588,14 +588,12 @@ struct E5M2 : F16 {
 struct E2M3 : F16 {
     static constexpr bool kChunked = true;
     static constexpr int kDtype = kE2M3;
-    static constexpr bool kDistances = false; // dot products only
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp6x8<false>((uint32_t)v[0], (uint32_t)v[1]); }
 };
 struct E3M2 : F16 {
     static constexpr bool kChunked = true;
     static constexpr int kDtype = kE3M2;
-    static constexpr bool kDistances = false; // dot products only
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp6x8<true>((uint32_t)v[0], (uint32_t)v[1]); }
 };
@@ -603,7 +601,6 @@ struct E3M2 : F16 {
  *  as they are: none of u8's offset arithmetic. */
 struct I4 : I8 {
     static constexpr int kDtype = kI4;
-    static constexpr bool kDistances = false; // dot products only
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_i4x16<true>((uint32_t)v[0], (uint32_t)v[1]); }
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); }
@@ -618,7 +615,6 @@ struct U1 : I8 {
 };
 struct U4 : I8 {
     static constexpr int kDtype = kU4;
-    static constexpr bool kDistances = false; // dot products only
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_i4x16<false>((uint32_t)v[0], (uint32_t)v[1]); }
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); }

@@ -334,9 +334,13 @@ NK_AMD_DEFINE_BACKEND_DISTANCES_(e4m3, nk_e4m3_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(e5m2, nk_e5m2_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DISTANCES_(e5m2, nk_e5m2_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(e2m3, nk_e2m3_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(e2m3, nk_e2m3_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(e3m2, nk_e3m2_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(i4, nk_i4x2_t, nk_i32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(i4, nk_i4x2_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(u4, nk_u4x2_t, nk_u32_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(u4, nk_u4x2_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(u1, nk_u1x8_t, nk_u32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(f32, nk_f32_t, nk_f64_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(f64, nk_f64_t, nk_f64_t)

@@ -116,9 +116,13 @@ NK_AMD_DISPATCH_DISTANCES_(e4m3, nk_e4m3_t)
 NK_AMD_DISPATCH_DOTS_(e5m2, nk_e5m2_t, nk_f32_t)
 NK_AMD_DISPATCH_DISTANCES_(e5m2, nk_e5m2_t)
 NK_AMD_DISPATCH_DOTS_(e2m3, nk_e2m3_t, nk_f32_t)
+NK_AMD_DISPATCH_DISTANCES_(e2m3, nk_e2m3_t)
 NK_AMD_DISPATCH_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
+NK_AMD_DISPATCH_DISTANCES_(e3m2, nk_e3m2_t)
 NK_AMD_DISPATCH_DOTS_(i4, nk_i4x2_t, nk_i32_t)
+NK_AMD_DISPATCH_DISTANCES_(i4, nk_i4x2_t)
 NK_AMD_DISPATCH_DOTS_(u4, nk_u4x2_t, nk_u32_t)
+NK_AMD_DISPATCH_DISTANCES_(u4, nk_u4x2_t)
 NK_AMD_DISPATCH_DOTS_(u1, nk_u1x8_t, nk_u32_t)
 NK_AMD_DISPATCH_DOTS_(f32, nk_f32_t, nk_f64_t)
 NK_AMD_DISPATCH_DOTS_(f64, nk_f64_t, nk_f64_t)
@@ -193,8 +197,12 @@ NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t i
         case nk_bf16_k:
         case nk_f16_k:
         case nk_e4m3_k:
-        case nk_e5m2_k: return nk_f32_k;
-        default: return nk_dtype_unknown_k; /* (the 6-bit floats and 4-bit integers have the dot-product kinds only) */
+        case nk_e5m2_k:
+        case nk_e2m3_k:
+        case nk_e3m2_k:
+        case nk_i4_k:
+        case nk_u4_k: return nk_f32_k;
+        default: return nk_dtype_unknown_k; /* (u1, f32 and f64 have the dot-product kinds only) */
         }
     }
     if (kind != nk_kernel_dots_packed_k && kind != nk_kernel_dots_symmetric_k) return nk_dtype_unknown_k;

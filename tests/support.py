@@ -26,13 +26,19 @@ OUTPUT = {"i8": np.int32, "u8": np.uint32, "f16": np.float32, "bf16": np.float32
           "i4": np.int32, "u4": np.uint32, "e2m3": np.float32, "e3m2": np.float32, "u1": np.uint32,
           "f32": np.float64, "f64": np.float64}
 FLOAT_DTYPES = ("bf16", "f16", "e4m3", "e5m2")
-ALL_DTYPES = ("i8", "u8") + FLOAT_DTYPES  # the types with every kind: packed dots, packed distances, symmetric
-# the types with the dot-product kinds only: 6-bit floats (one per byte), 4-bit integers (two per byte), bits (eight)
+ALL_DTYPES = ("i8", "u8") + FLOAT_DTYPES  # the six types of the headline path
+# the narrow types: 6-bit floats (one per byte), 4-bit integers (two per byte), bits (eight; dot-product kinds only)
 NARROW_FLOAT_DTYPES = ("e2m3", "e3m2")
 NARROW_INT_DTYPES = ("i4", "u4", "u1")
 NARROW_DTYPES = NARROW_FLOAT_DTYPES + NARROW_INT_DTYPES
 DIMENSIONS_PER_VALUE = {"i4": 2, "u4": 2, "u1": 8}
 WIDE_DTYPES = ("f32", "f64")  # f64 results; the dot-product kinds only
+DISTANCE_DTYPES = ALL_DTYPES + ("e2m3", "e3m2", "i4", "u4")  # the types with the distance kinds, packed and symmetric
+INTEGER_DTYPES = ("i8", "u8", "i4", "u4", "u1")  # bit-exact everywhere
+# The reference's distance kernels take their sums of squares from the host-dispatched nk_reduce_moments_<T>, and the
+# AVX2 one of i4 squares negative values as if they were unsigned (reduce/haswell.h:3629-3633), so for i4 only the
+# serial kernels (restated by the oracle, nk_reduce_moments_i4_serial) can stand next to the f64 truth.
+DISPATCHED_DISTANCES_UNUSABLE = ("i4",)
 
 
 def depth_of(dtype: str, matrix: np.ndarray) -> int:
@@ -110,12 +116,12 @@ class Oracle:
     def row_sumsq(self, dtype: str, x: np.ndarray) -> np.ndarray:
         """Per-row sum of squares as the serial backend computes it: u32 for the integer types, f32 otherwise."""
         out = np.empty(x.shape[0], dtype=np.uint32)
-        self.lib.nko_row_sumsq(CODES[dtype], _ptr(x), x.shape[0], x.shape[1], x.strides[0], _ptr(out))
-        return out if dtype in ("i8", "u8") else out.view(np.float32)
+        self.lib.nko_row_sumsq(CODES[dtype], _ptr(x), x.shape[0], depth_of(dtype, x), x.strides[0], _ptr(out))
+        return out if dtype in INTEGER_DTYPES else out.view(np.float32)
 
     def spatials_packed(self, metric: str, dtype: str, a: np.ndarray, b: np.ndarray) -> np.ndarray:
         """`nk_angulars_packed_<dtype>_serial` ("angular") / `nk_euclideans_packed_<dtype>_serial` ("euclidean")."""
-        m, k = a.shape
+        m, k = a.shape[0], depth_of(dtype, a)
         n = b.shape[0]
         c = np.empty((m, n), dtype=np.float32)
         self.lib.nko_serial_spatials(CODES[dtype], METRICS[metric], _ptr(a), _ptr(b), _ptr(c), m, n, k, a.strides[0],
@@ -124,7 +130,7 @@ class Oracle:
 
     def spatials_truth(self, metric: str, dtype: str, a: np.ndarray, b: np.ndarray) -> np.ndarray:
         """The distances from f64 dots and f64 norms."""
-        m, k = a.shape
+        m, k = a.shape[0], depth_of(dtype, a)
         n = b.shape[0]
         c = np.empty((m, n), dtype=np.float64)
         self.lib.nko_spatials_f64(CODES[dtype], METRICS[metric], _ptr(a), _ptr(b), _ptr(c), m, n, k, a.strides[0],
@@ -215,7 +221,7 @@ class Reference:
 
     def spatials_packed(self, kind: int, dtype: str, a: np.ndarray, b: np.ndarray, viable: int = CAP_SERIAL) -> np.ndarray:
         """`nk_angulars_packed_<dtype>` / `nk_euclideans_packed_<dtype>` of the chosen backend, f32 results."""
-        m, k = a.shape
+        m, k = a.shape[0], depth_of(dtype, a)
         n = b.shape[0]
         packed = self.pack(dtype, b, viable)
         c = np.empty((m, n), dtype=np.float32)

@@ -89,7 +89,19 @@ def test_lookup_and_capabilities():
         fn, cap = find(lib, ord("Y"), code, CAP_GFX950)  # symmetric hamming distances: not on this path
         assert fn and cap == 0
     assert find(lib, ord("G"), 1 << 20, CAP_GFX950) == (None, 0)  # f64c: unknown dtype -> null kernel
-    for name in ("e2m3", "e3m2", "i4", "u4", "u1", "f32", "f64"):  # the dot-product kinds only
+    for name in ("e2m3", "e3m2", "i4", "u4"):  # every kind as well; dot products in their own widened types
+        code = api.DTYPES[name][0]
+        for kind, stem in ((ord("P"), "nk_dots_packed_size_"), (ord("Q"), "nk_dots_pack_"), (ord("G"), "nk_dots_packed_"),
+                           (ord("y"), "nk_dots_symmetric_"), (ord("N"), "nk_angulars_packed_"), (ord("E"), "nk_euclideans_packed_"),
+                           (ord("n"), "nk_angulars_symmetric_"), (ord("D"), "nk_euclideans_symmetric_")):
+            fn, cap = find(lib, kind, code, CAP_GFX950 | 1)
+            assert fn == ctypes.cast(getattr(lib, f"{stem}{name}_gfx950"), ctypes.c_void_p).value and cap == CAP_GFX950
+            assert ctypes.cast(getattr(lib, f"{stem}{name}"), ctypes.c_void_p).value  # the dispatched entry point
+        expected = {"i4": 1 << 4, "u4": 1 << 8}.get(name, 1 << 11)
+        assert lib.nk_kernel_output_dtype(ord("G"), code) == lib.nk_kernel_output_dtype(ord("y"), code) == expected
+        for kind in (ord("N"), ord("E"), ord("n"), ord("D")):
+            assert lib.nk_kernel_output_dtype(kind, code) == 1 << 11
+    for name in ("u1", "f32", "f64"):  # the dot-product kinds only
         code = api.DTYPES[name][0]
         for kind, stem in ((ord("P"), "nk_dots_packed_size_"), (ord("Q"), "nk_dots_pack_"), (ord("G"), "nk_dots_packed_"),
                            (ord("y"), "nk_dots_symmetric_")):
@@ -98,7 +110,7 @@ def test_lookup_and_capabilities():
         for kind in (ord("N"), ord("E"), ord("n"), ord("D")):
             fn, cap = find(lib, kind, code, CAP_GFX950)
             assert fn and cap == 0
-        expected = {"i4": 1 << 4, "u4": 1 << 8, "u1": 1 << 8, "f32": 1 << 10, "f64": 1 << 10}.get(name, 1 << 11)
+        expected = {"u1": 1 << 8, "f32": 1 << 10, "f64": 1 << 10}[name]
         assert lib.nk_kernel_output_dtype(ord("G"), code) == lib.nk_kernel_output_dtype(ord("y"), code) == expected
         assert lib.nk_kernel_output_dtype(ord("N"), code) == 0
     out = {"i8": 1 << 4, "u8": 1 << 8, "bf16": 1 << 11, "f16": 1 << 11, "e4m3": 1 << 11, "e5m2": 1 << 11}
@@ -189,4 +201,4 @@ def test_python_mirror_validates_arguments():
     with pytest.raises(TypeError):
         nk.angulars_symmetric(cpu, "f16c")
     with pytest.raises(TypeError):
-        nk.euclideans_symmetric(cpu, "i4")  # the 4-bit integers have the dot-product kinds only
+        nk.euclideans_symmetric(cpu, "u1")  # single bits have the dot-product kinds only

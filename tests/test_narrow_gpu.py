@@ -10,7 +10,11 @@ and the bits to i8, B at pack time and A on its way into LDS.
     unpacked nibbles;
   * e2m3 / e3m2: the float gate of tests/test_dots_gpu.py against the serial restatement and the host-dispatched kernel;
     where every partial sum is exact in f32 (short depths: all values are multiples of 1/16 below 32) bit-exact as well;
-  * the widening itself: all 256 byte values, on the A side and on the B side, one at a time against a unit vector.
+  * the widening itself: all 256 byte values, on the A side and on the B side, one at a time against a unit vector;
+  * the distance kinds of e2m3, e3m2, i4, u4 (`nk_{angulars,euclideans}_{packed,symmetric}_<T>`, reference
+    include/numkong/spatials/serial.h:143-240): the gates of tests/test_spatials_gpu.py and tests/test_symmetric_gpu.py
+    (f32 outputs: error against the f64 truth next to the serial kernel's; for i4 the serial kernel only, see
+    tests/support.py). u1 has no distance kinds and is refused.
 """
 import os
 
@@ -23,7 +27,8 @@ import numkong_amd as nk  # noqa: E402
 from tests import support  # noqa: E402
 from tests.support import NARROW_DTYPES, NARROW_FLOAT_DTYPES, NARROW_INT_DTYPES  # noqa: E402
 from tests.test_dots_gpu import DEV, assert_float_gate, best_dispatch, gpu_dots, to_gpu  # noqa: E402
-from tests.test_symmetric_gpu import POISON, gpu_symmetric, owned, reference_library  # noqa: E402
+from tests.test_spatials_gpu import assert_distance_gate, gpu_distances  # noqa: E402
+from tests.test_symmetric_gpu import POISON, check_distances, gpu_symmetric, owned, reference_library  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 
@@ -167,7 +172,8 @@ def test_symmetric_windows(oracle, dtype):
 @pytest.mark.parametrize("dtype", NARROW_DTYPES)
 def test_full_size_properties(oracle, dtype):
     """4096 x 4096 x 4096: the symmetric kind equals the packed kind with both sides the same on the upper triangle, bit
-    for bit; sampled rows agree with the oracle; the distance kinds are refused for these types."""
+    for bit; sampled rows agree with the oracle; the distance kinds equal their packed forms above the diagonal (u1: are
+    refused)."""
     count, depth = 4096, 4096
     rng = np.random.default_rng(89)
     vectors = support.random_matrix(oracle, dtype, count, depth, rng)
@@ -186,9 +192,52 @@ def test_full_size_properties(oracle, dtype):
     else:
         truth, magnitude = oracle.truth(dtype, vectors[rows], vectors)
         assert_float_gate(dtype, sample, serial, truth, magnitude, f"{dtype} full size")
+    if dtype != "u1":
+        for packed_kind, symmetric_kind in ((nk.angulars_packed, nk.angulars_symmetric), (nk.euclideans_packed, nk.euclideans_symmetric)):
+            both = packed_kind(gv, packed)
+            triangle = symmetric_kind(gv, dtype)
+            strict = torch.triu(torch.ones((count, count), dtype=torch.bool, device=DEV), 1)
+            assert torch.equal(triangle.view(torch.int32)[strict], both.view(torch.int32)[strict])
+            assert not torch.diagonal(triangle).any()
+        return
     with pytest.raises(TypeError):
         nk.angulars_packed(gv, packed)
     status = nk.library().nk_amd_spatials_packed_async(support.KIND_ANGULARS, support.CODES[dtype], gv.data_ptr(),
                                                        packed.buffer.data_ptr(), rectangle.data_ptr(), 8, 8, depth,
                                                        vectors.strides[0], count * 4, None)
     assert status != 0  # no distance kernels behind these types
+
+
+DISTANCE_NARROW = ("e2m3", "e3m2", "i4", "u4")
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", DISTANCE_NARROW)
+@pytest.mark.parametrize("config", [0, 2, 4])
+def test_packed_distances(oracle, dtype, metric, config):
+    """Storage columns x dimensions per value = depth: odd depths of the 4-bit types are the odd storage widths here."""
+    rng = np.random.default_rng(500 + config)
+    for m, n, k in [(1, 1, 1), (3, 5, 7), (33, 70, 200), (100, 37, 333), (257, 129, 1000), (40, 33, 4100)]:
+        a, b = support.random_matrix(oracle, dtype, m, k, rng), support.random_matrix(oracle, dtype, n, k, rng)
+        if m > 4 and n > 4:
+            a[1] = 0         # zero row
+            b[2] = a[3]      # identical rows: both distances cancel to ~0
+            b[4] = 0
+        got = gpu_distances(metric, dtype, a, b, config)
+        assert_distance_gate(oracle, metric, dtype, a, b, got, f"{dtype} {metric} {m}x{n}x{k} config {config}")
+        if m > 4 and n > 4:
+            assert got[1, 4] == 0
+            if metric == "angular":
+                assert (got[1] == 0).all()
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", DISTANCE_NARROW)
+def test_symmetric_distances(oracle, dtype, metric):
+    rng = np.random.default_rng(510)
+    for count, depth, row_start, row_count in [(5, 7, 0, 5), (300, 64, 100, 77), (700, 130, 333, 1000), (1000, 515, 37, 411)]:
+        vectors = support.random_matrix(oracle, dtype, count, depth, rng)
+        if count > 40:
+            vectors[2] = 0
+            vectors[9] = vectors[40]
+        check_distances(oracle, metric, dtype, vectors, row_start, row_count, 0, f"{dtype} {metric} {count}x{depth} rows {row_start}+{row_count}")

@@ -16,7 +16,7 @@ import numpy as np
 import pytest
 
 from tests import support
-from tests.support import ALL_DTYPES, FLOAT_DTYPES, NARROW_DTYPES, NARROW_FLOAT_DTYPES, STORAGE, WIDE_DTYPES
+from tests.support import ALL_DTYPES, DISTANCE_DTYPES, FLOAT_DTYPES, INTEGER_DTYPES, NARROW_DTYPES, NARROW_FLOAT_DTYPES, STORAGE, WIDE_DTYPES
 
 
 def same_floats(x, y):
@@ -151,9 +151,21 @@ def finite_inputs(oracle, dtype, rows, cols, rng):
     return x
 
 
-@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def reference_distance_inputs(oracle, dtype, rows, cols, rng):
+    """Inputs on which the reference's distance kernels can serve as the pin. They take their sums of squares from the
+    host-dispatched nk_reduce_moments_<T> (dots/serial.h:165-170), and the AVX2 one of i4 squares a nibble as if it
+    were unsigned (reduce/haswell.h:3629-3633: a table of 0..15 squared behind signed values, so -5 counts as 121),
+    unlike nk_reduce_moments_i4_serial, which the oracle follows and test_row_sums_of_squares pins bit for bit with
+    negative values. So i4 is compared on non-negative values here, where every backend agrees, and on signed values
+    against the f64 truth in test_four_bit_distances_follow_the_serial_moments."""
+    x = finite_inputs(oracle, dtype, rows, cols, rng)
+    return x & 0x77 if dtype == "i4" else x
+
+
+@pytest.mark.parametrize("dtype", DISTANCE_DTYPES)
 def test_row_sums_of_squares_match_reference_serial(oracle, reference, dtype):
-    """nk_reduce_moments_<T>_serial: exact integers, Neumaier-compensated f32 for the float types, bit for bit."""
+    """nk_reduce_moments_<T>_serial: exact integers (the 4-bit types count both halves of every byte they touch),
+    Neumaier-compensated f32 for the float types, bit for bit."""
     if reference is None:
         pytest.skip("reference build not present")
     rng = np.random.default_rng(21)
@@ -176,7 +188,8 @@ def reference_moments(reference, dtype):
     def sumsq_bits(row):
         row = np.ascontiguousarray(row)
         total, squares = np.zeros(1, np.uint64), np.zeros(1, np.uint64)
-        call(row.ctypes.data, row.size, row.itemsize, total.ctypes.data, squares.ctypes.data)
+        call(row.ctypes.data, row.size * support.DIMENSIONS_PER_VALUE.get(dtype, 1), row.itemsize, total.ctypes.data,
+             squares.ctypes.data)
         # integers: u64 sum of squares, truncated like dots/serial.h:154-164; floats: the f32 in the low half
         return int(squares[0]) & 0xFFFFFFFF
 
@@ -184,7 +197,7 @@ def reference_moments(reference, dtype):
 
 
 @pytest.mark.parametrize("metric", ["angular", "euclidean"])
-@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("dtype", DISTANCE_DTYPES)
 def test_packed_distances_match_reference_serial(oracle, reference, dtype, metric):
     """Integer types: every input of the finaliser is an exact integer, so the restated reciprocal square root
     and formulas must reproduce nk_{angulars,euclideans}_packed_<T>_serial bit for bit. Float types: the reference
@@ -195,13 +208,13 @@ def test_packed_distances_match_reference_serial(oracle, reference, dtype, metri
         pytest.skip("reference build not present")
     rng = np.random.default_rng(22)
     for m, n, k in [(1, 1, 1), (5, 7, 37), (33, 21, 300), (16, 16, 1024), (9, 4, 4099)]:
-        a, b = finite_inputs(oracle, dtype, m, k, rng), finite_inputs(oracle, dtype, n, k, rng)
+        a, b = reference_distance_inputs(oracle, dtype, m, k, rng), reference_distance_inputs(oracle, dtype, n, k, rng)
         if m > 4:
             a[1] = 0  # a zero row: the "product of norms is not positive" branch
             b[2] = a[3][:k] if n > 2 else b[0]  # identical rows: distance 0 up to rounding
         mine = oracle.spatials_packed(metric, dtype, a, b)
         ref = reference.spatials_packed(support.METRIC_KINDS[metric], dtype, a, b)
-        if dtype in ("i8", "u8"):
+        if dtype in INTEGER_DTYPES:
             assert np.array_equal(mine.view(np.uint32), ref.view(np.uint32)), (dtype, metric, m, n, k)
         else:
             u = 2.0 ** -24
@@ -215,12 +228,13 @@ def test_packed_distances_match_reference_serial(oracle, reference, dtype, metri
 
 
 @pytest.mark.parametrize("metric", ["angular", "euclidean"])
-@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("dtype", DISTANCE_DTYPES)
 def test_packed_distances_closed_forms(oracle, dtype, metric):
     """Known answers that need no reference: orthogonal rows are at angular 1 / euclidean sqrt(|a|^2 + |b|^2),
     a row against itself at 0, against its double (same direction) at angular 0 / euclidean |a|, zero rows at 0."""
-    one = {"i8": 1, "u8": 1, "bf16": 0x3F80, "f16": 0x3C00, "e4m3": 0x38, "e5m2": 0x3C}[dtype]
-    two = {"i8": 2, "u8": 2, "bf16": 0x4000, "f16": 0x4000, "e4m3": 0x40, "e5m2": 0x40}[dtype]
+    # (the 4-bit types: the value in the low half of a byte, 0 in the high half)
+    one = {"i8": 1, "u8": 1, "bf16": 0x3F80, "f16": 0x3C00, "e4m3": 0x38, "e5m2": 0x3C, "e2m3": 0x08, "e3m2": 0x0C, "i4": 1, "u4": 1}[dtype]
+    two = {"i8": 2, "u8": 2, "bf16": 0x4000, "f16": 0x4000, "e4m3": 0x40, "e5m2": 0x40, "e2m3": 0x10, "e3m2": 0x10, "i4": 2, "u4": 2}[dtype]
     k = 64
     rows = np.zeros((4, k), dtype=support.STORAGE[dtype])
     rows[0, :16] = one   # |.|^2 = 16
@@ -235,6 +249,20 @@ def test_packed_distances_closed_forms(oracle, dtype, metric):
         expected = np.array([[0, np.sqrt(32), 4, 4], [np.sqrt(32), 0, np.sqrt(80), 4], [4, np.sqrt(80), 0, 8], [4, 4, 8, 0]])
     assert np.allclose(truth, expected, atol=1e-12)
     assert np.allclose(got, expected, atol=2e-6)
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", ["i4", "u4"])
+def test_four_bit_distances_follow_the_serial_moments(oracle, dtype, metric):
+    """Signed and unsigned 4-bit values over their full range, odd depths included (both halves of the last byte count,
+    reduce/serial.h:373-404): the restated kernels against the distances from f64 dots and norms. All inputs of the
+    finaliser are exact integers, so what is left is its own few f32 roundings."""
+    rng = np.random.default_rng(23)
+    for m, n, k in [(3, 5, 1), (9, 7, 19), (12, 33, 257)]:
+        a, b = support.random_matrix(oracle, dtype, m, k, rng), support.random_matrix(oracle, dtype, n, k, rng)
+        got, truth = oracle.spatials_packed(metric, dtype, a, b).astype(np.float64), oracle.spatials_truth(metric, dtype, a, b)
+        scale = 1.0 if metric == "angular" else np.maximum(truth, 1.0)
+        assert (np.abs(got - truth) <= 4e-7 * scale).all(), (dtype, metric, m, n, k)
 
 
 def upper_window(count, row_start, row_count):
@@ -265,7 +293,7 @@ def test_symmetric_dots_match_reference_serial(oracle, reference, dtype):
 
 
 @pytest.mark.parametrize("metric", ["angular", "euclidean"])
-@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("dtype", DISTANCE_DTYPES)
 def test_symmetric_distances_match_reference_serial(oracle, reference, dtype, metric):
     """nk_{angulars,euclideans}_symmetric_<T>_serial: integers bit for bit, floats to the tolerance of the packed
     distances above (the same host-dispatched norms enter); the diagonal is exactly 0 in both."""
@@ -276,7 +304,7 @@ def test_symmetric_distances_match_reference_serial(oracle, reference, dtype, me
         # (the reference's distance kinds do not clamp a window that runs past the last vector, unlike its dots
         # kind, dots/serial.h:2380 against :2815-2821: such a call is outside its contract and is not made here)
         row_count = min(row_count, count - row_start)
-        vectors = finite_inputs(oracle, dtype, count, depth, rng)
+        vectors = reference_distance_inputs(oracle, dtype, count, depth, rng)
         if count > 40:
             vectors[2] = 0
             vectors[9] = vectors[40]  # identical vectors off the diagonal
@@ -285,7 +313,7 @@ def test_symmetric_distances_match_reference_serial(oracle, reference, dtype, me
         own = upper_window(count, row_start, row_count)
         assert not mine[~own].any()
         assert not np.diag(mine).any() and not np.diag(ref)[row_start:row_start + row_count].any()
-        if dtype in ("i8", "u8"):
+        if dtype in INTEGER_DTYPES:
             assert np.array_equal(mine.view(np.uint32)[own], ref.view(np.uint32)[own]), (dtype, metric, count, row_start)
             continue
         u = 2.0 ** -24
@@ -298,7 +326,7 @@ def test_symmetric_distances_match_reference_serial(oracle, reference, dtype, me
             assert ((np.abs(x - y) <= 8 * u * np.abs(y)) | (np.abs(x * x - y * y) <= 8 * u * np.maximum(norms, 1e-30))).all()
 
 
-@pytest.mark.parametrize("dtype", ALL_DTYPES)
+@pytest.mark.parametrize("dtype", DISTANCE_DTYPES)
 def test_symmetric_equals_packed_with_both_sides_the_same(oracle, dtype):
     """Needs no reference: the upper triangle of the symmetric kinds is the packed kinds with B = A (same per-pair
     arithmetic), the diagonal of the distances is 0, and the row windows tile the full call."""
@@ -507,7 +535,7 @@ def test_golden_vectors(oracle, name):
         assert same_floats(mine.view(np.float32), data["dots_serial"].view(np.float32))
         for metric, key in (("angular", "angulars_serial"), ("euclidean", "euclideans_serial")):
             mine, ref = oracle.symmetric(metric, dtype, vectors, row_start, row_count).astype(np.float64), data[key].astype(np.float64)
-            if dtype in ("i8", "u8"):
+            if dtype in INTEGER_DTYPES:
                 assert np.array_equal(mine, ref), (dtype, metric)
             elif metric == "angular":
                 assert np.abs(mine - ref).max() <= 8 * u
@@ -520,7 +548,7 @@ def test_golden_vectors(oracle, name):
         norms = oracle.row_sumsq(dtype, a).astype(np.float64)[:, None] + oracle.row_sumsq(dtype, b).astype(np.float64)[None, :]
         for metric, key in (("angular", "angulars_serial"), ("euclidean", "euclideans_serial")):
             mine, ref = oracle.spatials_packed(metric, dtype, a, b).astype(np.float64), data[key].astype(np.float64)
-            if dtype in ("i8", "u8"):
+            if dtype in INTEGER_DTYPES:
                 assert np.array_equal(mine, ref), (dtype, metric)
             elif metric == "angular":
                 assert np.abs(mine - ref).max() <= 8 * u
