@@ -185,54 +185,58 @@ NK_DYNAMIC void nk_dots_packed_f64(nk_f64_t const *a, void const *b_packed, nk_f
                                    nk_size_t width, nk_size_t depth, nk_size_t a_stride, nk_size_t c_stride);
 
 /* Distances over the same packed B, in one pass: result[i][j] = angular (1 - cosine) or euclidean distance between
- * row i of A and row j of B, f32 results for these ten types. Reference: include/numkong/spatials.h:139-300. */
-#define NK_AMD_DECLARE_SPATIALS_(T, in_t)                                                                              \
-    NK_DYNAMIC void nk_angulars_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *result, nk_size_t rows,     \
+ * row i of A and row j of B, f32 results (f64 for f32 and f64 inputs). Reference: include/numkong/spatials.h:72-300. */
+#define NK_AMD_DECLARE_SPATIALS_(T, in_t, r_t)                                                                            \
+    NK_DYNAMIC void nk_angulars_packed_##T(in_t const *a, void const *b_packed, r_t *result, nk_size_t rows,     \
                                            nk_size_t cols, nk_size_t depth, nk_size_t a_stride, nk_size_t r_stride);  \
-    NK_DYNAMIC void nk_euclideans_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *result, nk_size_t rows,   \
+    NK_DYNAMIC void nk_euclideans_packed_##T(in_t const *a, void const *b_packed, r_t *result, nk_size_t rows,   \
                                              nk_size_t cols, nk_size_t depth, nk_size_t a_stride, nk_size_t r_stride);
-NK_AMD_DECLARE_SPATIALS_(i8, nk_i8_t)
-NK_AMD_DECLARE_SPATIALS_(u8, nk_u8_t)
-NK_AMD_DECLARE_SPATIALS_(bf16, nk_bf16_t)
-NK_AMD_DECLARE_SPATIALS_(f16, nk_f16_t)
-NK_AMD_DECLARE_SPATIALS_(e4m3, nk_e4m3_t)
-NK_AMD_DECLARE_SPATIALS_(e5m2, nk_e5m2_t)
-NK_AMD_DECLARE_SPATIALS_(e2m3, nk_e2m3_t)
-NK_AMD_DECLARE_SPATIALS_(e3m2, nk_e3m2_t)
-NK_AMD_DECLARE_SPATIALS_(i4, nk_i4x2_t)
-NK_AMD_DECLARE_SPATIALS_(u4, nk_u4x2_t)
+NK_AMD_DECLARE_SPATIALS_(i8, nk_i8_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(u8, nk_u8_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(bf16, nk_bf16_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(f16, nk_f16_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(e4m3, nk_e4m3_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(e5m2, nk_e5m2_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(e2m3, nk_e2m3_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(e3m2, nk_e3m2_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(i4, nk_i4x2_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(u4, nk_u4x2_t, nk_f32_t)
+NK_AMD_DECLARE_SPATIALS_(f32, nk_f32_t, nk_f64_t)
+NK_AMD_DECLARE_SPATIALS_(f64, nk_f64_t, nk_f64_t)
 #undef NK_AMD_DECLARE_SPATIALS_
 
 /* All pairs of one set of vectors: result[i][j] for i in [row_start, row_start + row_count), j >= i, is the dot
- * product (widened, as above) or the angular / euclidean distance (f32) of vectors i and j; the distance of a vector
+ * product (widened, as above) or the angular / euclidean distance (f32; f64 for f32 and f64 inputs) of vectors i and j; the distance of a vector
  * from itself is exactly 0. Only that upper triangle of the window is written; a caller that wants the full matrix
  * mirrors it (python/distance.c:865-872) and splits the rows among its threads with the window arguments. Reference:
  * include/numkong/dots.h:298-359, include/numkong/spatials.h:76-120, 245-275; include/numkong/dots/serial.h:2361-2435,
  * 2802-2878 for the semantics. */
-#define NK_AMD_DECLARE_SYMMETRIC_(T, in_t, out_t)                                                                      \
+#define NK_AMD_DECLARE_SYMMETRIC_(T, in_t, out_t, r_t)                                                                    \
     NK_DYNAMIC void nk_dots_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,              \
                                           nk_size_t stride, out_t *result, nk_size_t result_stride,                   \
                                           nk_size_t row_start, nk_size_t row_count);                                  \
     NK_DYNAMIC void nk_angulars_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,          \
-                                              nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,            \
+                                              nk_size_t stride, r_t *result, nk_size_t result_stride,            \
                                               nk_size_t row_start, nk_size_t row_count);                              \
     NK_DYNAMIC void nk_euclideans_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,        \
-                                                nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,          \
+                                                nk_size_t stride, r_t *result, nk_size_t result_stride,          \
                                                 nk_size_t row_start, nk_size_t row_count);
-NK_AMD_DECLARE_SYMMETRIC_(i8, nk_i8_t, nk_i32_t)
-NK_AMD_DECLARE_SYMMETRIC_(u8, nk_u8_t, nk_u32_t)
-NK_AMD_DECLARE_SYMMETRIC_(bf16, nk_bf16_t, nk_f32_t)
-NK_AMD_DECLARE_SYMMETRIC_(f16, nk_f16_t, nk_f32_t)
-NK_AMD_DECLARE_SYMMETRIC_(e4m3, nk_e4m3_t, nk_f32_t)
-NK_AMD_DECLARE_SYMMETRIC_(e5m2, nk_e5m2_t, nk_f32_t)
-NK_AMD_DECLARE_SYMMETRIC_(e2m3, nk_e2m3_t, nk_f32_t)
-NK_AMD_DECLARE_SYMMETRIC_(e3m2, nk_e3m2_t, nk_f32_t)
-NK_AMD_DECLARE_SYMMETRIC_(i4, nk_i4x2_t, nk_i32_t)
-NK_AMD_DECLARE_SYMMETRIC_(u4, nk_u4x2_t, nk_u32_t)
+NK_AMD_DECLARE_SYMMETRIC_(i8, nk_i8_t, nk_i32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(u8, nk_u8_t, nk_u32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(bf16, nk_bf16_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(f16, nk_f16_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(e4m3, nk_e4m3_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(e5m2, nk_e5m2_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(e2m3, nk_e2m3_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(e3m2, nk_e3m2_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(i4, nk_i4x2_t, nk_i32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(u4, nk_u4x2_t, nk_u32_t, nk_f32_t)
+NK_AMD_DECLARE_SYMMETRIC_(f32, nk_f32_t, nk_f64_t, nk_f64_t)
+NK_AMD_DECLARE_SYMMETRIC_(f64, nk_f64_t, nk_f64_t, nk_f64_t)
 #undef NK_AMD_DECLARE_SYMMETRIC_
 
-/* The 1-bit type and the two wide types (f32, f64) have the dot-product kinds only (packed above, symmetric here),
- * with their backend-suffixed names; their distance kinds resolve to the error stubs. */
+/* The 1-bit type has the dot-product kinds only (packed above, symmetric here), with their backend-suffixed names;
+ * its distance kinds resolve to the error stubs. */
 #define NK_AMD_DECLARE_DOTS_ONLY_(T, in_t, out_t)                                                                      \
     NK_DYNAMIC void nk_dots_symmetric_##T(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,              \
                                           nk_size_t stride, out_t *result, nk_size_t result_stride,                   \
@@ -247,8 +251,6 @@ NK_AMD_DECLARE_SYMMETRIC_(u4, nk_u4x2_t, nk_u32_t)
                                                    nk_size_t stride, out_t *result, nk_size_t result_stride,          \
                                                    nk_size_t row_start, nk_size_t row_count);
 NK_AMD_DECLARE_DOTS_ONLY_(u1, nk_u1x8_t, nk_u32_t)
-NK_AMD_DECLARE_DOTS_ONLY_(f32, nk_f32_t, nk_f64_t)
-NK_AMD_DECLARE_DOTS_ONLY_(f64, nk_f64_t, nk_f64_t)
 #undef NK_AMD_DECLARE_DOTS_ONLY_
 
 /* Capability and lookup API. Reference: c/numkong.c:767-768, 831-913. */
@@ -266,38 +268,40 @@ NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t i
 
 /* The gfx950 kernels by their backend-suffixed names, as the reference exposes `_serial`, `_haswell`, ...
  * (include/numkong/dots.h:361-1877). Same prototypes as the dispatched entry points above. */
-#define NK_AMD_DECLARE_BACKEND_(T, in_t, out_t)                                                                        \
+#define NK_AMD_DECLARE_BACKEND_(T, in_t, out_t, r_t)                                                                      \
     NK_DYNAMIC nk_size_t nk_dots_packed_size_##T##_gfx950(nk_size_t width, nk_size_t depth);                           \
     NK_DYNAMIC void nk_dots_pack_##T##_gfx950(in_t const *b, nk_size_t width, nk_size_t depth, nk_size_t b_stride,     \
                                               void *b_packed);                                                         \
     NK_DYNAMIC void nk_dots_packed_##T##_gfx950(in_t const *a, void const *b_packed, out_t *c, nk_size_t height,       \
                                                 nk_size_t width, nk_size_t depth, nk_size_t a_stride,                  \
                                                 nk_size_t c_stride);                                 \
-    NK_DYNAMIC void nk_angulars_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,  \
+    NK_DYNAMIC void nk_angulars_packed_##T##_gfx950(in_t const *a, void const *b_packed, r_t *c, nk_size_t height,  \
                                                     nk_size_t width, nk_size_t depth, nk_size_t a_stride,                 \
                                                     nk_size_t c_stride);                                                  \
-    NK_DYNAMIC void nk_euclideans_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height, \
+    NK_DYNAMIC void nk_euclideans_packed_##T##_gfx950(in_t const *a, void const *b_packed, r_t *c, nk_size_t height, \
                                                       nk_size_t width, nk_size_t depth, nk_size_t a_stride,               \
                                                       nk_size_t c_stride);                                                \
     NK_DYNAMIC void nk_dots_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,         \
                                                    nk_size_t stride, out_t *result, nk_size_t result_stride,              \
                                                    nk_size_t row_start, nk_size_t row_count);                             \
     NK_DYNAMIC void nk_angulars_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,     \
-                                                       nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,       \
+                                                       nk_size_t stride, r_t *result, nk_size_t result_stride,       \
                                                        nk_size_t row_start, nk_size_t row_count);                         \
     NK_DYNAMIC void nk_euclideans_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,   \
-                                                         nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,     \
+                                                         nk_size_t stride, r_t *result, nk_size_t result_stride,     \
                                                          nk_size_t row_start, nk_size_t row_count);
-NK_AMD_DECLARE_BACKEND_(i8, nk_i8_t, nk_i32_t)
-NK_AMD_DECLARE_BACKEND_(u8, nk_u8_t, nk_u32_t)
-NK_AMD_DECLARE_BACKEND_(bf16, nk_bf16_t, nk_f32_t)
-NK_AMD_DECLARE_BACKEND_(f16, nk_f16_t, nk_f32_t)
-NK_AMD_DECLARE_BACKEND_(e4m3, nk_e4m3_t, nk_f32_t)
-NK_AMD_DECLARE_BACKEND_(e5m2, nk_e5m2_t, nk_f32_t)
-NK_AMD_DECLARE_BACKEND_(e2m3, nk_e2m3_t, nk_f32_t)
-NK_AMD_DECLARE_BACKEND_(e3m2, nk_e3m2_t, nk_f32_t)
-NK_AMD_DECLARE_BACKEND_(i4, nk_i4x2_t, nk_i32_t)
-NK_AMD_DECLARE_BACKEND_(u4, nk_u4x2_t, nk_u32_t)
+NK_AMD_DECLARE_BACKEND_(i8, nk_i8_t, nk_i32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(u8, nk_u8_t, nk_u32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(bf16, nk_bf16_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(f16, nk_f16_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(e4m3, nk_e4m3_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(e5m2, nk_e5m2_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(e2m3, nk_e2m3_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(e3m2, nk_e3m2_t, nk_f32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(i4, nk_i4x2_t, nk_i32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(u4, nk_u4x2_t, nk_u32_t, nk_f32_t)
+NK_AMD_DECLARE_BACKEND_(f32, nk_f32_t, nk_f64_t, nk_f64_t)
+NK_AMD_DECLARE_BACKEND_(f64, nk_f64_t, nk_f64_t, nk_f64_t)
 #undef NK_AMD_DECLARE_BACKEND_
 
 /* Additions without a counterpart in the reference. */

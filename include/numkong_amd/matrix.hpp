@@ -115,41 +115,45 @@ struct u1x8_t {
     }
 };
 
-/** The distance kinds exist for every type but u1, f32 and f64; `distances<T>` names their entry points. */
+/** The distance kinds exist for every type but u1; `distances<T>` names their entry points and their result type
+ *  (f32; f64 for f32 and f64 inputs). */
 template <typename value_type_>
 struct distances;
-#define NK_AMD_DEFINE_DISTANCES_(tag, name)                                                                           \
+#define NK_AMD_DEFINE_DISTANCES_(tag, name, result)                                                                           \
     template <>                                                                                                   \
     struct distances<tag> {                                                                               \
         using raw_t = tag::raw_t;                                                                         \
-        static void angulars_packed(raw_t const *a, void const *b, nk_f32_t *c, nk_size_t m, nk_size_t n,         \
+        using distance_t = result;                                                                         \
+        static void angulars_packed(raw_t const *a, void const *b, distance_t *c, nk_size_t m, nk_size_t n,         \
                                     nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) noexcept {               \
             nk_angulars_packed_##name(a, b, c, m, n, k, a_stride, c_stride);                                      \
         }                                                                                                         \
-        static void euclideans_packed(raw_t const *a, void const *b, nk_f32_t *c, nk_size_t m, nk_size_t n,       \
+        static void euclideans_packed(raw_t const *a, void const *b, distance_t *c, nk_size_t m, nk_size_t n,       \
                                       nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) noexcept {             \
             nk_euclideans_packed_##name(a, b, c, m, n, k, a_stride, c_stride);                                    \
         }                                                                                                         \
-        static void angulars_symmetric(raw_t const *v, nk_size_t n, nk_size_t k, nk_size_t stride, nk_f32_t *out, \
+        static void angulars_symmetric(raw_t const *v, nk_size_t n, nk_size_t k, nk_size_t stride, distance_t *out, \
                                        nk_size_t out_stride, nk_size_t row_start, nk_size_t row_count) noexcept { \
             nk_angulars_symmetric_##name(v, n, k, stride, out, out_stride, row_start, row_count);                 \
         }                                                                                                         \
         static void euclideans_symmetric(raw_t const *v, nk_size_t n, nk_size_t k, nk_size_t stride,              \
-                                         nk_f32_t *out, nk_size_t out_stride, nk_size_t row_start,                \
+                                         distance_t *out, nk_size_t out_stride, nk_size_t row_start,                \
                                          nk_size_t row_count) noexcept {                                          \
             nk_euclideans_symmetric_##name(v, n, k, stride, out, out_stride, row_start, row_count);               \
         }                                                                                                         \
     };
-NK_AMD_DEFINE_DISTANCES_(i8_t, i8)
-NK_AMD_DEFINE_DISTANCES_(u8_t, u8)
-NK_AMD_DEFINE_DISTANCES_(bf16_t, bf16)
-NK_AMD_DEFINE_DISTANCES_(f16_t, f16)
-NK_AMD_DEFINE_DISTANCES_(e4m3_t, e4m3)
-NK_AMD_DEFINE_DISTANCES_(e5m2_t, e5m2)
-NK_AMD_DEFINE_DISTANCES_(e2m3_t, e2m3)
-NK_AMD_DEFINE_DISTANCES_(e3m2_t, e3m2)
-NK_AMD_DEFINE_DISTANCES_(i4x2_t, i4)
-NK_AMD_DEFINE_DISTANCES_(u4x2_t, u4)
+NK_AMD_DEFINE_DISTANCES_(i8_t, i8, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(u8_t, u8, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(bf16_t, bf16, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(f16_t, f16, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(e4m3_t, e4m3, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(e5m2_t, e5m2, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(e2m3_t, e2m3, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(e3m2_t, e3m2, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(i4x2_t, i4, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(u4x2_t, u4, nk_f32_t)
+NK_AMD_DEFINE_DISTANCES_(f32_t, f32, nk_f64_t)
+NK_AMD_DEFINE_DISTANCES_(f64_t, f64, nk_f64_t)
 #undef NK_AMD_DEFINE_DISTANCES_
 
 /** Bytes of device memory; what `packed_matrix` keeps its image in unless told otherwise. */
@@ -256,14 +260,14 @@ bool dots_packed(typename value_type_::raw_t const *a, packed_matrix<value_type_
 }
 template <typename value_type_, typename allocator_type_>
 bool angulars_packed(typename value_type_::raw_t const *a, packed_matrix<value_type_, allocator_type_> const &b,
-                     nk_f32_t *c, std::size_t row_count, std::size_t a_stride_bytes, std::size_t c_stride_bytes) noexcept {
+                     typename distances<value_type_>::distance_t *c, std::size_t row_count, std::size_t a_stride_bytes, std::size_t c_stride_bytes) noexcept {
     if (b.empty()) return false;
     distances<value_type_>::angulars_packed(a, b.data(), c, row_count, b.rows(), b.depth(), a_stride_bytes, c_stride_bytes);
     return true;
 }
 template <typename value_type_, typename allocator_type_>
 bool euclideans_packed(typename value_type_::raw_t const *a, packed_matrix<value_type_, allocator_type_> const &b,
-                       nk_f32_t *c, std::size_t row_count, std::size_t a_stride_bytes, std::size_t c_stride_bytes) noexcept {
+                       typename distances<value_type_>::distance_t *c, std::size_t row_count, std::size_t a_stride_bytes, std::size_t c_stride_bytes) noexcept {
     if (b.empty()) return false;
     distances<value_type_>::euclideans_packed(a, b.data(), c, row_count, b.rows(), b.depth(), a_stride_bytes, c_stride_bytes);
     return true;
@@ -278,14 +282,14 @@ void dots_symmetric(typename value_type_::raw_t const *vectors, std::size_t coun
 }
 template <typename value_type_>
 void angulars_symmetric(typename value_type_::raw_t const *vectors, std::size_t count, std::size_t depth,
-                        std::size_t stride_bytes, nk_f32_t *result, std::size_t result_stride_bytes, std::size_t row_start,
+                        std::size_t stride_bytes, typename distances<value_type_>::distance_t *result, std::size_t result_stride_bytes, std::size_t row_start,
                         std::size_t row_count) noexcept {
     distances<value_type_>::angulars_symmetric(vectors, count, depth, stride_bytes, result, result_stride_bytes, row_start,
                                                row_count);
 }
 template <typename value_type_>
 void euclideans_symmetric(typename value_type_::raw_t const *vectors, std::size_t count, std::size_t depth,
-                          std::size_t stride_bytes, nk_f32_t *result, std::size_t result_stride_bytes,
+                          std::size_t stride_bytes, typename distances<value_type_>::distance_t *result, std::size_t result_stride_bytes,
                           std::size_t row_start, std::size_t row_count) noexcept {
     distances<value_type_>::euclideans_symmetric(vectors, count, depth, stride_bytes, result, result_stride_bytes, row_start,
                                                  row_count);

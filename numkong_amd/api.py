@@ -44,7 +44,7 @@ DTYPES = {
 
 
 # the types that also have the distance kinds (the 6-bit floats and 4-bit integers have dot products only)
-DISTANCE_DTYPES = ("i8", "u8", "bf16", "f16", "e4m3", "e5m2", "e2m3", "e3m2", "i4", "u4")
+DISTANCE_DTYPES = ("i8", "u8", "bf16", "f16", "e4m3", "e5m2", "e2m3", "e3m2", "i4", "u4", "f32", "f64")
 
 
 class NumKongAmdError(RuntimeError):
@@ -229,18 +229,25 @@ def _needs_distances(dtype: str) -> None:
         raise TypeError(f"dtype {dtype!r} has the dot-product kinds only; distances need one of {DISTANCE_DTYPES}")
 
 
+def _distance_dtype(dtype) -> str:
+    """float32 distances, float64 for f32 and f64 inputs (reference: include/numkong/spatials.h:72-137)."""
+    return "float64" if dtype in ("f32", "f64") else "float32"
+
+
 def angulars_packed(a, packed: PackedMatrix, out=None):
-    """Angular distances ``1 - cos(a_i, b_j)`` as float32 (reference: ``nk_angulars_packed_<dtype>``)."""
+    """Angular distances ``1 - cos(a_i, b_j)`` as float32, float64 for f32 and f64 inputs (reference:
+    ``nk_angulars_packed_<dtype>``)."""
     if isinstance(packed, PackedMatrix):
         _needs_distances(packed.dtype)
-    return _packed_product("nk_angulars_packed_", "float32", a, packed, out)
+    return _packed_product("nk_angulars_packed_", _distance_dtype(getattr(packed, "dtype", None)), a, packed, out)
 
 
 def euclideans_packed(a, packed: PackedMatrix, out=None):
-    """Euclidean distances ``|a_i - b_j|`` as float32 (reference: ``nk_euclideans_packed_<dtype>``)."""
+    """Euclidean distances ``|a_i - b_j|`` as float32, float64 for f32 and f64 inputs (reference:
+    ``nk_euclideans_packed_<dtype>``)."""
     if isinstance(packed, PackedMatrix):
         _needs_distances(packed.dtype)
-    return _packed_product("nk_euclideans_packed_", "float32", a, packed, out)
+    return _packed_product("nk_euclideans_packed_", _distance_dtype(getattr(packed, "dtype", None)), a, packed, out)
 
 
 def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_row, end_row):
@@ -281,12 +288,14 @@ def dots_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
 
 
 def angulars_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
-    """Upper triangle of the pairwise angular distances as float32; the diagonal is exactly 0."""
+    """Upper triangle of the pairwise angular distances as float32 (float64 for f32 and f64 inputs); the diagonal is
+    exactly 0."""
     _needs_distances(dtype)
-    return _symmetric("nk_angulars_symmetric_", "float32", vectors, dtype, out, start_row, end_row)
+    return _symmetric("nk_angulars_symmetric_", _distance_dtype(dtype), vectors, dtype, out, start_row, end_row)
 
 
 def euclideans_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
-    """Upper triangle of the pairwise euclidean distances as float32; the diagonal is exactly 0."""
+    """Upper triangle of the pairwise euclidean distances as float32 (float64 for f32 and f64 inputs); the diagonal is
+    exactly 0."""
     _needs_distances(dtype)
-    return _symmetric("nk_euclideans_symmetric_", "float32", vectors, dtype, out, start_row, end_row)
+    return _symmetric("nk_euclideans_symmetric_", _distance_dtype(dtype), vectors, dtype, out, start_row, end_row)

@@ -25,19 +25,21 @@ typedef struct {
         dots_packed_i4, dots_packed_u4, dots_packed_u1, dots_packed_f32, dots_packed_f64;
     nk_dots_packed_punned_t angulars_packed_i8, angulars_packed_u8, angulars_packed_bf16, angulars_packed_f16,
         angulars_packed_e4m3, angulars_packed_e5m2, angulars_packed_e2m3, angulars_packed_e3m2, angulars_packed_i4,
-        angulars_packed_u4;
+        angulars_packed_u4, angulars_packed_f32, angulars_packed_f64;
     nk_dots_packed_punned_t euclideans_packed_i8, euclideans_packed_u8, euclideans_packed_bf16, euclideans_packed_f16,
         euclideans_packed_e4m3, euclideans_packed_e5m2, euclideans_packed_e2m3, euclideans_packed_e3m2,
-        euclideans_packed_i4, euclideans_packed_u4;
+        euclideans_packed_i4, euclideans_packed_u4, euclideans_packed_f32, euclideans_packed_f64;
     nk_dots_symmetric_punned_t dots_symmetric_i8, dots_symmetric_u8, dots_symmetric_bf16, dots_symmetric_f16,
         dots_symmetric_e4m3, dots_symmetric_e5m2, dots_symmetric_e2m3, dots_symmetric_e3m2,
         dots_symmetric_i4, dots_symmetric_u4, dots_symmetric_u1, dots_symmetric_f32, dots_symmetric_f64;
     nk_dots_symmetric_punned_t angulars_symmetric_i8, angulars_symmetric_u8, angulars_symmetric_bf16,
         angulars_symmetric_f16, angulars_symmetric_e4m3, angulars_symmetric_e5m2, angulars_symmetric_e2m3,
-        angulars_symmetric_e3m2, angulars_symmetric_i4, angulars_symmetric_u4;
+        angulars_symmetric_e3m2, angulars_symmetric_i4, angulars_symmetric_u4, angulars_symmetric_f32,
+        angulars_symmetric_f64;
     nk_dots_symmetric_punned_t euclideans_symmetric_i8, euclideans_symmetric_u8, euclideans_symmetric_bf16,
         euclideans_symmetric_f16, euclideans_symmetric_e4m3, euclideans_symmetric_e5m2, euclideans_symmetric_e2m3,
-        euclideans_symmetric_e3m2, euclideans_symmetric_i4, euclideans_symmetric_u4;
+        euclideans_symmetric_e3m2, euclideans_symmetric_i4, euclideans_symmetric_u4, euclideans_symmetric_f32,
+        euclideans_symmetric_f64;
 } nk_implementations_t;
 
 extern nk_implementations_t nk_dispatch_table;
@@ -77,11 +79,11 @@ NK_AMD_DECLARE_DISPATCH_(f64)
 #undef NK_AMD_DECLARE_DISPATCH_
 
 /**
- *  Body shared by the dispatch_<T>.c files of the ten types with every kind. The reference walks a ladder of CPU ISAs per dtype
+ *  Body shared by the dispatch_<T>.c files of the twelve types with every kind. The reference walks a ladder of CPU ISAs per dtype
  *  (c/dispatch_i8.c:9-323); here there is one backend, so the ladder has one rung, and a kind this
  *  library does not implement falls through to the reference's error fallback (c/dispatch_i8.c:321-322).
  */
-#define NK_AMD_DEFINE_DISPATCH_(T)                                                                                    \
+#define NK_AMD_DEFINE_DISPATCH_WITH_(T, dots_stub, symmetric_stub)                                                                                  \
     void nk_dispatch_##T##_find_(nk_capability_t v, nk_kernel_kind_t k, nk_kernel_punned_t *m, nk_capability_t *c) { \
         typedef nk_kernel_punned_t m_t;                                                                               \
         if (v & nk_cap_gfx950_k) switch (k) {                                                                         \
@@ -108,10 +110,10 @@ NK_AMD_DECLARE_DISPATCH_(f64)
         case nk_kernel_dots_pack_k: *m = (m_t)nk_error_pack_, *c = 0; return;                                        \
         case nk_kernel_dots_packed_k:                                                                                 \
         case nk_kernel_angulars_packed_k:                                                                             \
-        case nk_kernel_euclideans_packed_k: *m = (m_t)nk_error_dots_, *c = 0; return;                                \
+        case nk_kernel_euclideans_packed_k: *m = (m_t)dots_stub, *c = 0; return;                       \
         case nk_kernel_dots_symmetric_k:                                                                              \
         case nk_kernel_angulars_symmetric_k:                                                                          \
-        case nk_kernel_euclideans_symmetric_k: *m = (m_t)nk_error_dots_symmetric_, *c = 0; return;                   \
+        case nk_kernel_euclideans_symmetric_k: *m = (m_t)symmetric_stub, *c = 0; return;       \
         default: *m = (m_t)nk_error_dense_, *c = 0; return;                                                          \
         }                                                                                                             \
     }                                                                                                                 \
@@ -134,7 +136,11 @@ NK_AMD_DECLARE_DISPATCH_(f64)
                                 (nk_kernel_punned_t *)&t->euclideans_symmetric_##T, &used);                           \
     }
 
-/** The same for the types that have the dot-product kinds only (u1, and with 8-byte outputs f32 and f64). */
+#define NK_AMD_DEFINE_DISPATCH_(T) NK_AMD_DEFINE_DISPATCH_WITH_(T, nk_error_dots_, nk_error_dots_symmetric_)
+/** ... and for the two types whose outputs are 8 bytes wide (f32, f64). */
+#define NK_AMD_DEFINE_DISPATCH_WIDE_(T) NK_AMD_DEFINE_DISPATCH_WITH_(T, nk_error_dots_wide_, nk_error_dots_symmetric_wide_)
+
+/** The same for the type that has the dot-product kinds only (u1). */
 #define NK_AMD_DEFINE_DISPATCH_DOTS_WITH_(T, dots_stub, symmetric_stub)                                               \
     void nk_dispatch_##T##_find_(nk_capability_t v, nk_kernel_kind_t k, nk_kernel_punned_t *m, nk_capability_t *c) { \
         typedef nk_kernel_punned_t m_t;                                                                               \
@@ -171,9 +177,6 @@ NK_AMD_DECLARE_DISPATCH_(f64)
     }
 
 #define NK_AMD_DEFINE_DISPATCH_DOTS_(T) NK_AMD_DEFINE_DISPATCH_DOTS_WITH_(T, nk_error_dots_, nk_error_dots_symmetric_)
-/** ... and for the two types whose outputs are 8 bytes wide. */
-#define NK_AMD_DEFINE_DISPATCH_WIDE_(T) \
-    NK_AMD_DEFINE_DISPATCH_DOTS_WITH_(T, nk_error_dots_wide_, nk_error_dots_symmetric_wide_)
 
 #ifdef __cplusplus
 }

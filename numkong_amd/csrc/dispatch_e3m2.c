@@ -3,7 +3,7 @@
  *  @file numkong_amd/csrc/dispatch_e3m2.c
  *
  *  Counterpart of the reference's c/dispatch_e3m2.c (`nk_dispatch_e3m2_find_`, `nk_dispatch_e3m2_init_`), for the kinds
- *  this backend serves for this type: the packed dots (size, pack, product) and the symmetric dots.
+ *  this backend serves: the packed dots (size, pack, product), the packed distances and the symmetric kinds.
  */
 #include "dispatch.h"
 

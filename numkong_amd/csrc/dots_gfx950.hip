@@ -199,9 +199,8 @@ static int product_async(int dtype, int metric, void const *a, void const *b_pac
     hipStream_t stream = (hipStream_t)stream_;
     if (!m || !n) return 0;
     if (dtype == kF32 || dtype == kF64) { // f64 results, a kernel of their own
-        if (metric != 0) return fail_msg("nk_hip_dots_packed: f32 and f64 have the dot-product kinds only");
         if (!c || !b_packed || (k && !a)) return fail_msg("nk_hip_dots_packed: NULL operand");
-        hipError_t const status = wide_product(dtype, a, b_packed, c, m, n, k, a_stride, c_stride, stream, triangle != nullptr, shift);
+        hipError_t const status = wide_product(dtype, a, b_packed, c, m, n, k, a_stride, c_stride, stream, triangle != nullptr, shift, metric);
         return status == hipSuccess ? 0 : fail(status, "nk_hip_dots_packed (f32 / f64)");
     }
     Geometry geo;

@@ -93,9 +93,10 @@ struct WideGeometry {
 };
 bool wide_geometry(int dtype, size_t n, size_t k, WideGeometry &g);
 hipError_t wide_pack(int dtype, void const *b, size_t n, size_t k, size_t b_stride, void *b_packed, hipStream_t stream);
-/** `triangle`: only the outputs with col >= row + shift (the symmetric kinds). */
+/** `triangle`: only the outputs with col >= row + shift (the symmetric kinds). `metric`: 0 dot products, 1 angular,
+ *  2 euclidean distances. */
 hipError_t wide_product(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n, size_t k,
-                        size_t a_stride, size_t c_stride, hipStream_t stream, bool triangle, uint32_t shift);
+                        size_t a_stride, size_t c_stride, hipStream_t stream, bool triangle, uint32_t shift, int metric);
 
 extern int g_forced_config; // 0: the heuristic picks the tile shape; see nk_hip_set_tile_config
 extern int g_variant;       // timing experiments of tuning builds

@@ -21,6 +21,10 @@
  */
 #include "dots_gfx950.hpp"
 
+// Every floating-point operation in this file rounds on its own (the compensated sums depend on it; the fused
+// multiply-adds that are meant are written as such).
+#pragma clang fp contract(off)
+
 namespace {
 
 constexpr int kWideTile = 64;  // rows and columns of C per workgroup
@@ -34,7 +38,74 @@ struct WideArgs {
     uint64_t a_stride, c_stride;
     uint32_t m, n, k, n_padded, k_padded;
     uint32_t tri_shift, tri_mask; // symmetric form: store only col >= row + tri_shift (mask all ones), see GemmArgs
+    int metric;                   // 0: dot products, 1: angular, 2: euclidean distances (f64, like the products)
 };
+
+/** A running sum in two numbers: the rounded sum and what the additions so far have lost (each addition's error is
+ *  recovered exactly by TwoSum). `value()` is then within a rounding of the exact sum of the terms. */
+struct CompensatedSum {
+    double sum = 0, lost = 0;
+    __device__ __forceinline__ void add(double term) {
+#pragma clang fp contract(off)
+        double const tentative = sum + term;
+        double const recovered = tentative - sum;
+        lost += (sum - (tentative - recovered)) + (term - recovered);
+        sum = tentative;
+    }
+    __device__ __forceinline__ void add(CompensatedSum const &other) { add(other.sum), lost += other.lost; }
+    __device__ __forceinline__ double value() const { return sum + lost; }
+};
+
+/** The reference's f64 reciprocal square root (scalar/serial.h:35-45): bit-trick estimate, four Newton steps; and its
+ *  finalisers for f32 and f64 inputs (spatial/serial.h:281-302). Contraction off: every operation rounds on its own. */
+__device__ __forceinline__ double wide_rsqrt(double number) {
+#pragma clang fp contract(off)
+    double y = __builtin_bit_cast(double, 0x5FE6EB50C7B537A9ull - (__builtin_bit_cast(uint64_t, number) >> 1));
+#pragma unroll
+    for (int step = 0; step < 4; ++step) y = y * (1.5 - 0.5 * number * y * y);
+    return y;
+}
+__device__ __forceinline__ double wide_distance(int metric, double dot, double query, double target) {
+#pragma clang fp contract(off)
+    if (metric == 1) {
+        double const product = query * target;
+        if (product > 0) {
+            double const result = 1.0 - dot * wide_rsqrt(product);
+            return result > 0 ? result : 0;
+        }
+        return dot == 0 ? 0.0 : 1.0;
+    }
+    double const squared = query + target - 2.0 * dot;
+    return squared > 0 ? squared * wide_rsqrt(squared) : 0.0;
+}
+
+/** Sum of squares of every row of B (f32 or f64, row-major) in f64, behind the image's matrix: one wavefront per
+ *  row, a compensated sum per lane over every 64th element, the lanes folded the same way. The reference sums the
+ *  rounded squares one after the other with a compensation (reduce/serial.h:50-92); this is the same quantity to
+ *  within a rounding, in another order. */
+template <bool F64>
+__global__ __launch_bounds__(256) void wide_norms_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
+                                                         uint32_t k, uint32_t n_padded, double *__restrict__ norms) {
+    uint32_t const lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_padded) return;
+    CompensatedSum total;
+    if (row < n) {
+        uint8_t const *source = b + (uint64_t)row * b_stride;
+        for (uint32_t at = lane; at < k; at += 64) {
+#pragma clang fp contract(off)
+            double const value = F64 ? ((double const *)source)[at] : (double)((float const *)source)[at];
+            total.add(value * value);
+        }
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        CompensatedSum other;
+        other.sum = __shfl_xor(total.sum, offset), other.lost = __shfl_xor(total.lost, offset);
+        total.add(other);
+    }
+    if (lane == 0) norms[row] = total.value(); // (padding columns: 0)
+}
+
 
 /** B (n rows of k elements, row-major, f32 or f64) -> k-major f64 with zero padding; 32 x 32 blocks through LDS so
  *  that both sides are touched in runs. */
@@ -92,9 +163,12 @@ __device__ __forceinline__ double fold_compensated(double const (&lane)[4]) {
     return running + error;
 }
 
+template <bool NORMS>
 __global__ __launch_bounds__(256) void dots_f64_compensated_kernel(WideArgs g) {
     __shared__ double a_lds[2][kWideDepth][kWideTile + 1];
     __shared__ double b_lds[2][kWideDepth][kWideTile];
+    __shared__ double row_parts[NORMS ? kWideTile : 1][4][2]; // distances: four partial sums of squares per row of A
+    __shared__ double row_norms[NORMS ? kWideTile : 1];
     uint32_t const tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     uint32_t const row0 = blockIdx.y * kWideTile, col0 = blockIdx.x * kWideTile;
     // symmetric form: a tile wholly left of the diagonal has nothing to store
@@ -130,6 +204,7 @@ __global__ __launch_bounds__(256) void dots_f64_compensated_kernel(WideArgs g) {
     uint8_t const *a_source = g.a + (uint64_t)(row0 + a_row < g.m ? row0 + a_row : 0) * g.a_stride;
     bool const a_exists = row0 + a_row < g.m;
     double a_next[2], b_next[2];
+    CompensatedSum squares; // distances: of this thread's share of its row of A
     auto fetch = [&](uint32_t k0) {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
@@ -137,6 +212,7 @@ __global__ __launch_bounds__(256) void dots_f64_compensated_kernel(WideArgs g) {
             double value = 0;
             if (a_exists && at < g.k) value = ((double const *)a_source)[at];
             a_next[e] = value;
+            if (NORMS) squares.add(value * value);
         }
         double const *b_source = g.b + (uint64_t)(k0 + b_k) * g.n_padded + col0 + b_col; // (inside the padded image)
         b_next[0] = b_source[0], b_next[1] = b_source[1];
@@ -176,13 +252,36 @@ __global__ __launch_bounds__(256) void dots_f64_compensated_kernel(WideArgs g) {
         buffer ^= 1;
     }
 
+    double column_norm[4];
+    if (NORMS) {
+        row_parts[a_row][tid & 3][0] = squares.sum, row_parts[a_row][tid & 3][1] = squares.lost;
+        __syncthreads();
+        if (tid < kWideTile) {
+            CompensatedSum total;
+#pragma unroll
+            for (int part = 0; part < 4; ++part) {
+                CompensatedSum one;
+                one.sum = row_parts[tid][part][0], one.lost = row_parts[tid][part][1];
+                total.add(one);
+            }
+            row_norms[tid] = total.value();
+        }
+        __syncthreads();
+        double const *norms = g.b + (uint64_t)g.k_padded * g.n_padded; // behind the matrix, one per padded column
+#pragma unroll
+        for (int j = 0; j < 4; ++j) column_norm[j] = norms[col0 + tx + 16 * j];
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         uint32_t const row = row0 + ty + 16 * i;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             uint32_t const col = col0 + tx + 16 * j;
-            double const result = fold_compensated(acc[i][j]);
+            double result = fold_compensated(acc[i][j]);
+            if (NORMS) {
+                result = wide_distance(g.metric, result, row_norms[ty + 16 * i], column_norm[j]);
+                if (g.tri_mask && row + g.tri_shift == col) result = 0; // a vector and itself: exactly 0
+            }
             if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col)
                 *(global_f64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8) = result;
         }
@@ -208,6 +307,7 @@ constexpr int kMatrixBStride = kMatrixCols + 4;      // doubles per staged depth
  *  wavefronts per SIMD cover each other's LDS waits. A is staged as f32, [row][k] so that one 16-byte read gives a
  *  lane the four operands (r = 0..3) of its row and depth group; B comes from the k-major f64 image into [k][column].
  */
+template <bool NORMS>
 __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
     typedef double __attribute__((ext_vector_type(4))) f64x4_t;
     typedef double __attribute__((ext_vector_type(2))) f64x2_t;
@@ -216,6 +316,8 @@ __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
     typedef __attribute__((address_space(1))) uint64_t global_u64_t;
     __shared__ __attribute__((aligned(16))) float a_lds[2][kMatrixRows][kMatrixAStride];
     __shared__ __attribute__((aligned(16))) double b_lds[2][kMatrixDepth][kMatrixBStride];
+    __shared__ double row_parts[NORMS ? kMatrixRows : 1][4][2]; // distances: four partial sums of squares per row of A
+    __shared__ double row_norms[NORMS ? kMatrixRows : 1];
     uint32_t const tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     uint32_t const row0 = blockIdx.y * kMatrixRows, col0 = blockIdx.x * kMatrixCols;
     // symmetric form: a tile wholly left of the diagonal has nothing to store
@@ -249,12 +351,17 @@ __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
     bool const aligned = ((((uint64_t)g.a) | g.a_stride) & 15) == 0;
     f32x4_t a_next;
     f64x2_t b_next;
+    CompensatedSum squares; // distances: of this thread's share of its row of A
     auto fetch = [&](uint32_t k0) {
         uint32_t const at = k0 + a_k;
         if (aligned && at + 4 <= g.k) a_next = *(f32x4_t const *)(a_source + (uint64_t)at * 4);
         else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) a_next[e] = at + e < g.k ? ((float const *)a_source)[at + e] : 0.f;
+        }
+        if (NORMS) { // four exact squares summed with three roundings of their own small sum, then one compensated addition
+            double const x0 = a_next[0], x1 = a_next[1], x2 = a_next[2], x3 = a_next[3];
+            squares.add(__builtin_fma(x0, x0, __builtin_fma(x1, x1, __builtin_fma(x2, x2, x3 * x3))));
         }
         b_next = *(f64x2_t const *)(g.b + (uint64_t)(k0 + b_k) * g.n_padded + col0 + b_col); // (inside the padded image)
     };
@@ -294,18 +401,37 @@ __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
         buffer ^= 1;
     }
 
+    double column_norm[2];
+    if (NORMS) {
+        row_parts[a_row][tid & 3][0] = squares.sum, row_parts[a_row][tid & 3][1] = squares.lost;
+        __syncthreads();
+        if (tid < kMatrixRows) {
+            CompensatedSum total;
+#pragma unroll
+            for (int part = 0; part < 4; ++part) {
+                CompensatedSum one;
+                one.sum = row_parts[tid][part][0], one.lost = row_parts[tid][part][1];
+                total.add(one);
+            }
+            row_norms[tid] = total.value();
+        }
+        __syncthreads();
+        double const *norms = g.b + (uint64_t)g.k_padded * g.n_padded; // behind the matrix, one per padded column
+#pragma unroll
+        for (int j = 0; j < 2; ++j) column_norm[j] = norms[col0 + wave_col + 16 * j + in_block];
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            uint32_t const row = row0 + wave_row + 16 * i + 4 * v + depth_group;
+            uint32_t const in_tile = wave_row + 16 * i + 4 * v + depth_group, row = row0 + in_tile;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 uint32_t const col = col0 + wave_col + 16 * j + in_block;
-                double result;
-                {
-#pragma clang fp contract(off)
-                    result = ((acc[i][j][0][v] + acc[i][j][1][v]) + acc[i][j][2][v]) + acc[i][j][3][v];
+                double result = ((acc[i][j][0][v] + acc[i][j][1][v]) + acc[i][j][2][v]) + acc[i][j][3][v];
+                if (NORMS) {
+                    result = wide_distance(g.metric, result, row_norms[in_tile], column_norm[j]);
+                    if (g.tri_mask && row + g.tri_shift == col) result = 0; // a vector and itself: exactly 0
                 }
                 if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col)
                     *(global_f64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8) = result;
@@ -331,7 +457,7 @@ bool wide_geometry(int dtype, size_t n, size_t k, WideGeometry &g) {
     g.n = (uint32_t)n, g.k = (uint32_t)k;
     g.n_padded = (uint32_t)((n + kWideTile - 1) / kWideTile * kWideTile);
     g.k_padded = (uint32_t)((k + 31) / 32 * 32); // the pack kernel writes whole 32 x 32 blocks
-    g.total_bytes = sizeof(PackedHeader) + (uint64_t)g.n_padded * g.k_padded * 8;
+    g.total_bytes = sizeof(PackedHeader) + (uint64_t)g.n_padded * g.k_padded * 8 + (uint64_t)g.n_padded * 8; // matrix, then sums of squares
     return true;
 }
 
@@ -353,12 +479,19 @@ hipError_t wide_pack(int dtype, void const *b, size_t n, size_t k, size_t b_stri
     if (grid.y > 65535) return hipErrorInvalidValue;
     if (dtype == kF64) hipLaunchKernelGGL(pack_wide_kernel<true>, grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, out, h);
     else hipLaunchKernelGGL(pack_wide_kernel<false>, grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, out, h);
+    hipError_t const status = hipGetLastError();
+    if (status != hipSuccess) return status;
+    double *norms = out + (uint64_t)g.n_padded * g.k_padded;
+    dim3 const norms_grid((g.n_padded + 3) / 4);
+    if (dtype == kF64) hipLaunchKernelGGL(wide_norms_kernel<true>, norms_grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, norms);
+    else hipLaunchKernelGGL(wide_norms_kernel<false>, norms_grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, norms);
     return hipGetLastError();
 }
 
 hipError_t wide_product(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n, size_t k,
-                        size_t a_stride, size_t c_stride, hipStream_t stream, bool triangle, uint32_t shift) {
+                        size_t a_stride, size_t c_stride, hipStream_t stream, bool triangle, uint32_t shift, int metric) {
     WideGeometry geo;
+    if (metric < 0 || metric > 2) return hipErrorInvalidValue;
     if (!wide_geometry(dtype, n, k, geo)) return hipErrorInvalidValue;
     if (m > 0x7FFFFFFFull) return hipErrorInvalidValue;
     if (((uintptr_t)c | c_stride) & 7) return hipErrorInvalidValue;
@@ -378,14 +511,14 @@ hipError_t wide_product(int dtype, void const *a, void const *b_packed, void *c,
     g.a = (uint8_t const *)a, g.b = (double const *)((uint8_t const *)b_packed + sizeof(PackedHeader)), g.c = (uint8_t *)c;
     g.a_stride = a_stride, g.c_stride = c_stride;
     g.m = (uint32_t)m, g.n = geo.n, g.k = geo.k, g.n_padded = geo.n_padded, g.k_padded = geo.k_padded;
-    g.tri_shift = shift, g.tri_mask = tri_mask;
+    g.tri_shift = shift, g.tri_mask = tri_mask, g.metric = metric;
     dim3 const grid(geo.n_padded / kWideTile, (uint32_t)((m + kWideTile - 1) / kWideTile));
     if (grid.y > 65535) return hipErrorInvalidValue;
-    if (dtype == kF64) hipLaunchKernelGGL(dots_f64_compensated_kernel, grid, dim3(256), 0, stream, g);
-    else {
-        dim3 const matrix_grid(geo.n_padded / kMatrixCols, (uint32_t)((m + kMatrixRows - 1) / kMatrixRows));
-        hipLaunchKernelGGL(dots_f32_matrix_kernel, matrix_grid, dim3(512), 0, stream, g);
-    }
+    dim3 const matrix_grid(geo.n_padded / kMatrixCols, (uint32_t)((m + kMatrixRows - 1) / kMatrixRows));
+    if (dtype == kF64 && metric) hipLaunchKernelGGL(dots_f64_compensated_kernel<true>, grid, dim3(256), 0, stream, g);
+    else if (dtype == kF64) hipLaunchKernelGGL(dots_f64_compensated_kernel<false>, grid, dim3(256), 0, stream, g);
+    else if (metric) hipLaunchKernelGGL(dots_f32_matrix_kernel<true>, matrix_grid, dim3(512), 0, stream, g);
+    else hipLaunchKernelGGL(dots_f32_matrix_kernel<false>, matrix_grid, dim3(512), 0, stream, g);
     return hipGetLastError();
 }
 

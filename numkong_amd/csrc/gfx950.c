@@ -124,7 +124,7 @@ static void nk_amd_pack_(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t
     if (staged_p) nk_hip_free(staged_p);
 }
 
-/** `metric`: 0 dot products, 1 angular distances, 2 euclidean distances; all outputs are 4 bytes wide. */
+/** `metric`: 0 dot products, 1 angular distances, 2 euclidean distances; outputs are 4 bytes wide, 8 for f32 and f64 inputs. */
 static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void const *b_packed, void *c, nk_size_t m,
                            nk_size_t n, nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {
     nk_amd_error_[0] = 0;
@@ -297,50 +297,52 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
                           row_count);                                                                              \
     }
 
-#define NK_AMD_DEFINE_BACKEND_DISTANCES_(T, in_t)                                                                   \
-    void nk_angulars_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,       \
+#define NK_AMD_DEFINE_BACKEND_DISTANCES_(T, in_t, r_t)                                                                 \
+    void nk_angulars_packed_##T##_gfx950(in_t const *a, void const *b_packed, r_t *c, nk_size_t height,       \
                                          nk_size_t width, nk_size_t depth, nk_size_t a_stride,                     \
                                          nk_size_t c_stride) {                                                     \
         nk_amd_packed_(nk_##T##_k, 1, a, b_packed, c, height, width, depth, a_stride, c_stride);                   \
     }                                                                                                              \
-    void nk_euclideans_packed_##T##_gfx950(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t height,     \
+    void nk_euclideans_packed_##T##_gfx950(in_t const *a, void const *b_packed, r_t *c, nk_size_t height,     \
                                            nk_size_t width, nk_size_t depth, nk_size_t a_stride,                   \
                                            nk_size_t c_stride) {                                                   \
         nk_amd_packed_(nk_##T##_k, 2, a, b_packed, c, height, width, depth, a_stride, c_stride);                   \
     }                                                                                                              \
     void nk_angulars_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,         \
-                                            nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,           \
+                                            nk_size_t stride, r_t *result, nk_size_t result_stride,           \
                                             nk_size_t row_start, nk_size_t row_count) {                            \
         nk_amd_symmetric_(nk_##T##_k, 1, vectors, vectors_count, depth, stride, result, result_stride, row_start,  \
                           row_count);                                                                              \
     }                                                                                                              \
     void nk_euclideans_symmetric_##T##_gfx950(in_t const *vectors, nk_size_t vectors_count, nk_size_t depth,       \
-                                              nk_size_t stride, nk_f32_t *result, nk_size_t result_stride,         \
+                                              nk_size_t stride, r_t *result, nk_size_t result_stride,         \
                                               nk_size_t row_start, nk_size_t row_count) {                          \
         nk_amd_symmetric_(nk_##T##_k, 2, vectors, vectors_count, depth, stride, result, result_stride, row_start,  \
                           row_count);                                                                              \
     }
 
 NK_AMD_DEFINE_BACKEND_DOTS_(i8, nk_i8_t, nk_i32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(i8, nk_i8_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(i8, nk_i8_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(u8, nk_u8_t, nk_u32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(u8, nk_u8_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(u8, nk_u8_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(bf16, nk_bf16_t, nk_f32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(bf16, nk_bf16_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(bf16, nk_bf16_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(f16, nk_f16_t, nk_f32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(f16, nk_f16_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(f16, nk_f16_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(e4m3, nk_e4m3_t, nk_f32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(e4m3, nk_e4m3_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(e4m3, nk_e4m3_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(e5m2, nk_e5m2_t, nk_f32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(e5m2, nk_e5m2_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(e5m2, nk_e5m2_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(e2m3, nk_e2m3_t, nk_f32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(e2m3, nk_e2m3_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(e2m3, nk_e2m3_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(e3m2, nk_e3m2_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(e3m2, nk_e3m2_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(i4, nk_i4x2_t, nk_i32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(i4, nk_i4x2_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(i4, nk_i4x2_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(u4, nk_u4x2_t, nk_u32_t)
-NK_AMD_DEFINE_BACKEND_DISTANCES_(u4, nk_u4x2_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(u4, nk_u4x2_t, nk_f32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(u1, nk_u1x8_t, nk_u32_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(f32, nk_f32_t, nk_f64_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(f32, nk_f32_t, nk_f64_t)
 NK_AMD_DEFINE_BACKEND_DOTS_(f64, nk_f64_t, nk_f64_t)
+NK_AMD_DEFINE_BACKEND_DISTANCES_(f64, nk_f64_t, nk_f64_t)

@@ -80,52 +80,54 @@ void nk_error_dots_symmetric_wide_(void const *vectors, nk_size_t n_vectors, nk_
         nk_dispatch_table.dots_symmetric_##T(vectors, n, k, stride, result, result_stride, row_start, row_count); \
     }
 
-#define NK_AMD_DISPATCH_DISTANCES_(T, in_t)                                                                     \
-    NK_DYNAMIC void nk_angulars_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t m,       \
+#define NK_AMD_DISPATCH_DISTANCES_(T, in_t, r_t)                                                                   \
+    NK_DYNAMIC void nk_angulars_packed_##T(in_t const *a, void const *b_packed, r_t *c, nk_size_t m,       \
                                            nk_size_t n, nk_size_t k, nk_size_t a_stride, nk_size_t c_stride) {  \
         nk_dispatch_table.angulars_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                     \
     }                                                                                                           \
-    NK_DYNAMIC void nk_euclideans_packed_##T(in_t const *a, void const *b_packed, nk_f32_t *c, nk_size_t m,     \
+    NK_DYNAMIC void nk_euclideans_packed_##T(in_t const *a, void const *b_packed, r_t *c, nk_size_t m,     \
                                              nk_size_t n, nk_size_t k, nk_size_t a_stride,                      \
                                              nk_size_t c_stride) {                                              \
         nk_dispatch_table.euclideans_packed_##T(a, b_packed, c, m, n, k, a_stride, c_stride);                   \
     }                                                                                                           \
     NK_DYNAMIC void nk_angulars_symmetric_##T(in_t const *vectors, nk_size_t n, nk_size_t k, nk_size_t stride,  \
-                                              nk_f32_t *result, nk_size_t result_stride, nk_size_t row_start,   \
+                                              r_t *result, nk_size_t result_stride, nk_size_t row_start,   \
                                               nk_size_t row_count) {                                            \
         nk_dispatch_table.angulars_symmetric_##T(vectors, n, k, stride, result, result_stride, row_start,       \
                                                  row_count);                                                    \
     }                                                                                                           \
     NK_DYNAMIC void nk_euclideans_symmetric_##T(in_t const *vectors, nk_size_t n, nk_size_t k, nk_size_t stride, \
-                                                nk_f32_t *result, nk_size_t result_stride, nk_size_t row_start, \
+                                                r_t *result, nk_size_t result_stride, nk_size_t row_start, \
                                                 nk_size_t row_count) {                                          \
         nk_dispatch_table.euclideans_symmetric_##T(vectors, n, k, stride, result, result_stride, row_start,     \
                                                    row_count);                                                  \
     }
 
 NK_AMD_DISPATCH_DOTS_(i8, nk_i8_t, nk_i32_t)
-NK_AMD_DISPATCH_DISTANCES_(i8, nk_i8_t)
+NK_AMD_DISPATCH_DISTANCES_(i8, nk_i8_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(u8, nk_u8_t, nk_u32_t)
-NK_AMD_DISPATCH_DISTANCES_(u8, nk_u8_t)
+NK_AMD_DISPATCH_DISTANCES_(u8, nk_u8_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(bf16, nk_bf16_t, nk_f32_t)
-NK_AMD_DISPATCH_DISTANCES_(bf16, nk_bf16_t)
+NK_AMD_DISPATCH_DISTANCES_(bf16, nk_bf16_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(f16, nk_f16_t, nk_f32_t)
-NK_AMD_DISPATCH_DISTANCES_(f16, nk_f16_t)
+NK_AMD_DISPATCH_DISTANCES_(f16, nk_f16_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(e4m3, nk_e4m3_t, nk_f32_t)
-NK_AMD_DISPATCH_DISTANCES_(e4m3, nk_e4m3_t)
+NK_AMD_DISPATCH_DISTANCES_(e4m3, nk_e4m3_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(e5m2, nk_e5m2_t, nk_f32_t)
-NK_AMD_DISPATCH_DISTANCES_(e5m2, nk_e5m2_t)
+NK_AMD_DISPATCH_DISTANCES_(e5m2, nk_e5m2_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(e2m3, nk_e2m3_t, nk_f32_t)
-NK_AMD_DISPATCH_DISTANCES_(e2m3, nk_e2m3_t)
+NK_AMD_DISPATCH_DISTANCES_(e2m3, nk_e2m3_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(e3m2, nk_e3m2_t, nk_f32_t)
-NK_AMD_DISPATCH_DISTANCES_(e3m2, nk_e3m2_t)
+NK_AMD_DISPATCH_DISTANCES_(e3m2, nk_e3m2_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(i4, nk_i4x2_t, nk_i32_t)
-NK_AMD_DISPATCH_DISTANCES_(i4, nk_i4x2_t)
+NK_AMD_DISPATCH_DISTANCES_(i4, nk_i4x2_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(u4, nk_u4x2_t, nk_u32_t)
-NK_AMD_DISPATCH_DISTANCES_(u4, nk_u4x2_t)
+NK_AMD_DISPATCH_DISTANCES_(u4, nk_u4x2_t, nk_f32_t)
 NK_AMD_DISPATCH_DOTS_(u1, nk_u1x8_t, nk_u32_t)
 NK_AMD_DISPATCH_DOTS_(f32, nk_f32_t, nk_f64_t)
+NK_AMD_DISPATCH_DISTANCES_(f32, nk_f32_t, nk_f64_t)
 NK_AMD_DISPATCH_DOTS_(f64, nk_f64_t, nk_f64_t)
+NK_AMD_DISPATCH_DISTANCES_(f64, nk_f64_t, nk_f64_t)
 
 NK_DYNAMIC int nk_uses_dynamic_dispatch(void) { return 1; }
 
@@ -191,7 +193,7 @@ NK_DYNAMIC void nk_find_kernel_punned(nk_kernel_kind_t kind, nk_dtype_t dtype, n
 NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t input) {
     if (kind == nk_kernel_angulars_packed_k || kind == nk_kernel_euclideans_packed_k ||
         kind == nk_kernel_angulars_symmetric_k || kind == nk_kernel_euclideans_symmetric_k) {
-        switch (input) { /* reference: include/numkong/numkong.h:46-51; f32 for every type served here */
+        switch (input) { /* reference: include/numkong/numkong.h:46-51 */
         case nk_i8_k:
         case nk_u8_k:
         case nk_bf16_k:
@@ -202,7 +204,9 @@ NK_DYNAMIC nk_dtype_t nk_kernel_output_dtype(nk_kernel_kind_t kind, nk_dtype_t i
         case nk_e3m2_k:
         case nk_i4_k:
         case nk_u4_k: return nk_f32_k;
-        default: return nk_dtype_unknown_k; /* (u1, f32 and f64 have the dot-product kinds only) */
+        case nk_f32_k:
+        case nk_f64_k: return nk_f64_k;
+        default: return nk_dtype_unknown_k; /* (u1 has the dot-product kinds only) */
         }
     }
     if (kind != nk_kernel_dots_packed_k && kind != nk_kernel_dots_symmetric_k) return nk_dtype_unknown_k;

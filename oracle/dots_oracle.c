@@ -250,6 +250,13 @@ static float element_f32(int dtype, void const *row, size_t i) {
     }
 }
 
+/* The same as f64, which also covers the two wide types. */
+static double element_f64(int dtype, void const *row, size_t i) {
+    if (dtype == NKO_F32) return (double)((float const *)row)[i];
+    if (dtype == NKO_F64) return ((double const *)row)[i];
+    return (double)element_f32(dtype, row, i);
+}
+
 NKO_API void nko_decode(int dtype, void const *src, size_t count, float *dst) {
     for (size_t i = 0; i < count; ++i) dst[i] = element_f32(dtype, src, i);
 }
@@ -466,16 +473,71 @@ static float serial_from_dot(int dtype, int metric, uint32_t dot_bits, uint32_t 
     return root;
 }
 
+/** Sum of squares of one f32 or f64 row in f64: Neumaier-compensated running sum of the squares, one element after
+ *  the other, as nk_reduce_moments_{f32,f64}_serial (reduce/serial.h:50-92). */
+static double row_sumsq_wide(int dtype, void const *row, size_t depth) {
+    double running = 0, compensation = 0;
+    for (size_t l = 0; l < depth; ++l) {
+        double const value = element_f64(dtype, row, l);
+        double const squared = value * value;
+        double const tentative = running + squared;
+        if (running >= squared) compensation += (running - tentative) + squared;
+        else compensation += (squared - tentative) + running;
+        running = tentative;
+    }
+    return running + compensation;
+}
+
+NKO_API void nko_row_sumsq_wide(int dtype, void const *x, size_t rows, size_t depth, size_t stride, double *out) {
+    for (size_t i = 0; i < rows; ++i) out[i] = row_sumsq_wide(dtype, (unsigned char const *)x + i * stride, depth);
+}
+
+/** scalar/serial.h:35-47: the bit-trick estimate refined by four Newton steps, all in f64. */
+static double serial_rsqrt_wide(double number) {
+    uint64_t bits;
+    memcpy(&bits, &number, 8);
+    bits = 0x5FE6EB50C7B537A9ull - (bits >> 1);
+    double y;
+    memcpy(&y, &bits, 8);
+    for (int step = 0; step < 4; ++step) y = y * (1.5 - 0.5 * number * y * y);
+    return y;
+}
+
+/** spatial/serial.h:281-302: the f64 finalisers of the f32 and f64 inputs. */
+static double serial_from_dot_wide(int metric, double dot, double query, double target) {
+    if (metric == 1) {
+        double const product = query * target;
+        if (product > 0) {
+            double const result = 1.0 - dot * serial_rsqrt_wide(product);
+            return result > 0 ? result : 0;
+        }
+        return dot == 0 ? 0.0 : 1.0;
+    }
+    double const squared = query + target - 2.0 * dot;
+    return squared > 0 ? squared * serial_rsqrt_wide(squared) : 0.0;
+}
+
 NKO_API void nko_serial_dots(int dtype, void const *a, void const *b, void *c, size_t rows, size_t columns, size_t depth,
                              size_t a_stride, size_t b_stride, size_t c_stride);
 
 /** nk_angulars_packed_<T>_serial (metric 1) / nk_euclideans_packed_<T>_serial (metric 2) from unpacked B:
  *  the serial product, then the finaliser per element with the row's and the column's sum of squares. */
-NKO_API void nko_serial_spatials(int dtype, int metric, void const *a, void const *b, float *c, size_t rows,
+NKO_API void nko_serial_spatials(int dtype, int metric, void const *a, void const *b, void *c, size_t rows,
                                  size_t columns, size_t depth, size_t a_stride, size_t b_stride, size_t c_stride) {
+    nko_serial_dots(dtype, a, b, c, rows, columns, depth, a_stride, b_stride, c_stride); /* (= pack + packed, per pair) */
+    if (dtype == NKO_F32 || dtype == NKO_F64) { /* f64 dots, f64 sums of squares, f64 results */
+        double *target_norms = (double *)__builtin_malloc(columns * sizeof(double) + 8);
+        nko_row_sumsq_wide(dtype, b, columns, depth, b_stride, target_norms);
+        for (size_t i = 0; i < rows; ++i) {
+            double const query_norm = row_sumsq_wide(dtype, (unsigned char const *)a + i * a_stride, depth);
+            double *row = (double *)((unsigned char *)c + i * c_stride);
+            for (size_t j = 0; j < columns; ++j) row[j] = serial_from_dot_wide(metric, row[j], query_norm, target_norms[j]);
+        }
+        __builtin_free(target_norms);
+        return;
+    }
     uint32_t *target_norms = (uint32_t *)__builtin_malloc(columns * sizeof(uint32_t) + 4);
     nko_row_sumsq(dtype, b, columns, depth, b_stride, target_norms);
-    nko_serial_dots(dtype, a, b, c, rows, columns, depth, a_stride, b_stride, c_stride); /* (= pack + packed, per pair) */
     for (size_t i = 0; i < rows; ++i) {
         uint32_t const query_norm = row_sumsq_bits(dtype, (unsigned char const *)a + i * a_stride, depth);
         uint32_t *row = (uint32_t *)((unsigned char *)c + i * c_stride);
@@ -493,12 +555,12 @@ NKO_API void nko_spatials_f64(int dtype, int metric, void const *a, void const *
     for (size_t i = 0; i < rows; ++i) {
         unsigned char const *a_row = (unsigned char const *)a + i * a_stride;
         double query = 0;
-        for (size_t l = 0; l < depth; ++l) query += (double)element_f32(dtype, a_row, l) * (double)element_f32(dtype, a_row, l);
+        for (size_t l = 0; l < depth; ++l) query += element_f64(dtype, a_row, l) * element_f64(dtype, a_row, l);
         for (size_t j = 0; j < columns; ++j) {
             unsigned char const *b_row = (unsigned char const *)b + j * b_stride;
             double dot = 0, target = 0;
             for (size_t l = 0; l < depth; ++l) {
-                double const x = element_f32(dtype, a_row, l), y = element_f32(dtype, b_row, l);
+                double const x = element_f64(dtype, a_row, l), y = element_f64(dtype, b_row, l);
                 dot += x * y, target += y * y;
             }
             double result;
@@ -604,17 +666,25 @@ NKO_API void nko_serial_dots(int dtype, void const *a, void const *b, void *c, s
 NKO_API void nko_serial_symmetric(int dtype, int metric, void const *vectors, size_t count, size_t depth, size_t stride,
                                   void *result, size_t result_stride, size_t row_start, size_t row_count) {
     size_t const row_end = row_start + row_count < count ? row_start + row_count : count;
+    int const wide = dtype == NKO_F32 || dtype == NKO_F64; /* (8-byte outputs, f64 sums of squares) */
     uint32_t *norms = NULL;
-    if (metric) {
+    double *wide_norms = NULL;
+    if (metric && !wide) {
         norms = (uint32_t *)__builtin_malloc(count * sizeof(uint32_t) + 4);
         nko_row_sumsq(dtype, vectors, count, depth, stride, norms);
+    }
+    if (metric && wide) {
+        wide_norms = (double *)__builtin_malloc(count * sizeof(double) + 8);
+        nko_row_sumsq_wide(dtype, vectors, count, depth, stride, wide_norms);
     }
     for (size_t i = row_start; i < row_end; ++i) {
         unsigned char const *a_row = (unsigned char const *)vectors + i * stride;
         uint32_t *out = (uint32_t *)((unsigned char *)result + i * result_stride);
         for (size_t j = i; j < count; ++j) {
-            if (dtype == NKO_F32 || dtype == NKO_F64) { /* (dot-product kind only, 8-byte outputs) */
-                ((double *)out)[j] = serial_dot_wide(dtype, a_row, (unsigned char const *)vectors + j * stride, depth);
+            if (wide) {
+                double const dot = serial_dot_wide(dtype, a_row, (unsigned char const *)vectors + j * stride, depth);
+                if (!metric) ((double *)out)[j] = dot;
+                else ((double *)out)[j] = i == j ? 0.0 : serial_from_dot_wide(metric, dot, wide_norms[i], wide_norms[j]);
                 continue;
             }
             uint32_t const dot = serial_dot_bits(dtype, a_row, (unsigned char const *)vectors + j * stride, depth);
@@ -623,6 +693,7 @@ NKO_API void nko_serial_symmetric(int dtype, int metric, void const *vectors, si
         }
     }
     if (norms) __builtin_free(norms);
+    if (wide_norms) __builtin_free(wide_norms);
 }
 
 #pragma endregion Symmetric kinds

@@ -118,7 +118,11 @@ def main():
         np.savez_compressed(os.path.join(out, f"wide_{dtype}.npz"), dtype=dtype, a=a, b=b,
                             c_serial=reference.dots_packed(dtype, a, b), vectors=vectors, row_start=row_start,
                             row_count=row_count,
-                            symmetric_serial=np.where(own, reference.symmetric("dots", dtype, vectors, row_start, row_count), 0.0))
+                            symmetric_serial=np.where(own, reference.symmetric("dots", dtype, vectors, row_start, row_count), 0.0),
+                            angulars_serial=reference.spatials_packed(support.KIND_ANGULARS, dtype, a, b),
+                            euclideans_serial=reference.spatials_packed(support.KIND_EUCLIDEANS, dtype, a, b),
+                            angulars_symmetric_serial=np.where(own, reference.symmetric("angular", dtype, vectors, row_start, row_count), 0.0),
+                            euclideans_symmetric_serial=np.where(own, reference.symmetric("euclidean", dtype, vectors, row_start, row_count), 0.0))
     print("wrote", len(os.listdir(out)) - 1, "fixtures to", out)
 
 

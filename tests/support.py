@@ -33,7 +33,9 @@ NARROW_INT_DTYPES = ("i4", "u4", "u1")
 NARROW_DTYPES = NARROW_FLOAT_DTYPES + NARROW_INT_DTYPES
 DIMENSIONS_PER_VALUE = {"i4": 2, "u4": 2, "u1": 8}
 WIDE_DTYPES = ("f32", "f64")  # f64 results; the dot-product kinds only
-DISTANCE_DTYPES = ALL_DTYPES + ("e2m3", "e3m2", "i4", "u4")  # the types with the distance kinds, packed and symmetric
+DISTANCE_DTYPES = ALL_DTYPES + ("e2m3", "e3m2", "i4", "u4")  # the types with the distance kinds (f32 results), packed and symmetric
+# ... and f32 and f64, whose distances are f64
+DISTANCE_OUTPUT = {**{t: np.float32 for t in DISTANCE_DTYPES}, "f32": np.float64, "f64": np.float64}
 INTEGER_DTYPES = ("i8", "u8", "i4", "u4", "u1")  # bit-exact everywhere
 # The reference's distance kernels take their sums of squares from the host-dispatched nk_reduce_moments_<T>, and the
 # AVX2 one of i4 squares negative values as if they were unsigned (reduce/haswell.h:3629-3633), so for i4 only the
@@ -73,6 +75,7 @@ class Oracle:
         lib.nko_serial_packed.argtypes = [_i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
         lib.nko_dots_f64.argtypes = [_i32, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
         lib.nko_row_sumsq.argtypes = [_i32, _vp, _sz, _sz, _sz, _vp]
+        lib.nko_row_sumsq_wide.argtypes = [_i32, _vp, _sz, _sz, _sz, _vp]
         lib.nko_serial_spatials.argtypes = [_i32, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz]
         lib.nko_spatials_f64.argtypes = [_i32, _i32, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]
         lib.nko_serial_symmetric.argtypes = [_i32, _i32, _vp, _sz, _sz, _sz, _vp, _sz, _sz, _sz]
@@ -114,7 +117,12 @@ class Oracle:
         return c
 
     def row_sumsq(self, dtype: str, x: np.ndarray) -> np.ndarray:
-        """Per-row sum of squares as the serial backend computes it: u32 for the integer types, f32 otherwise."""
+        """Per-row sum of squares as the serial backend computes it: u32 for the integer types, f64 for f32 and f64
+        inputs, f32 otherwise."""
+        if dtype in WIDE_DTYPES:
+            wide = np.empty(x.shape[0], dtype=np.float64)
+            self.lib.nko_row_sumsq_wide(CODES[dtype], _ptr(x), x.shape[0], x.shape[1], x.strides[0], _ptr(wide))
+            return wide
         out = np.empty(x.shape[0], dtype=np.uint32)
         self.lib.nko_row_sumsq(CODES[dtype], _ptr(x), x.shape[0], depth_of(dtype, x), x.strides[0], _ptr(out))
         return out if dtype in INTEGER_DTYPES else out.view(np.float32)
@@ -123,7 +131,7 @@ class Oracle:
         """`nk_angulars_packed_<dtype>_serial` ("angular") / `nk_euclideans_packed_<dtype>_serial` ("euclidean")."""
         m, k = a.shape[0], depth_of(dtype, a)
         n = b.shape[0]
-        c = np.empty((m, n), dtype=np.float32)
+        c = np.empty((m, n), dtype=DISTANCE_OUTPUT[dtype])
         self.lib.nko_serial_spatials(CODES[dtype], METRICS[metric], _ptr(a), _ptr(b), _ptr(c), m, n, k, a.strides[0],
                                      b.strides[0], c.strides[0])
         return c
@@ -143,7 +151,7 @@ class Oracle:
         not given): only result[i][j], i in the row window, j >= i, is written."""
         count, depth = vectors.shape[0], depth_of(dtype, vectors)
         if out is None:
-            out = np.zeros((count, count), dtype=OUTPUT[dtype] if metric == "dots" else np.float32)
+            out = np.zeros((count, count), dtype=OUTPUT[dtype] if metric == "dots" else DISTANCE_OUTPUT[dtype])
         rows = count - row_start if row_count is None else row_count
         self.lib.nko_serial_symmetric(CODES[dtype], SYMMETRIC_METRICS[metric], _ptr(vectors), count, depth,
                                       vectors.strides[0], _ptr(out), out.strides[0], row_start, rows)
@@ -224,7 +232,7 @@ class Reference:
         m, k = a.shape[0], depth_of(dtype, a)
         n = b.shape[0]
         packed = self.pack(dtype, b, viable)
-        c = np.empty((m, n), dtype=np.float32)
+        c = np.empty((m, n), dtype=DISTANCE_OUTPUT[dtype])
         self.kernel(kind, dtype, viable)[0](_ptr(a), _ptr(packed), _ptr(c), m, n, k, a.strides[0], c.strides[0])
         return c
 
@@ -233,11 +241,21 @@ class Reference:
         """The chosen backend's symmetric kernel into `out` (count x count; fresh and zeroed when not given)."""
         count, depth = vectors.shape[0], depth_of(dtype, vectors)
         if out is None:
-            out = np.zeros((count, count), dtype=OUTPUT[dtype] if metric == "dots" else np.float32)
+            out = np.zeros((count, count), dtype=OUTPUT[dtype] if metric == "dots" else DISTANCE_OUTPUT[dtype])
         rows = count - row_start if row_count is None else row_count
         self.kernel(SYMMETRIC_KINDS[metric], dtype, viable)[0](_ptr(vectors), count, depth, vectors.strides[0], _ptr(out),
                                                                out.strides[0], row_start, rows)
         return out
+
+
+def wide_distances_agree(metric, mine, ref, norms, ulps=16):
+    """f64 distances from the same f64 dot products: what differs between two evaluations is the summation order of the
+    sums of squares (a rounding or two of f64) and the last bits of the square root. Angular is 1 - x with |x| <= 1, so
+    the difference is absolute; euclidean is a root of a difference that can cancel to a residue of the norms' size."""
+    u = 2.0 ** -53
+    if metric == "angular":
+        return bool((np.abs(mine - ref) <= ulps * u).all())
+    return bool(((np.abs(mine - ref) <= ulps * u * np.abs(ref)) | (np.abs(mine * mine - ref * ref) <= ulps * u * norms)).all())
 
 
 def load_oracle() -> Oracle:

@@ -53,8 +53,9 @@ def test_packed_size_formula():
             assert nk.dots_packed_size(t, n, k) == 64 + tiles * chunks * 512 + tiles * 256, (t, n, k)
         assert nk.dots_packed_size(t, 0, 0) == 64
         assert nk.dots_packed_size(t, 1 << 40, 8) == 0  # dimensions beyond 32 bits are refused, as the error stub does
-    # the two wide types keep f64 values k-major: header + 8 bytes x (n padded to 64) x (k padded to 32)
-    assert nk.dots_packed_size("f32", 100, 70) == nk.dots_packed_size("f64", 100, 70) == 64 + 8 * 128 * 96
+    # the two wide types keep f64 values k-major: header + 8 bytes x (n padded to 64) x (k padded to 32), and a sum of
+    # squares per padded column behind them
+    assert nk.dots_packed_size("f32", 100, 70) == nk.dots_packed_size("f64", 100, 70) == 64 + 8 * 128 * 96 + 8 * 128
     with pytest.raises(TypeError):
         nk.dots_packed_size("f16c", 4, 4)
 
@@ -89,7 +90,7 @@ def test_lookup_and_capabilities():
         fn, cap = find(lib, ord("Y"), code, CAP_GFX950)  # symmetric hamming distances: not on this path
         assert fn and cap == 0
     assert find(lib, ord("G"), 1 << 20, CAP_GFX950) == (None, 0)  # f64c: unknown dtype -> null kernel
-    for name in ("e2m3", "e3m2", "i4", "u4"):  # every kind as well; dot products in their own widened types
+    for name in ("e2m3", "e3m2", "i4", "u4", "f32", "f64"):  # every kind as well; dot products in their own widened types
         code = api.DTYPES[name][0]
         for kind, stem in ((ord("P"), "nk_dots_packed_size_"), (ord("Q"), "nk_dots_pack_"), (ord("G"), "nk_dots_packed_"),
                            (ord("y"), "nk_dots_symmetric_"), (ord("N"), "nk_angulars_packed_"), (ord("E"), "nk_euclideans_packed_"),
@@ -97,11 +98,11 @@ def test_lookup_and_capabilities():
             fn, cap = find(lib, kind, code, CAP_GFX950 | 1)
             assert fn == ctypes.cast(getattr(lib, f"{stem}{name}_gfx950"), ctypes.c_void_p).value and cap == CAP_GFX950
             assert ctypes.cast(getattr(lib, f"{stem}{name}"), ctypes.c_void_p).value  # the dispatched entry point
-        expected = {"i4": 1 << 4, "u4": 1 << 8}.get(name, 1 << 11)
+        expected = {"i4": 1 << 4, "u4": 1 << 8, "f32": 1 << 10, "f64": 1 << 10}.get(name, 1 << 11)
         assert lib.nk_kernel_output_dtype(ord("G"), code) == lib.nk_kernel_output_dtype(ord("y"), code) == expected
-        for kind in (ord("N"), ord("E"), ord("n"), ord("D")):
-            assert lib.nk_kernel_output_dtype(kind, code) == 1 << 11
-    for name in ("u1", "f32", "f64"):  # the dot-product kinds only
+        for kind in (ord("N"), ord("E"), ord("n"), ord("D")):  # f32 distances, f64 for the two wide types
+            assert lib.nk_kernel_output_dtype(kind, code) == (1 << 10 if name in ("f32", "f64") else 1 << 11)
+    for name in ("u1",):  # the dot-product kinds only
         code = api.DTYPES[name][0]
         for kind, stem in ((ord("P"), "nk_dots_packed_size_"), (ord("Q"), "nk_dots_pack_"), (ord("G"), "nk_dots_packed_"),
                            (ord("y"), "nk_dots_symmetric_")):
@@ -110,7 +111,7 @@ def test_lookup_and_capabilities():
         for kind in (ord("N"), ord("E"), ord("n"), ord("D")):
             fn, cap = find(lib, kind, code, CAP_GFX950)
             assert fn and cap == 0
-        expected = {"u1": 1 << 8, "f32": 1 << 10, "f64": 1 << 10}[name]
+        expected = {"u1": 1 << 8}[name]
         assert lib.nk_kernel_output_dtype(ord("G"), code) == lib.nk_kernel_output_dtype(ord("y"), code) == expected
         assert lib.nk_kernel_output_dtype(ord("N"), code) == 0
     out = {"i8": 1 << 4, "u8": 1 << 8, "bf16": 1 << 11, "f16": 1 << 11, "e4m3": 1 << 11, "e5m2": 1 << 11}

@@ -435,6 +435,73 @@ def test_wide_products_match_reference_serial(oracle, reference, dtype):
         assert not mine[~own].any()
 
 
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", WIDE_DTYPES)
+def test_wide_distances_match_reference_serial(oracle, reference, dtype, metric):
+    """nk_{angulars,euclideans}_{packed,symmetric}_{f32,f64}_serial (f64 results): the sums of squares bit for bit
+    against nk_reduce_moments_{f32,f64}_serial, the distances to 16 units of 2^-53 (the reference takes its sums of
+    squares from the host-dispatched moments, whose order differs; dots and finaliser are restated exactly)."""
+    if reference is None:
+        pytest.skip("reference build not present")
+    import ctypes
+
+    rng = np.random.default_rng(68)
+    fn, cap = ctypes.c_void_p(), ctypes.c_uint64()
+    reference.lib.nk_find_kernel_punned(ord("R"), support.CODES[dtype], support.CAP_SERIAL, ctypes.byref(fn), ctypes.byref(cap))
+    moments = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p)(fn.value)
+    for kind in ("default", "lognormal"):
+        for m, n, k in [(1, 1, 1), (5, 7, 37), (33, 21, 300), (9, 4, 4099)]:
+            a, b = support.random_matrix(oracle, dtype, m, k, rng, kind), support.random_matrix(oracle, dtype, n, k, rng, kind)
+            if m > 4:
+                a[1] = 0
+                b[2] = a[3]
+            squares = oracle.row_sumsq(dtype, a)
+            for i in range(m):
+                total, sumsq = np.zeros(1), np.zeros(1)
+                moments(a[i].ctypes.data, k, a.itemsize, total.ctypes.data, sumsq.ctypes.data)
+                assert squares[i:i + 1].view(np.uint64)[0] == sumsq.view(np.uint64)[0], (dtype, kind, m, k, i)
+            norms = squares[:, None] + oracle.row_sumsq(dtype, b)[None, :]
+            mine = oracle.spatials_packed(metric, dtype, a, b)
+            ref = reference.spatials_packed(support.METRIC_KINDS[metric], dtype, a, b)
+            assert mine.dtype == ref.dtype == np.float64
+            assert support.wide_distances_agree(metric, mine, ref, norms), (dtype, metric, kind, m, n, k)
+            truth = oracle.spatials_truth(metric, dtype, a, b)  # plain f64 sums: a loose band against a common mistake
+            assert support.wide_distances_agree(metric, mine, truth, norms, ulps=64 * k)
+    for count, depth, row_start, row_count in SYMMETRIC_CASES[:6]:
+        row_count = min(row_count, count - row_start)
+        vectors = support.random_matrix(oracle, dtype, count, depth, rng)
+        if count > 40:
+            vectors[2] = 0
+            vectors[9] = vectors[40]
+        own = upper_window(count, row_start, row_count)
+        mine = oracle.symmetric(metric, dtype, vectors, row_start, row_count)
+        ref = reference.symmetric(metric, dtype, vectors, row_start, row_count)
+        assert not mine[~own].any() and not np.diag(mine).any() and not np.diag(ref)[row_start:row_start + row_count].any()
+        squares = oracle.row_sumsq(dtype, vectors)
+        assert support.wide_distances_agree(metric, mine[own], ref[own], (squares[:, None] + squares[None, :])[own]), (dtype, metric, count)
+        strict = np.triu(np.ones((count, count), dtype=bool), 1) & own
+        packed = oracle.spatials_packed(metric, dtype, vectors, vectors)
+        assert np.array_equal(mine[strict].view(np.uint64), packed[strict].view(np.uint64))
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", WIDE_DTYPES)
+def test_wide_distances_closed_forms(oracle, dtype, metric):
+    """Needs no reference: orthogonal rows, a row against itself and its double, a zero row (the layout of
+    test_packed_distances_closed_forms), to a few units of 2^-53."""
+    k = 64
+    rows = np.zeros((4, k), dtype=support.STORAGE[dtype])
+    rows[0, :16] = 1
+    rows[1, 16:32] = 1
+    rows[2, :16] = 2
+    got = oracle.spatials_packed(metric, dtype, rows, rows)
+    if metric == "angular":
+        expected = np.array([[0, 1, 0, 0], [1, 0, 1, 0], [0, 1, 0, 0], [0, 0, 0, 0]], dtype=np.float64)
+    else:
+        expected = np.array([[0, np.sqrt(32), 4, 4], [np.sqrt(32), 0, np.sqrt(80), 4], [4, np.sqrt(80), 0, 8], [4, 4, 8, 0]])
+    assert np.abs(got - expected).max() <= 8 * 2.0 ** -53 * 8
+
+
 def test_wide_products_closed_forms(oracle):
     """Needs no reference. Small integers: every sum is exact in f64, so both kinds equal the int64 product. f64 only:
     sums that plain f64 gets wrong and a sum in twice the working precision gets right: 1e100 + 1 - 1e100 = 1, and a
@@ -518,6 +585,12 @@ def test_golden_vectors(oracle, name):
         assert np.array_equal(oracle.dots_packed(dtype, a, b).view(np.uint64), data["c_serial"].view(np.uint64))
         mine = oracle.symmetric("dots", dtype, vectors, int(data["row_start"]), int(data["row_count"]))
         assert np.array_equal(mine.view(np.uint64), data["symmetric_serial"].view(np.uint64))
+        norms = oracle.row_sumsq(dtype, a)[:, None] + oracle.row_sumsq(dtype, b)[None, :]
+        squares = oracle.row_sumsq(dtype, vectors)
+        for metric, key in (("angular", "angulars"), ("euclidean", "euclideans")):  # f64 distances: 16 units of 2^-53
+            assert support.wide_distances_agree(metric, oracle.spatials_packed(metric, dtype, a, b), data[key + "_serial"], norms)
+            mine = oracle.symmetric(metric, dtype, vectors, int(data["row_start"]), int(data["row_count"]))
+            assert support.wide_distances_agree(metric, mine, data[key + "_symmetric_serial"], squares[:, None] + squares[None, :])
     elif name.startswith("narrow_"):
         dtype, a, b, vectors = str(data["dtype"]), data["a"], data["b"], data["vectors"]
         assert same_floats(oracle.dots_packed(dtype, a, b).view(np.float32), data["c_serial"].view(np.float32))

@@ -8,6 +8,14 @@ kernels (f32: the f64 MFMA, whose chain of fused multiply-adds along its depth a
 keep the reference's own accumulators per output in the reference's own order along k, so the bar here is the
 integer one: BIT-EXACT against the oracle's restatement of the serial kernels (which tests/test_oracle.py pins bit for
 bit against the reference library), not a tolerance.
+
+The distance kinds (`nk_{angulars,euclideans}_{packed,symmetric}_{f32,f64}`, f64 results; reference
+include/numkong/spatials/serial.h:41-72, finalisers include/numkong/spatial/serial.h:281-302) finalise those same dot
+products with the reference's own f64 arithmetic (bit-trick reciprocal square root, four Newton steps), so what can differ
+from the serial kernel is the order in which the sums of squares are added up: a rounding or two of f64. Tolerance: 16
+units of 2^-53, absolute for angular (a value in [0, 2]), relative for euclidean or, where two nearly equal vectors
+cancel, of the sum of the two norms under the root (tests/support.py: wide_distances_agree); the oracle is pinned against
+the reference's serial kernels to the same tolerance in tests/test_oracle.py.
 """
 import os
 
@@ -64,7 +72,7 @@ def test_c_abi_strides_host_pointers_and_mismatch(oracle, dtype):
     a_wide, b_wide = support.random_matrix(oracle, dtype, m, k + pad, rng), support.random_matrix(oracle, dtype, n, k + pad, rng)
     a, b = np.ascontiguousarray(a_wide[:, :k]), np.ascontiguousarray(b_wide[:, :k])
     size = getattr(lib, f"nk_dots_packed_size_{dtype}")(n, k)
-    assert size == 64 + 8 * 64 * (-(-k // 32) * 32)  # header + f64 x (n padded to 64) x (k padded to 32)
+    assert size == 64 + 8 * 64 * (-(-k // 32) * 32) + 8 * 64  # header + f64 x (n padded to 64) x (k padded to 32) + sums of squares
     packed = np.zeros(size, np.uint8)
     getattr(lib, f"nk_dots_pack_{dtype}")(b_wide.ctypes.data, n, k, b_wide.strides[0], packed.ctypes.data)
     c = np.full((m, n + 2), np.float64(-7.0))
@@ -80,8 +88,6 @@ def test_c_abi_strides_host_pointers_and_mismatch(oracle, dtype):
                                           a.strides[0], n * 8, torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert status == 0 and (out.cpu().numpy().view(np.uint64) == 0xFFFFFFFFFFFFFFFF).all()
-    with pytest.raises(TypeError):
-        nk.angulars_packed(ga, other)  # dot-product kinds only
 
 
 @pytest.mark.parametrize("dtype", WIDE_DTYPES)
@@ -109,6 +115,13 @@ def test_golden_vectors(oracle, name):
     out = torch.zeros((count, count), dtype=torch.float64, device=DEV)
     nk.dots_symmetric(to_gpu(vectors), dtype, out=out, start_row=row_start, end_row=row_start + row_count)
     assert same_bits(out.cpu().numpy(), data["symmetric_serial"])
+    norms = oracle.row_sumsq(dtype, a)[:, None] + oracle.row_sumsq(dtype, b)[None, :]
+    squares = oracle.row_sumsq(dtype, vectors)
+    for metric, key, call in (("angular", "angulars", nk.angulars_symmetric), ("euclidean", "euclideans", nk.euclideans_symmetric)):
+        assert support.wide_distances_agree(metric, gpu_wide_distances(metric, dtype, a, b), data[key + "_serial"], norms)
+        out = torch.zeros((count, count), dtype=torch.float64, device=DEV)
+        call(to_gpu(vectors), dtype, out=out, start_row=row_start, end_row=row_start + row_count)
+        assert support.wide_distances_agree(metric, out.cpu().numpy(), data[key + "_symmetric_serial"], squares[:, None] + squares[None, :])
 
 
 @pytest.mark.parametrize("dtype", WIDE_DTYPES)
@@ -127,3 +140,69 @@ def test_full_size_properties(oracle, dtype):
     rows = np.array([0, 1001, 2047])
     sample = rectangle[torch.from_numpy(rows).to(DEV)].cpu().numpy()
     assert same_bits(sample, oracle.dots_packed(dtype, vectors[rows], vectors))
+
+
+def gpu_wide_distances(metric, dtype, a, b):
+    call = {"angular": nk.angulars_packed, "euclidean": nk.euclideans_packed}[metric]
+    return call(to_gpu(a), nk.dots_pack(to_gpu(b), dtype)).cpu().numpy()
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", WIDE_DTYPES)
+def test_packed_distances(oracle, dtype, metric):
+    rng = np.random.default_rng(905)
+    for kind in ("default", "lognormal"):
+        for m, n, k in SHAPES:
+            a, b = support.random_matrix(oracle, dtype, m, k, rng, kind), support.random_matrix(oracle, dtype, n, k, rng, kind)
+            if m > 4 and n > 4:
+                a[1] = 0         # zero row
+                b[2] = a[3]      # identical rows
+                b[4] = 0
+            got = gpu_wide_distances(metric, dtype, a, b)
+            assert got.dtype == np.float64 and np.isfinite(got).all()
+            serial = oracle.spatials_packed(metric, dtype, a, b)
+            norms = oracle.row_sumsq(dtype, a)[:, None] + oracle.row_sumsq(dtype, b)[None, :]
+            assert support.wide_distances_agree(metric, got, serial, norms), f"{dtype} {metric} {kind} {m}x{n}x{k}"
+            if m > 4 and n > 4:
+                assert got[1, 4] == 0
+                if metric == "angular":
+                    assert (got[1] == 0).all()
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", WIDE_DTYPES)
+def test_symmetric_distances(oracle, dtype, metric):
+    rng = np.random.default_rng(906)
+    call = {"angular": nk.angulars_symmetric, "euclidean": nk.euclideans_symmetric}[metric]
+    for count, depth, row_start, row_count in [(5, 8, 0, 5), (300, 64, 100, 77), (700, 131, 333, 1000), (130, 515, 0, 130)]:
+        vectors = support.random_matrix(oracle, dtype, count, depth, rng, "lognormal")
+        if count > 40:
+            vectors[2] = 0
+            vectors[9] = vectors[40]
+        row_count = min(row_count, count - row_start)
+        out = torch.full((count, count), POISON, dtype=torch.int64, device=DEV).view(torch.float64)
+        call(to_gpu(vectors), dtype, out=out, start_row=row_start, end_row=row_start + row_count)
+        bits = out.view(torch.int64).cpu().numpy().view(np.uint64)
+        own = owned(count, row_start, row_count)
+        assert (bits[~own] == POISON).all()
+        window = np.arange(row_start, row_start + row_count)
+        assert (bits[window, window] == 0).all()  # a vector and itself: exactly 0
+        got, serial = bits.view(np.float64), oracle.symmetric(metric, dtype, vectors, row_start, row_count)
+        squares = oracle.row_sumsq(dtype, vectors)
+        assert support.wide_distances_agree(metric, got[own], serial[own], (squares[:, None] + squares[None, :])[own]), (dtype, metric, count)
+
+
+@pytest.mark.parametrize("dtype", WIDE_DTYPES)
+def test_distances_through_the_c_abi_with_host_pointers(oracle, dtype):
+    rng = np.random.default_rng(907)
+    lib = nk.library()
+    m, n, k = 19, 45, 203
+    a, b = support.random_matrix(oracle, dtype, m, k, rng), support.random_matrix(oracle, dtype, n, k, rng)
+    packed = np.zeros(getattr(lib, f"nk_dots_packed_size_{dtype}")(n, k), np.uint8)
+    getattr(lib, f"nk_dots_pack_{dtype}")(b.ctypes.data, n, k, b.strides[0], packed.ctypes.data)
+    norms = oracle.row_sumsq(dtype, a)[:, None] + oracle.row_sumsq(dtype, b)[None, :]
+    for metric, stem in (("angular", "nk_angulars_packed_"), ("euclidean", "nk_euclideans_packed_")):
+        c = np.full((m, n + 1), -7.0)
+        getattr(lib, stem + dtype)(a.ctypes.data, packed.ctypes.data, c.ctypes.data, m, n, k, a.strides[0], c.strides[0])
+        assert not lib.nk_amd_last_error() and (c[:, n] == -7.0).all()
+        assert support.wide_distances_agree(metric, c[:, :n], oracle.spatials_packed(metric, dtype, a, b), norms)
