@@ -12,8 +12,8 @@
  *
  *  `dtype` arguments take the `nk_dtype_t` codes of <numkong_amd/dots.h> (reference:
  *  include/numkong/types.h:923-952): nk_i8_k, nk_u8_k, nk_bf16_k, nk_f16_k, nk_e4m3_k, nk_e5m2_k, nk_e2m3_k, nk_e3m2_k,
- *  nk_i4_k, nk_u4_k (every kind), and nk_u1_k, nk_f32_k, nk_f64_k (the dot-product kinds). Depth counts dimensions, so
- *  4-bit values or bits for the sub-byte types; f32 and f64 write 8-byte f64 outputs.
+ *  nk_i4_k, nk_u4_k, nk_f32_k, nk_f64_k (every kind), and nk_u1_k (the dot-product kinds). Depth counts dimensions, so
+ *  4-bit values or bits for the sub-byte types; f32 and f64 write 8-byte f64 outputs, distances included.
  */
 #ifndef NUMKONG_AMD_HIP_ABI_H
 #define NUMKONG_AMD_HIP_ABI_H
@@ -46,7 +46,7 @@ int nk_hip_stream_synchronize(void *stream);
 
 /**
  *  Bytes of the gfx950 packed image of an (n x k) B matrix: 64-byte header, MFMA-fragment tiles,
- *  per-column compensation terms, per-column sums of squares (f32 / f64: header and k-major f64 values). Replaces `nk_dots_packed_size_<T>_<isa>`
+ *  per-column compensation terms, per-column sums of squares (f32 / f64: header, k-major f64 values, f64 sums of squares). Replaces `nk_dots_packed_size_<T>_<isa>`
  *  (reference: include/numkong/dots/serial.h:245-271). Returns 0 for an unsupported dtype or when
  *  n or k do not fit 32 bits.
  */
@@ -69,7 +69,7 @@ int nk_hip_dots_packed_async(int dtype, void const *a, void const *b_packed, voi
 
 /**
  *  Distances instead of dot products, in one pass: C[i][j] = angular (metric 1) or euclidean (metric 2) distance
- *  between row i of A and row j of B, as f32, from the same MFMA product, the per-column sums of squares that
+ *  between row i of A and row j of B, as f32 (f64 for f32 and f64 inputs), from the same MFMA product, the per-column sums of squares that
  *  `nk_hip_dots_pack_async` leaves in the image and the per-row sums of squares gathered while A is staged.
  *  Replaces `nk_angulars_packed_<T>_<isa>` / `nk_euclideans_packed_<T>_<isa>`
  *  (reference: include/numkong/dots/serial.h:2756-2800, include/numkong/spatial/serial.h:257-344).

@@ -157,8 +157,8 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
     }
     if (g.n_tiles && terms) {
         if (g.k_chunks) {
-            // by what the image holds: signed bytes (i8 and the widened 4-bit types), offset u8, bf16, f16 (and what is widened to it)
-            auto kernel = dtype == kI8 || dtype == kI4 || dtype == kU4 || dtype == kU1
+            // by what the image holds: signed bytes (i8, the widened 4-bit types and bits, e2m3 as 8 x its values), offset u8, bf16, f16 (and what is widened to it)
+            auto kernel = dtype == kI8 || dtype == kI4 || dtype == kU4 || dtype == kU1 || dtype == kE2M3
                               ? column_terms_kernel<0>
                               : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
             hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(256), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);

@@ -25,7 +25,7 @@
  *  is the MFMA operand-fragment order, and B goes from HBM to registers with one coalesced 128-bit load
  *  per lane per step, never through LDS. Which k sits in which operand slot of the instruction does not
  *  matter as long as A and B agree, and they do: A fragments are read from LDS with the same rule.
- *  e4m3 and e5m2 are stored widened to f16 (see packed_bytes_of), so their chunks hold 8 values.
+ *  e4m3, e5m2 and e3m2 are stored widened to f16 (see packed_bytes_of), so their chunks hold 8 values.
  *
  *  u8 has no unsigned MFMA. B is stored as b' = b ^ 0x80 (signed b - 128), A is turned into
  *  a' = a ^ 0x80 on its way into LDS, and  sum(a*b) = sum(a'*b') + 128*sum(a) + 128*sum(b')  (mod 2^32)
@@ -188,14 +188,15 @@ inline int elem_bits_of(int dtype) {
  *  keep only about 14 bits (1 + 2^-14 comes back as 1), far from the f32 accumulation of the reference's
  *  kernels (dot/serial.h:522-600). e4m3 and e5m2 are therefore widened, exactly, to f16 and run on the f16
  *  MFMA, whose products and sums are kept to full f32 precision: B at pack time, A on its way into LDS.
- *  The 6-bit floats go the same way (every e2m3 / e3m2 value is an f16 value), and the 4-bit integers are
- *  widened to i8 for the i8 MFMA, and so are single bits (0 or 1: their dot product is the popcount of the AND). */
+ *  e3m2 goes the same way (every e3m2 value is an f16 value). e2m3 values are multiples of 1/8 below 8 in magnitude:
+ *  eight times each is an i8 value, and the i8 MFMA sums their products exactly at twice the f16 rate. The 4-bit
+ *  integers are widened to i8 as well, and so are single bits (0 or 1: their dot product is the popcount of the AND). */
 inline int packed_bytes_of(int dtype) {
     switch (dtype) {
     case kE4M3:
     case kE5M2:
-    case kE2M3:
     case kE3M2: return 2;
+    case kE2M3: // (as i8 values, eight times the e2m3 value)
     case kI4:
     case kU4:
     case kU1: return 1;
@@ -279,7 +280,8 @@ __device__ __forceinline__ v4i widen_fp8x8(uint32_t lo, uint32_t hi) {
  *  subnormals and no Inf/NaN (e2m3: 2 exponent bits, bias 1; e3m2: 3 exponent bits, bias 3; reference decoders:
  *  cast/serial.h:1318-1330, 1455-1470), so the exponent and mantissa bits, moved under an f16's sign bit, read as the
  *  value scaled by a power of two, subnormals included: one packed multiply by 2^14 (e2m3) or 2^12 (e3m2) finishes
- *  two values at a time. Bits 6 and 7 of a byte are ignored, as the reference does.
+ *  two values at a time. Bits 6 and 7 of a byte are ignored, as the reference does. In use for e3m2; e2m3 has the
+ *  cheaper integer route of widen_e2m3x4.
  */
 template <bool E3M2>
 __device__ __forceinline__ v4i widen_fp6x8(uint32_t lo, uint32_t hi) {
@@ -297,6 +299,28 @@ __device__ __forceinline__ v4i widen_fp6x8(uint32_t lo, uint32_t hi) {
         out[pair] = __builtin_bit_cast(int, value);
     }
     return out;
+}
+
+/**
+ *  Four e2m3 values, one per byte -> four i8 values, each EIGHT TIMES the e2m3 value: with 2 exponent bits (bias 1) and
+ *  3 mantissa bits every e2m3 value is a multiple of 1/8 of magnitude at most 7.5, so 8 x is an integer in [-60, 60]
+ *  (reference decoder: cast/serial.h:1318-1330). Products of two such integers summed in i32 are exact, 64 times the
+ *  dot product, and the i8 MFMA runs at twice the rate of the f16 one. All four bytes at once: with x = the low five
+ *  bits (e, m), the magnitude is x for e <= 1 (m, or 8 + m), x + (x & 15) for e = 2 (16 + 2 m) and
+ *  x + (x & 15) + 2 (x & 7) for e = 3 (32 + 4 m); no byte ever carries into its neighbour. The three per-byte masks
+ *  (the two above and 0xFF for a set sign bit) come from 8-entry byte tables indexed by bits 3..5 of each byte, one
+ *  v_perm_b32 each. Negative values by 0x80 - magnitude, flipped back. Bits 6 and 7 of a byte are ignored, as the
+ *  reference does.
+ */
+__device__ __forceinline__ uint32_t widen_e2m3x4(uint32_t codes) {
+    uint32_t const index = (codes >> 3) & 0x07070707u; // e + 4 * sign, per byte
+    uint32_t const negate = __builtin_amdgcn_perm(0xFFFFFFFFu, 0x00000000u, index);  // 0xFF where the sign bit is set
+    uint32_t const from_two = __builtin_amdgcn_perm(0x0F0F0000u, 0x0F0F0000u, index); // 0x0F where e >= 2
+    uint32_t const at_three = __builtin_amdgcn_perm(0x07000000u, 0x07000000u, index); // 0x07 where e == 3
+    uint32_t const low = codes & 0x1F1F1F1Fu;
+    uint32_t const magnitude = low + (low & from_two) + ((low & at_three) << 1);
+    uint32_t const negative = (0x80808080u - magnitude) ^ 0x80808080u;
+    return (negative & negate) | (magnitude & ~negate);
 }
 
 /** Sixteen 4-bit integers (two dwords; the even dimension in the low nibble) -> sixteen i8 values: the low nibbles
@@ -324,13 +348,13 @@ __device__ __forceinline__ v4i widen_u1x16(uint32_t bits) {
     return out;
 }
 
-/** Widening of the source bytes behind one 16-byte chunk, by kind: 1 e4m3, 2 e5m2, 3 e2m3, 4 e3m2 (8 bytes to f16);
- *  5 i4, 6 u4 (8 bytes to i8); 7 u1 (2 bytes to i8). */
+/** Widening of the source bytes behind one 16-byte chunk, by kind: 1 e4m3, 2 e5m2, 4 e3m2 (8 bytes to f16);
+ *  5 i4, 6 u4 (8 bytes to i8); 7 u1 (2 bytes to i8). Kind 3, e2m3, turns 16 bytes into 16 i8 values in place
+ *  (widen_e2m3x4) and does not come through here. */
 template <int WIDEN>
 __device__ __forceinline__ v4i widen_chunk(uint32_t lo, uint32_t hi) {
     if constexpr (WIDEN == 1) return widen_fp8x8<false>(lo, hi);
     else if constexpr (WIDEN == 2) return widen_fp8x8<true>(lo, hi);
-    else if constexpr (WIDEN == 3) return widen_fp6x8<false>(lo, hi);
     else if constexpr (WIDEN == 4) return widen_fp6x8<true>(lo, hi);
     else if constexpr (WIDEN == 5) return widen_i4x16<true>(lo, hi);
     else if constexpr (WIDEN == 6) return widen_i4x16<false>(lo, hi);
@@ -354,13 +378,14 @@ inline int widen_kind_of(int dtype) {
 /**
  *  One thread per 16-byte chunk of the image. A block of 256 threads covers 32 rows x 8 chunks: reads are
  *  128 (64 for the widened types) contiguous bytes per row, writes are eight 512-byte runs. WIDEN: 0 copies the
- *  elements, otherwise the kind of widen_chunk (8 source bytes per chunk).
+ *  elements, 3 rewrites e2m3 bytes as i8 values in place, otherwise the kind of widen_chunk (8 or 2 source bytes per
+ *  chunk).
  */
 template <int WIDEN>
 __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
                                                    uint64_t k_src_bytes, uint32_t k_chunks, uint8_t *__restrict__ data,
                                                    int avec, uint32_t xr, PackedHeader header) {
-    constexpr int kSrcChunk = WIDEN == 0 ? 16 : (WIDEN == 7 ? 2 : 8);
+    constexpr int kSrcChunk = WIDEN == 0 || WIDEN == 3 ? 16 : (WIDEN == 7 ? 2 : 8);
     if (blockIdx.x == 0 && threadIdx.x == 0) *(PackedHeader *)(data - sizeof(PackedHeader)) = header; // (64 bytes in front of the tiles)
     uint32_t const groups = k_chunks / kStageChunks;
     uint32_t const tile = blockIdx.x / groups;
@@ -373,12 +398,16 @@ __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b
     v4i v = {0, 0, 0, 0};
     if (valid > 0) {
         uint8_t const *src = b + row * b_stride + (uint64_t)c * kSrcChunk;
-        if (!WIDEN && valid == 16 && avec >= 16) {
+        if ((WIDEN == 0 || WIDEN == 3) && valid == 16 && avec >= 16) {
             v = *(v4i const *)src;
             v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
         }
         else { v = load_chunk_guarded(src, valid, avec, xr); }
-        if constexpr (WIDEN != 0) v = widen_chunk<WIDEN>((uint32_t)v[0], (uint32_t)v[1]);
+        if constexpr (WIDEN == 3) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) v[w] = (int)widen_e2m3x4((uint32_t)v[w]);
+        }
+        else if constexpr (WIDEN != 0) v = widen_chunk<WIDEN>((uint32_t)v[0], (uint32_t)v[1]);
     }
     *(v4i *)(data + (((uint64_t)tile * k_chunks + c) * kTileRows + r) * kChunkBytes) = v;
 }
@@ -585,13 +614,19 @@ struct E5M2 : F16 {
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<true>((uint32_t)v[0], (uint32_t)v[1]); }
 };
-/** The 6-bit floats run widened to f16 as well; see widen_fp6x8. */
-struct E2M3 : F16 {
-    static constexpr bool kChunked = true;
+/** e2m3 runs as i8 values eight times as large on the i8 MFMA (see widen_e2m3x4): sums are exact integers, 64 times
+ *  the dot product, converted to f32 once in the epilogue (one rounding for sums beyond 2^24, none below). */
+struct E2M3 : I8 {
     static constexpr int kDtype = kE2M3;
-    static constexpr int kSrcChunk = 8;
-    static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp6x8<false>((uint32_t)v[0], (uint32_t)v[1]); }
+    static __device__ __forceinline__ v4i widen(v4i v) {
+        v4i out;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) out[w] = (int)widen_e2m3x4((uint32_t)v[w]);
+        return out;
+    }
+    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); } // 64 x the sum of squares
 };
+/** e3m2 runs widened to f16 (its values times 16 do not fit i8); see widen_fp6x8. */
 struct E3M2 : F16 {
     static constexpr bool kChunked = true;
     static constexpr int kDtype = kE3M2;
@@ -631,7 +666,16 @@ template <class T>
 __device__ __forceinline__ float norm_as_f32(uint32_t bits) {
     if (T::kDtype == kI8 || T::kDtype == kI4) return (float)(int)bits;
     if (T::kDtype == kU8 || T::kDtype == kU4) return (float)bits;
+    if (T::kDtype == kE2M3) return (float)bits * 0.015625f; // integer sums of squares of 8 x the values
     return __builtin_bit_cast(float, bits);
+}
+
+/** What the accumulators hold -> what the caller gets, as 32-bit patterns: as they are, except that e2m3 sums are
+ *  integers, 64 times the f32 result. */
+template <class T>
+__device__ __forceinline__ uint32_t finished_dot(uint32_t bits) {
+    if (T::kDtype == kE2M3) return __builtin_bit_cast(uint32_t, (float)(int)bits * 0.015625f);
+    return bits;
 }
 
 /** METRIC: 1 angular, 2 euclidean. `query` and `target` are the row's and the column's sums of squares as f32
@@ -1341,7 +1385,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                         int const r_fixed = i * 32 + 8 * (v / 4) + (v % 4); // row of lanes 0..31; lanes 32..63 are 4 rows below
                         // a named copy: bit-casting the vector element expression itself reads lane 0
                         auto const element = total.finish(acc, i, j, v);
-                        uint32_t bits = __builtin_bit_cast(uint32_t, element);
+                        uint32_t bits = finished_dot<T>(__builtin_bit_cast(uint32_t, element));
                         if (T::kUnsigned) {
                             // the terms of 4 consecutive rows in one LDS read
                             if (v % 4 == 0) row_term4 = *(v4i const *)&row_terms[i * 32 + 8 * (v / 4) + 4 * half];

@@ -17,7 +17,9 @@
  *
  *  Either way every output keeps the reference's own accumulators and takes its terms in the reference's own order
  *  along k, so the results are those of its serial kernels bit for bit. B comes from an image that is already k-major
- *  f64: [64-byte header][k padded to 32][n padded to 64] doubles, zeros in the padding.
+ *  f64: [64-byte header][k padded to 32][n padded to 64] doubles, zeros in the padding, then a sum of squares per
+ *  padded column for the distance kinds (`nk_{angulars,euclideans}_{packed,symmetric}_{f32,f64}`, reference
+ *  include/numkong/spatials/serial.h:41-72), which finalise the same dot products in the epilogue.
  */
 #include "dots_gfx950.hpp"
 

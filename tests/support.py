@@ -32,7 +32,7 @@ NARROW_FLOAT_DTYPES = ("e2m3", "e3m2")
 NARROW_INT_DTYPES = ("i4", "u4", "u1")
 NARROW_DTYPES = NARROW_FLOAT_DTYPES + NARROW_INT_DTYPES
 DIMENSIONS_PER_VALUE = {"i4": 2, "u4": 2, "u1": 8}
-WIDE_DTYPES = ("f32", "f64")  # f64 results; the dot-product kinds only
+WIDE_DTYPES = ("f32", "f64")  # f64 results, for the dot products and for the distances
 DISTANCE_DTYPES = ALL_DTYPES + ("e2m3", "e3m2", "i4", "u4")  # the types with the distance kinds (f32 results), packed and symmetric
 # ... and f32 and f64, whose distances are f64
 DISTANCE_OUTPUT = {**{t: np.float32 for t in DISTANCE_DTYPES}, "f32": np.float64, "f64": np.float64}
