@@ -208,6 +208,9 @@ inline bool make_geometry(int dtype, size_t n, size_t k, Geometry &g) {
     int const bits = elem_bits_of(dtype);
     if (!bits) return false;
     if (n > 0x7FFFFFFFull || k > 0x3FFFFFFFull) return false;
+    // e2m3 sums 64 x its products in i32: 60 * 60 * k must stay below 2^31 (the reference sums in f32 and has no
+    // such bound; rows this deep are refused like dimensions beyond 32 bits)
+    if (dtype == kE2M3 && k > 0x7FFFFFFFull / 3600) return false;
     g.elem_bytes = (uint32_t)(bits + 7) / 8, g.packed_bytes = (uint32_t)packed_bytes_of(dtype), g.n = (uint32_t)n, g.k = (uint32_t)k;
     g.k_src_bytes = ((uint64_t)k * bits + 7) / 8; // (sub-byte types: whole bytes, as the reference loads them, cast/serial.h:519-538)
     g.k_bytes = bits < 8 ? g.k_src_bytes * (8 / bits) * g.packed_bytes : (uint64_t)k * g.packed_bytes;

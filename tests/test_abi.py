@@ -53,6 +53,8 @@ def test_packed_size_formula():
             assert nk.dots_packed_size(t, n, k) == 64 + tiles * chunks * 512 + tiles * 256, (t, n, k)
         assert nk.dots_packed_size(t, 0, 0) == 64
         assert nk.dots_packed_size(t, 1 << 40, 8) == 0  # dimensions beyond 32 bits are refused, as the error stub does
+    # e2m3 sums integers 64 times its products in i32: depths where 60 * 60 * k passes 2^31 are refused
+    assert nk.dots_packed_size("e2m3", 8, 596523) > 0 and nk.dots_packed_size("e2m3", 8, 596524) == 0
     # the two wide types keep f64 values k-major: header + 8 bytes x (n padded to 64) x (k padded to 32), and a sum of
     # squares per padded column behind them
     assert nk.dots_packed_size("f32", 100, 70) == nk.dots_packed_size("f64", 100, 70) == 64 + 8 * 128 * 96 + 8 * 128
