@@ -50,6 +50,7 @@ MEASURED_TRAFFIC = {
     ("i8", 8192, 8192, 8192, "symmetric"): 8.9050e8,   # all kernels of one call: pack, tile lists, two product launches
     ("bf16", 8192, 8192, 8192, "symmetric"): 2.3554e9,
     ("i4", 8192, 8192, 8192): 8.1447e8,
+    ("e2m3", 8192, 8192, 8192): 1.1173e9,
     ("u1", 8192, 8192, 8192): 6.1474e8,
     ("f32", 4096, 4096, 4096): 2.0132e9,
     ("f64", 4096, 4096, 4096): 3.8853e9,
