@@ -36,7 +36,7 @@ MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2":
              "i4": "widened to i8, priced against the i8 MFMA peak", "u4": "widened to i8, priced against the i8 MFMA peak",
              "u1": "bits widened to i8 zeros and ones, priced against the i8 MFMA peak",
              "f32": "exact f32 products summed in f64 on the f64 MFMA (78.6 TFLOP/s), four sums per output as in the reference",
-             "f64": "compensated f64 sums on the vector units: about 17 f64 operations per multiply-add, priced as 2"}
+             "f64": "compensated f64 sums on the vector units: 10 f64 instructions per multiply-add, priced as the 2 flops of one"}
 HBM_PEAK = 8000.0
 # HBM-side bytes per launch (L2 <-> fabric) from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --probe`,
 # each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
