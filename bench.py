@@ -200,7 +200,7 @@ def time_gpu(dtype, m, n, k, steps, warmup, metric="dots"):
     return result
 
 
-def cpu_baseline(dtype, m, n, k, budget_rows=2048):
+def cpu_baseline(dtype, m, n, k, budget_rows=8192):
     """The reference's own dots path on the host cores: B packed once, A split into 64-row tiles handed out
     dynamically to one thread per core (python/matrix.c:466-483, python/matrix.h:18), best-dispatch kernel.
     Falls back to this repository's scalar oracle on a smaller sample if the reference build is absent."""
