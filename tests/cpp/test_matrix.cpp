@@ -151,6 +151,44 @@ int main() {
                 if (c[i * n + j] != sum) ok = false;
             }
         expect(ok, "i4 dots_packed: exact against sign-extended nibbles");
+        // distances of the 4-bit type: f32, from the same image
+        std::vector<nk_f32_t> angular(m * n);
+        ok = angulars_packed(a.data(), packed, angular.data(), m, bytes, n * 4);
+        for (std::size_t i = 0; i < m && ok; ++i)
+            for (std::size_t j = 0; j < n; ++j) {
+                double dot = 0, aa = 0, bb = 0;
+                for (std::size_t l = 0; l < bytes; ++l)
+                    for (int high = 0; high < 2; ++high) {
+                        double const x = nibble(a[i * bytes + l], high), y = nibble(b[j * bytes + l], high);
+                        dot += x * y, aa += x * x, bb += y * y;
+                    }
+                double const expected = aa * bb > 0 ? std::fmax(1.0 - dot / std::sqrt(aa * bb), 0.0) : (dot == 0 ? 0.0 : 1.0);
+                if (std::fabs(angular[i * n + j] - expected) > 1e-5) ok = false;
+            }
+        expect(ok, "i4 angulars_packed: within 1e-5 of the f64 formula");
+    }
+
+    { // f32: f64 results for the products and for the distances
+        std::normal_distribution<float> normal;
+        std::vector<nk_f32_t> a(m * k), b(n * k);
+        for (auto &x : a) x = normal(generator);
+        for (auto &x : b) x = normal(generator);
+        auto packed = packed_matrix<f32_t>::try_pack(b.data(), n, k, k * 4);
+        std::vector<nk_f64_t> c(m * n), euclidean(m * n);
+        bool ok = dots_packed(a.data(), packed, c.data(), m, k * 4, n * 8) &&
+                  euclideans_packed(a.data(), packed, euclidean.data(), m, k * 4, n * 8);
+        for (std::size_t i = 0; i < m && ok; ++i)
+            for (std::size_t j = 0; j < n; ++j) {
+                double lanes[4] = {0, 0, 0, 0}, squared = 0; // the reference's four sums by k mod 4
+                for (std::size_t l = 0; l < k; ++l) {
+                    lanes[l & 3] += static_cast<double>(a[i * k + l]) * b[j * k + l];
+                    double const d = static_cast<double>(a[i * k + l]) - b[j * k + l];
+                    squared += d * d;
+                }
+                if (c[i * n + j] != ((lanes[0] + lanes[1]) + lanes[2]) + lanes[3]) ok = false;
+                if (std::fabs(euclidean[i * n + j] - std::sqrt(squared)) > 1e-12 * std::sqrt(squared)) ok = false;
+            }
+        expect(ok, "f32 dots_packed: bit-exact against four f64 sums by k mod 4; euclideans_packed: f64, within 1e-12");
     }
 
     { // symmetric: upper triangle of a row window, the rest left alone
