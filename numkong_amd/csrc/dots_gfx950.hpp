@@ -532,6 +532,7 @@ struct I8 {
     static constexpr int kDtype = kI8;
     static constexpr bool kUnsigned = false;
     static constexpr bool kDistances = true; // the distance kinds are built for this type (NORMS kernels)
+    static constexpr bool kPrewiden = false; // widen A in place, ahead of its LDS write, spread over two k-steps
     /** Sum of the squares of the source values behind one staged chunk (`raw`: as loaded, `wide`: as it goes to LDS). */
     static __device__ __forceinline__ norm_t sumsq(v4i raw, v4i) {
         int sum = 0;
@@ -562,6 +563,7 @@ struct BF16 {
     static constexpr int kDtype = kBF16;
     static constexpr bool kUnsigned = false;
     static constexpr bool kDistances = true;
+    static constexpr bool kPrewiden = false;
     /** The 8 products are exact in f32; their short sum is rounded a few times, the long sum runs in f64. */
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) {
         float sum = 0;
@@ -587,6 +589,7 @@ struct F16 {
     static constexpr int kDtype = kF16;
     static constexpr bool kUnsigned = false;
     static constexpr bool kDistances = true;
+    static constexpr bool kPrewiden = false;
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { // also e4m3 / e5m2, which are f16 by then
         typedef _Float16 v2h __attribute__((ext_vector_type(2)));
         float sum = 0;
@@ -621,6 +624,7 @@ struct E5M2 : F16 {
  *  the dot product, converted to f32 once in the epilogue (one rounding for sums beyond 2^24, none below). */
 struct E2M3 : I8 {
     static constexpr int kDtype = kE2M3;
+    static constexpr bool kPrewiden = true; // 13 operations per dword: too many to sit in front of the LDS writes
     static __device__ __forceinline__ v4i widen(v4i v) {
         v4i out;
 #pragma unroll
@@ -1060,22 +1064,50 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // `s` is the stage the registers hold: the bytes of its chunk that lie past the end of the row are cleared
     // (for whole stages the masks come out as all ones; no branch either way).
     int const a_tail = (int)(uint32_t)g.k_src_bytes - (int)(a_pos * T::kSrcChunk); // bytes of the row from this thread's chunk on, stage 0
-    auto store_a = [&](auto buffer_tag, auto slot_tag, uint32_t s, uint32_t mine) {
-        constexpr int buffer = decltype(buffer_tag)::value, slot = decltype(slot_tag)::value;
-        uint8_t *dst = lds + buffer * kStageLds;
+    // What a stage reads past the end of its row of A must become zero for the float types (the image's zero padding
+    // times a NaN is a NaN), for u8's row sums and for the sums of squares of the distances. The integer products
+    // need no such care: whatever is read there meets zeros of the image.
+    constexpr bool kMaskTail = NORMS || T::kUnsigned || !__is_same(typename T::acc_t, v16i);
+    auto masks_of = [&](uint32_t s, uint32_t (&keep)[(T::kSrcChunk + 3) / 4]) {
         int const left = a_tail - (int)(s * kSrcStage);
-        constexpr int kSrcWords = (T::kSrcChunk + 3) / 4;
-        uint32_t keep[kSrcWords];
 #pragma unroll
-        for (int w = 0; w < kSrcWords; ++w) {
+        for (int w = 0; w < (T::kSrcChunk + 3) / 4; ++w) {
             int const over = left - 4 * w, bytes = over < 0 ? 0 : (over > 4 ? 4 : over);
             keep[w] = bytes == 4 ? 0xFFFFFFFFu : ((1u << (8 * bytes)) - 1u);
         }
+    };
+    // Half of the staged chunks of stage `s`, masked and widened where they are (types with kPrewiden): what
+    // store_a would do right in front of its LDS writes, done a k-step or two earlier among that k-step's MFMAs.
+    auto prewiden = [&](auto slot_tag, uint32_t s, auto half_tag) {
+        constexpr int slot = decltype(slot_tag)::value, half_of = decltype(half_tag)::value;
+        constexpr int kSrcWords = (T::kSrcChunk + 3) / 4;
+        uint32_t keep[kSrcWords];
+        if (kMaskTail) masks_of(s, keep);
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            if (i * 2 / kLoads != half_of) continue;
+            v4i v = a_reg[slot][i];
+            if (kMaskTail) {
+#pragma unroll
+                for (int w = 0; w < kSrcWords; ++w) v[w] &= (int)keep[w];
+            }
+            a_reg[slot][i] = T::widen(v);
+        }
+    };
+    auto store_a = [&](auto buffer_tag, auto slot_tag, uint32_t s, uint32_t mine, auto widened_tag) {
+        constexpr int buffer = decltype(buffer_tag)::value, slot = decltype(slot_tag)::value;
+        constexpr bool widened = decltype(widened_tag)::value != 0; // prewiden has been over these registers
+        uint8_t *dst = lds + buffer * kStageLds;
+        constexpr int kSrcWords = (T::kSrcChunk + 3) / 4;
+        uint32_t keep[kSrcWords];
+        if (!widened && kMaskTail) masks_of(s, keep);
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             v4i v = a_reg[slot][i];
+            if (!widened && kMaskTail) {
 #pragma unroll
-            for (int w = 0; w < kSrcWords; ++w) v[w] &= (int)keep[w];
+                for (int w = 0; w < kSrcWords; ++w) v[w] &= (int)keep[w];
+            }
             // (without a next tile to stage for, what is staged past the end is dropped)
             uint32_t const set = across && !mine ? sums_here ^ (uint32_t)(kLoads * NT) : sums_here;
             v4i const raw = v;
@@ -1084,7 +1116,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 add_row_sum(i, across ? sum : sum * mine, set);
                 v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
             }
-            v4i const wide = T::widen(v);
+            v4i const wide = widened ? v : T::widen(v);
             if (NORMS) {
                 norm_t const squares = T::sumsq(raw, wide);
                 add_row_norm(i, across || mine ? squares : (norm_t)0, set);
@@ -1118,14 +1150,16 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // Scheduling hints for one k-step. Masks: 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write.
     // Fragment reads go one-to-one with the first TM MFMAs; the global loads of the k-step (TN of B
     // and a quarter of A) are spread over the remaining MFMAs; k-step 2 also carries the LDS writes.
-    auto schedule_k_step = [&](auto writes_tag) {
+    auto schedule_k_step = [&](auto writes_tag, auto vector_tag) {
         constexpr bool writes = decltype(writes_tag)::value != 0;
+        constexpr int vector = decltype(vector_tag)::value; // vector operations to put behind every MFMA (0x002)
         constexpr int loads = TN + (kLoads >= 4 ? kLoads / 4 : 1);
         constexpr int rest = TM * (TN - 1);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if constexpr (vector > 0) __builtin_amdgcn_sched_group_barrier(0x002, vector, 0);
         }
         if constexpr (rest == 0) {
             if (writes) __builtin_amdgcn_sched_group_barrier(0x200, kLoads, 0);
@@ -1138,6 +1172,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 if (i * loads / rest != (i + 1) * loads / rest || (loads > rest && i == 0))
                     __builtin_amdgcn_sched_group_barrier(0x020, loads > rest ? loads : 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if constexpr (vector > 0) __builtin_amdgcn_sched_group_barrier(0x002, vector, 0);
             }
             if (writes && kLoads > rest) __builtin_amdgcn_sched_group_barrier(0x200, kLoads - rest, 0);
         }
@@ -1147,6 +1182,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // this one again when nothing follows: loads of valid memory that nobody uses).
     auto stage = [&](auto parity_tag, uint32_t s) {
         constexpr int P = decltype(parity_tag)::value;
+        // vector operations behind each MFMA of the k-steps that widen in place: their share of half the chunks
+        constexpr int kSpread = T::kPrewiden ? (kLoads * 28 + TM * TN - 1) / (TM * TN) : 0;
         bool const wrap2 = s + 2 >= fast, wrap3 = s + 3 >= fast;
         uint32_t const s2 = wrap2 ? s + 2 - fast : s + 2, s3 = wrap3 ? s + 3 - fast : s + 3;
         TileView const &a2 = wrap2 ? nxt : cur, &a3 = wrap3 ? nxt : cur, &b2 = a2;
@@ -1154,28 +1191,31 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
         multiply(slot_c<P>(), slot_c<0>());
         if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<0>()), load_a(a2, s2, slot_c<P>(), slot_c<2>());
-        schedule_k_step(slot_c<0>());
+        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<0>());
+        schedule_k_step(slot_c<0>(), slot_c<kSpread>());
         __builtin_amdgcn_sched_barrier(0);
         if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
         multiply(slot_c<P>(), slot_c<1>());
         if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<1>()), load_a(a2, s2, slot_c<P>(), slot_c<3>());
-        schedule_k_step(slot_c<0>());
+        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<1>());
+        schedule_k_step(slot_c<0>(), slot_c<kSpread>());
         __builtin_amdgcn_sched_barrier(0);
         if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
         multiply(slot_c<P>(), slot_c<2>());
         if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<2>());
         // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
         // at the previous barrier); then its registers start being refilled with A(s+3).
-        if (!(DBG & 8)) store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, s + 1 < fast ? 1u : 0u);
+        if (!(DBG & 8))
+            store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, s + 1 < fast ? 1u : 0u, slot_c<T::kPrewiden ? 1 : 0>());
         if (!(DBG & 1)) load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
-        schedule_k_step(slot_c<1>());
+        schedule_k_step(slot_c<1>(), slot_c<0>());
         __builtin_amdgcn_sched_barrier(0);
         if (!(DBG & 4)) __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         if (!(DBG & 2)) read_frags(slot_c<P ^ 1>(), slot_c<0>(), slot_c<0>());
         multiply(slot_c<P>(), slot_c<3>());
         if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<3>()), load_a(a3, s3, slot_c<P ^ 1>(), slot_c<1>());
-        schedule_k_step(slot_c<0>());
+        schedule_k_step(slot_c<0>(), slot_c<0>());
     };
 
     // Fills the pipeline for a tile: stages 0 and 1 on their way, A(0) in LDS, its first fragments read.
@@ -1187,7 +1227,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         load_a_all(cur, 1, slot_c<1>());
         load_b(cur, 1, slot_c<1>(), slot_c<0>()), load_b(cur, 1, slot_c<1>(), slot_c<1>());
         load_b(cur, 1, slot_c<1>(), slot_c<2>()), load_b(cur, 1, slot_c<1>(), slot_c<3>());
-        store_a(slot_c<0>(), slot_c<0>(), 0u, 1u);
+        store_a(slot_c<0>(), slot_c<0>(), 0u, 1u, slot_c<0>());
         // the first half of A(2), as k-steps 2 and 3 of a stage "-1" would have issued it
         // (with two stages in all it is A(0) again, which nobody uses)
         uint32_t const third = fast > 2 ? 2 : 0;
