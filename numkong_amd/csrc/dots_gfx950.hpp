@@ -893,7 +893,18 @@ __global__ __launch_bounds__(256) void triangle_tiles_kernel(TriangleGrids grids
  *  needs a quarter of the store instructions but writes 32-byte pieces of 32 different rows; it measured
  *  12 % slower on the square shapes and 9 % slower on the retrieval shape.)
  */
-template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, int DBG = 0>
+/** Does a row of A stop short inside a stage's reads, or does the kernel read one stage more than the rows hold (the
+ *  image's depth is padded to an even number of stages)? The types whose arithmetic cares (tail_matters_for) clear such
+ *  bytes on their way into LDS; kernels compiled with WHOLE are for depths that fill an even number of stages exactly
+ *  and leave those masks out of the loop. */
+template <class T, bool NORMS>
+constexpr bool tail_matters_for() {
+    // floats (the image's zero padding times a NaN is a NaN), u8's row sums, the sums of squares of the distances;
+    // the integer products need no care: whatever is read there meets zeros of the image
+    return NORMS || T::kUnsigned || !__is_same(typename T::acc_t, v16i);
+}
+
+template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, int DBG = 0, bool WHOLE = false>
 __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChunked ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
     typedef typename T::acc_t acc_t;
     constexpr int BM = TM * 32;
@@ -1064,10 +1075,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // `s` is the stage the registers hold: the bytes of its chunk that lie past the end of the row are cleared
     // (for whole stages the masks come out as all ones; no branch either way).
     int const a_tail = (int)(uint32_t)g.k_src_bytes - (int)(a_pos * T::kSrcChunk); // bytes of the row from this thread's chunk on, stage 0
-    // What a stage reads past the end of its row of A must become zero for the float types (the image's zero padding
-    // times a NaN is a NaN), for u8's row sums and for the sums of squares of the distances. The integer products
-    // need no such care: whatever is read there meets zeros of the image.
-    constexpr bool kMaskTail = NORMS || T::kUnsigned || !__is_same(typename T::acc_t, v16i);
+    constexpr bool kMaskTail = !WHOLE && tail_matters_for<T, NORMS>();
     auto masks_of = [&](uint32_t s, uint32_t (&keep)[(T::kSrcChunk + 3) / 4]) {
         int const left = a_tail - (int)(s * kSrcStage);
 #pragma unroll
@@ -1533,9 +1541,15 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
     uint32_t const stages = g.k_chunks / kStageChunks;
     bool const across = g.avec >= (T::kSrcChunk < 4 ? T::kSrcChunk : 4) && stages >= 4 && !(g_variant & 1);
     bool const norms = g.metric != 0;
+    // depths that fill an even number of stages exactly: the pipelined kernel without the tail masks
+    bool const whole = across && g.k_src_bytes % (2 * kStageChunks * T::kSrcChunk) == 0;
     void (*kernel)(GemmArgs) = across ? dots_packed_kernel<T, TM, TN, true, false> : dots_packed_kernel<T, TM, TN, false, false>;
+    if constexpr (tail_matters_for<T, false>()) {
+        if (whole) kernel = dots_packed_kernel<T, TM, TN, true, false, 0, true>;
+    }
     if constexpr (T::kDistances) {
         if (norms) kernel = across ? dots_packed_kernel<T, TM, TN, true, true> : dots_packed_kernel<T, TM, TN, false, true>;
+        if (norms && whole) kernel = dots_packed_kernel<T, TM, TN, true, true, 0, true>;
     }
     else if (norms) return hipErrorInvalidValue;
 #ifdef NK_TUNE // timing experiments that leave parts of the loop out (results are wrong on purpose)
@@ -1551,8 +1565,8 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
     }
 #endif
     // Persistent grid: as many workgroups as fit on the device at once (queried once per kernel).
-    static int resident_of[4] = {0, 0, 0, 0};
-    int &resident = resident_of[(across ? 1 : 0) + (norms ? 2 : 0)];
+    static int resident_of[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int &resident = resident_of[(across ? 1 : 0) + (norms ? 2 : 0) + (whole ? 4 : 0)];
     if (!resident) {
         int per_cu = 0, device = 0;
         hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (void const *)kernel, 256, 0);
