@@ -42,17 +42,17 @@ HBM_PEAK = 8000.0
 # each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
 # the summaries are under profiles/. Not re-measured by a plain run: counters need the profiler.
 MEASURED_TRAFFIC = {
-    ("i8", 8192, 8192, 8192): 1.0816e9,
-    ("bf16", 8192, 8192, 8192): 2.4328e9,
-    ("e4m3", 8192, 8192, 8192): 1.8864e9,
-    ("i8", 1024, 1 << 20, 768): 5.5057e9,
-    ("i8", 1024, 1 << 20, 768, "angular"): 5.3857e9,
-    ("i8", 8192, 8192, 8192, "symmetric"): 8.9050e8,   # all kernels of one call: pack, tile lists, two product launches
-    ("bf16", 8192, 8192, 8192, "symmetric"): 2.3554e9,
-    ("i4", 8192, 8192, 8192): 8.1447e8,
+    ("i8", 8192, 8192, 8192): 1.0821e9,
+    ("bf16", 8192, 8192, 8192): 2.5800e9,
+    ("e4m3", 8192, 8192, 8192): 1.8859e9,
+    ("i8", 1024, 1 << 20, 768): 5.4921e9,
+    ("i8", 1024, 1 << 20, 768, "angular"): 5.3914e9,
+    ("i8", 8192, 8192, 8192, "symmetric"): 8.9150e8,   # all kernels of one call: pack, tile lists, two product launches
+    ("bf16", 8192, 8192, 8192, "symmetric"): 2.5219e9,
+    ("i4", 8192, 8192, 8192): 8.1530e8,
     ("e2m3", 8192, 8192, 8192): 1.1173e9,
-    ("u1", 8192, 8192, 8192): 6.1474e8,
-    ("f32", 4096, 4096, 4096): 2.0132e9,
+    ("u1", 8192, 8192, 8192): 6.1481e8,
+    ("f32", 4096, 4096, 4096): 2.0133e9,
     ("f64", 4096, 4096, 4096): 3.8853e9,
 }
 HEADLINE = ("i8", 8192, 8192, 8192)
