@@ -1491,8 +1491,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
 struct TileConfig {
     int tm, tn;
 };
-// Index 0 is "choose for me"; 1.. are explicit.
-constexpr TileConfig kConfigs[] = {{0, 0}, {8, 2}, {4, 2}, {4, 1}, {2, 1}};
+// Index 0 is "choose for me"; 1.. are explicit (5: e2m3 only).
+constexpr TileConfig kConfigs[] = {{0, 0}, {8, 2}, {4, 2}, {4, 1}, {2, 1}, {4, 4}};
 constexpr int kConfigCount = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
 
@@ -1597,6 +1597,9 @@ hipError_t launch_config(GemmArgs &g, hipStream_t stream, TriangleScratch const 
         else return launch_one<T, 8, 2>(g, stream, triangle, slots_only);
     case 2: return launch_one<T, 4, 2>(g, stream, triangle, slots_only);
     case 3: return launch_one<T, 4, 1>(g, stream, triangle, slots_only);
+    case 5:
+        if constexpr (T::kDtype != kE2M3) return hipErrorInvalidValue;
+        else return launch_one<T, 4, 4>(g, stream, triangle, slots_only);
     default: return launch_one<T, 2, 1>(g, stream, triangle, slots_only);
     }
 }
@@ -1623,6 +1626,9 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream, TriangleScratch const *
         // (measured on 1024 x 1,048,576 x 768: 2.17 against 2.33 ms angular, 1.98 against 2.07 ms euclidean).
         if (args.metric != 0 && best < 3 && args.k_chunks / kStageChunks <= 8 && tiles_of(args, 3) >= 256) best = 3;
         if (T::kChunked && best == 1) best = 2; // two accumulator sets do not fit the 256 x 256 tile
+        // e2m3 pays 13 vector operations for every dword of A it stages: a 128 x 512 tile (every wavefront 128 x 128)
+        // stages half as much A per MFMA as 256 x 256 (8192^3: 0.51 against 0.59 ms; for i8 itself the two are equal)
+        if (T::kDtype == kE2M3 && !triangle && args.metric == 0 && first == 1 && tiles_of(args, 5) >= 256) best = 5;
         return best;
     };
     if (chosen_here) config = choose(g, 1);

@@ -241,3 +241,15 @@ def test_symmetric_distances(oracle, dtype, metric):
             vectors[2] = 0
             vectors[9] = vectors[40]
         check_distances(oracle, metric, dtype, vectors, row_start, row_count, 0, f"{dtype} {metric} {count}x{depth} rows {row_start}+{row_count}")
+
+
+def test_e2m3_wide_tile(oracle):
+    """The 128 x 512 tile that large e2m3 products take (tile configuration 5): exact on shapes off its edges (every
+    e2m3 sum below 2^24 / 64 is exact in f32) and equal to the default shape bit for bit."""
+    rng = np.random.default_rng(520)
+    for m, n, k in [(1, 1, 1), (130, 33, 200), (257, 1100, 515), (100, 513, 4100)]:
+        a, b = support.random_matrix(oracle, "e2m3", m, k, rng), support.random_matrix(oracle, "e2m3", n, k, rng)
+        got = gpu_dots("e2m3", a, b, config=5)
+        exact = oracle.decode("e2m3", a).astype(np.float64) @ oracle.decode("e2m3", b).astype(np.float64).T
+        assert np.array_equal(got.astype(np.float64), exact), (m, n, k)
+        assert np.array_equal(got.view(np.uint32), gpu_dots("e2m3", a, b).view(np.uint32))
