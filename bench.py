@@ -50,7 +50,7 @@ MEASURED_TRAFFIC = {
     ("i8", 8192, 8192, 8192, "symmetric"): 8.9150e8,   # all kernels of one call: pack, tile lists, two product launches
     ("bf16", 8192, 8192, 8192, "symmetric"): 2.5219e9,
     ("i4", 8192, 8192, 8192): 8.1530e8,
-    ("e2m3", 8192, 8192, 8192): 1.1173e9,
+    ("e2m3", 8192, 8192, 8192): 1.1190e9,
     ("u1", 8192, 8192, 8192): 6.1481e8,
     ("f32", 4096, 4096, 4096): 2.0133e9,
     ("f64", 4096, 4096, 4096): 3.8853e9,
