@@ -50,15 +50,26 @@
  *      the AND over whole bytes)
  *          include/numkong/cast/serial.h:533-538, 1280-1330, 1418-1470, include/numkong/dot/serial.h:602-800
  *      Pinned bit for bit against nk_cast_serial (all 256 byte values decode; encoder on finite probes incl. every
- *      tie) and nk_dots_packed_<T>_serial / nk_dots_symmetric_<T>_serial; their distance kinds are not restated
- *      (and not built).
+ *      tie) and nk_dots_packed_<T>_serial / nk_dots_symmetric_<T>_serial.
+ *      Distance kinds of e2m3, e3m2, i4, u4 (u1 has none): the finalisers above over these products and the sums of
+ *      squares of include/numkong/reduce/serial.h:323-404 (the 4-bit types count both halves of every byte they
+ *      touch). Sums of squares pinned bit for bit against nk_reduce_moments_<T>_serial; distances against
+ *      nk_{angulars,euclideans}_{packed,symmetric}_<T>_serial: bit for bit for u4, for i4 on non-negative values (the
+ *      reference's distance kernels take their norms from the host-dispatched moments, and its AVX2 i4 moments square
+ *      negative values as unsigned, include/numkong/reduce/haswell.h:3629-3633) and on signed values against the f64
+ *      formulas; the 6-bit floats to the tolerance of the other float types.
  *
- *    - the two wide types, products only (packed and symmetric), f64 results: f32 by four f64 lane sums, f64 by the
+ *    - the two wide types (packed and symmetric), f64 results: f32 by four f64 lane sums, f64 by the
  *      compensated two-lane sum with its compensated fold
  *          include/numkong/dot/serial.h:262-335, include/numkong/scalar/serial.h:128-136, include/numkong/reduce/serial.h:33-48
  *      Pinned bit for bit against nk_dots_packed_{f32,f64}_serial / nk_dots_symmetric_{f32,f64}_serial, and by what
  *      the arithmetic fixes: integer-valued inputs (exact), and for f64 a sum that cancels catastrophically in plain
  *      f64 and comes out right only if the compensation works.
+ *      Their distance kinds: Neumaier-compensated f64 sums of squares (include/numkong/reduce/serial.h:50-92), the f64
+ *      reciprocal square root (bit trick + four Newton steps, include/numkong/scalar/serial.h:35-47) and the finalisers
+ *      of include/numkong/spatial/serial.h:281-302. Sums of squares pinned bit for bit against
+ *      nk_reduce_moments_{f32,f64}_serial; distances against nk_{angulars,euclideans}_{packed,symmetric}_{f32,f64}_serial
+ *      to 16 units of 2^-53 (their norms come from the host-dispatched moments), and against closed forms.
  *
  *  Parity unpinned: the per-column norms of FLOAT types in the serial packed image as stored bytes (the
  *  reference computes them with the host-dispatched nk_reduce_moments_*, whose summation order is not restated
