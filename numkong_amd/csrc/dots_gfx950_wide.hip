@@ -291,9 +291,10 @@ __global__ __launch_bounds__(256) void dots_f64_compensated_kernel(WideArgs g) {
 }
 
 constexpr int kMatrixRows = 128, kMatrixCols = 64; // rows and columns of C per workgroup of the f32 matrix kernel
-constexpr int kMatrixDepth = 16;                     // k per step: four MFMA depths for each of the four sums
-constexpr int kMatrixAStride = kMatrixDepth + 4;     // floats per staged row of A: 16-byte reads of 16 rows spread over all banks
-constexpr int kMatrixBStride = kMatrixCols + 4;      // doubles per staged depth of B
+constexpr int kMatrixDepth = 32;                     // k per step: two groups of four MFMA depths for each of the four sums
+// A row of staged A is 128 bytes of f32, eight 16-byte units; unit u of row r sits at position u ^ (r % 8), so that the
+// eight lanes of an LDS cycle, which read the same unit of eight consecutive rows, or write the eight units of one row,
+// spread over all banks without padding. Two stages of A and of B (f64, [k][column]) fill the 64 KiB exactly.
 
 /**
  *  f32 inputs on the f64 matrix cores. `v_mfma_f64_16x16x4_f64` is, per output, a chain of four fused multiply-adds in
@@ -316,10 +317,12 @@ __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
     typedef float __attribute__((ext_vector_type(4))) f32x4_t;
     typedef __attribute__((address_space(1))) double global_f64_t;
     typedef __attribute__((address_space(1))) uint64_t global_u64_t;
-    __shared__ __attribute__((aligned(16))) float a_lds[2][kMatrixRows][kMatrixAStride];
-    __shared__ __attribute__((aligned(16))) double b_lds[2][kMatrixDepth][kMatrixBStride];
-    __shared__ double row_parts[NORMS ? kMatrixRows : 1][4][2]; // distances: four partial sums of squares per row of A
-    __shared__ double row_norms[NORMS ? kMatrixRows : 1];
+    __shared__ __attribute__((aligned(16))) float a_lds[2][kMatrixRows][kMatrixDepth];
+    __shared__ __attribute__((aligned(16))) double b_lds[2][kMatrixDepth][kMatrixCols];
+    // distances: four partial sums of squares per row of A and their total, in the B stages once the loop is over
+    double(*row_parts)[4][2] = (double(*)[4][2]) & b_lds[0][0][0];
+    double *row_norms = &b_lds[1][0][0];
+    static_assert(sizeof(double) * kMatrixRows * 8 <= sizeof(b_lds) / 2, "the partial sums fit one stage of B");
     uint32_t const tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     uint32_t const row0 = blockIdx.y * kMatrixRows, col0 = blockIdx.x * kMatrixCols;
     // symmetric form: a tile wholly left of the diagonal has nothing to store
@@ -345,67 +348,94 @@ __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = f64x4_t {0, 0, 0, 0};
 
-    // staging: A: thread t brings 4 consecutive k of row t / 4; B: 2 consecutive columns of depth t / 32
-    uint32_t const a_row = tid >> 2, a_k = (tid & 3) * 4;
+    // staging: A: thread t brings 8 consecutive k of row t / 4; B: 2 consecutive columns of depths t / 32 and 16 + t / 32
+    uint32_t const a_row = tid >> 2, a_k = (tid & 3) * 8;
     uint32_t const b_k = tid >> 5, b_col = (tid & 31) * 2;
     uint32_t const a_from = row0 + a_row < g.m ? row0 + a_row : g.m - 1; // (rows past the end repeat the last; never stored)
     uint8_t const *a_source = g.a + (uint64_t)a_from * g.a_stride;
     bool const aligned = ((((uint64_t)g.a) | g.a_stride) & 15) == 0;
-    f32x4_t a_next;
-    f64x2_t b_next;
+    f32x4_t a_next[2];
+    f64x2_t b_next[2];
     CompensatedSum squares; // distances: of this thread's share of its row of A
     auto fetch = [&](uint32_t k0) {
-        uint32_t const at = k0 + a_k;
-        if (aligned && at + 4 <= g.k) a_next = *(f32x4_t const *)(a_source + (uint64_t)at * 4);
-        else {
+        // One decision for the whole wavefront: a per-lane choice between the two ways to load would put a wait for the
+        // loads between them, in front of the MFMAs that are there to cover it.
+        bool const whole = aligned && k0 + kMatrixDepth <= g.k;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) a_next[e] = at + e < g.k ? ((float const *)a_source)[at + e] : 0.f;
+        for (int h = 0; h < 2; ++h) {
+            uint32_t const at = k0 + a_k + 4 * h;
+            if (whole) a_next[h] = *(f32x4_t const *)(a_source + (uint64_t)at * 4);
+            else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) a_next[h][e] = at + e < g.k ? ((float const *)a_source)[at + e] : 0.f;
+            }
+            b_next[h] = *(f64x2_t const *)(g.b + (uint64_t)(k0 + b_k + 16 * h) * g.n_padded + col0 + b_col); // (inside the padded image)
         }
-        if (NORMS) { // four exact squares summed with three roundings of their own small sum, then one compensated addition
-            double const x0 = a_next[0], x1 = a_next[1], x2 = a_next[2], x3 = a_next[3];
-            squares.add(__builtin_fma(x0, x0, __builtin_fma(x1, x1, __builtin_fma(x2, x2, x3 * x3))));
+    };
+    auto stash = [&](int buffer) { // (the first use of what fetch() asked for: the wait for it sits here, behind a group of MFMAs)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            *(f32x4_t *)&a_lds[buffer][a_row][4 * ((a_k / 4 + h) ^ (a_row & 7))] = a_next[h];
+            *(f64x2_t *)&b_lds[buffer][b_k + 16 * h][b_col] = b_next[h];
+            if (NORMS) { // four exact squares summed with three roundings of their own small sum, then one compensated addition
+                double const x0 = a_next[h][0], x1 = a_next[h][1], x2 = a_next[h][2], x3 = a_next[h][3];
+                squares.add(__builtin_fma(x0, x0, __builtin_fma(x1, x1, __builtin_fma(x2, x2, x3 * x3))));
+            }
         }
-        b_next = *(f64x2_t const *)(g.b + (uint64_t)(k0 + b_k) * g.n_padded + col0 + b_col); // (inside the padded image)
     };
-    auto stash = [&](int buffer) {
-        *(f32x4_t *)&a_lds[buffer][a_row][a_k] = a_next;
-        *(f64x2_t *)&b_lds[buffer][b_k][b_col] = b_next;
+    struct Operands {
+        double a[2][4], b[2][4]; // [row or column block][sum r]
     };
-
-    uint32_t const depth = (g.k + kMatrixDepth - 1) & ~(uint32_t)(kMatrixDepth - 1); // (the image is padded to 32)
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    int buffer = 0;
-    for (uint32_t k0 = 0; k0 < depth; k0 += kMatrixDepth) {
-        bool const more = k0 + kMatrixDepth < depth;
-        if (more) fetch(k0 + kMatrixDepth);
-        double a_operand[2][4], b_operand[2][4];
+    auto read_operands = [&](int buffer, int group, Operands &operands) { // 16 depths: 16 group + r + 4 (lane / 16)
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            f32x4_t const quad = *(f32x4_t const *)&a_lds[buffer][wave_row + 16 * i + in_block][4 * depth_group];
+            uint32_t const row = wave_row + 16 * i + in_block;
+            f32x4_t const quad = *(f32x4_t const *)&a_lds[buffer][row][4 * ((4 * group + depth_group) ^ (row & 7))];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) a_operand[i][r] = (double)quad[r];
+            for (int r = 0; r < 4; ++r) operands.a[i][r] = (double)quad[r];
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) b_operand[j][r] = b_lds[buffer][r + 4 * depth_group][wave_col + 16 * j + in_block];
+            for (int r = 0; r < 4; ++r)
+                operands.b[j][r] = b_lds[buffer][16 * group + r + 4 * depth_group][wave_col + 16 * j + in_block];
+    };
+    auto multiply = [&](Operands const &operands) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    acc[i][j][r] = __builtin_amdgcn_mfma_f64_16x16x4f64(a_operand[i][r], b_operand[j][r], acc[i][j][r], 0, 0, 0);
+                    acc[i][j][r] = __builtin_amdgcn_mfma_f64_16x16x4f64(operands.a[i][r], operands.b[j][r], acc[i][j][r], 0, 0, 0);
+    };
+
+    uint32_t const depth = (g.k + kMatrixDepth - 1) & ~(uint32_t)(kMatrixDepth - 1); // (the image is padded to 32)
+    // One barrier per step, in the middle of its MFMAs: the first half's operands were read behind the previous barrier,
+    // the second half's before this one, so every read of a stage precedes the barrier that lets the next writes into it,
+    // and no wave waits on LDS with the matrix pipe idle.
+    static_assert(kMatrixDepth == 32, "two groups of 16 depths per step");
+    Operands first, second;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    read_operands(0, 0, first);
+    int buffer = 0;
+    for (uint32_t k0 = 0; k0 < depth; k0 += kMatrixDepth) {
+        bool const more = k0 + kMatrixDepth < depth;
+        if (more) fetch(k0 + kMatrixDepth);
+        read_operands(buffer, 1, second);
+        multiply(first);
         if (more) stash(buffer ^ 1);
         __syncthreads();
+        if (more) read_operands(buffer ^ 1, 0, first);
+        multiply(second);
         buffer ^= 1;
     }
 
     double column_norm[2];
     if (NORMS) {
-        row_parts[a_row][tid & 3][0] = squares.sum, row_parts[a_row][tid & 3][1] = squares.lost;
+        row_parts[a_row][tid & 3][0] = squares.sum, row_parts[a_row][tid & 3][1] = squares.lost; // (no read of a stage follows the loop's last barrier)
         __syncthreads();
         if (tid < kMatrixRows) {
             CompensatedSum total;
