@@ -21,6 +21,7 @@
  *  padded column for the distance kinds (`nk_{angulars,euclideans}_{packed,symmetric}_{f32,f64}`, reference
  *  include/numkong/spatials/serial.h:41-72), which finalise the same dot products in the epilogue.
  */
+#include <type_traits>
 #include "dots_gfx950.hpp"
 
 // Every floating-point operation in this file rounds on its own (the compensated sums depend on it; the fused
@@ -306,9 +307,11 @@ constexpr int kMatrixDepth = 32;                     // k per step: two groups o
  *  reference does, and four instructions (r = 0..3) consume 16 depths. Zero padding past the last depth adds products
  *  of +0, which leave a sum that started at +0 unchanged (such a sum is never -0).
  *
- *  512 threads, 8 wavefronts as 4 x 2, each 32 x 32 outputs = 2 x 2 blocks x 4 sums = 128 accumulator registers; two
- *  wavefronts per SIMD cover each other's LDS waits. A is staged as f32, [row][k] so that one 16-byte read gives a
- *  lane the four operands (r = 0..3) of its row and depth group; B comes from the k-major f64 image into [k][column].
+ *  512 threads, 8 wavefronts as 4 x 2, each 32 x 32 outputs = 2 x 2 blocks x 4 sums = 128 accumulator registers, two
+ *  wavefronts per SIMD. A is staged as f32, [row][k] so that one 16-byte read gives a lane the four operands
+ *  (r = 0..3) of its row and depth group, and widened where it is multiplied; B comes from the k-major f64 image into
+ *  [k][column]. A step is 32 depths = 32 MFMAs per wavefront; loads from memory are asked for a whole step before the
+ *  stash that takes them, and the stash, the barrier and the reads of LDS sit between groups of MFMAs.
  */
 template <bool NORMS>
 __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
@@ -357,10 +360,10 @@ __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
     f32x4_t a_next[2];
     f64x2_t b_next[2];
     CompensatedSum squares; // distances: of this thread's share of its row of A
-    auto fetch = [&](uint32_t k0) {
-        // One decision for the whole wavefront: a per-lane choice between the two ways to load would put a wait for the
-        // loads between them, in front of the MFMAs that are there to cover it.
-        bool const whole = aligned && k0 + kMatrixDepth <= g.k;
+    // `whole`: the step lies inside the rows of A and they can be read 16 bytes at a time. It is a compile-time choice, one
+    // loop for each: where both ways to load sit in one loop, waits for the loads come between them, in front of the MFMAs
+    // that are there to cover them.
+    auto fetch = [&](uint32_t k0, auto whole) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             uint32_t const at = k0 + a_k + 4 * h;
@@ -384,15 +387,14 @@ __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
         }
     };
     struct Operands {
-        double a[2][4], b[2][4]; // [row or column block][sum r]
+        f32x4_t a[2];   // [row block]: as staged, widened where it is multiplied: nothing between two groups of MFMAs waits on LDS
+        double b[2][4]; // [column block][sum r]
     };
     auto read_operands = [&](int buffer, int group, Operands &operands) { // 16 depths: 16 group + r + 4 (lane / 16)
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             uint32_t const row = wave_row + 16 * i + in_block;
-            f32x4_t const quad = *(f32x4_t const *)&a_lds[buffer][row][4 * ((4 * group + depth_group) ^ (row & 7))];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) operands.a[i][r] = (double)quad[r];
+            operands.a[i] = *(f32x4_t const *)&a_lds[buffer][row][4 * ((4 * group + depth_group) ^ (row & 7))];
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j)
@@ -400,38 +402,58 @@ __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
             for (int r = 0; r < 4; ++r)
                 operands.b[j][r] = b_lds[buffer][16 * group + r + 4 * depth_group][wave_col + 16 * j + in_block];
     };
-    auto multiply = [&](Operands const &operands) {
+    auto multiply = [&](Operands const &operands, int from, int to) { // sums `from` up to `to`, 4 MFMAs each
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+        for (int r = from; r < to; ++r)
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    acc[i][j][r] = __builtin_amdgcn_mfma_f64_16x16x4f64(operands.a[i][r], operands.b[j][r], acc[i][j][r], 0, 0, 0);
+                    acc[i][j][r] = __builtin_amdgcn_mfma_f64_16x16x4f64((double)operands.a[i][r], operands.b[j][r], acc[i][j][r], 0, 0, 0);
     };
 
     uint32_t const depth = (g.k + kMatrixDepth - 1) & ~(uint32_t)(kMatrixDepth - 1); // (the image is padded to 32)
-    // One barrier per step, in the middle of its MFMAs: the first half's operands were read behind the previous barrier,
-    // the second half's before this one, so every read of a stage precedes the barrier that lets the next writes into it,
+    // One barrier per step, in the middle of its MFMAs: the first group's operands were read behind the previous barrier,
+    // the second group's before this one, so every read of a stage precedes the barrier that lets the next writes into it,
     // and no wave waits on LDS with the matrix pipe idle.
     static_assert(kMatrixDepth == 32, "two groups of 16 depths per step");
     Operands first, second;
-    fetch(0);
+    std::false_type const piecewise;
+    std::true_type const whole;
+    fetch(0, piecewise);
     stash(0);
+    if (kMatrixDepth < depth) fetch(kMatrixDepth, piecewise);
     __syncthreads();
     read_operands(0, 0, first);
     int buffer = 0;
-    for (uint32_t k0 = 0; k0 < depth; k0 += kMatrixDepth) {
-        bool const more = k0 + kMatrixDepth < depth;
-        if (more) fetch(k0 + kMatrixDepth);
+    // One step: 32 MFMAs, and between them, where none of it holds the matrix pipe up: the stash of the step after this one
+    // (its stage was last read before the previous barrier), the request for the step after that, the barrier, and the
+    // reads of LDS, each asked for at least 8 MFMAs before its use. The scheduler is held to this order.
+    auto step = [&](uint32_t k0, auto whole) { // (a whole step: neither the last nor the one before it)
+        bool const more = whole || k0 + kMatrixDepth < depth;
         read_operands(buffer, 1, second);
-        multiply(first);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(first, 0, 4);
+        __builtin_amdgcn_sched_barrier(0);
         if (more) stash(buffer ^ 1);
-        __syncthreads();
+        if (whole || k0 + 2 * kMatrixDepth < depth) fetch(k0 + 2 * kMatrixDepth, whole); // a whole step ahead of its stash()
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(second, 0, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        // a barrier that orders LDS only: __syncthreads() would also wait for the loads just asked for
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
         if (more) read_operands(buffer ^ 1, 0, first);
-        multiply(second);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(second, 2, 4);
+        __builtin_amdgcn_sched_barrier(0);
         buffer ^= 1;
-    }
+    };
+    uint32_t k0 = 0;
+    if (aligned)
+        for (; k0 + 3 * kMatrixDepth <= g.k; k0 += kMatrixDepth) step(k0, whole);
+    for (; k0 < depth; k0 += kMatrixDepth) step(k0, piecewise);
 
     double column_norm[2];
     if (NORMS) {
