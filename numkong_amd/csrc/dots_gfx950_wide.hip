@@ -286,7 +286,7 @@ __global__ __launch_bounds__(256) void dots_f64_compensated_kernel(WideArgs g) {
                 if (g.tri_mask && row + g.tri_shift == col) result = 0; // a vector and itself: exactly 0
             }
             if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col)
-                *(global_f64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8) = result;
+                __builtin_nontemporal_store(result, (global_f64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8));
         }
     }
 }
@@ -488,7 +488,7 @@ __global__ __launch_bounds__(512) void dots_f32_matrix_kernel(WideArgs g) {
                     if (g.tri_mask && row + g.tri_shift == col) result = 0; // a vector and itself: exactly 0
                 }
                 if (row < g.m && col < g.n && ((row + g.tri_shift) & g.tri_mask) <= col)
-                    *(global_f64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8) = result;
+                    __builtin_nontemporal_store(result, (global_f64_t *)(g.c + (uint64_t)row * g.c_stride + (uint64_t)col * 8));
             }
         }
 }
