@@ -42,16 +42,16 @@ HBM_PEAK = 8000.0
 # each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
 # the summaries are under profiles/. Not re-measured by a plain run: counters need the profiler.
 MEASURED_TRAFFIC = {
-    ("i8", 8192, 8192, 8192): 1.0821e9,
-    ("bf16", 8192, 8192, 8192): 2.5800e9,
-    ("e4m3", 8192, 8192, 8192): 1.8859e9,
-    ("i8", 1024, 1 << 20, 768): 5.4921e9,
-    ("i8", 1024, 1 << 20, 768, "angular"): 5.3914e9,
-    ("i8", 8192, 8192, 8192, "symmetric"): 8.9150e8,   # all kernels of one call: pack, tile lists, two product launches
-    ("bf16", 8192, 8192, 8192, "symmetric"): 2.5219e9,
-    ("i4", 8192, 8192, 8192): 8.1530e8,
-    ("e2m3", 8192, 8192, 8192): 1.1190e9,
-    ("u1", 8192, 8192, 8192): 6.1481e8,
+    ("i8", 8192, 8192, 8192): 1.0816e9,
+    ("bf16", 8192, 8192, 8192): 2.4588e9,
+    ("e4m3", 8192, 8192, 8192): 1.8833e9,
+    ("i8", 1024, 1 << 20, 768): 5.1137e9,
+    ("i8", 1024, 1 << 20, 768, "angular"): 5.1117e9,
+    ("i8", 8192, 8192, 8192, "symmetric"): 8.8783e8,   # all kernels of one call: pack, tile lists, two product launches
+    ("bf16", 8192, 8192, 8192, "symmetric"): 2.4161e9,
+    ("i4", 8192, 8192, 8192): 8.1106e8,
+    ("e2m3", 8192, 8192, 8192): 1.1188e9,
+    ("u1", 8192, 8192, 8192): 6.0883e8,
     ("f32", 4096, 4096, 4096): 2.0133e9,
     ("f64", 4096, 4096, 4096): 3.8853e9,
 }
