@@ -141,6 +141,45 @@ def time_symmetric(dtype, n, k, steps, warmup, metric):
     return out
 
 
+PACKS = [("i8", 8192, 8192), ("bf16", 8192, 8192), ("i8", 1 << 20, 768), ("f32", 4096, 4096)]
+
+
+def time_pack(dtype, n, k, steps, warmup):
+    """nk_dots_pack alone (every kernel it launches): B read once, its image written once, so HBM bounds it."""
+    import torch
+
+    import numkong_amd as nk
+    from numkong_amd import api
+
+    lib = nk.library()
+    b = make_operands(dtype, 1, n, k)[1]
+    size = api.dots_packed_size(dtype, n, k)
+    image = torch.empty(size, dtype=torch.uint8, device="cuda:0")
+    code, row_bytes = api.DTYPES[dtype][0], b.shape[1] * b.element_size()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        if lib.nk_amd_dots_pack_async(code, b.data_ptr(), n, k, row_bytes, image.data_ptr(), stream):
+            raise RuntimeError(lib.nk_hip_last_error().decode())
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record()
+    for _ in range(steps):
+        step()
+    end.record()
+    torch.cuda.synchronize()
+    device_ms = begin.elapsed_time(end) / steps
+    algorithmic = n * row_bytes + size
+    del b, image
+    torch.cuda.empty_cache()
+    return {"kernel_ms": device_ms, "roofline": {"bound": "hbm", "achieved": algorithmic / (device_ms * 1e-3) / 1e9, "peak": HBM_PEAK,
+                                                 "unit": "GB/s", "frac": algorithmic / (device_ms * 1e-3) / 1e9 / HBM_PEAK, "traffic": None,
+                                                 "note": f"{n * row_bytes} bytes of B read + {size} bytes of image written"}}
+
+
 def time_gpu(dtype, m, n, k, steps, warmup, metric="dots"):
     import torch
 
@@ -316,6 +355,8 @@ def main():
             name = f"{dtype}_{on}x{ok}_{metric}" if metric in SYMMETRIC_KINDS else f"{dtype}_{om}x{on}x{ok}" + ("" if metric == "dots" else "_" + metric)
             line["others"][name] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"],
                                                          "roofline": r["roofline"]}
+        for dtype, on, ok in PACKS:
+            line["others"][f"pack_{dtype}_{on}x{ok}"] = time_pack(dtype, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2))
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.dtype, m, n, k)
     print(json.dumps(line))
