@@ -115,6 +115,24 @@ def test_deep_rows(oracle, dtype, metric):
     assert_distance_gate(oracle, metric, dtype, a, b, gpu_distances(metric, dtype, a, b), f"{dtype} {metric} deep")
 
 
+@pytest.mark.parametrize("metric", METRICS)
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_wide_magnitudes(oracle, dtype, metric):
+    """Log-normal magnitudes with random signs, and rows scaled apart by powers of two: the sums of squares add terms
+    many binades apart (bf16 takes the short sum of 8 squares with the two-element dot instruction)."""
+    rng = np.random.default_rng(77)
+    for m, n, k in [(40, 70, 777), (64, 96, 4096)]:
+        a, b = finite_inputs(oracle, dtype, m, k, rng, "lognormal"), finite_inputs(oracle, dtype, n, k, rng, "lognormal")
+        if dtype == "bf16":  # whole rows moved by 2^-20 .. 2^20 through the exponent field
+            for matrix in (a, b):
+                shift = rng.integers(-20, 21, size=matrix.shape[0]).astype(np.int32)
+                bits = matrix.view(np.uint16).astype(np.int32)
+                moved = np.clip(((bits >> 7) & 0xFF) + shift[:, None], 1, 254)
+                matrix.view(np.uint16)[:] = np.where((bits & 0x7FFF) == 0, bits, (bits & 0x807F) | (moved << 7)).astype(np.uint16)
+        got = gpu_distances(metric, dtype, a, b)
+        assert_distance_gate(oracle, metric, dtype, a, b, got, f"{dtype} {metric} {m}x{n}x{k} wide magnitudes")
+
+
 @pytest.mark.parametrize("name", sorted(f for f in os.listdir(support.GOLDEN_DIR) if f.startswith("spatials_")))
 def test_golden_vectors(oracle, name):
     """Inputs and serial-kernel outputs recorded from the reference library."""
