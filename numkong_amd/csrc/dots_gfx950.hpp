@@ -720,7 +720,10 @@ __device__ __forceinline__ uint32_t distance_from_dot(uint32_t dot_bits, float q
         float root = __builtin_amdgcn_rsqf(product);
         float const residual = __builtin_fmaf(-(product * root), root, 1.0f);
         root = __builtin_fmaf(root * 0.5f, residual, root);
-        float const unclipped = __builtin_fmaxf(__builtin_fmaf(-dot, root, 1.0f), 0.0f);
+        float unclipped = __builtin_fmaxf(__builtin_fmaf(-dot, root, 1.0f), 0.0f);
+        // Where the dot product squared is the product of the norms exactly (one non-zero term, values of a few bits),
+        // a division by a correctly rounded square root gives a cosine of exactly 1 or -1, and so does this.
+        if (__builtin_fmaf(dot, dot, -product) == 0.0f) unclipped = dot > 0 ? 0.0f : 2.0f;
         result = product > 0 ? unclipped : (dot == 0 ? 0.0f : 1.0f);
     }
     else {

@@ -5,7 +5,10 @@ oracle's restatement of the serial kernels. Integers and the two wide types bit 
 gate of tests/test_dots_gpu.py (mean error against the f64 truth at most twice the serial kernel's, NaN / Inf masks
 identical). The shapes straddle every tile edge and every path through the kernels: the pipelined loop with and
 without tail masks, the guarded loop for rows that are not dword-aligned, depths from 1 to a few stages.
+`NK_RANDOM_CASES` (default 10 per type) and `NK_RANDOM_SEED` (default 7000) widen or move the sample.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -34,8 +37,8 @@ def embedded(oracle, dtype, rows, cols, rng, pad, offset):
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES + NARROW_DTYPES + WIDE_DTYPES)
 def test_random_shapes_strides_and_offsets(oracle, dtype):
-    rng = np.random.default_rng(7000 + sorted(api.DTYPES).index(dtype))
-    for case in range(10):
+    rng = np.random.default_rng(int(os.environ.get("NK_RANDOM_SEED", "7000")) + sorted(api.DTYPES).index(dtype))
+    for case in range(int(os.environ.get("NK_RANDOM_CASES", "10"))):
         m, n = int(rng.integers(1, 300)), int(rng.integers(1, 700))
         cols = int(rng.choice([int(rng.integers(1, 40)), int(rng.integers(40, 1100)), 64 * int(rng.integers(1, 17))]))
         pad_a, pad_b = int(rng.integers(0, 9)), int(rng.integers(0, 9))
@@ -52,3 +55,33 @@ def test_random_shapes_strides_and_offsets(oracle, dtype):
         else:
             truth, magnitude = oracle.truth(dtype, a, b)
             assert_float_gate(dtype, got, serial, truth, magnitude, where, best_dispatch(dtype, a, b))
+
+
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", ALL_DTYPES + WIDE_DTYPES)
+def test_random_distances_strides_and_offsets(oracle, dtype, metric):
+    """The packed distances (`nk_angulars_packed_<T>`, `nk_euclideans_packed_<T>`, reference
+    include/numkong/spatials.h:139-266) over the same kind of embedded operands: the six 8- and 16-bit types through
+    the gate of tests/test_spatials_gpu.py, f32 and f64 within 16 units of 2^-53 of the serial restatement."""
+    from tests.test_spatials_gpu import GPU_CALL, assert_distance_gate
+
+    rng = np.random.default_rng(int(os.environ.get("NK_RANDOM_SEED", "7000")) + 100 + sorted(api.DTYPES).index(dtype))
+    for case in range(max(1, int(os.environ.get("NK_RANDOM_CASES", "10")) // 2)):
+        m, n = int(rng.integers(1, 300)), int(rng.integers(1, 400))
+        cols = int(rng.choice([int(rng.integers(1, 40)), int(rng.integers(40, 1100)), 64 * int(rng.integers(1, 17))]))
+        pad_a, pad_b = int(rng.integers(0, 9)), int(rng.integers(0, 9))
+        off_a, off_b = int(rng.integers(0, 5)), int(rng.integers(0, 5))
+        a, ga = embedded(oracle, dtype, m, cols, rng, pad_a, off_a)
+        b, gb = embedded(oracle, dtype, n, cols, rng, pad_b, off_b)
+        if dtype == "e5m2":  # the reference-rule encoder overflows to Inf: keep the distances finite
+            keep = lambda x: np.where((x & 0x7F) > 0x7B, (x & 0x80) | 0x7B, x).astype(x.dtype)
+            a, b = keep(a), keep(b)
+            ga, gb = to_gpu(np.pad(a, ((0, 0), (off_a, pad_a))))[:, off_a:off_a + cols], to_gpu(np.pad(b, ((0, 0), (off_b, pad_b))))[:, off_b:off_b + cols]
+        where = f"{dtype} {metric} case {case}: {m}x{n}x{cols} pads {pad_a},{pad_b} offsets {off_a},{off_b}"
+        got = GPU_CALL[metric](ga, nk.dots_pack(gb, dtype)).cpu().numpy()
+        if dtype in WIDE_DTYPES:
+            serial = oracle.spatials_packed(metric, dtype, a, b)
+            norms = oracle.row_sumsq(dtype, a)[:, None] + oracle.row_sumsq(dtype, b)[None, :]
+            assert got.dtype == np.float64 and support.wide_distances_agree(metric, got, serial, norms), where
+        else:
+            assert_distance_gate(oracle, metric, dtype, a, b, got, where)
