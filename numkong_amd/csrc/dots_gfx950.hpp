@@ -457,7 +457,7 @@ __global__ __launch_bounds__(256) void column_terms_kernel(uint8_t const *__rest
     int sum = 0;
     uint32_t squares = 0;
     double squares_f64 = 0;
-    for (uint32_t c = first; c < k_chunks; c += 8) {
+    auto take = [&](uint32_t c) {
         v4i const v = *(v4i const *)(base + (uint64_t)c * kTileChunkBytes);
         if (KIND == 0) {
 #pragma unroll
@@ -471,6 +471,13 @@ __global__ __launch_bounds__(256) void column_terms_kernel(uint8_t const *__rest
             }
         }
         else { squares_f64 += chunk_sumsq_f64<KIND == 2>(v); }
+    };
+    if (KIND < 2) { // four loads in flight per lane (i8 8192 x 8192: the whole pack 42 -> 32 us); the f64 chain of the floats gains nothing from it
+#pragma unroll 4
+        for (uint32_t c = first; c < k_chunks; c += 8) take(c);
+    }
+    else {
+        for (uint32_t c = first; c < k_chunks; c += 8) take(c);
     }
     part_sum[first][row] = sum, part_squares[first][row] = squares, part_f64[first][row] = squares_f64;
     __syncthreads();
