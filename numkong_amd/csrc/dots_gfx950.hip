@@ -161,7 +161,7 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
             auto kernel = dtype == kI8 || dtype == kI4 || dtype == kU4 || dtype == kU1 || dtype == kE2M3
                               ? column_terms_kernel<0>
                               : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
-            hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(256), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);
+            hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(32 * kColumnParts), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);
         }
         else {
             uint64_t const count = 2 * (uint64_t)g.n_tiles * kTileRows; // both arrays, back to back

@@ -442,17 +442,19 @@ __device__ __forceinline__ double chunk_sumsq_f64(v4i v) {
  *  the row, mod 2^32; zero for the other types) and the column's sum of squares, which the angular and
  *  euclidean products need (reference: the norms behind the packed rows, dots/serial.h:326-332): exact mod
  *  2^32 for the integer types, accumulated in f64 and rounded once to f32 for the float types.
- *  Four wavefronts per tile: lane l of wavefront w owns row l % 32 and every eighth chunk starting at 2 w + l / 32.
+ *  Sixteen wavefronts per tile (a tile is all the parallelism a workgroup has, and 8192 rows are only 256 tiles):
+ *  lane l of wavefront w owns row l % 32 and every 32nd chunk starting at 2 w + l / 32.
  *  KIND: 0 i8, 1 u8, 2 bf16, 3 f16 (and fp8, stored widened to f16).
  */
+constexpr int kColumnParts = 32; // 32-lane groups of a workgroup of column_terms_kernel, each with a share of the chunks
 template <int KIND>
-__global__ __launch_bounds__(256) void column_terms_kernel(uint8_t const *__restrict__ data, uint32_t k_chunks, uint32_t k,
+__global__ __launch_bounds__(32 * kColumnParts) void column_terms_kernel(uint8_t const *__restrict__ data, uint32_t k_chunks, uint32_t k,
                                                            uint32_t *__restrict__ sums, uint32_t *__restrict__ norms) {
-    __shared__ int part_sum[8][32];
-    __shared__ uint32_t part_squares[8][32];
-    __shared__ double part_f64[8][32];
+    __shared__ int part_sum[kColumnParts][32];
+    __shared__ uint32_t part_squares[kColumnParts][32];
+    __shared__ double part_f64[kColumnParts][32];
     uint32_t const tile = blockIdx.x;
-    uint32_t const first = threadIdx.x >> 5, row = threadIdx.x & 31; // chunk residue mod 8, row of the tile
+    uint32_t const first = threadIdx.x >> 5, row = threadIdx.x & 31; // chunk residue mod 32, row of the tile
     uint8_t const *base = data + (uint64_t)tile * k_chunks * kTileChunkBytes + row * kChunkBytes;
     int sum = 0;
     uint32_t squares = 0;
@@ -474,17 +476,17 @@ __global__ __launch_bounds__(256) void column_terms_kernel(uint8_t const *__rest
     };
     if (KIND < 2) { // four loads in flight per lane (i8 8192 x 8192: the whole pack 42 -> 32 us); the f64 chain of the floats gains nothing from it
 #pragma unroll 4
-        for (uint32_t c = first; c < k_chunks; c += 8) take(c);
+        for (uint32_t c = first; c < k_chunks; c += kColumnParts) take(c);
     }
     else {
-        for (uint32_t c = first; c < k_chunks; c += 8) take(c);
+        for (uint32_t c = first; c < k_chunks; c += kColumnParts) take(c);
     }
     part_sum[first][row] = sum, part_squares[first][row] = squares, part_f64[first][row] = squares_f64;
     __syncthreads();
     if (threadIdx.x < 32) {
         sum = 0, squares = 0, squares_f64 = 0;
 #pragma unroll
-        for (int part = 0; part < 8; ++part) sum += part_sum[part][row], squares += part_squares[part][row], squares_f64 += part_f64[part][row];
+        for (int part = 0; part < kColumnParts; ++part) sum += part_sum[part][row], squares += part_squares[part][row], squares_f64 += part_f64[part][row];
         // u8 is stored as b - 128 (and its padding as 0): sum(b^2) = sum((b - 128)^2) + 256 * sum(b - 128) + 128^2 * k
         if (KIND == 1) squares += 256u * (uint32_t)sum + 16384u * k;
         sums[(uint64_t)tile * kTileRows + row] = (uint32_t)sum * 128u;
