@@ -1,12 +1,18 @@
 """Throughput of the packed batched-dots path on one MI355X, with its roofline and a CPU baseline.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype i8] [--shape M N K] [--no-others] [--no-cpu]
+                    [--no-vendor] [--no-ceiling]
 
 One "step" is one packed product C = A * B^T over one synthetic batch (B is packed once, before the timed
 region, as the reference's own benchmark does: bench/bench.hpp:238-255). The headline workload is the
 i8 -> i32 product at M = N = K = 8192; bf16 and e4m3 at the same shape and the HBM-bound retrieval shape
 (1024 queries x 1,048,576 vectors x 768) are measured the same way and reported under "others".
 gso/s = 2*M*N*K / seconds / 1e9 (bench/bench.hpp:257). All operands are resident in HBM before timing.
+Every step sits between two events of its own on the launch stream: `kernel_ms` is the mean over the timed region,
+`kernel_ms_median` and `kernel_ms_min` come from the per-step pairs (include/numkong/dots/README.md:127-135 quotes
+medians). `others` also holds, measured in the same process on the same box: the vendor library's GEMM on the same
+operands (`vendor_*`: torch._int_mm / torch.matmul, which run hipBLASLt; timing only) and the rate an MFMA-only loop
+sustains (`mfma_ceiling`, numkong_amd/lib/mfma_probes), so that a reader can tell the kernel from the part.
 
 The symmetric kinds (`--metric symmetric`, `symmetric-angular`, `symmetric-euclidean`; N vectors of depth K, M is
 ignored) time the whole call as the reference's benchmark does (bench/bench.hpp:397-438): packing the vectors,
@@ -29,9 +35,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 # MI355X published dense peaks, in T(FL)OP/s, for the MFMA the dtype runs on; HBM3E in GB/s.
-MFMA_PEAK = {"i8": 5000.0, "u8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "e4m3": 2500.0, "e5m2": 2500.0,
+MFMA_PEAK = {"i8": 5000.0, "u8": 5000.0, "bf16": 2500.0, "f16": 2500.0, "e4m3": 5000.0, "e5m2": 5000.0,
              "e2m3": 5000.0, "e3m2": 2500.0, "i4": 5000.0, "u4": 5000.0, "u1": 5000.0, "f32": 78.6, "f64": 78.6}
-MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2": "widened to f16, priced against the f16 MFMA peak",
+F16_ROUTE = ("e4m3", "e5m2")  # run widened to f16 on the f16 MFMA (2500): `frac` is against the fp8 peak, `frac_f16` against the instruction's
+MFMA_NOTE = {"e4m3": "widened to f16 (the fp8 MFMA keeps 14 bits of a lane's sums): frac is against the fp8 peak of 5000, frac_f16 against the f16 MFMA it runs on",
+             "e5m2": "widened to f16 (the fp8 MFMA keeps 14 bits of a lane's sums): frac is against the fp8 peak of 5000, frac_f16 against the f16 MFMA it runs on",
              "e2m3": "as i8 values eight times as large (exact), priced against the i8 MFMA peak", "e3m2": "widened to f16, priced against the f16 MFMA peak",
              "i4": "widened to i8, priced against the i8 MFMA peak", "u4": "widened to i8, priced against the i8 MFMA peak",
              "u1": "bits widened to i8 zeros and ones, priced against the i8 MFMA peak",
@@ -40,34 +48,38 @@ MFMA_NOTE = {"e4m3": "widened to f16, priced against the f16 MFMA peak", "e5m2":
 HBM_PEAK = 8000.0
 # HBM-side bytes per launch (L2 <-> fabric) from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --probe`,
 # each scaled by what the same counter reads for a 1 GiB elementwise kernel (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
-# the summaries are under profiles/. Not re-measured by a plain run: counters need the profiler.
-MEASURED_TRAFFIC = {
-    ("i8", 8192, 8192, 8192): 1.0817e9,
-    ("bf16", 8192, 8192, 8192): 2.5718e9,
-    ("e4m3", 8192, 8192, 8192): 1.8833e9,
-    ("i8", 1024, 1 << 20, 768): 5.1129e9,
-    ("i8", 1024, 1 << 20, 768, "angular"): 5.1118e9,
-    ("i8", 8192, 8192, 8192, "symmetric"): 8.8783e8,   # all kernels of one call: pack, tile lists, two product launches
-    ("bf16", 8192, 8192, 8192, "symmetric"): 2.4161e9,
-    ("i4", 8192, 8192, 8192): 8.1106e8,
-    ("e2m3", 8192, 8192, 8192): 1.1188e9,
-    ("u1", 8192, 8192, 8192): 6.0883e8,
-    ("f32", 4096, 4096, 4096): 2.0133e9,
-    ("f64", 4096, 4096, 4096): 3.8853e9,
-}
+# kept, with the commands, in profiles/traffic.json. Not re-measured by a plain run: counters need the profiler.
+def measured_traffic(*key):
+    global _TRAFFIC
+    if _TRAFFIC is None:
+        try:
+            with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+                _TRAFFIC = json.load(f)["bytes_per_launch"]
+        except (OSError, ValueError, KeyError):
+            _TRAFFIC = {}
+    return _TRAFFIC.get("_".join(str(part) for part in key))
+
+
+_TRAFFIC = None
 HEADLINE = ("i8", 8192, 8192, 8192)
-OTHERS = [("bf16", 8192, 8192, 8192, "dots"), ("e4m3", 8192, 8192, 8192, "dots"), ("i8", 1024, 1 << 20, 768, "dots"),
+OTHERS = [("bf16", 8192, 8192, 8192, "dots"), ("e4m3", 8192, 8192, 8192, "dots"), ("e5m2", 8192, 8192, 8192, "dots"),
+          ("f16", 8192, 8192, 8192, "dots"), ("i8", 8192, 8191, 1000, "dots"), ("f16", 8192, 8191, 1000, "dots"),
+          ("bf16", 4096, 4096, 4096, "dots"), ("i8", 2048, 2048, 2048, "dots"),
+          ("i8", 1024, 1 << 20, 768, "dots"), ("u8", 1024, 1 << 20, 768, "dots"),
           ("i8", 1024, 1 << 20, 768, "angular"), ("i8", 8192, 8192, 8192, "symmetric"), ("bf16", 8192, 8192, 8192, "symmetric"),
           ("i4", 8192, 8192, 8192, "dots"), ("e2m3", 8192, 8192, 8192, "dots"), ("u1", 8192, 8192, 8192, "dots"),
           ("f32", 4096, 4096, 4096, "dots"), ("f64", 4096, 4096, 4096, "dots")]
+VENDOR = [("i8", 8192, 8192, 8192), ("bf16", 8192, 8192, 8192), ("f16", 8192, 8192, 8192)]
 KINDS = {"angular": ord("N"), "euclidean": ord("E")}  # nk_kernel_angulars_packed_k, nk_kernel_euclideans_packed_k
 # nk_kernel_dots_symmetric_k, nk_kernel_angulars_symmetric_k, nk_kernel_euclideans_symmetric_k
 SYMMETRIC_KINDS = {"symmetric": ord("y"), "symmetric-angular": ord("n"), "symmetric-euclidean": ord("D")}
 
 
 def make_operands(dtype, m, n, k, seed=42):
-    """Synthetic inputs of BASELINE's families, generated on the GPU: ints uniform over the full range,
-    bf16/f16 N(0,1), fp8 N(0,1) scaled to half the largest finite value with 1 % zeros."""
+    """Synthetic inputs of BASELINE's families, generated on the GPU: ints uniform over the full range, bf16 N(0,1),
+    f16 log-normal(0,1) magnitudes with random signs, fp8 N(0,1) scaled to half the largest finite value with 1 %
+    zeros (clamped to the finite range before the cast: e5m2's literal configuration overflows to Inf and is almost
+    all NaN, which the parity tests cover)."""
     import torch
 
     g = torch.Generator(device="cuda:0").manual_seed(seed)
@@ -88,12 +100,35 @@ def make_operands(dtype, m, n, k, seed=42):
         if dtype == "bf16":
             return z.to(torch.bfloat16).view(torch.int16)
         if dtype == "f16":
-            return z.to(torch.float16).view(torch.int16)
+            sign = torch.randint(0, 2, (rows, k), device="cuda:0", generator=g).float() * 2 - 1
+            return (torch.exp(z) * sign).to(torch.float16).view(torch.int16)
         top = 448.0 if dtype == "e4m3" else 57344.0
         z = (z * (0.5 * top)).clamp(-top, top)  # torch's cast has no saturation: clamp first
         z = z * (torch.rand((rows, k), device="cuda:0", generator=g) >= 0.01)
         return z.to(torch.float8_e4m3fn if dtype == "e4m3" else torch.float8_e5m2).view(torch.uint8)
     return one(m), one(n)
+
+
+def timed_steps(step, steps, warmup):
+    """`warmup` untimed calls of `step`, then `steps` timed ones, each between two events of its own on torch's
+    current stream (the stream the kernels are launched on). Returns wall ms per step and the device times in ms:
+    mean over the whole region, median and minimum of the per-step pairs."""
+    import torch
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    wall = time.perf_counter()
+    marks[0].record()
+    for at in range(steps):
+        step()
+        marks[at + 1].record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - wall) * 1e3 / steps
+    each = sorted(marks[at].elapsed_time(marks[at + 1]) for at in range(steps))
+    median = each[steps // 2] if steps % 2 else 0.5 * (each[steps // 2 - 1] + each[steps // 2])
+    return wall, {"kernel_ms": marks[0].elapsed_time(marks[steps]) / steps, "kernel_ms_median": median, "kernel_ms_min": each[0]}
 
 
 def time_symmetric(dtype, n, k, steps, warmup, metric):
@@ -118,23 +153,13 @@ def time_symmetric(dtype, n, k, steps, warmup, metric):
         if status:
             raise RuntimeError(lib.nk_hip_last_error().decode())
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    wall = time.perf_counter()
-    begin.record()
-    for _ in range(steps):
-        step()
-    end.record()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - wall) * 1e3 / steps
-    device_ms = begin.elapsed_time(end) / steps
+    wall, times = timed_steps(step, steps, warmup)
+    device_ms = times["kernel_ms"]
     ops = 1.0 * n * (n + 1) * k
     achieved = ops / (device_ms * 1e-3) / 1e12
-    out = {"ms_per_step": wall, "kernel_ms": device_ms, "gso_per_s": ops / (wall * 1e-3) / 1e9,
+    out = {"ms_per_step": wall, **times, "gso_per_s": ops / (wall * 1e-3) / 1e9,
            "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK[dtype], "unit": "TFLOP/s",
-                        "frac": achieved / MFMA_PEAK[dtype], "traffic": MEASURED_TRAFFIC.get((dtype, n, n, k, metric)),
+                        "frac": achieved / MFMA_PEAK[dtype], "traffic": measured_traffic(dtype, n, n, k, metric),
                         "note": "whole call (pack + tile list + product) over the operations of the upper triangle"}}
     del vectors, result, workspace
     torch.cuda.empty_cache()
@@ -162,20 +187,12 @@ def time_pack(dtype, n, k, steps, warmup):
         if lib.nk_amd_dots_pack_async(code, b.data_ptr(), n, k, row_bytes, image.data_ptr(), stream):
             raise RuntimeError(lib.nk_hip_last_error().decode())
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    begin.record()
-    for _ in range(steps):
-        step()
-    end.record()
-    torch.cuda.synchronize()
-    device_ms = begin.elapsed_time(end) / steps
+    _, times = timed_steps(step, steps, warmup)
+    device_ms = times["kernel_ms"]
     algorithmic = n * row_bytes + size
     del b, image
     torch.cuda.empty_cache()
-    return {"kernel_ms": device_ms, "roofline": {"bound": "hbm", "achieved": algorithmic / (device_ms * 1e-3) / 1e9, "peak": HBM_PEAK,
+    return {**times, "roofline": {"bound": "hbm", "achieved": algorithmic / (device_ms * 1e-3) / 1e9, "peak": HBM_PEAK,
                                                  "unit": "GB/s", "frac": algorithmic / (device_ms * 1e-3) / 1e9 / HBM_PEAK, "traffic": None,
                                                  "note": f"{n * row_bytes} bytes of B read + {size} bytes of image written"}}
 
@@ -208,35 +225,62 @@ def time_gpu(dtype, m, n, k, steps, warmup, metric="dots"):
         if status:
             raise RuntimeError(lib.nk_hip_last_error().decode())
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    wall = time.perf_counter()
-    begin.record()
-    for _ in range(steps):
-        step()
-    end.record()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - wall) * 1e3 / steps
-    device_ms = begin.elapsed_time(end) / steps
+    wall, times = timed_steps(step, steps, warmup)
+    device_ms = times["kernel_ms"]
     ops = 2.0 * m * n * k
-    result = {"ms_per_step": wall, "kernel_ms": device_ms, "gso_per_s": ops / (wall * 1e-3) / 1e9}
+    result = {"ms_per_step": wall, **times, "gso_per_s": ops / (wall * 1e-3) / 1e9}
     if m * n >= 64 * k * 8 and dtype in ("i8", "u8") and n >= 1 << 18:  # retrieval shape: HBM-bound on C and the packed stream
         algorithmic = (m + n) * row_bytes + m * n * 4
         result["roofline"] = {"bound": "hbm", "achieved": algorithmic / (device_ms * 1e-3) / 1e9, "peak": HBM_PEAK,
                               "unit": "GB/s", "frac": algorithmic / (device_ms * 1e-3) / 1e9 / HBM_PEAK,
-                              "traffic": MEASURED_TRAFFIC.get((dtype, m, n, k) if metric == "dots" else (dtype, m, n, k, metric))}
+                              "traffic": measured_traffic(*((dtype, m, n, k) if metric == "dots" else (dtype, m, n, k, metric)))}
     else:
         achieved = ops / (device_ms * 1e-3) / 1e12
         result["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK[dtype], "unit": "TFLOP/s",
                               "frac": achieved / MFMA_PEAK[dtype],
-                              "traffic": MEASURED_TRAFFIC.get((dtype, m, n, k) if metric == "dots" else (dtype, m, n, k, metric))}
+                              "traffic": measured_traffic(*((dtype, m, n, k) if metric == "dots" else (dtype, m, n, k, metric)))}
+        if dtype in F16_ROUTE:
+            result["roofline"]["frac_f16"] = achieved / MFMA_PEAK["f16"]
         if dtype in MFMA_NOTE:
             result["roofline"]["note"] = MFMA_NOTE[dtype]
     del a, packed, c
     torch.cuda.empty_cache()
     return result
+
+
+def time_vendor(dtype, m, n, k, steps, warmup):
+    """The vendor library's GEMM (hipBLASLt through torch) on operands of the same family in the same process: what
+    this part gives a tuned kernel of the same shape. Timing only; nothing of it is used by the product."""
+    import torch
+
+    a, b = make_operands(dtype, m, n, k)
+    if dtype == "i8":
+        bt = b.t()  # (k x n) view of the row-major B: the library picks its own transposed kernel
+        step = lambda: torch._int_mm(a, bt)
+    else:
+        view = torch.bfloat16 if dtype == "bf16" else torch.float16
+        av, bt = a.view(view), b.view(view).t()
+        step = lambda: torch.matmul(av, bt)
+    _, times = timed_steps(step, steps, warmup)
+    achieved = 2.0 * m * n * k / (times["kernel_ms"] * 1e-3) / 1e12
+    del a, b
+    torch.cuda.empty_cache()
+    return {**times, "tops": achieved, "frac": achieved / MFMA_PEAK[dtype],
+            "what": "torch._int_mm (i8 -> i32)" if dtype == "i8" else f"torch.matmul ({dtype} -> {dtype}, f32 accumulation)"}
+
+
+def mfma_ceiling():
+    """The rate an MFMA-only loop sustains on this box (numkong_amd/lib/mfma_probes ceiling), as a child process."""
+    import subprocess
+
+    probe = os.path.join(ROOT, "numkong_amd", "lib", "mfma_probes")
+    if not os.path.exists(probe):
+        return {"error": "numkong_amd/lib/mfma_probes is not built"}
+    try:
+        done = subprocess.run([probe, "ceiling", "--json"], capture_output=True, text=True, timeout=120)
+        return json.loads(done.stdout) if done.returncode == 0 else {"error": done.stderr[-300:]}
+    except (OSError, ValueError, subprocess.TimeoutExpired) as failure:
+        return {"error": str(failure)}
 
 
 def cpu_baseline(dtype, m, n, k, budget_rows=8192):
@@ -250,7 +294,8 @@ def cpu_baseline(dtype, m, n, k, budget_rows=8192):
     oracle = support.load_oracle()
     reference = support.load_reference()
     rng = np.random.default_rng(42)
-    cores = max(1, min(16, len(os.sched_getaffinity(0))))
+    allowed = sorted(os.sched_getaffinity(0))  # every core this process may run on, one pinned thread each
+    cores = max(1, len(allowed))
     if reference is None:
         rows, cols = 16, min(n, 256)
         a = support.random_matrix(oracle, dtype, rows, k, rng)
@@ -278,7 +323,11 @@ def cpu_baseline(dtype, m, n, k, budget_rows=8192):
         for start in range(0, rows, tile):
             tiles.put(start)
 
-        def worker():
+        def worker(cpu):
+            try:
+                os.sched_setaffinity(0, {cpu})  # (0 = the calling thread)
+            except OSError:
+                pass
             reference.lib.nk_configure_thread(ctypes.c_uint64(viable))
             while True:
                 try:
@@ -289,7 +338,7 @@ def cpu_baseline(dtype, m, n, k, budget_rows=8192):
                 dots_fn(a.ctypes.data + start * a.strides[0], packed.ctypes.data, c.ctypes.data + start * c.strides[0],
                         count, cols, k, a.strides[0], c.strides[0])
 
-        threads = [threading.Thread(target=worker) for _ in range(cores)]
+        threads = [threading.Thread(target=worker, args=(cpu,)) for cpu in allowed]
         begin = time.perf_counter()
         for t in threads:
             t.start()
@@ -298,10 +347,12 @@ def cpu_baseline(dtype, m, n, k, budget_rows=8192):
         return time.perf_counter() - begin
 
     run_once()
-    best = min(run_once() for _ in range(3))
-    return {"value": 2.0 * rows * cols * k / best / 1e9, "unit": "gso/s", "cores": cores, "kind": "reference",
-            "kernel_capability": hex(used),
-            "sample": f"{rows} rows of A x {cols} packed rows of B x depth {k}, 64-row tiles over {cores} threads, best of 3"}
+    runs = sorted(run_once() for _ in range(3))
+    best, median = runs[0], runs[1]
+    return {"value": 2.0 * rows * cols * k / best / 1e9, "median": 2.0 * rows * cols * k / median / 1e9, "unit": "gso/s",
+            "cores": cores, "online_cores": os.cpu_count(), "kind": "reference", "kernel_capability": hex(used),
+            "sample": (f"{rows} rows of A x {cols} packed rows of B x depth {k}, 64-row tiles handed to {cores} pinned threads "
+                       "(every core the process may use), best and median of 3 after a warm-up run")}
 
 
 def main():
@@ -316,6 +367,8 @@ def main():
                              "one of the symmetric kinds over N vectors of depth K")
     parser.add_argument("--no-others", action="store_true")
     parser.add_argument("--no-cpu", action="store_true")
+    parser.add_argument("--no-vendor", action="store_true", help="skip the vendor GEMM timings (others.vendor_*)")
+    parser.add_argument("--no-ceiling", action="store_true", help="skip the MFMA-only loop (others.mfma_ceiling)")
     parser.add_argument("--probe", action="store_true",
                         help="for rocprofv3 --pmc runs: launch a plain 1 GiB elementwise copy kernel 3 times, then the selected product 3 times, nothing else")
     args = parser.parse_args()
@@ -346,17 +399,24 @@ def main():
                                 "row-major in HBM, packed inside the timed call") if args.metric in SYMMETRIC_KINDS else
                                (f"{args.dtype} packed {args.metric} C = A * B^T, M={m} N={n} K={k}, A row-major in HBM, "
                                 "B packed once outside the timed region, C overwritten")},
-        "kernel_ms": head["kernel_ms"], "roofline": head["roofline"],
+        "kernel_ms": head["kernel_ms"], "kernel_ms_median": head["kernel_ms_median"], "kernel_ms_min": head["kernel_ms_min"],
+        "roofline": head["roofline"],
     }
     if not args.no_others:
         line["others"] = {}
         for dtype, om, on, ok, metric in OTHERS:
             r = time_gpu(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2), metric)
             name = f"{dtype}_{on}x{ok}_{metric}" if metric in SYMMETRIC_KINDS else f"{dtype}_{om}x{on}x{ok}" + ("" if metric == "dots" else "_" + metric)
-            line["others"][name] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"],
-                                                         "roofline": r["roofline"]}
+            line["others"][name] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"], "kernel_ms_median": r["kernel_ms_median"],
+                                    "kernel_ms_min": r["kernel_ms_min"], "roofline": r["roofline"]}
         for dtype, on, ok in PACKS:
             line["others"][f"pack_{dtype}_{on}x{ok}"] = time_pack(dtype, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2))
+    if not args.no_vendor:
+        line.setdefault("others", {})
+        for dtype, om, on, ok in VENDOR:
+            line["others"][f"vendor_{dtype}_{om}x{on}x{ok}"] = time_vendor(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2))
+    if not args.no_ceiling:
+        line.setdefault("others", {})["mfma_ceiling"] = mfma_ceiling()
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.dtype, m, n, k)
     print(json.dumps(line))

@@ -45,6 +45,40 @@ int nk_hip_memcpy2d_d2h(void *dst, size_t dst_pitch, void const *src, size_t src
 int nk_hip_stream_synchronize(void *stream);
 
 /**
+ *  Per-thread state of the synchronous entry points, so that host threads calling at the same time (the reference's
+ *  callers hand 64-row slices of A to a thread each against one shared packed B, python/matrix.c:466-483) neither share
+ *  a stream nor allocate per call. Everything is created on first use by the calling thread and released when the
+ *  thread ends or by `nk_hip_thread_release`.
+ *   - `nk_hip_thread_stream(which)`, which = 0 or 1: the thread's own streams (blocking streams at the default
+ *     priority: ordered against the legacy default stream, independent of each other). NULL on failure.
+ *   - `nk_hip_thread_buffer(slot, pinned, bytes, &ptr)`: a staging buffer of at least `bytes` (device memory, or pinned
+ *     host memory when `pinned` is non-zero) that lives in slot 0..7 until a larger one is asked for there.
+ *   - `nk_hip_event_record / _synchronize`, `nk_hip_stream_wait_event`: the thread's events 0..7 (waiting for one
+ *     that was never recorded returns at once).
+ */
+void *nk_hip_thread_stream(int which);
+int nk_hip_thread_buffer(int slot, int pinned, size_t bytes, void **ptr);
+size_t nk_hip_thread_cached_bytes(void);
+void nk_hip_thread_release(void);
+int nk_hip_event_record(int which, void *stream);
+int nk_hip_event_synchronize(int which);
+int nk_hip_stream_wait_event(void *stream, int which);
+
+/**
+ *  Device copies of packed images that the caller keeps in host memory (what `malloc(nk_dots_packed_size_T(n, k))`
+ *  gives a caller of the reference's interface). `find` looks the image up by the number its pack call left in its
+ *  header and, when found (returns 1), hands out the device copy and counts the caller as a user until `release`.
+ *  `adopt` gives the cache a device copy the caller has just uploaded with `nk_hip_malloc` memory (returns 1: the cache
+ *  owns it now, the caller is its first user and calls `release` when done; 0: not taken, the caller frees it).
+ *  Copies nobody is using are dropped, least recently used first, beyond 4 images or NK_AMD_IMAGE_CACHE_BYTES
+ *  (default 8 GiB); `clear` drops all of them.
+ */
+int nk_hip_image_cache_find(void const *host_image, size_t total_bytes, void **device_image);
+int nk_hip_image_cache_adopt(void const *host_image, size_t total_bytes, void *device_image);
+void nk_hip_image_cache_release(void *device_image);
+void nk_hip_image_cache_clear(void);
+
+/**
  *  Bytes of the gfx950 packed image of an (n x k) B matrix: 64-byte header, MFMA-fragment tiles,
  *  per-column compensation terms, per-column sums of squares (f32 / f64: header, k-major f64 values, f64 sums of squares). Replaces `nk_dots_packed_size_<T>_<isa>`
  *  (reference: include/numkong/dots/serial.h:245-271). Returns 0 for an unsupported dtype or when
@@ -95,7 +129,10 @@ int nk_hip_symmetric_async(int dtype, int metric, void const *vectors, size_t n,
 /** Fill the m x n block of 32-bit outputs with `value` (used for the 0xFF error convention). */
 int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_t value, void *stream);
 
-/** Tile-shape override for experiments: 0 = heuristic, otherwise a configuration index. */
+/** TEST HOOK, not part of the product interface: forces the tile shape of the calling thread's launches (0 = the
+ *  heuristic picks; 1..5 = 256x256, 128x256, 128x128, 64x128, 128x512; bit 7: a forced shape may still split a
+ *  triangle). The tests use it to run every shape over the same small cases; thread-local, so it never reaches
+ *  another thread's calls. */
 void nk_hip_set_tile_config(int config);
 
 /** Thread-local text of the last failure in this layer ("" if none). */

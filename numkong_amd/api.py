@@ -105,6 +105,8 @@ def library() -> ctypes.CDLL:
     lib.nk_hip_set_tile_config.restype = None
     lib.nk_hip_device_count.restype = i32
     lib.nk_capabilities.restype = ctypes.c_uint64
+    lib.nk_configure_thread.argtypes = [ctypes.c_uint64]
+    lib.nk_configure_thread.restype = i32
     lib.nk_capabilities_compiled.restype = ctypes.c_uint64
     lib.nk_capabilities_available.restype = ctypes.c_uint64
     lib.nk_find_kernel_punned.restype = None

@@ -8,10 +8,47 @@
  */
 #include "dots_gfx950.hpp"
 
+#include <pthread.h>
+#include <time.h>
+#include <unistd.h>
+
+#include <stdlib.h>
+
+#include <new>
+
 namespace nk_gfx950 {
-int g_forced_config = 0;
-int g_variant = 0;
-int g_cu_count = 0;
+
+static thread_local int t_forced_config = 0;
+int forced_tile_config() { return t_forced_config; }
+
+uint64_t next_image_nonce() {
+    static std::atomic<uint64_t> counter {0};
+    static uint64_t const base = [] {
+        struct timespec now;
+        clock_gettime(CLOCK_REALTIME, &now);
+        return (uint64_t)now.tv_sec * 1000000007ull ^ (uint64_t)now.tv_nsec << 20 ^ (uint64_t)getpid() << 44;
+    }();
+    uint64_t x = base + 0x9E3779B97F4A7C15ull * (counter.fetch_add(1, std::memory_order_relaxed) + 1); // (splitmix64)
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    x ^= x >> 31;
+    return x ? x : 1;
+}
+
+int compute_unit_count() {
+    static std::atomic<int> cached {0};
+    int units = cached.load(std::memory_order_relaxed);
+    if (units) return units;
+    int device = 0;
+    hipDeviceProp_t properties;
+    if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&properties, device) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    cached.store(properties.multiProcessorCount, std::memory_order_relaxed);
+    return properties.multiProcessorCount;
+}
+
 } // namespace nk_gfx950
 
 namespace {
@@ -26,6 +63,56 @@ int fail(hipError_t e, char const *what) {
 int fail_msg(char const *what) {
     snprintf(g_last_error, sizeof(g_last_error), "%s", what);
     return -1;
+}
+
+/**
+ *  What a host thread keeps between synchronous calls: its streams, the events that order its staging pipeline, and
+ *  device and pinned staging buffers that only ever grow. Created on first use, released when the thread ends (a
+ *  pthread key's destructor: it runs for threads that exit, not at process exit, when the HIP runtime may already be
+ *  gone).
+ */
+constexpr int kThreadStreams = 2, kThreadEvents = 8, kThreadSlots = 8;
+struct CachedBuffer {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+struct ThreadContext {
+    hipStream_t stream[kThreadStreams] = {};
+    hipEvent_t event[kThreadEvents] = {};
+    CachedBuffer device[kThreadSlots], pinned[kThreadSlots];
+    void release(bool everything) {
+        for (int slot = 0; slot < kThreadSlots; ++slot) {
+            if (device[slot].ptr) (void)hipFree(device[slot].ptr);
+            if (pinned[slot].ptr) (void)hipHostFree(pinned[slot].ptr);
+            device[slot] = CachedBuffer(), pinned[slot] = CachedBuffer();
+        }
+        if (!everything) return;
+        for (hipEvent_t &e : event)
+            if (e) (void)hipEventDestroy(e), e = nullptr;
+        for (hipStream_t &s : stream)
+            if (s) (void)hipStreamDestroy(s), s = nullptr;
+        (void)hipGetLastError();
+    }
+};
+pthread_key_t g_context_key;
+pthread_once_t g_context_once = PTHREAD_ONCE_INIT;
+void destroy_thread_context(void *raw) {
+    ThreadContext *context = (ThreadContext *)raw;
+    context->release(true);
+    delete context;
+}
+void make_context_key() { (void)pthread_key_create(&g_context_key, destroy_thread_context); }
+ThreadContext *thread_context() {
+    (void)pthread_once(&g_context_once, make_context_key);
+    ThreadContext *context = (ThreadContext *)pthread_getspecific(g_context_key);
+    if (!context) {
+        context = new (std::nothrow) ThreadContext();
+        if (context && pthread_setspecific(g_context_key, context) != 0) {
+            delete context;
+            context = nullptr;
+        }
+    }
+    return context;
 }
 
 } // namespace
@@ -65,6 +152,83 @@ int nk_hip_free(void *ptr) {
     hipError_t e = hipFree(ptr);
     return e == hipSuccess ? 0 : fail(e, "hipFree");
 }
+
+void *nk_hip_thread_stream(int which) {
+    ThreadContext *context = thread_context();
+    if (!context || which < 0 || which >= kThreadStreams) return nullptr;
+    if (!context->stream[which]) {
+        // (a blocking stream at the default priority: ordered against the legacy default stream in both directions,
+        // so operands produced there are complete before this work starts, and independent of other threads' streams)
+        hipError_t e = hipStreamCreateWithFlags(&context->stream[which], hipStreamDefault);
+        if (e != hipSuccess) {
+            context->stream[which] = nullptr;
+            fail(e, "hipStreamCreateWithFlags");
+            return nullptr;
+        }
+    }
+    return (void *)context->stream[which];
+}
+
+int nk_hip_thread_buffer(int slot, int pinned, size_t bytes, void **ptr) {
+    ThreadContext *context = thread_context();
+    if (!context || slot < 0 || slot >= kThreadSlots) return fail_msg("nk_hip_thread_buffer: no such slot");
+    CachedBuffer &buffer = pinned ? context->pinned[slot] : context->device[slot];
+    if (buffer.bytes < bytes) {
+        hipError_t e = hipSuccess;
+        if (buffer.ptr) e = pinned ? hipHostFree(buffer.ptr) : hipFree(buffer.ptr);
+        buffer.ptr = nullptr, buffer.bytes = 0;
+        if (e != hipSuccess) return fail(e, "nk_hip_thread_buffer (release)");
+        size_t const rounded = (bytes + 0xFFFFF) & ~(size_t)0xFFFFF; // whole MiB: a slightly larger call does not reallocate
+        e = pinned ? hipHostMalloc(&buffer.ptr, rounded, hipHostMallocDefault) : hipMalloc(&buffer.ptr, rounded);
+        if (e != hipSuccess) {
+            buffer.ptr = nullptr;
+            return fail(e, pinned ? "hipHostMalloc" : "hipMalloc");
+        }
+        buffer.bytes = rounded;
+    }
+    *ptr = buffer.ptr;
+    return 0;
+}
+
+size_t nk_hip_thread_cached_bytes(void) {
+    ThreadContext *context = thread_context();
+    size_t total = 0;
+    if (context)
+        for (int slot = 0; slot < kThreadSlots; ++slot) total += context->device[slot].bytes + context->pinned[slot].bytes;
+    return total;
+}
+
+void nk_hip_thread_release(void) {
+    ThreadContext *context = thread_context();
+    if (context) context->release(false);
+}
+
+int nk_hip_event_record(int which, void *stream) {
+    ThreadContext *context = thread_context();
+    if (!context || which < 0 || which >= kThreadEvents) return fail_msg("nk_hip_event_record: no such event");
+    if (!context->event[which]) {
+        hipError_t e = hipEventCreateWithFlags(&context->event[which], hipEventDisableTiming);
+        if (e != hipSuccess) {
+            context->event[which] = nullptr;
+            return fail(e, "hipEventCreateWithFlags");
+        }
+    }
+    hipError_t e = hipEventRecord(context->event[which], (hipStream_t)stream);
+    return e == hipSuccess ? 0 : fail(e, "hipEventRecord");
+}
+int nk_hip_event_synchronize(int which) {
+    ThreadContext *context = thread_context();
+    if (!context || which < 0 || which >= kThreadEvents) return fail_msg("nk_hip_event_synchronize: no such event");
+    if (!context->event[which]) return 0; // never recorded: nothing to wait for
+    hipError_t e = hipEventSynchronize(context->event[which]);
+    return e == hipSuccess ? 0 : fail(e, "hipEventSynchronize");
+}
+int nk_hip_stream_wait_event(void *stream, int which) {
+    ThreadContext *context = thread_context();
+    if (!context || which < 0 || which >= kThreadEvents || !context->event[which]) return fail_msg("nk_hip_stream_wait_event: no such event");
+    hipError_t e = hipStreamWaitEvent((hipStream_t)stream, context->event[which], 0);
+    return e == hipSuccess ? 0 : fail(e, "hipStreamWaitEvent");
+}
 int nk_hip_memcpy_h2d(void *dst, void const *src, size_t bytes, void *stream) {
     if (!bytes) return 0;
     hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream);
@@ -94,6 +258,103 @@ int nk_hip_stream_synchronize(void *stream) {
     return e == hipSuccess ? 0 : fail(e, "hipStreamSynchronize");
 }
 
+/**
+ *  Device copies of packed images that live in host memory. A caller of the reference's interface allocates the image
+ *  with malloc, so every product would have to upload it again; instead the upload is kept and found again by the
+ *  number that the pack call left in the image's header (images are opaque: only a pack call changes one, and every
+ *  pack call leaves a new number). Least recently used copies that no call is using are dropped beyond 4 entries or
+ *  `budget` bytes.
+ */
+namespace {
+struct CachedImage {
+    uint64_t nonce, total_bytes, last_use;
+    uint32_t dtype, n, k;
+    void *device;
+    int users;
+};
+constexpr int kCachedImages = 4;
+CachedImage g_images[kCachedImages];
+uint64_t g_image_clock = 0;
+pthread_mutex_t g_image_lock = PTHREAD_MUTEX_INITIALIZER;
+size_t image_budget() {
+    static size_t const budget = [] {
+        char const *text = getenv("NK_AMD_IMAGE_CACHE_BYTES");
+        return text ? (size_t)strtoull(text, nullptr, 10) : (size_t)8 << 30;
+    }();
+    return budget;
+}
+bool header_of_host_image(void const *image, size_t total_bytes, PackedHeader &h) {
+    if (!image || total_bytes < sizeof(PackedHeader)) return false;
+    memcpy(&h, image, sizeof(h));
+    return h.magic == kMagic && h.version == kVersion && h.nonce != 0 && h.total_bytes == total_bytes;
+}
+} // namespace
+
+int nk_hip_image_cache_find(void const *host_image, size_t total_bytes, void **device_image) {
+    PackedHeader h;
+    *device_image = nullptr;
+    if (!header_of_host_image(host_image, total_bytes, h)) return 0;
+    int found = 0;
+    pthread_mutex_lock(&g_image_lock);
+    for (CachedImage &entry : g_images)
+        if (entry.device && entry.nonce == h.nonce && entry.total_bytes == total_bytes && entry.dtype == h.dtype &&
+            entry.n == h.n && entry.k == h.k) {
+            entry.users++, entry.last_use = ++g_image_clock;
+            *device_image = entry.device, found = 1;
+            break;
+        }
+    pthread_mutex_unlock(&g_image_lock);
+    return found;
+}
+
+int nk_hip_image_cache_adopt(void const *host_image, size_t total_bytes, void *device_image) {
+    PackedHeader h;
+    if (!device_image || !header_of_host_image(host_image, total_bytes, h) || total_bytes > image_budget()) return 0;
+    void *dropped[kCachedImages] = {};
+    int adopted = 0;
+    pthread_mutex_lock(&g_image_lock);
+    // room: a free entry, or the least recently used one that nobody is using; and the byte budget
+    for (;;) {
+        size_t held = 0;
+        CachedImage *vacant = nullptr, *oldest = nullptr;
+        for (CachedImage &entry : g_images) {
+            if (!entry.device) { vacant = vacant ? vacant : &entry; continue; }
+            held += entry.total_bytes;
+            if (!entry.users && (!oldest || entry.last_use < oldest->last_use)) oldest = &entry;
+        }
+        if (vacant && held + total_bytes <= image_budget()) {
+            *vacant = CachedImage {h.nonce, total_bytes, ++g_image_clock, h.dtype, h.n, h.k, device_image, 1};
+            adopted = 1;
+            break;
+        }
+        if (!oldest) break; // everything is in use: the caller keeps its copy for the call and frees it
+        for (void *&slot : dropped)
+            if (!slot) { slot = oldest->device; break; }
+        oldest->device = nullptr;
+    }
+    pthread_mutex_unlock(&g_image_lock);
+    for (void *image : dropped)
+        if (image) (void)hipFree(image);
+    return adopted;
+}
+
+void nk_hip_image_cache_release(void *device_image) {
+    pthread_mutex_lock(&g_image_lock);
+    for (CachedImage &entry : g_images)
+        if (entry.device == device_image && entry.users > 0) entry.users--;
+    pthread_mutex_unlock(&g_image_lock);
+}
+
+void nk_hip_image_cache_clear(void) {
+    void *dropped[kCachedImages] = {};
+    pthread_mutex_lock(&g_image_lock);
+    for (int i = 0; i < kCachedImages; ++i)
+        if (g_images[i].device && !g_images[i].users) dropped[i] = g_images[i].device, g_images[i].device = nullptr;
+    pthread_mutex_unlock(&g_image_lock);
+    for (void *image : dropped)
+        if (image) (void)hipFree(image);
+}
+
 size_t nk_hip_dots_packed_size(int dtype, size_t n, size_t k) {
     WideGeometry wide;
     if (wide_geometry(dtype, n, k, wide)) return (size_t)wide.total_bytes;
@@ -121,7 +382,7 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
     memset(&h, 0, sizeof(h));
     h.magic = kMagic, h.version = kVersion, h.dtype = (uint32_t)dtype, h.elem_bytes = g.packed_bytes;
     h.n = g.n, h.k = g.k, h.n_tiles = g.n_tiles, h.k_chunks = g.k_chunks;
-    h.data_offset = sizeof(PackedHeader);
+    h.nonce = next_image_nonce();
     h.sums_offset = sizeof(PackedHeader) + g.data_bytes;
     h.norms_offset = h.sums_offset + g.sums_bytes;
     h.total_bytes = g.total_bytes;
@@ -322,8 +583,7 @@ int nk_hip_symmetric_async(int dtype, int metric, void const *vectors, size_t n,
 }
 
 void nk_hip_set_tile_config(int config) {
-    g_forced_config = config & 0xFF; // (bit 7: a forced shape may still hand the narrow end of a triangle to small tiles)
-    g_variant = (config >> 8) & 0xFF;
+    t_forced_config = config & 0xFF; // (bit 7: a forced shape may still hand the narrow end of a triangle to small tiles)
 }
 
 char const *nk_hip_last_error(void) { return g_last_error; }

@@ -36,6 +36,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <stddef.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -98,9 +99,12 @@ hipError_t wide_pack(int dtype, void const *b, size_t n, size_t k, size_t b_stri
 hipError_t wide_product(int dtype, void const *a, void const *b_packed, void *c, size_t m, size_t n, size_t k,
                         size_t a_stride, size_t c_stride, hipStream_t stream, bool triangle, uint32_t shift, int metric);
 
-extern int g_forced_config; // 0: the heuristic picks the tile shape; see nk_hip_set_tile_config
-extern int g_variant;       // timing experiments of tuning builds
-extern int g_cu_count;      // compute units of the device, asked once
+/** A fresh non-zero number for the header of a newly packed image. */
+uint64_t next_image_nonce();
+/** Tile shape forced by nk_hip_set_tile_config for the calling thread (0: the heuristic picks). */
+int forced_tile_config();
+/** Compute units of the current device, asked once per process. */
+int compute_unit_count();
 
 } // namespace nk_gfx950
 
@@ -134,7 +138,7 @@ enum : int {
 };
 
 constexpr uint32_t kMagic = 0x35394B4Eu; // "NK95"
-constexpr uint32_t kVersion = 3;
+constexpr uint32_t kVersion = 4;
 constexpr int kChunkBytes = 16;   // bytes of K per lane per operand load
 constexpr int kTileRows = 32;     // B rows per tile = MFMA N
 constexpr int kStageChunks = 8;   // chunks of K per pipeline stage (128 bytes per row)
@@ -150,7 +154,7 @@ struct PackedHeader {
     uint32_t k;        // logical depth in elements
     uint32_t n_tiles;  // ceil(n / 32)
     uint32_t k_chunks; // padded depth in 16-byte chunks, multiple of 8
-    uint64_t data_offset;
+    uint64_t nonce; // a number no other pack call of this process (and, in practice, of any) has used; 0: none
     uint64_t sums_offset; // u32 x (32 * n_tiles): 128 * sum(b') per column for u8, zeros otherwise
     uint64_t total_bytes;
     uint64_t norms_offset; // u32 or f32 x (32 * n_tiles): sum(b^2) per column (exact mod 2^32 for the integer types)
@@ -752,10 +756,6 @@ __device__ __forceinline__ uint32_t distance_from_dot(uint32_t dot_bits, float q
 
 #pragma region Packed product
 
-#ifdef NK_TUNE
-__device__ unsigned long long g_debug_clocks[8];
-#endif
-
 template <int V>
 struct slot_c {
     static constexpr int value = V;
@@ -935,7 +935,7 @@ constexpr bool tail_matters_for() {
     return NORMS || T::kUnsigned || !__is_same(typename T::acc_t, v16i);
 }
 
-template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, int DBG = 0, bool WHOLE = false>
+template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, bool WHOLE = false>
 __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChunked ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
     typedef typename T::acc_t acc_t;
     constexpr int BM = TM * 32;
@@ -1227,33 +1227,32 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         uint32_t const s2 = wrap2 ? s + 2 - fast : s + 2, s3 = wrap3 ? s + 3 - fast : s + 3;
         TileView const &a2 = wrap2 ? nxt : cur, &a3 = wrap3 ? nxt : cur, &b2 = a2;
         __builtin_amdgcn_sched_barrier(0);
-        if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
+        read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
         multiply(slot_c<P>(), slot_c<0>());
-        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<0>()), load_a(a2, s2, slot_c<P>(), slot_c<2>());
+        load_b(b2, s2, slot_c<P>(), slot_c<0>()), load_a(a2, s2, slot_c<P>(), slot_c<2>());
         if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<0>());
         schedule_k_step(slot_c<0>(), slot_c<kSpread>());
         __builtin_amdgcn_sched_barrier(0);
-        if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
+        read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
         multiply(slot_c<P>(), slot_c<1>());
-        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<1>()), load_a(a2, s2, slot_c<P>(), slot_c<3>());
+        load_b(b2, s2, slot_c<P>(), slot_c<1>()), load_a(a2, s2, slot_c<P>(), slot_c<3>());
         if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<1>());
         schedule_k_step(slot_c<0>(), slot_c<kSpread>());
         __builtin_amdgcn_sched_barrier(0);
-        if (!(DBG & 2)) read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
+        read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
         multiply(slot_c<P>(), slot_c<2>());
-        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<2>());
+        load_b(b2, s2, slot_c<P>(), slot_c<2>());
         // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
         // at the previous barrier); then its registers start being refilled with A(s+3).
-        if (!(DBG & 8))
-            store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, s + 1 < fast ? 1u : 0u, slot_c<T::kPrewiden ? 1 : 0>());
-        if (!(DBG & 1)) load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
+        store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, s + 1 < fast ? 1u : 0u, slot_c<T::kPrewiden ? 1 : 0>());
+        load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
         schedule_k_step(slot_c<1>(), slot_c<0>());
         __builtin_amdgcn_sched_barrier(0);
-        if (!(DBG & 4)) __syncthreads();
+        __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        if (!(DBG & 2)) read_frags(slot_c<P ^ 1>(), slot_c<0>(), slot_c<0>());
+        read_frags(slot_c<P ^ 1>(), slot_c<0>(), slot_c<0>());
         multiply(slot_c<P>(), slot_c<3>());
-        if (!(DBG & 1)) load_b(b2, s2, slot_c<P>(), slot_c<3>()), load_a(a3, s3, slot_c<P ^ 1>(), slot_c<1>());
+        load_b(b2, s2, slot_c<P>(), slot_c<3>()), load_a(a3, s3, slot_c<P ^ 1>(), slot_c<1>());
         schedule_k_step(slot_c<0>(), slot_c<0>());
     };
 
@@ -1280,10 +1279,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     }
 
     for (uint32_t tile = blockIdx.x; tile < tile_count; tile += gridDim.x) {
-#ifdef NK_TUNE
-        unsigned long long const debug_t0 = clock64(), debug_tw0 = wall_clock64();
-        unsigned long long debug_t1 = 0, debug_t2 = 0;
-#endif
         cur = view_of(tile);
         bool const has_next = across && tile + gridDim.x < tile_count;
         nxt = view_of(has_next ? tile + gridDim.x : tile);
@@ -1308,14 +1303,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         total.clear();
 
         {
-#ifdef NK_TUNE
-            unsigned long long const debug_c0 = clock64(), debug_w0 = wall_clock64();
-#endif
             if (across || fast > 0) { // (always, when the pipeline runs across tiles: the host checked)
                 if constexpr (!across) prime();
-#ifdef NK_TUNE
-                debug_t1 = clock64();
-#endif
                 uint32_t until_fold = g.chunk_stages;
                 for (uint32_t s = 0; s < fast; s += 2) {
                     stage(slot_c<0>(), s);
@@ -1331,14 +1320,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-#ifdef NK_TUNE
-            if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + (tile_count > 45 * gridDim.x ? 40 : 1) * gridDim.x) {
-                g_debug_clocks[0] = clock64() - debug_c0, g_debug_clocks[1] = wall_clock64() - debug_w0;
-                g_debug_clocks[2] = fast;
-                g_debug_clocks[3] = debug_c0 - debug_t0, g_debug_clocks[4] = debug_t1 - debug_c0;
-            }
-            debug_t2 = clock64();
-#endif
 
             // Remaining stages: the ragged end of K, or everything when A cannot be read with vector loads.
             if (!across && fast < stages) {
@@ -1438,8 +1419,10 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         typedef __attribute__((address_space(4))) GemmArgs const late_args_t;
         late_args_t *late = (late_args_t *)__builtin_amdgcn_kernarg_segment_ptr();
         asm volatile("" : "+s"(late));
+        // (the distance kinds force the diagonal to zero in the masked copy only: a part of a tile that holds a
+        // diagonal element, even its corner alone, is not interior for them)
         bool const interior = row0 + BM <= late->m && col0 + 32 * TN <= late->n &&
-                              (((row0 + (BM - 1) + late->tri_shift) & late->tri_mask) <= col0);
+                              (((row0 + (BM - 1) + (NORMS ? 1u : 0u) + late->tri_shift) & late->tri_mask) <= col0);
         bool const nothing = ((row0 + late->tri_shift) & late->tri_mask) > col0 + (32 * TN - 1);
         global_u8_t *c_tile = (global_u8_t *)late->c + (uint64_t)row0 * late->c_stride + (uint64_t)col0 * 4;
         auto store_all = [&](auto masked_tag, auto metric_tag) {
@@ -1486,7 +1469,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                             // a vector's distance from itself is exactly 0 (dots/serial.h:2871-2876)
                             if (metric != 0 && r_fixed - j * 32 == diagonal) bits = 0;
                         }
-                        if ((!(DBG & 16) || bits == 0x12345678u) && keep) // (timing experiment: almost no stores)
+                        if (keep)
                             __builtin_nontemporal_store(bits, (global_u32_t *)(row_base + lane_offset));
                         row_base += (v % 4 == 3 ? 5 : 1) * row_step;
                         asm volatile("" : "+s"(row_base));
@@ -1512,12 +1495,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             if (interior) store_all(slot_c<0>(), slot_c<0>());
             else store_all(slot_c<1>(), slot_c<0>());
         }
-#ifdef NK_TUNE
-        if (blockIdx.x == 7 && tid == 0 && tile == blockIdx.x + (g.tile_count > 45 * gridDim.x ? 40 : 1) * gridDim.x) {
-            g_debug_clocks[5] = clock64() - debug_t2, g_debug_clocks[6] = clock64() - debug_t0;
-            g_debug_clocks[7] = wall_clock64() - debug_tw0;
-        }
-#endif
     }
 }
 
@@ -1572,45 +1549,31 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
     // The pipeline runs across tile boundaries when the pipelined loop takes the stages of a tile (A readable
     // with dword loads) and there are enough of them to prefetch three ahead.
     uint32_t const stages = g.k_chunks / kStageChunks;
-    bool const across = g.avec >= (T::kSrcChunk < 4 ? T::kSrcChunk : 4) && stages >= 4 && !(g_variant & 1);
+    bool const across = g.avec >= (T::kSrcChunk < 4 ? T::kSrcChunk : 4) && stages >= 4;
     bool const norms = g.metric != 0;
     // depths that fill an even number of stages exactly: the pipelined kernel without the tail masks
     bool const whole = across && g.k_src_bytes % (2 * kStageChunks * T::kSrcChunk) == 0;
     void (*kernel)(GemmArgs) = across ? dots_packed_kernel<T, TM, TN, true, false> : dots_packed_kernel<T, TM, TN, false, false>;
     if constexpr (tail_matters_for<T, false>()) {
-        if (whole) kernel = dots_packed_kernel<T, TM, TN, true, false, 0, true>;
+        if (whole) kernel = dots_packed_kernel<T, TM, TN, true, false, true>;
     }
     if constexpr (T::kDistances) {
         if (norms) kernel = across ? dots_packed_kernel<T, TM, TN, true, true> : dots_packed_kernel<T, TM, TN, false, true>;
-        if (norms && whole) kernel = dots_packed_kernel<T, TM, TN, true, true, 0, true>;
+        if (norms && whole) kernel = dots_packed_kernel<T, TM, TN, true, true, true>;
     }
     else if (norms) return hipErrorInvalidValue;
-#ifdef NK_TUNE // timing experiments that leave parts of the loop out (results are wrong on purpose)
-    if constexpr (TM == 8 && TN == 2 && T::kDtype == kI8) {
-        switch (g_variant >> 2) {
-        case 1: kernel = dots_packed_kernel<T, TM, TN, false, false, 1>; break;
-        case 2: kernel = dots_packed_kernel<T, TM, TN, false, false, 2>; break;
-        case 3: kernel = dots_packed_kernel<T, TM, TN, false, false, 4>; break;
-        case 4: kernel = dots_packed_kernel<T, TM, TN, false, false, 16>; break;
-        case 5: kernel = dots_packed_kernel<T, TM, TN, false, false, 17>; break;
-        default: break;
-        }
-    }
-#endif
-    // Persistent grid: as many workgroups as fit on the device at once (queried once per kernel).
-    static int resident_of[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    int &resident = resident_of[(across ? 1 : 0) + (norms ? 2 : 0) + (whole ? 4 : 0)];
+    // Persistent grid: as many workgroups as fit on the device at once (queried once per kernel; threads that
+    // ask at the same time store the same number).
+    static std::atomic<int> resident_of[8];
+    std::atomic<int> &slot = resident_of[(across ? 1 : 0) + (norms ? 2 : 0) + (whole ? 4 : 0)];
+    int resident = slot.load(std::memory_order_relaxed);
     if (!resident) {
-        int per_cu = 0, device = 0;
+        int per_cu = 0;
         hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (void const *)kernel, 256, 0);
         if (e != hipSuccess) return e;
-        if (!g_cu_count) {
-            hipDeviceProp_t properties;
-            if ((e = hipGetDevice(&device)) != hipSuccess) return e;
-            if ((e = hipGetDeviceProperties(&properties, device)) != hipSuccess) return e;
-            g_cu_count = properties.multiProcessorCount;
-        }
-        resident = (per_cu > 0 ? per_cu : 1) * (g_cu_count > 0 ? g_cu_count : 256);
+        int const units = compute_unit_count();
+        resident = (per_cu > 0 ? per_cu : 1) * (units > 0 ? units : 256);
+        slot.store(resident, std::memory_order_relaxed);
     }
     if (slots_only) {
         *slots_only = resident;
@@ -1639,7 +1602,8 @@ hipError_t launch_config(GemmArgs &g, hipStream_t stream, TriangleScratch const 
 
 template <class T>
 hipError_t launch_typed(GemmArgs &g, hipStream_t stream, TriangleScratch const *triangle) {
-    int config = g_forced_config & 0x7F;
+    int const forced = forced_tile_config();
+    int config = forced & 0x7F;
     bool const chosen_here = config <= 0 || config >= kConfigCount;
     auto tiles_of = [&](GemmArgs const &args, int c) {
         uint64_t const bm = kConfigs[c].tm * 32, bn = (uint64_t)kConfigs[c].tn * 128;
@@ -1681,7 +1645,7 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream, TriangleScratch const *
     // is mostly empty costs as much as a full one. When that last round would be less than half full, the tile rows
     // from the top that fill whole rounds go to this tile shape and the rows below them, the narrow end of the
     // triangle, to a second launch with small tiles that spreads them over the whole device.
-    if (triangle && (chosen_here || (g_forced_config & 0x80)) && config < 4) {
+    if (triangle && (chosen_here || (forced & 0x80)) && config < 4) {
         int slots = 0;
         GemmArgs probe = g;
         hipError_t e = launch_config<T>(probe, stream, triangle, config, &slots);

@@ -523,7 +523,7 @@ hipError_t wide_pack(int dtype, void const *b, size_t n, size_t k, size_t b_stri
     memset(&h, 0, sizeof(h));
     h.magic = kMagic, h.version = kVersion, h.dtype = (uint32_t)dtype, h.elem_bytes = 8;
     h.n = g.n, h.k = g.k, h.n_tiles = g.n_padded / kWideTile, h.k_chunks = g.k_padded;
-    h.data_offset = sizeof(PackedHeader), h.sums_offset = h.norms_offset = h.total_bytes = g.total_bytes;
+    h.nonce = next_image_nonce(), h.sums_offset = h.norms_offset = h.total_bytes = g.total_bytes;
     double *out = (double *)((uint8_t *)b_packed + sizeof(PackedHeader));
     if (!g.n_padded || !g.k_padded) {
         hipLaunchKernelGGL(write_header_kernel, dim3(1), dim3(64), 0, stream, (PackedHeader *)b_packed, h);

@@ -7,14 +7,21 @@
  *  kernels (include/numkong/dots.h:361-1877). Plain C over the thin HIP ABI of <numkong_amd/hip_abi.h>.
  *
  *  The reference's kernels take caller-owned pointers and return nothing (include/numkong/dots.h:84-98);
- *  so do these. A pointer the GPU can address is used in place; a plain host pointer is staged through
- *  a temporary device buffer that lives for the duration of the call (the one hidden allocation of this
- *  library). Failures follow c/numkong.c:195-216: size 0, pack is a no-op, the product fills C with 0xFF.
+ *  so do these. A pointer the GPU can address is used in place; a plain host pointer is staged through pinned and
+ *  device buffers that the calling thread keeps between calls (up to 1 GiB; the hidden allocations of this library,
+ *  with the device copies of host-resident packed images). Every call runs on streams of the calling thread, so
+ *  threads that call at the same time do not wait for each other, and is complete when it returns.
+ *  Failures follow c/numkong.c:195-216: size 0, pack is a no-op, the product fills C with 0xFF.
  */
+#define _GNU_SOURCE /* sysconf */
+#include <pthread.h>
+#include <stdatomic.h>
 #include <stddef.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
+#include <unistd.h>
 
 #include "dispatch.h"
 #include "numkong_amd/hip_abi.h"
@@ -58,7 +65,8 @@ static size_t nk_amd_round_up_(size_t x, size_t to) { return (x + to - 1) / to *
 static void nk_amd_fill_error_(void *c, int c_kind, size_t m, size_t n, size_t c_stride, size_t out_bytes) {
     if (!c || !m || !n) return;
     if (c_kind == 1) { /* (as 32-bit words: two per f64 output) */
-        if (nk_hip_fill_rows_async(c, m, n * out_bytes / 4, c_stride, 0xFFFFFFFFu, NULL) == 0) nk_hip_stream_synchronize(NULL);
+        void *stream = nk_hip_thread_stream(0);
+        if (nk_hip_fill_rows_async(c, m, n * out_bytes / 4, c_stride, 0xFFFFFFFFu, stream) == 0) nk_hip_stream_synchronize(stream);
         return;
     }
     for (size_t row = 0; row < m; ++row) memset((char *)c + row * c_stride, 0xFF, n * out_bytes);
@@ -85,6 +93,173 @@ static nk_size_t nk_amd_packed_size_(nk_dtype_t dtype, nk_size_t n, nk_size_t k)
     return nk_hip_dots_packed_size((int)dtype, n, k);
 }
 
+#pragma region Staging of host operands
+
+/*  Plain host memory reaches the GPU through pinned bounce buffers that the calling thread keeps between calls
+ *  (hip_abi.h: nk_hip_thread_buffer), in pieces, so that the copy into the bounce buffer, the transfer and whatever the
+ *  GPU does with the previous piece overlap. Copies of 16 MiB and more between pageable and pinned memory are split
+ *  over a few short-lived helper threads: one core moves about 10 GB/s, the link several times that.
+ *  Pinned slots: 0, 1 uploads; 2, 3 downloads; 4, 5 row chunks of A; 6, 7 row chunks of C. Events: the same numbers
+ *  for the slot's last transfer (4, 5: everything queued for a row chunk); 6: the packed image is on the device. */
+enum {
+    nk_amd_piece_bytes_k = 8u << 20,      /* one bounce-buffer piece of a plain upload or download */
+    nk_amd_chunk_bytes_k = 32u << 20,     /* what a row chunk of the product moves in one direction, about */
+    nk_amd_parallel_copy_k = 16u << 20,   /* host copies from this size on get helper threads */
+    nk_amd_keep_cached_k = 1u << 30,      /* staging memory a thread may keep between calls */
+};
+enum { nk_amd_slot_a_k = 0, nk_amd_slot_c_k = 2, nk_amd_slot_b_k = 4, nk_amd_slot_image_k = 5, nk_amd_slot_result_k = 6 };
+
+typedef struct {
+    char *dst;
+    char const *src;
+    size_t dst_stride, src_stride, width, rows;
+} nk_amd_copy_job_t_;
+
+static void *nk_amd_copy_worker_(void *raw) {
+    nk_amd_copy_job_t_ const *job = (nk_amd_copy_job_t_ const *)raw;
+    for (size_t row = 0; row < job->rows; ++row) memcpy(job->dst + row * job->dst_stride, job->src + row * job->src_stride, job->width);
+    return NULL;
+}
+
+static int nk_amd_copy_threads_(void) {
+    static _Atomic int cached = 0;
+    int threads = atomic_load_explicit(&cached, memory_order_relaxed);
+    if (threads) return threads;
+    char const *text = getenv("NK_AMD_COPY_THREADS");
+    long const online = sysconf(_SC_NPROCESSORS_ONLN);
+    threads = text ? atoi(text) : (int)(online / 2);
+    threads = threads < 1 ? 1 : (threads > 8 ? 8 : threads);
+    atomic_store_explicit(&cached, threads, memory_order_relaxed);
+    return threads;
+}
+
+/** `rows` runs of `width` bytes between host buffers, on this thread and, for large copies, a few helpers. */
+static void nk_amd_copy_rows_(void *dst, size_t dst_stride, void const *src, size_t src_stride, size_t width, size_t rows) {
+    if (!width || !rows) return;
+    if (dst_stride == width && src_stride == width && rows > 1) { /* one run: cut it where it suits the threads */
+        size_t const total = width * rows, unit = 1u << 16;
+        nk_amd_copy_rows_(dst, unit, src, unit, unit, total / unit);
+        memcpy((char *)dst + total / unit * unit, (char const *)src + total / unit * unit, total % unit);
+        return;
+    }
+    int threads = width * rows >= nk_amd_parallel_copy_k ? nk_amd_copy_threads_() : 1;
+    if ((size_t)threads > rows) threads = (int)rows;
+    nk_amd_copy_job_t_ jobs[8];
+    pthread_t helpers[8];
+    int started[8] = {0};
+    size_t const share = (rows + (size_t)threads - 1) / (size_t)threads;
+    for (int t = 0; t < threads; ++t) {
+        size_t const first = (size_t)t * share, last = first + share < rows ? first + share : rows;
+        jobs[t].dst = (char *)dst + first * dst_stride, jobs[t].src = (char const *)src + first * src_stride;
+        jobs[t].dst_stride = dst_stride, jobs[t].src_stride = src_stride, jobs[t].width = width;
+        jobs[t].rows = first < last ? last - first : 0;
+        if (t > 0 && jobs[t].rows) started[t] = pthread_create(&helpers[t], NULL, nk_amd_copy_worker_, &jobs[t]) == 0;
+    }
+    for (int t = 0; t < threads; ++t)
+        if (t == 0 || !started[t]) nk_amd_copy_worker_(&jobs[t]); /* this thread's share, and any a helper could not take */
+    for (int t = 1; t < threads; ++t)
+        if (started[t]) pthread_join(helpers[t], NULL);
+}
+
+/** Host rows -> device rows on `stream`, through pinned pieces 0 and 1. Returns with the last transfers in flight. */
+static int nk_amd_upload_(void *dst, size_t dst_pitch, void const *src, size_t src_pitch, size_t width, size_t rows,
+                          void *stream) {
+    if (!width || !rows) return 0;
+    size_t piece_rows = nk_amd_piece_bytes_k / width;
+    piece_rows = piece_rows < 1 ? 1 : (piece_rows > rows ? rows : piece_rows);
+    int status = 0;
+    for (size_t first = 0, piece = 0; first < rows && !status; first += piece_rows, ++piece) {
+        int const slot = (int)(piece & 1);
+        size_t const count = rows - first < piece_rows ? rows - first : piece_rows;
+        void *bounce = NULL;
+        if ((status = nk_hip_event_synchronize(slot))) break; /* the transfer that last used this piece is done */
+        if ((status = nk_hip_thread_buffer(slot, 1, piece_rows * width, &bounce))) break;
+        nk_amd_copy_rows_(bounce, width, (char const *)src + first * src_pitch, src_pitch, width, count);
+        status = nk_hip_memcpy2d_h2d((char *)dst + first * dst_pitch, dst_pitch, bounce, width, width, count, stream);
+        if (!status) status = nk_hip_event_record(slot, stream);
+    }
+    return status;
+}
+
+/** Device rows -> host rows, through pinned pieces 2 and 3; complete on return. */
+static int nk_amd_download_(void *dst, size_t dst_pitch, void const *src, size_t src_pitch, size_t width, size_t rows,
+                            void *stream) {
+    if (!width || !rows) return 0;
+    size_t piece_rows = nk_amd_piece_bytes_k / width;
+    piece_rows = piece_rows < 1 ? 1 : (piece_rows > rows ? rows : piece_rows);
+    size_t const pieces = (rows + piece_rows - 1) / piece_rows;
+    void *bounce[2] = {NULL, NULL};
+    int status = nk_hip_thread_buffer(2, 1, piece_rows * width, &bounce[0]);
+    if (!status) status = nk_hip_thread_buffer(3, 1, piece_rows * width, &bounce[1]);
+    /* piece p is queued before piece p - 1 is copied out of its bounce buffer */
+    for (size_t piece = 0; piece <= pieces && !status; ++piece) {
+        if (piece < pieces) {
+            size_t const first = piece * piece_rows, count = rows - first < piece_rows ? rows - first : piece_rows;
+            status = nk_hip_memcpy2d_d2h(bounce[piece & 1], width, (char const *)src + first * src_pitch, src_pitch, width, count, stream);
+            if (!status) status = nk_hip_event_record(2 + (int)(piece & 1), stream);
+        }
+        if (piece > 0 && !status) {
+            size_t const first = (piece - 1) * piece_rows, count = rows - first < piece_rows ? rows - first : piece_rows;
+            status = nk_hip_event_synchronize(2 + (int)((piece - 1) & 1));
+            if (!status) nk_amd_copy_rows_((char *)dst + first * dst_pitch, dst_pitch, bounce[(piece - 1) & 1], width, width, count);
+        }
+    }
+    return status;
+}
+
+/** The same for one run of bytes (a packed image), taken as rows of 1 MiB and a tail. */
+static int nk_amd_upload_flat_(void *dst, void const *src, size_t bytes, void *stream) {
+    size_t const unit = 1u << 20, whole = bytes / unit;
+    int status = nk_amd_upload_(dst, unit, src, unit, unit, whole, stream);
+    if (!status) status = nk_amd_upload_((char *)dst + whole * unit, bytes % unit, (char const *)src + whole * unit, bytes % unit, bytes % unit, 1, stream);
+    return status;
+}
+static int nk_amd_download_flat_(void *dst, void const *src, size_t bytes, void *stream) {
+    size_t const unit = 1u << 20, whole = bytes / unit;
+    int status = nk_amd_download_(dst, unit, src, unit, unit, whole, stream);
+    if (!status) status = nk_amd_download_((char *)dst + whole * unit, bytes % unit, (char const *)src + whole * unit, bytes % unit, bytes % unit, 1, stream);
+    return status;
+}
+
+/** What a synchronous call leaves behind: nothing in flight, and no more staging memory than a thread should keep. */
+static void nk_amd_settle_(void) {
+    (void)nk_hip_stream_synchronize(nk_hip_thread_stream(0));
+    (void)nk_hip_stream_synchronize(nk_hip_thread_stream(1));
+    if (nk_hip_thread_cached_bytes() > nk_amd_keep_cached_k) nk_hip_thread_release();
+}
+
+/**
+ *  The packed image where the GPU can read it. A device (or device-addressable) image is used in place. A host image
+ *  is looked up among the device copies of earlier calls and uploaded on `stream` when it is new; `*owned` is then 1
+ *  for a copy this call must free and 2 for one to hand back to the cache (nk_amd_drop_image_).
+ */
+static int nk_amd_image_on_device_(void const *b_packed, size_t total, void *stream, void const **device, int *owned) {
+    *owned = 0, *device = b_packed;
+    if (nk_hip_pointer_kind(b_packed) != 0) return 0;
+    void *copy = NULL;
+    if (nk_hip_image_cache_find(b_packed, total, &copy)) {
+        *device = copy, *owned = 2;
+        return 0;
+    }
+    int status = nk_hip_malloc(&copy, total);
+    if (status) return status;
+    status = nk_amd_upload_flat_(copy, b_packed, total, stream);
+    if (status) {
+        (void)nk_hip_stream_synchronize(stream);
+        nk_hip_free(copy);
+        return status;
+    }
+    *device = copy;
+    *owned = nk_hip_image_cache_adopt(b_packed, total, copy) ? 2 : 1;
+    return 0;
+}
+static void nk_amd_drop_image_(void const *device, int owned) {
+    if (owned == 2) nk_hip_image_cache_release((void *)device);
+    if (owned == 1) nk_hip_free((void *)device);
+}
+
+#pragma endregion Staging of host operands
+
 static void nk_amd_pack_(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t k, nk_size_t b_stride,
                          void *b_packed) {
     nk_amd_error_[0] = 0;
@@ -97,31 +272,36 @@ static void nk_amd_pack_(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_pack: no HIP device");
         return;
     }
+    void *stream = nk_hip_thread_stream(0);
     int const b_kind = (n && k) ? nk_hip_pointer_kind(b) : 1;
     int const p_kind = nk_hip_pointer_kind(b_packed);
     void *staged_b = NULL, *staged_p = NULL;
     void const *device_b = b;
     void *device_p = b_packed;
     size_t device_b_stride = b_stride;
-    int status = 0;
+    int status = stream ? 0 : -1;
 
-    if (b_kind == 0) {
+    if (!status && b_kind == 0) {
         size_t const row_bytes = nk_amd_row_bytes_(dtype, k);
         device_b_stride = nk_amd_round_up_(row_bytes, 16);
-        status = nk_hip_malloc(&staged_b, n * device_b_stride);
-        if (!status) status = nk_hip_memcpy2d_h2d(staged_b, device_b_stride, b, b_stride, row_bytes, n, NULL);
+        status = nk_hip_thread_buffer(nk_amd_slot_b_k, 0, n * device_b_stride, &staged_b);
+        if (!status) status = nk_amd_upload_(staged_b, device_b_stride, b, b_stride, row_bytes, n, stream);
         device_b = staged_b;
     }
-    if (!status && p_kind == 0) {
+    if (!status && p_kind == 0) { /* (a buffer of its own: the device copy outlives the call, as the cached image) */
         status = nk_hip_malloc(&staged_p, total);
         device_p = staged_p;
     }
-    if (!status) status = nk_hip_dots_pack_async((int)dtype, device_b, n, k, device_b_stride, device_p, NULL);
-    if (!status && staged_p) status = nk_hip_memcpy_d2h(b_packed, staged_p, total, NULL);
-    if (!status) status = nk_hip_stream_synchronize(NULL);
+    if (!status) status = nk_hip_dots_pack_async((int)dtype, device_b, n, k, device_b_stride, device_p, stream);
+    if (!status && staged_p) status = nk_amd_download_flat_(b_packed, staged_p, total, stream);
+    if (!status) status = nk_hip_stream_synchronize(stream);
     if (status) nk_amd_set_error_("nk_dots_pack");
-    if (staged_b) nk_hip_free(staged_b);
-    if (staged_p) nk_hip_free(staged_p);
+    if (staged_p) {
+        /* the host image is what the caller multiplies with next: its device copy is kept for those calls */
+        if (!status && nk_hip_image_cache_adopt(b_packed, total, staged_p)) nk_hip_image_cache_release(staged_p);
+        else nk_hip_free(staged_p);
+    }
+    nk_amd_settle_();
 }
 
 /** `metric`: 0 dot products, 1 angular distances, 2 euclidean distances; outputs are 4 bytes wide, 8 for f32 and f64 inputs. */
@@ -143,45 +323,73 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
         return;
     }
     int const a_kind = k ? nk_hip_pointer_kind(a) : 1;
-    int const p_kind = nk_hip_pointer_kind(b_packed);
-    void *staged_a = NULL, *staged_p = NULL, *staged_c = NULL;
-    void const *device_a = a, *device_p = b_packed;
-    void *device_c = c;
-    size_t device_a_stride = a_stride, device_c_stride = c_stride;
-    int status = 0;
+    void *streams[2] = {nk_hip_thread_stream(0), nk_hip_thread_stream(1)};
+    void const *device_p = b_packed;
+    int image_owned = 0;
+    int status = streams[0] && streams[1] ? 0 : -1;
+    if (!status) status = nk_amd_image_on_device_(b_packed, total, streams[0], &device_p, &image_owned);
 
-    if (a_kind == 0) {
-        size_t const row_bytes = nk_amd_row_bytes_(dtype, k);
-        device_a_stride = nk_amd_round_up_(row_bytes, 16);
-        status = nk_hip_malloc(&staged_a, m * device_a_stride);
-        if (!status) status = nk_hip_memcpy2d_h2d(staged_a, device_a_stride, a, a_stride, row_bytes, m, NULL);
-        device_a = staged_a;
+    size_t const row_bytes = nk_amd_row_bytes_(dtype, k);
+    size_t const a_pitch = nk_amd_round_up_(row_bytes, 16), c_pitch = nk_amd_round_up_(n * out_bytes, 16);
+    if (!status && a_kind != 0 && c_kind != 0) { /* everything where the GPU reads it: one launch */
+        status = metric == 0 ? nk_hip_dots_packed_async((int)dtype, a, device_p, c, m, n, k, a_stride, c_stride, streams[0])
+                             : nk_hip_spatials_packed_async((int)dtype, metric, a, device_p, c, m, n, k, a_stride, c_stride, streams[0]);
     }
-    if (!status && p_kind == 0) {
-        status = nk_hip_malloc(&staged_p, total);
-        if (!status) status = nk_hip_memcpy_h2d(staged_p, b_packed, total, NULL);
-        device_p = staged_p;
+    else if (!status) {
+        /* Rows of A go up and rows of C come down in chunks, alternating between the thread's two streams, so that
+         * the upload of one chunk, the product of the one before it and the copy of the one before that out of its
+         * bounce buffer run at the same time. */
+        size_t const heavier = (a_kind == 0 ? a_pitch : 0) > (c_kind == 0 ? c_pitch : 0) ? a_pitch : c_pitch;
+        size_t chunk = nk_amd_chunk_bytes_k / (heavier ? heavier : 1);
+        chunk = chunk >= 256 ? chunk / 256 * 256 : 64; /* whole tiles of the product kernels */
+        if (chunk > m) chunk = m;
+        size_t const chunks = (m + chunk - 1) / chunk;
+        void *device_a[2] = {NULL, NULL}, *device_c[2] = {NULL, NULL}, *bounce_a[2] = {NULL, NULL}, *bounce_c[2] = {NULL, NULL};
+        for (int half = 0; half < 2 && !status; ++half) {
+            if (a_kind == 0) status = nk_hip_thread_buffer(nk_amd_slot_a_k + half, 0, chunk * a_pitch, &device_a[half]);
+            if (!status && a_kind == 0) status = nk_hip_thread_buffer(4 + half, 1, chunk * a_pitch, &bounce_a[half]);
+            if (!status && c_kind == 0) status = nk_hip_thread_buffer(nk_amd_slot_c_k + half, 0, chunk * c_pitch, &device_c[half]);
+            if (!status && c_kind == 0) status = nk_hip_thread_buffer(6 + half, 1, chunk * c_pitch, &bounce_c[half]);
+        }
+        /* the image may still be on its way up stream 0: stream 1 waits for it */
+        if (!status) status = nk_hip_event_record(6, streams[0]);
+        if (!status) status = nk_hip_stream_wait_event(streams[1], 6);
+        for (size_t at = 0; at <= chunks && !status; ++at) {
+            if (at < chunks) {
+                int const half = (int)(at & 1);
+                size_t const first = at * chunk, rows = m - first < chunk ? m - first : chunk;
+                void const *chunk_a = (char const *)a + first * a_stride;
+                void *chunk_c = (char *)c + first * c_stride;
+                size_t chunk_a_stride = a_stride, chunk_c_stride = c_stride;
+                if (a_kind == 0) { /* (this half's buffers were last used two chunks ago: drained below) */
+                    nk_amd_copy_rows_(bounce_a[half], a_pitch, chunk_a, a_stride, row_bytes, rows);
+                    status = nk_hip_memcpy_h2d(device_a[half], bounce_a[half], rows * a_pitch, streams[half]);
+                    chunk_a = device_a[half], chunk_a_stride = a_pitch;
+                }
+                if (c_kind == 0) chunk_c = device_c[half], chunk_c_stride = c_pitch;
+                if (!status)
+                    status = metric == 0 ? nk_hip_dots_packed_async((int)dtype, chunk_a, device_p, chunk_c, rows, n, k, chunk_a_stride, chunk_c_stride, streams[half])
+                                         : nk_hip_spatials_packed_async((int)dtype, metric, chunk_a, device_p, chunk_c, rows, n, k, chunk_a_stride, chunk_c_stride, streams[half]);
+                if (!status && c_kind == 0) status = nk_hip_memcpy_d2h(bounce_c[half], device_c[half], rows * c_pitch, streams[half]);
+                if (!status) status = nk_hip_event_record(4 + half, streams[half]);
+            }
+            if (at > 0 && !status) { /* the chunk before: wait for it and hand its rows of C to the caller */
+                int const half = (int)((at - 1) & 1);
+                size_t const first = (at - 1) * chunk, rows = m - first < chunk ? m - first : chunk;
+                status = nk_hip_event_synchronize(4 + half);
+                if (!status && c_kind == 0) nk_amd_copy_rows_((char *)c + first * c_stride, c_stride, bounce_c[half], c_pitch, n * out_bytes, rows);
+            }
+        }
     }
-    if (!status && c_kind == 0) {
-        device_c_stride = nk_amd_round_up_(n * out_bytes, 16);
-        status = nk_hip_malloc(&staged_c, m * device_c_stride);
-        device_c = staged_c;
-    }
-    if (!status && metric == 0)
-        status = nk_hip_dots_packed_async((int)dtype, device_a, device_p, device_c, m, n, k, device_a_stride,
-                                          device_c_stride, NULL);
-    if (!status && metric != 0)
-        status = nk_hip_spatials_packed_async((int)dtype, metric, device_a, device_p, device_c, m, n, k, device_a_stride,
-                                              device_c_stride, NULL);
-    if (!status && staged_c) status = nk_hip_memcpy2d_d2h(c, c_stride, staged_c, device_c_stride, n * out_bytes, m, NULL);
-    if (!status) status = nk_hip_stream_synchronize(NULL);
+    if (!status) status = nk_hip_stream_synchronize(streams[0]);
+    if (!status) status = nk_hip_stream_synchronize(streams[1]);
     if (status) {
         nk_amd_set_error_("nk_dots_packed");
+        nk_amd_settle_();
         nk_amd_fill_error_(c, c_kind, m, n, c_stride, out_bytes);
     }
-    if (staged_a) nk_hip_free(staged_a);
-    if (staged_p) nk_hip_free(staged_p);
-    if (staged_c) nk_hip_free(staged_c);
+    nk_amd_drop_image_(device_p, image_owned);
+    nk_amd_settle_();
 }
 
 nk_size_t nk_amd_symmetric_workspace_size(nk_dtype_t dtype, nk_size_t vectors_count, nk_size_t depth,
@@ -236,46 +444,46 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
     size_t const row_end = row_count < n - row_start ? row_start + row_count : n;
     size_t const first = row_start / 32 * 32; /* vectors and result columns from here on take part */
     int const v_kind = k ? nk_hip_pointer_kind(vectors) : 1;
+    void *stream = nk_hip_thread_stream(0);
     void *staged_v = NULL, *staged_r = NULL, *workspace = NULL;
     /* device views, addressed as if they started at vector 0 / result element (0, 0) */
     char const *device_v = (char const *)vectors;
     char *device_r = (char *)result;
     size_t device_stride = stride, device_r_stride = result_stride;
-    int status = nk_hip_malloc(&workspace, workspace_bytes);
+    int status = stream ? nk_hip_thread_buffer(nk_amd_slot_image_k, 0, workspace_bytes + 256, &workspace) : -1;
+    if (!status) workspace = (void *)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
 
     if (!status && v_kind == 0) {
         size_t const row_bytes = nk_amd_row_bytes_(dtype, k);
         device_stride = nk_amd_round_up_(row_bytes, 16);
-        status = nk_hip_malloc(&staged_v, (n - first) * device_stride);
+        status = nk_hip_thread_buffer(nk_amd_slot_b_k, 0, (n - first) * device_stride, &staged_v);
         if (!status)
-            status = nk_hip_memcpy2d_h2d(staged_v, device_stride, (char const *)vectors + first * stride, stride,
-                                         row_bytes, n - first, NULL);
+            status = nk_amd_upload_(staged_v, device_stride, (char const *)vectors + first * stride, stride, row_bytes,
+                                    n - first, stream);
         device_v = (char const *)staged_v - first * device_stride;
     }
     char *host_window = (char *)result + row_start * result_stride + first * out_bytes;
     if (!status && r_kind == 0) {
         device_r_stride = nk_amd_round_up_((n - first) * out_bytes, 16);
-        status = nk_hip_malloc(&staged_r, (row_end - row_start) * device_r_stride);
+        status = nk_hip_thread_buffer(nk_amd_slot_result_k, 0, (row_end - row_start) * device_r_stride, &staged_r);
         if (!status)
-            status = nk_hip_memcpy2d_h2d(staged_r, device_r_stride, host_window, result_stride, (n - first) * out_bytes,
-                                         row_end - row_start, NULL);
+            status = nk_amd_upload_(staged_r, device_r_stride, host_window, result_stride, (n - first) * out_bytes,
+                                    row_end - row_start, stream);
         device_r = (char *)staged_r - row_start * device_r_stride - first * out_bytes;
     }
     if (!status)
         status = nk_hip_symmetric_async((int)dtype, metric, device_v, n, k, device_stride, device_r, device_r_stride,
-                                        row_start, row_count, workspace, workspace_bytes, NULL);
+                                        row_start, row_count, workspace, workspace_bytes, stream);
     if (!status && staged_r)
-        status = nk_hip_memcpy2d_d2h(host_window, result_stride, staged_r, device_r_stride, (n - first) * out_bytes,
-                                     row_end - row_start, NULL);
-    if (!status) status = nk_hip_stream_synchronize(NULL);
-    else (void)nk_hip_stream_synchronize(NULL);
+        status = nk_amd_download_(host_window, result_stride, staged_r, device_r_stride, (n - first) * out_bytes,
+                                  row_end - row_start, stream);
+    if (!status) status = nk_hip_stream_synchronize(stream);
     if (status) {
         nk_amd_set_error_("nk_dots_symmetric");
+        nk_amd_settle_();
         nk_amd_fill_symmetric_error_(result, r_kind, n, result_stride, out_bytes);
     }
-    if (staged_v) nk_hip_free(staged_v);
-    if (staged_r) nk_hip_free(staged_r);
-    if (workspace) nk_hip_free(workspace);
+    nk_amd_settle_();
 }
 
 #define NK_AMD_DEFINE_BACKEND_DOTS_(T, in_t, out_t)                                                                     \

@@ -8,6 +8,7 @@
  *  symmetric kinds, the error stubs (:78-81, :195-227), the capability and lookup API
  *  (:767-768, :831-913) and initialisation when the library is loaded (:916-919).
  */
+#include <stdatomic.h>
 #include <string.h>
 
 #include "dispatch.h"
@@ -131,10 +132,13 @@ NK_AMD_DISPATCH_DISTANCES_(f64, nk_f64_t, nk_f64_t)
 
 NK_DYNAMIC int nk_uses_dynamic_dispatch(void) { return 1; }
 
-/** The reference needs this once per thread for AMX tile permission (include/README.md:531-532); here
- *  there is no per-thread state to prepare. */
+/** The reference needs this once per thread for AMX tile permission (include/README.md:531-532). Here it creates
+ *  the calling thread's streams ahead of its first product, when a GPU is there; calling it is optional. */
 NK_DYNAMIC int nk_configure_thread(nk_capability_t capabilities) {
-    (void)capabilities;
+    if ((capabilities & nk_cap_gfx950_k) && (nk_capabilities() & nk_cap_gfx950_k)) {
+        (void)nk_hip_thread_stream(0);
+        (void)nk_hip_thread_stream(1);
+    }
     return 1;
 }
 
@@ -142,10 +146,12 @@ NK_DYNAMIC nk_capability_t nk_capabilities_compiled(void) { return nk_cap_serial
 
 /** Probes for a GPU on first use, not when the library is loaded, so that loading never starts HIP. */
 NK_DYNAMIC nk_capability_t nk_capabilities(void) {
-    static nk_capability_t cached = nk_cap_any_k;
-    if (cached != nk_cap_any_k) return cached;
-    cached = nk_cap_serial_k | (nk_hip_device_count() > 0 ? nk_cap_gfx950_k : 0);
-    return cached;
+    static _Atomic nk_capability_t cached = nk_cap_any_k; /* (threads that ask at the same time store the same answer) */
+    nk_capability_t known = atomic_load_explicit(&cached, memory_order_relaxed);
+    if (known != nk_cap_any_k) return known;
+    known = nk_cap_serial_k | (nk_hip_device_count() > 0 ? nk_cap_gfx950_k : 0);
+    atomic_store_explicit(&cached, known, memory_order_relaxed);
+    return known;
 }
 
 NK_DYNAMIC nk_capability_t nk_capabilities_available(void) { return nk_capabilities() & nk_capabilities_compiled(); }

@@ -258,6 +258,34 @@ def wide_distances_agree(metric, mine, ref, norms, ulps=16):
     return bool(((np.abs(mine - ref) <= ulps * u * np.abs(ref)) | (np.abs(mine * mine - ref * ref) <= ulps * u * norms)).all())
 
 
+def ulp_distance_f32(actual: np.ndarray, expected: np.ndarray) -> np.ndarray:
+    """Units in the last place between two f32 arrays, the way the reference's tests count them (test/test.hpp:400-441):
+    the distance between the bit patterns on the number line, the two zeros one step apart from nothing."""
+    def ordered(x):
+        bits = np.ascontiguousarray(x, dtype=np.float32).view(np.int32).astype(np.int64)
+        return np.where(bits < 0, -(bits & 0x7FFFFFFF), bits)
+    return np.abs(ordered(actual) - ordered(expected))
+
+
+ULP_TABLE_HEADER = f"{'kernel':<40s} {'max abs err':>12s} {'max rel err':>12s} {'mean ulp':>10s} {'max ulp':>12s} {'exact':>10s}"
+
+
+def ulp_table_row(name: str, actual: np.ndarray, truth: np.ndarray) -> str:
+    """One row of the reference's accuracy table for a mixed-precision reduction (test/test.hpp:491-514): largest
+    absolute and relative error against the f64 truth rounded to f32, mean and largest distance in units in the last
+    place, outputs that match exactly. Pairs with a NaN or an infinity on either side are skipped, as there."""
+    expected = truth.astype(np.float32)
+    use = np.isfinite(actual) & np.isfinite(expected)
+    got, want = actual[use].astype(np.float32), expected[use]
+    if not got.size:
+        return f"{name:<40s} (no finite outputs)"
+    absolute = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    relative = np.where(want != 0, absolute / np.maximum(np.abs(want.astype(np.float64)), 1e-300), absolute)
+    ulps = ulp_distance_f32(got, want)
+    return (f"{name:<40s} {absolute.max():12.2e} {relative.max():12.2e} {ulps.mean():10.1f} {int(ulps.max()):12d} "
+            f"{int((ulps == 0).sum()):10d}")
+
+
 def load_oracle() -> Oracle:
     if not os.path.exists(ORACLE_PATH):
         subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), os.path.join(ROOT, "oracle", "liboracle.so")])

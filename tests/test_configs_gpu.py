@@ -39,15 +39,35 @@ def exact_rows(dtype, a, b, rows):
     return torch.cat([sub @ as_f64(dtype, b[j:j + 65536]).T for j in range(0, b.shape[0], 65536)], dim=1)
 
 
-def sampled_oracle_gate(oracle, dtype, a, b, c, rows, cols):
+ULP_ROWS = []  # the reference-style accuracy table of this run, printed once at the end of the module
+
+
+@pytest.fixture(scope="module", autouse=True)
+def ulp_table(request):
+    yield
+    if ULP_ROWS:
+        capture = request.config.pluginmanager.getplugin("capturemanager")
+        with capture.global_and_fixture_disabled():
+            print("\n" + support.ULP_TABLE_HEADER)
+            print("\n".join(ULP_ROWS), flush=True)
+
+
+def sampled_oracle_gate(oracle, dtype, a, b, c, rows, cols, label=None):
+    """The float gate on a sample of rows and columns of the full result, next to both reference kernels, and the
+    sample's rows of the reference-style accuracy table (test/test.hpp:491-514)."""
     a_host = a[rows].cpu().numpy()
     b_host = b[cols].cpu().numpy()
     if a_host.dtype == np.int16:
         a_host, b_host = a_host.view(np.uint16), b_host.view(np.uint16)
     got = c[rows][:, cols].cpu().numpy()
     truth, magnitude = oracle.truth(dtype, a_host, b_host)
-    assert_float_gate(dtype, got, oracle.dots_packed(dtype, a_host, b_host), truth, magnitude, f"{dtype} sample",
-                      best_dispatch(dtype, a_host, b_host))
+    serial, dispatched = oracle.dots_packed(dtype, a_host, b_host), best_dispatch(dtype, a_host, b_host)
+    shape = label or f"{a.shape[0]}x{b.shape[0]}x{a.shape[1]}"
+    ULP_ROWS.append(support.ulp_table_row(f"dots_packed_{dtype}_gfx950 {shape}", got, truth))
+    ULP_ROWS.append(support.ulp_table_row(f"dots_packed_{dtype}_serial {shape}", serial, truth))
+    if dispatched is not None:
+        ULP_ROWS.append(support.ulp_table_row(f"dots_packed_{dtype} (host dispatch) {shape}", dispatched, truth))
+    assert_float_gate(dtype, got, serial, truth, magnitude, f"{dtype} sample", dispatched)
 
 
 def tiling_invariance(dtype, a, packed, c):
@@ -106,7 +126,7 @@ def test_config3_fp8_8192_cubed(oracle, dtype):
         a2, b2 = clamp(a), clamp(b)
         c2 = nk.dots_packed(a2, nk.dots_pack(b2, dtype))
         assert torch.isfinite(c2[probe]).all()
-        sampled_oracle_gate(oracle, dtype, a2, b2, c2, rows, cols)
+        sampled_oracle_gate(oracle, dtype, a2, b2, c2, rows, cols, "8192x8192x8192 clamped")
 
 
 @pytest.mark.parametrize("dtype", ["i8", "u8"])

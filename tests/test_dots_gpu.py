@@ -10,6 +10,7 @@ and, when the reference build oracle/_ref is present, the kernel the reference d
   gate:  mean(e_gpu) <= 2 * mean(e_ref) + 2^-24 / sqrt(count)   (the slack only matters for a handful of outputs)
          max(e_gpu)  <= 2 * max(max(e_ref), floor)         floor = 2^-24 against the serial kernel (one f32 rounding unit
                                                             of the magnitude sum), 2.5 * 2^-24 against the dispatched one
+         every element: |c_gpu - truth| <= 2 * max(|c_ref - truth|, 2.5 * 2^-24 * sum|a*b|)
          NaN, +Inf and -Inf masks identical to the serial kernel's (the reference's AVX-512 e5m2 kernels do
          not propagate Inf/NaN, so masks are not compared with them and their non-finite outputs are skipped).
 
@@ -67,6 +68,9 @@ def best_dispatch(dtype, a, b):
     return None if reference is None else reference.dots_packed(dtype, a, b, viable=reference.capabilities)
 
 
+PER_ELEMENT_FLOOR = 2.5  # `c` of the per-element bound below, in units of 2^-24 of sum|a*b|
+
+
 def assert_float_gate(dtype, got, serial, truth, magnitude, where="", dispatched=None):
     assert np.array_equal(np.isnan(got), np.isnan(serial)), f"NaN mask differs {where}"
     assert np.array_equal(np.isposinf(got), np.isposinf(serial)), f"+Inf mask differs {where}"
@@ -83,6 +87,13 @@ def assert_float_gate(dtype, got, serial, truth, magnitude, where="", dispatched
         assert e_gpu.mean() <= 2 * e_ref.mean() + slack, f"mean error {e_gpu.mean():.3e} vs {name} {e_ref.mean():.3e} {where}"
         floor = U if name == "serial" else 2.5 * U
         assert e_gpu.max() <= 2 * max(e_ref.max(), floor), f"max error {e_gpu.max():.3e} vs {name} {e_ref.max():.3e} {where}"
+        # Every element on its own: |c - truth| <= 2 * max(|c_ref - truth|, c * 2^-24 * sum|a*b|). The floor guards the
+        # elements where the reference kernel happens to land on the truth; c = 2.5 is five roundings of f32 at the
+        # magnitude of the whole sum, what a short chain of MFMA partial sums (each rounded once) can add up to.
+        bound = 2 * np.maximum(e_ref, PER_ELEMENT_FLOOR * U)
+        worst = int(np.argmax(e_gpu - bound))
+        assert (e_gpu <= bound).all(), (f"{int((e_gpu > bound).sum())} of {e_gpu.size} elements past the per-element bound vs {name}; "
+                                        f"worst {e_gpu[worst]:.3e} against its reference's {e_ref[worst]:.3e} {where}")
 
 
 def check(oracle, dtype, a, b, config=0, where=""):

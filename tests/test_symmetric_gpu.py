@@ -149,6 +149,21 @@ def test_distance_windows_every_tile_config(oracle, dtype, metric, config):
                         f"{dtype} {metric} {count}x{depth} rows {row_start}+{row_count} config {config}")
 
 
+@pytest.mark.parametrize("metric", ["angular", "euclidean"])
+@pytest.mark.parametrize("dtype", ALL_DTYPES + ("e3m2", "i4"))
+@pytest.mark.parametrize("config", [0, 1, 2, 3, 4])
+def test_diagonal_in_the_corner_of_a_tile(oracle, dtype, metric, config):
+    """Windows that start one row past a 32-row boundary: the diagonal then runs through the bottom-left corner of
+    32-row blocks, the only element of such a block on it. The self-distance must still be exactly 0
+    (dots/serial.h:2866-2871), for every tile shape."""
+    rng = np.random.default_rng(650 + config)
+    for row_start in (1, 33, 65, 129):
+        count, depth, row_count = 330, 64 if dtype != "i4" else 96, 200
+        vectors = finite_inputs(oracle, dtype, count, depth, rng)
+        check_distances(oracle, metric, dtype, vectors, row_start, row_count, config,
+                        f"{dtype} {metric} {count}x{depth} rows {row_start}+{row_count} config {config}")
+
+
 @pytest.mark.parametrize("name", sorted(f for f in os.listdir(support.GOLDEN_DIR) if f.startswith("symmetric_")))
 def test_golden_vectors(oracle, name):
     """Inputs and serial-kernel outputs recorded from the reference library (owned elements, zeros elsewhere)."""
