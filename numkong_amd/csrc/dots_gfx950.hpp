@@ -63,6 +63,9 @@ struct GemmArgs {
     // Symmetric products (C = A x A^T, upper triangle): only elements with col >= row + tri_shift are stored
     // (`tri_mask` all ones; 0 switches the test off), and the tiles to compute come as a list.
     uint32_t tri_shift, tri_mask;
+    // Store-bound shapes: workgroup b starts b * stagger_ticks / gridDim.x ticks of the 100 MHz clock late, so that the
+    // compute phases of some compute units fall into the store phases of others (0: all start together).
+    uint32_t stagger_ticks;
     uint32_t tile_count;       // tiles_m * tiles_n, or the length of the list
     uint32_t const *tile_list; // (tile row, tile column) pairs in walking order, or NULL for the full grid
 };
@@ -1071,6 +1074,13 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         }
         return;
     }
+    // Persistent workgroups that all start at once stay in step: every compute unit multiplies while none stores,
+    // then all of them store at once and share the memory bandwidth, and the two phases add up. Started at evenly
+    // spread times instead, some compute while others store, and a shallow product runs at the rate of its stores.
+    if (g.stagger_ticks) {
+        unsigned long long const until = wall_clock64() + (unsigned long long)blockIdx.x * g.stagger_ticks / gridDim.x;
+        while (wall_clock64() < until) __builtin_amdgcn_s_sleep(4);
+    }
     TileView cur, nxt;
     acc_t acc[TM][TN];
     constexpr bool kChunked = T::kChunked;
@@ -1580,6 +1590,15 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
         return hipSuccess;
     }
     uint32_t const blocks = (uint32_t)(tiles < (uint64_t)resident ? tiles : (uint64_t)resident);
+    // Shallow products with several tiles per workgroup are bound by their stores: spread the starts over about the
+    // time one round of tiles takes to store (the chip writes some 5.5 TB/s in this pattern; ticks of 10 ns).
+    g.stagger_ticks = 0;
+    if (stages <= 16 && tiles >= 4 * (uint64_t)blocks) {
+        double const round_bytes = (double)BM * BN * 4 * blocks;
+        g.stagger_ticks = (uint32_t)(round_bytes / 5.5e12 * 1e8);
+    }
+    int const forced = forced_tile_config();
+    if (forced >> 8) g.stagger_ticks = (uint32_t)(forced >> 8) - 1; // (test hook: bits 8.. = ticks + 1)
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, g);
     return hipGetLastError();
 }

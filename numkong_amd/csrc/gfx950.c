@@ -136,7 +136,8 @@ static int nk_amd_copy_threads_(void) {
 /** `rows` runs of `width` bytes between host buffers, on this thread and, for large copies, a few helpers. */
 static void nk_amd_copy_rows_(void *dst, size_t dst_stride, void const *src, size_t src_stride, size_t width, size_t rows) {
     if (!width || !rows) return;
-    if (dst_stride == width && src_stride == width && rows > 1) { /* one run: cut it where it suits the threads */
+    if (dst_stride == width && src_stride == width && width != (1u << 16) && rows > 1) {
+        /* one run of bytes: cut it into 64 KiB rows, which divide evenly among the threads, and a tail */
         size_t const total = width * rows, unit = 1u << 16;
         nk_amd_copy_rows_(dst, unit, src, unit, unit, total / unit);
         memcpy((char *)dst + total / unit * unit, (char const *)src + total / unit * unit, total % unit);

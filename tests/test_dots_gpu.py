@@ -221,9 +221,25 @@ def test_host_pointers_are_staged(oracle, dtype):
     assert (c[:, n:] == 7).all()
     device = gpu_dots(dtype, a, b)
     assert np.array_equal(np.ascontiguousarray(c[:, :n]).view(np.uint32), device.view(np.uint32))  # same kernel, same bits
-    # a packed image is relocatable bytes: device image == host image
+    # a packed image is relocatable bytes: device image == host image, but for the number that tells pack calls apart
+    # (header bytes 32..39), by which the library finds the device copy of a host image again
     image = nk.dots_pack(to_gpu(b), dtype).buffer.cpu().numpy()
+    nonce, other = packed[32:40].copy().view(np.uint64)[0], image[32:40].copy().view(np.uint64)[0]
+    assert nonce != 0 and other != 0 and nonce != other
+    image[32:40] = packed[32:40]
     assert np.array_equal(image, packed)
+    # the bytes stay valid wherever they are copied: a copy of the host image, and the device image brought to the host
+    for relocated in (packed.copy(), nk.dots_pack(to_gpu(b), dtype).buffer.cpu().numpy()):
+        again = np.full((m, n + 2), 7, OUTPUT[dtype])
+        getattr(lib, f"nk_dots_packed_{dtype}")(a.ctypes.data, relocated.ctypes.data, again.ctypes.data, m, n, k, a.strides[0], again.strides[0])
+        assert not lib.nk_amd_last_error()
+        assert np.array_equal(again.view(np.uint32), c.view(np.uint32))
+    # packing other rows into the same host buffer gives a new image, not the cached one's results
+    shuffled = np.ascontiguousarray(b[::-1])
+    getattr(lib, f"nk_dots_pack_{dtype}")(shuffled.ctypes.data, n, k, shuffled.strides[0], packed.ctypes.data)
+    again = np.full((m, n + 2), 7, OUTPUT[dtype])
+    getattr(lib, f"nk_dots_packed_{dtype}")(a.ctypes.data, packed.ctypes.data, again.ctypes.data, m, n, k, a.strides[0], again.strides[0])
+    assert np.array_equal(again[:, :n].view(np.uint32), c[:, :n][:, ::-1].view(np.uint32))
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
