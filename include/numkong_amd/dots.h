@@ -338,6 +338,20 @@ NK_DYNAMIC int nk_amd_symmetric_async(nk_kernel_kind_t kind, nk_dtype_t dtype, v
                                       nk_size_t result_stride, nk_size_t row_start, nk_size_t row_count, void *workspace,
                                       nk_size_t workspace_bytes, void *stream);
 
+/**
+ *  `nk_amd_symmetric_async` for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ *  loops, harnesses that forbid hipMalloc): no workspace argument, no allocation of any kind inside. It has no
+ *  counterpart in the reference. The scratch memory is a fixed array of `nk_amd_symmetric_static_capacity()` bytes
+ *  (32 MiB) that the library keeps in the memory of every GPU it runs on; a call that would need more
+ *  (`nk_amd_symmetric_workspace_size` says how much) returns non-zero and `nk_hip_last_error()` names both numbers.
+ *  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU race, so keep them on one stream.
+ */
+NK_DYNAMIC nk_size_t nk_amd_symmetric_static_capacity(void);
+NK_DYNAMIC int nk_amd_symmetric_static_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void const *vectors,
+                                             nk_size_t vectors_count, nk_size_t depth, nk_size_t stride, void *result,
+                                             nk_size_t result_stride, nk_size_t row_start, nk_size_t row_count,
+                                             void *stream);
+
 #ifdef __cplusplus
 }
 #endif

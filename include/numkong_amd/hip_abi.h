@@ -126,6 +126,17 @@ int nk_hip_symmetric_async(int dtype, int metric, void const *vectors, size_t n,
                            size_t result_stride, size_t row_start, size_t row_count, void *workspace,
                            size_t workspace_bytes, void *stream);
 
+/**
+ *  `nk_hip_symmetric_async` without a workspace argument and without any allocation: for callers that cannot call
+ *  hipMalloc (code under HIP graph capture, tight serving loops, harnesses that forbid it). The workspace is a fixed
+ *  array of `nk_hip_symmetric_static_capacity()` bytes (32 MiB) in device memory that the library holds on every GPU it
+ *  runs on; a call whose `nk_hip_symmetric_workspace_size` is larger fails with a message saying so. All calls on one
+ *  GPU share that array: calls that overlap there (two streams, two threads) race. No counterpart in the reference.
+ */
+size_t nk_hip_symmetric_static_capacity(void);
+int nk_hip_symmetric_static_async(int dtype, int metric, void const *vectors, size_t n, size_t k, size_t stride,
+                                  void *result, size_t result_stride, size_t row_start, size_t row_count, void *stream);
+
 /** Fill the m x n block of 32-bit outputs with `value` (used for the 0xFF error convention). */
 int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_t value, void *stream);
 

@@ -93,6 +93,10 @@ def library() -> ctypes.CDLL:
     lib.nk_amd_symmetric_workspace_size.argtypes = [i32, sz, sz, sz, sz]
     lib.nk_amd_symmetric_async.restype = i32
     lib.nk_amd_symmetric_async.argtypes = [i32, i32, vp, sz, sz, sz, vp, sz, sz, sz, vp, sz, vp]
+    lib.nk_amd_symmetric_static_capacity.restype = sz
+    lib.nk_amd_symmetric_static_capacity.argtypes = []
+    lib.nk_amd_symmetric_static_async.restype = i32
+    lib.nk_amd_symmetric_static_async.argtypes = [i32, i32, vp, sz, sz, sz, vp, sz, sz, sz, vp]
     lib.nk_amd_last_error.restype = ctypes.c_char_p
     lib.nk_amd_dots_pack_async.restype = i32
     lib.nk_amd_dots_pack_async.argtypes = [i32, vp, sz, sz, sz, vp, vp]

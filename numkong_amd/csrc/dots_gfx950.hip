@@ -582,6 +582,56 @@ int nk_hip_symmetric_async(int dtype, int metric, void const *vectors, size_t n,
                          result_stride, stream, &scratch, (uint32_t)(row_start - w.col_begin));
 }
 
+/**
+ *  The symmetric kinds for callers that cannot allocate: the workspace is a fixed array in device memory that belongs
+ *  to the library (each GPU the library runs on holds its own copy until the process ends), found once per device by
+ *  its symbol. Calls that overlap on one GPU share it and race; the array keeps the last call's contents, and nothing
+ *  in this path expects zeros there (the pack kernels write every byte of the image they read, padding included, and
+ *  the tile lists are written before they are read).
+ */
+constexpr size_t kStaticWorkspaceBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticWorkspaceBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void *> g_scratch_of_device[kMaxDevices];
+
+/** The address of `scratch` on the current device (the array's name is a host-side stand-in, not a device address). */
+static int static_workspace(void **workspace) {
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return fail(e, "hipGetDevice");
+    if (device < 0 || device >= kMaxDevices) return fail_msg("nk_hip_symmetric_static: device index out of range");
+    void *ptr = g_scratch_of_device[device].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) return fail(e, "hipGetSymbolAddress(scratch)");
+        g_scratch_of_device[device].store(ptr, std::memory_order_release);
+    }
+    *workspace = ptr;
+    return 0;
+}
+
+size_t nk_hip_symmetric_static_capacity(void) { return kStaticWorkspaceBytes; }
+
+int nk_hip_symmetric_static_async(int dtype, int metric, void const *vectors, size_t n, size_t k, size_t stride,
+                                  void *result, size_t result_stride, size_t row_start, size_t row_count, void *stream) {
+    if (row_start >= n || !row_count) return 0;
+    size_t const needed = nk_hip_symmetric_workspace_size(dtype, n, k, row_start, row_count);
+    if (!needed) return fail_msg("nk_hip_symmetric_static: unsupported dtype or dimensions");
+    if (needed > kStaticWorkspaceBytes) {
+        snprintf(g_last_error, sizeof(g_last_error),
+                 "nk_hip_symmetric_static: this call needs %zu bytes of workspace, the built-in one holds %zu; use "
+                 "nk_hip_symmetric_async with a workspace of the caller's",
+                 needed, kStaticWorkspaceBytes);
+        return -1;
+    }
+    void *workspace = nullptr;
+    int const status = static_workspace(&workspace);
+    if (status) return status;
+    return nk_hip_symmetric_async(dtype, metric, vectors, n, k, stride, result, result_stride, row_start, row_count,
+                                  workspace, kStaticWorkspaceBytes, stream);
+}
+
 void nk_hip_set_tile_config(int config) {
     t_forced_config = config; // (bits 0..6 the shape; bit 7: a forced shape may still hand the narrow end of a triangle to small tiles; bits 8..: start spread in 10 ns ticks + 1)
 }

@@ -414,6 +414,15 @@ int nk_amd_symmetric_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void const *
                                   result, result_stride, row_start, row_count, workspace, workspace_bytes, stream);
 }
 
+nk_size_t nk_amd_symmetric_static_capacity(void) { return nk_hip_symmetric_static_capacity(); }
+
+int nk_amd_symmetric_static_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void const *vectors, nk_size_t vectors_count,
+                                  nk_size_t depth, nk_size_t stride, void *result, nk_size_t result_stride,
+                                  nk_size_t row_start, nk_size_t row_count, void *stream) {
+    return nk_hip_symmetric_static_async((int)dtype, nk_amd_symmetric_metric_(kind), vectors, vectors_count, depth, stride,
+                                         result, result_stride, row_start, row_count, stream);
+}
+
 /** 0xFF over the whole n x n result, as the reference's stub does (c/numkong.c:218-227), 4 bytes per output. */
 static void nk_amd_fill_symmetric_error_(void *result, int kind, size_t n, size_t result_stride, size_t out_bytes) {
     nk_amd_fill_error_(result, kind, n, n, result_stride, out_bytes);
