@@ -401,7 +401,7 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
         if (blocks > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_pack: matrix too large");
         uint32_t const xr = dtype == kU8 ? 0x80808080u : 0u;
         void (*kernel)(uint8_t const *, uint64_t, uint32_t, uint64_t, uint32_t, uint8_t *, int, uint32_t, PackedHeader) = pack_kernel<0>;
-        switch (widen_kind_of(dtype)) {
+        switch (widen_kind_of(dtype, k)) {
         case 1: kernel = pack_kernel<1>; break;
         case 2: kernel = pack_kernel<2>; break;
         case 3: kernel = pack_kernel<3>; break;
@@ -409,6 +409,7 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
         case 5: kernel = pack_kernel<5>; break;
         case 6: kernel = pack_kernel<6>; break;
         case 7: kernel = pack_kernel<7>; break;
+        case 8: kernel = pack_kernel<8>; break;
         default: break;
         }
         hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride,
@@ -417,9 +418,9 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
         if (e != hipSuccess) return fail(e, "pack_kernel");
     }
     if (g.n_tiles && terms) {
-        if (g.k_chunks) {
+        if (g.k_chunks && dtype != kU1) { // (the 1-bit type has the dot-product kinds only, which read no terms: zeros)
             // by what the image holds: signed bytes (i8, the widened 4-bit types and bits, e2m3 as 8 x its values), offset u8, bf16, f16 (and what is widened to it)
-            auto kernel = dtype == kI8 || dtype == kI4 || dtype == kU4 || dtype == kU1 || dtype == kE2M3
+            auto kernel = dtype == kI8 || dtype == kI4 || dtype == kU4 || (dtype == kE2M3 && e2m3_as_integers(k))
                               ? column_terms_kernel<0>
                               : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
             hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(32 * kColumnParts), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);

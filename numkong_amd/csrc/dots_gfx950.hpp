@@ -166,9 +166,8 @@ static_assert(sizeof(PackedHeader) == 64, "header must stay 64 bytes");
 
 struct Geometry {
     uint32_t elem_bytes;   // bytes per element in the caller's A and B (1 for the 4-bit types, two to a byte)
-    uint32_t packed_bytes; // bytes per element in the image and in LDS (fp8 is widened to f16)
+    uint32_t packed_bytes; // bytes per element in the image and in LDS (fp8 is widened to f16; 0 for bits)
     uint32_t n, k, n_tiles, k_chunks;
-    uint64_t k_bytes;      // bytes of one packed row: k * packed_bytes
     uint64_t k_src_bytes;  // bytes of one source row
     uint64_t data_bytes, sums_bytes, norms_bytes, total_bytes;
 };
@@ -196,35 +195,53 @@ inline int elem_bits_of(int dtype) {
  *  kernels (dot/serial.h:522-600). e4m3 and e5m2 are therefore widened, exactly, to f16 and run on the f16
  *  MFMA, whose products and sums are kept to full f32 precision: B at pack time, A on its way into LDS.
  *  e3m2 goes the same way (every e3m2 value is an f16 value). e2m3 values are multiples of 1/8 below 8 in magnitude:
- *  eight times each is an i8 value, and the i8 MFMA sums their products exactly at twice the f16 rate. The 4-bit
- *  integers are widened to i8 as well, and so are single bits (0 or 1: their dot product is the popcount of the AND). */
-inline int packed_bytes_of(int dtype) {
+ *  eight times each is an i8 value, and the i8 MFMA sums their products exactly at twice the f16 rate, as long as the
+ *  i32 sums of 64 x the products cannot overflow (60 * 60 * k < 2^31); deeper rows take the f16 route like e3m2. The
+ *  4-bit integers are widened to i8 as well. Single bits stay bits in the image (sixteen to a chunk) and become i8
+ *  zeros and ones in registers, on both sides, right in front of the MFMA (their dot product is the popcount of the AND). */
+constexpr uint64_t kE2M3IntegerDepth = 0x7FFFFFFFull / 3600; // deepest e2m3 row whose i32 sums are safe
+inline bool e2m3_as_integers(size_t k) { return k <= kE2M3IntegerDepth; }
+
+/** Bytes per element in the image and in LDS (0: sub-byte, the 1-bit type). */
+inline int packed_bytes_of(int dtype, size_t k) {
     switch (dtype) {
     case kE4M3:
     case kE5M2:
     case kE3M2: return 2;
-    case kE2M3: // (as i8 values, eight times the e2m3 value)
+    case kE2M3: return e2m3_as_integers(k) ? 1 : 2; // (as i8 values, eight times the e2m3 value; or as f16)
     case kI4:
-    case kU4:
-    case kU1: return 1;
+    case kU4: return 1;
+    case kU1: return 0;
     default: return elem_bits_of(dtype) / 8;
     }
 }
+/** Source bytes of a row behind one chunk of the image (a chunk is what one lane feeds one MFMA: 16 bytes of operand). */
+inline int source_chunk_of(int dtype, size_t k) {
+    switch (dtype) {
+    case kE4M3:
+    case kE5M2:
+    case kE3M2:
+    case kI4:
+    case kU4: return 8;
+    case kE2M3: return e2m3_as_integers(k) ? 16 : 8;
+    case kU1: return 2;
+    default: return 16;
+    }
+}
+/** Bytes a chunk takes in the image: the 16 operand bytes, except for the 1-bit type, which keeps its 16 bits. */
+inline int image_chunk_of(int dtype) { return dtype == kU1 ? 2 : kChunkBytes; }
 
 inline bool make_geometry(int dtype, size_t n, size_t k, Geometry &g) {
     int const bits = elem_bits_of(dtype);
     if (!bits) return false;
     if (n > 0x7FFFFFFFull || k > 0x3FFFFFFFull) return false;
-    // e2m3 sums 64 x its products in i32: 60 * 60 * k must stay below 2^31 (the reference sums in f32 and has no
-    // such bound; rows this deep are refused like dimensions beyond 32 bits)
-    if (dtype == kE2M3 && k > 0x7FFFFFFFull / 3600) return false;
-    g.elem_bytes = (uint32_t)(bits + 7) / 8, g.packed_bytes = (uint32_t)packed_bytes_of(dtype), g.n = (uint32_t)n, g.k = (uint32_t)k;
+    g.elem_bytes = (uint32_t)(bits + 7) / 8, g.packed_bytes = (uint32_t)packed_bytes_of(dtype, k), g.n = (uint32_t)n, g.k = (uint32_t)k;
     g.k_src_bytes = ((uint64_t)k * bits + 7) / 8; // (sub-byte types: whole bytes, as the reference loads them, cast/serial.h:519-538)
-    g.k_bytes = bits < 8 ? g.k_src_bytes * (8 / bits) * g.packed_bytes : (uint64_t)k * g.packed_bytes;
-    uint64_t const chunks = (g.k_bytes + kChunkBytes - 1) / kChunkBytes;
+    uint64_t const source_chunk = (uint64_t)source_chunk_of(dtype, k);
+    uint64_t const chunks = (g.k_src_bytes + source_chunk - 1) / source_chunk;
     g.k_chunks = (uint32_t)((chunks + 2 * kStageChunks - 1) / (2 * kStageChunks) * (2 * kStageChunks)); // an even number of stages
     g.n_tiles = (uint32_t)((n + kTileRows - 1) / kTileRows);
-    g.data_bytes = (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes;
+    g.data_bytes = (uint64_t)g.n_tiles * g.k_chunks * kTileRows * image_chunk_of(dtype);
     g.sums_bytes = (uint64_t)g.n_tiles * kTileRows * sizeof(uint32_t);
     g.norms_bytes = g.sums_bytes;
     g.total_bytes = sizeof(PackedHeader) + g.data_bytes + g.sums_bytes + g.norms_bytes;
@@ -358,23 +375,24 @@ __device__ __forceinline__ v4i widen_u1x16(uint32_t bits) {
     return out;
 }
 
-/** Widening of the source bytes behind one 16-byte chunk, by kind: 1 e4m3, 2 e5m2, 4 e3m2 (8 bytes to f16);
- *  5 i4, 6 u4 (8 bytes to i8); 7 u1 (2 bytes to i8). Kind 3, e2m3, turns 16 bytes into 16 i8 values in place
- *  (widen_e2m3x4) and does not come through here. */
+/** Widening of the source bytes behind one 16-byte chunk, by kind: 1 e4m3, 2 e5m2, 4 e3m2, 8 e2m3 of deep rows (8
+ *  bytes to f16); 5 i4, 6 u4 (8 bytes to i8); 7 u1 (2 bytes to i8). Kind 3, e2m3 of rows that are not too deep, turns 16
+ *  bytes into 16 i8 values in place (widen_e2m3x4) and does not come through here. */
 template <int WIDEN>
 __device__ __forceinline__ v4i widen_chunk(uint32_t lo, uint32_t hi) {
     if constexpr (WIDEN == 1) return widen_fp8x8<false>(lo, hi);
     else if constexpr (WIDEN == 2) return widen_fp8x8<true>(lo, hi);
     else if constexpr (WIDEN == 4) return widen_fp6x8<true>(lo, hi);
+    else if constexpr (WIDEN == 8) return widen_fp6x8<false>(lo, hi);
     else if constexpr (WIDEN == 5) return widen_i4x16<true>(lo, hi);
     else if constexpr (WIDEN == 6) return widen_i4x16<false>(lo, hi);
     else return widen_u1x16(lo);
 }
-inline int widen_kind_of(int dtype) {
+inline int widen_kind_of(int dtype, size_t k) {
     switch (dtype) {
     case kE4M3: return 1;
     case kE5M2: return 2;
-    case kE2M3: return 3;
+    case kE2M3: return e2m3_as_integers(k) ? 3 : 8;
     case kE3M2: return 4;
     case kI4: return 5;
     case kU4: return 6;
@@ -388,14 +406,15 @@ inline int widen_kind_of(int dtype) {
 /**
  *  One thread per 16-byte chunk of the image. A block of 256 threads covers 32 rows x 8 chunks: reads are
  *  128 (64 for the widened types) contiguous bytes per row, writes are eight 512-byte runs. WIDEN: 0 copies the
- *  elements, 3 rewrites e2m3 bytes as i8 values in place, otherwise the kind of widen_chunk (8 or 2 source bytes per
- *  chunk).
+ *  elements, 3 rewrites e2m3 bytes as i8 values in place, 7 copies the 16 bits of a chunk of the 1-bit type as they
+ *  are (eight 64-byte runs), otherwise the kind of widen_chunk (8 source bytes per chunk).
  */
 template <int WIDEN>
 __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
                                                    uint64_t k_src_bytes, uint32_t k_chunks, uint8_t *__restrict__ data,
                                                    int avec, uint32_t xr, PackedHeader header) {
     constexpr int kSrcChunk = WIDEN == 0 || WIDEN == 3 ? 16 : (WIDEN == 7 ? 2 : 8);
+    constexpr int kImageChunk = WIDEN == 7 ? 2 : kChunkBytes;
     if (blockIdx.x == 0 && threadIdx.x == 0) *(PackedHeader *)(data - sizeof(PackedHeader)) = header; // (64 bytes in front of the tiles)
     uint32_t const groups = k_chunks / kStageChunks;
     uint32_t const tile = blockIdx.x / groups;
@@ -417,9 +436,11 @@ __global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b
 #pragma unroll
             for (int w = 0; w < 4; ++w) v[w] = (int)widen_e2m3x4((uint32_t)v[w]);
         }
-        else if constexpr (WIDEN != 0) v = widen_chunk<WIDEN>((uint32_t)v[0], (uint32_t)v[1]);
+        else if constexpr (WIDEN != 0 && WIDEN != 7) v = widen_chunk<WIDEN>((uint32_t)v[0], (uint32_t)v[1]);
     }
-    *(v4i *)(data + (((uint64_t)tile * k_chunks + c) * kTileRows + r) * kChunkBytes) = v;
+    uint8_t *at = data + (((uint64_t)tile * k_chunks + c) * kTileRows + r) * kImageChunk;
+    if constexpr (WIDEN == 7) *(uint16_t *)at = (uint16_t)v[0];
+    else *(v4i *)at = v;
 }
 
 /** Sum of the squares of the 8 values of a 16-byte chunk of bf16 (f32 = bits << 16) or f16, in f64. */
@@ -542,6 +563,10 @@ constexpr bool kHalfChunked = true;
 struct I8 {
     static constexpr bool kChunked = false; // fold the accumulator into a second one every few stages
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
+    static constexpr int kImageChunk = kChunkBytes; // bytes of one row's chunk in the image
+    static constexpr bool kEightfold = false; // the MFMA sees eight times the values (e2m3 as integers)
+    /** What a lane loaded from the image -> its MFMA operand. */
+    static __device__ __forceinline__ v4i operand_b(v4i loaded) { return loaded; }
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16i acc_t;
     typedef uint32_t norm_t; // what a row's sum of squares accumulates in
@@ -573,6 +598,9 @@ struct U8 : I8 {
 struct BF16 {
     static constexpr bool kChunked = kHalfChunked;
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
+    static constexpr int kImageChunk = kChunkBytes;
+    static constexpr bool kEightfold = false;
+    static __device__ __forceinline__ v4i operand_b(v4i loaded) { return loaded; }
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
     typedef double norm_t;
@@ -603,6 +631,9 @@ struct BF16 {
 struct F16 {
     static constexpr bool kChunked = kHalfChunked;
     static constexpr int kSrcChunk = 16; // source bytes of A behind one 16-byte LDS chunk
+    static constexpr int kImageChunk = kChunkBytes;
+    static constexpr bool kEightfold = false;
+    static __device__ __forceinline__ v4i operand_b(v4i loaded) { return loaded; }
     static __device__ __forceinline__ v4i widen(v4i v) { return v; }
     typedef v16f acc_t;
     typedef double norm_t;
@@ -658,6 +689,7 @@ struct E5M2 : F16 {
  *  the dot product, converted to f32 once in the epilogue (one rounding for sums beyond 2^24, none below). */
 struct E2M3 : I8 {
     static constexpr int kDtype = kE2M3;
+    static constexpr bool kEightfold = true;
     static constexpr bool kPrewiden = true; // 13 operations per dword: too many to sit in front of the LDS writes
     static __device__ __forceinline__ v4i widen(v4i v) {
         v4i out;
@@ -666,6 +698,15 @@ struct E2M3 : I8 {
         return out;
     }
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); } // 64 x the sum of squares
+};
+/** e2m3 rows too deep for exact i32 sums (see kE2M3IntegerDepth) run widened to f16 like e3m2: every e2m3 value is an
+ *  f16 value, the smallest non-zero one 1/8. */
+struct E2M3Deep : F16 {
+    static constexpr bool kChunked = true;
+    static constexpr int kDtype = kE2M3;
+    static constexpr int kSrcChunk = 8;
+    static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp6x8<false>((uint32_t)v[0], (uint32_t)v[1]); }
+    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return sumsq_of_normals(wide); }
 };
 /** e3m2 runs widened to f16 (its values times 16 do not fit i8); see widen_fp6x8. */
 struct E3M2 : F16 {
@@ -683,11 +724,14 @@ struct I4 : I8 {
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_i4x16<true>((uint32_t)v[0], (uint32_t)v[1]); }
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); }
 };
-/** Single bits run as i8 values 0 and 1: sixteen of them behind two source bytes. */
+/** Single bits run as i8 values 0 and 1: sixteen of them behind two source bytes, of A on its way into LDS and of B,
+ *  whose image keeps the bits, in registers between the load and the MFMA. */
 struct U1 : I8 {
     static constexpr int kDtype = kU1;
     static constexpr bool kDistances = false; // dot products only
     static constexpr int kSrcChunk = 2;
+    static constexpr int kImageChunk = 2;
+    static __device__ __forceinline__ v4i operand_b(v4i loaded) { return widen_u1x16((uint32_t)loaded[0]); }
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_u1x16((uint32_t)v[0]); }
     static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return I8::sumsq(wide, wide); }
 };
@@ -708,7 +752,7 @@ template <class T>
 __device__ __forceinline__ float norm_as_f32(uint32_t bits) {
     if (T::kDtype == kI8 || T::kDtype == kI4) return (float)(int)bits;
     if (T::kDtype == kU8 || T::kDtype == kU4) return (float)bits;
-    if (T::kDtype == kE2M3) return (float)bits * 0.015625f; // integer sums of squares of 8 x the values
+    if (T::kEightfold) return (float)bits * 0.015625f; // integer sums of squares of 8 x the values
     return __builtin_bit_cast(float, bits);
 }
 
@@ -716,7 +760,7 @@ __device__ __forceinline__ float norm_as_f32(uint32_t bits) {
  *  integers, 64 times the f32 result. */
 template <class T>
 __device__ __forceinline__ uint32_t finished_dot(uint32_t bits) {
-    if (T::kDtype == kE2M3) return __builtin_bit_cast(uint32_t, (float)(int)bits * 0.015625f);
+    if (T::kEightfold) return __builtin_bit_cast(uint32_t, (float)(int)bits * 0.015625f);
     return bits;
 }
 
@@ -963,7 +1007,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                           header->dtype == (uint32_t)T::kDtype && header->n == g.n && header->k == g.k &&
                           header->k_chunks == g.k_chunks && header->n_tiles == g.n_tiles;
     uint8_t const *data = g.bp + sizeof(PackedHeader);
-    uint32_t const *col_terms = (uint32_t const *)(data + (uint64_t)g.n_tiles * g.k_chunks * kTileChunkBytes);
+    constexpr int kImageTileChunk = kTileRows * T::kImageChunk; // one chunk of all 32 rows of a tile, as the image holds it
+    uint32_t const *col_terms = (uint32_t const *)(data + (uint64_t)g.n_tiles * g.k_chunks * kImageTileChunk);
     uint32_t const *col_norms = col_terms + (uint64_t)g.n_tiles * kTileRows;
 
     uint32_t const stages = g.k_chunks / kStageChunks;
@@ -992,7 +1037,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         a_off[i] = r * (uint32_t)g.a_stride + a_pos * T::kSrcChunk;
         a_lds[i] = r * kStageBytes + ((a_pos ^ ((r >> 1) & 7)) << 4);
     }
-    uint32_t const b_lane = lane * kChunkBytes;
+    uint32_t const b_lane = lane * T::kImageChunk;
 
     // Loads go through buffer descriptors: one scalar descriptor plus a 32-bit per-lane offset is the cheapest
     // address form to issue (a single address register per lane, no 64-bit vector adds), and a descriptor is
@@ -1017,7 +1062,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         // (whole aligned loads: an aligned A never ends in the middle of one that could fault)
         constexpr uint32_t kLoadAlign = T::kSrcChunk < 4 ? T::kSrcChunk : 4; // (2-byte loads for the 1-bit type)
         view.a_bytes = (rows_here - 1) * (uint32_t)g.a_stride + (((uint32_t)g.k_src_bytes + kLoadAlign - 1) & ~(kLoadAlign - 1));
-        uint32_t const tile_bytes = g.k_chunks * kTileChunkBytes;
+        uint32_t const tile_bytes = g.k_chunks * kImageTileChunk;
         uint32_t const first = view.col0 / 32 < g.n_tiles ? view.col0 / 32 : g.n_tiles - 1;
         view.b = data + (uint64_t)first * tile_bytes;
         uint64_t const left = (uint64_t)(g.n_tiles - first) * tile_bytes;
@@ -1177,10 +1222,15 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
         __amdgpu_buffer_rsrc_t const rsrc = b_rsrc_of(view);
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-            b_reg[slot][j][q] = __builtin_bit_cast(
-                v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_lane + q * 2 * kTileChunkBytes,
-                                                           view.b_tile[j] + s * (kStageChunks * kTileChunkBytes), 0));
+        for (int j = 0; j < TN; ++j) {
+            if constexpr (T::kImageChunk == 2) // (sixteen bits per lane: the rest of the register is never looked at)
+                b_reg[slot][j][q][0] = (int)(uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, b_lane + q * 2 * kImageTileChunk,
+                                                                                           view.b_tile[j] + s * (kStageChunks * kImageTileChunk), 0);
+            else
+                b_reg[slot][j][q] = __builtin_bit_cast(
+                    v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_lane + q * 2 * kImageTileChunk,
+                                                               view.b_tile[j] + s * (kStageChunks * kImageTileChunk), 0));
+        }
     };
     auto read_frags = [&](auto buffer_tag, auto q_tag, auto parity_tag) {
         constexpr int buffer = decltype(buffer_tag)::value, q = decltype(q_tag)::value,
@@ -1192,9 +1242,11 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     auto multiply = [&](auto slot_tag, auto q_tag) {
         constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j) {
+            v4i const b = T::operand_b(b_reg[slot][j][q]);
 #pragma unroll
-            for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[q & 1][i], b_reg[slot][j][q]);
+            for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[q & 1][i], b);
+        }
     };
     // Scheduling hints for one k-step. Masks: 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write.
     // Fragment reads go one-to-one with the first TM MFMAs; the global loads of the k-step (TN of B
@@ -1555,7 +1607,7 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
     // So are the per-lane C offsets: 4 rows plus the tile's width.
     if (4 * (uint64_t)g.c_stride + BN * 4 > 0xFFFFFFFFull) return hipErrorInvalidValue;
     // The offsets into a wavefront's B tiles are 32-bit as well.
-    if ((uint64_t)(TN + 1) * g.k_chunks * kTileChunkBytes > 0xFFFFFFFFull) return hipErrorInvalidValue;
+    if ((uint64_t)(TN + 1) * g.k_chunks * kTileRows * T::kImageChunk > 0xFFFFFFFFull) return hipErrorInvalidValue;
     // The pipeline runs across tile boundaries when the pipelined loop takes the stages of a tile (A readable
     // with dword loads) and there are enough of them to prefetch three ahead.
     uint32_t const stages = g.k_chunks / kStageChunks;

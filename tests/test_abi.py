@@ -53,8 +53,12 @@ def test_packed_size_formula():
             assert nk.dots_packed_size(t, n, k) == 64 + tiles * chunks * 512 + tiles * 256, (t, n, k)
         assert nk.dots_packed_size(t, 0, 0) == 64
         assert nk.dots_packed_size(t, 1 << 40, 8) == 0  # dimensions beyond 32 bits are refused, as the error stub does
-    # e2m3 sums integers 64 times its products in i32: depths where 60 * 60 * k passes 2^31 are refused
-    assert nk.dots_packed_size("e2m3", 8, 596523) > 0 and nk.dots_packed_size("e2m3", 8, 596524) == 0
+    # e2m3 is stored as i8 values (eight times as large) while the i32 sums of 64 x its products cannot overflow,
+    # 60 * 60 * k < 2^31, and widened to f16 like e3m2 beyond that depth: twice the bytes per element
+    assert nk.dots_packed_size("e2m3", 8, 596523) == 64 + -(-596523 // 256) * 16 * 512 + 256
+    assert nk.dots_packed_size("e2m3", 8, 596524) == 64 + -(-596524 // 128) * 16 * 512 + 256
+    # single bits stay bits: sixteen to a 2-byte chunk, 32 rows and 16 chunks to a unit
+    assert nk.dots_packed_size("u1", 100, 1000) == 64 + 4 * 64 * 64 + 4 * 256
     # the two wide types keep f64 values k-major: header + 8 bytes x (n padded to 64) x (k padded to 32), and a sum of
     # squares per padded column behind them
     assert nk.dots_packed_size("f32", 100, 70) == nk.dots_packed_size("f64", 100, 70) == 64 + 8 * 128 * 96 + 8 * 128

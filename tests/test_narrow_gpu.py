@@ -129,6 +129,47 @@ def test_deep_and_strided(oracle, dtype):
         assert_float_gate(dtype, got.view(np.float32), serial, truth, magnitude, f"{dtype} strided", best_dispatch(dtype, a_full, b_full))
 
 
+def test_e2m3_rows_too_deep_for_integer_sums(oracle):
+    """e2m3 runs as integers eight times as large on the i8 MFMA while 60 * 60 * depth stays below 2^31 (depth <=
+    596,523); deeper rows, which the reference takes like any others (dots/serial.h:2601-2678), run widened to f16.
+    Both sides of the switch, products and distances, against the serial restatement, the f64 truth and the kernel the
+    reference dispatches to; with all values at the format's largest magnitude the integer route's sums are the
+    largest they can be, and must still be exact."""
+    rng = np.random.default_rng(91)
+    for depth in (596_523, 596_524, 700_001):
+        a, b = support.random_matrix(oracle, "e2m3", 5, depth, rng), support.random_matrix(oracle, "e2m3", 37, depth, rng)
+        assert nk.dots_packed_size("e2m3", 37, depth) > 0
+        check(oracle, "e2m3", a, b, 0, f"e2m3 depth {depth}")
+        for metric in ("angular", "euclidean"):
+            assert_distance_gate(oracle, metric, "e2m3", a, b, gpu_distances(metric, "e2m3", a, b), f"e2m3 {metric} depth {depth}")
+    extreme = np.full((3, 596_523), 0x1F, np.uint8)  # +7.5 everywhere: 64 x the dot product is 3600 x depth, just below 2^31
+    extreme[1] = 0x3F                                # -7.5
+    got = gpu_dots("e2m3", extreme, extreme)
+    exact = np.float32(56.25 * 596_523) * np.array([[1, -1, 1], [-1, 1, -1], [1, -1, 1]], np.float32)
+    assert np.array_equal(got, exact)
+
+
+def test_u1_image_keeps_bits(oracle):
+    """The image of the 1-bit type holds the bits themselves, sixteen to a chunk (dots/serial.h:2680-2689 packs bytes
+    of bits as well): header + n / 8 * depth bytes rounded up to whole tiles and stages + the (unused) column terms;
+    chunk c of row r of tile t at ((t * chunks + c) * 32 + r) * 2."""
+    rng = np.random.default_rng(92)
+    for n, depth in [(70, 1000), (33, 4099), (1, 1)]:
+        b = support.random_matrix(oracle, "u1", n, depth, rng)
+        tiles, chunks = -(-n // 32), -(-(-(-depth // 16)) // 16) * 16
+        size = nk.dots_packed_size("u1", n, depth)
+        assert size == 64 + tiles * chunks * 64 + tiles * 256
+        image = nk.dots_pack(to_gpu(b), "u1").buffer.cpu().numpy()
+        assert image.size == size
+        masked = b.copy()  # (bits past the depth in the last byte are the caller's: whole bytes are taken, as the reference does)
+        padded = np.zeros((tiles * 32, chunks * 2), np.uint8)
+        padded[:n, : masked.shape[1]] = masked
+        expected = padded.reshape(tiles, 32, chunks, 2).transpose(0, 2, 1, 3).reshape(-1)
+        assert np.array_equal(image[64 : 64 + expected.size], expected)
+        assert not image[64 + expected.size :].any()
+    assert nk.dots_packed_size("u1", 8192, 8192) == 64 + 256 * 512 * 64 + 256 * 256  # 8 MiB of bits, not 64 MiB of bytes
+
+
 @pytest.mark.parametrize("name", sorted(f for f in os.listdir(support.GOLDEN_DIR) if f.startswith("narrow_")))
 def test_golden_vectors(oracle, name):
     """Inputs and serial-kernel outputs recorded from the reference library."""
