@@ -115,10 +115,10 @@ __global__ __launch_bounds__(256) void wide_norms_kernel(uint8_t const *__restri
 template <bool F64>
 __global__ __launch_bounds__(256) void pack_wide_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
                                                         uint32_t k, uint32_t n_padded, double *__restrict__ out,
-                                                        PackedHeader header) {
+                                                        PackedHeader header, uint32_t k_first) {
     __shared__ double block[32][33];
-    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *(PackedHeader *)((uint8_t *)out - sizeof(PackedHeader)) = header;
-    uint32_t const row0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && k_first == 0 && threadIdx.x == 0) *(PackedHeader *)((uint8_t *)out - sizeof(PackedHeader)) = header;
+    uint32_t const row0 = blockIdx.x * 32, k0 = k_first + blockIdx.y * 32; // (k_first: a grid covers 65535 blocks of depth at most)
     uint32_t const tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 32 x 8
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -506,7 +506,7 @@ namespace nk_gfx950 {
 
 bool wide_geometry(int dtype, size_t n, size_t k, WideGeometry &g) {
     if (dtype != kF32 && dtype != kF64) return false;
-    if (n > 0x7FFFFFFFull || k > 65535ull * 32) return false; // (one workgroup row of the pack grid per 32 depths)
+    if (n > 0x7FFFFFFFull || k > 0x3FFFFFFFull) return false;
     g.elem_bytes = dtype == kF64 ? 8 : 4;
     g.n = (uint32_t)n, g.k = (uint32_t)k;
     g.n_padded = (uint32_t)((n + kWideTile - 1) / kWideTile * kWideTile);
@@ -529,12 +529,15 @@ hipError_t wide_pack(int dtype, void const *b, size_t n, size_t k, size_t b_stri
         hipLaunchKernelGGL(write_header_kernel, dim3(1), dim3(64), 0, stream, (PackedHeader *)b_packed, h);
         return hipGetLastError();
     }
-    dim3 const grid(g.n_padded / 32, g.k_padded / 32);
-    if (grid.y > 65535) return hipErrorInvalidValue;
-    if (dtype == kF64) hipLaunchKernelGGL(pack_wide_kernel<true>, grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, out, h);
-    else hipLaunchKernelGGL(pack_wide_kernel<false>, grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, out, h);
-    hipError_t const status = hipGetLastError();
-    if (status != hipSuccess) return status;
+    // (the second grid dimension holds 65535 workgroups: deeper rows take several launches)
+    for (uint32_t k_first = 0; k_first < g.k_padded; k_first += 65535u * 32) {
+        uint32_t const depth_blocks = (g.k_padded - k_first) / 32 < 65535u ? (g.k_padded - k_first) / 32 : 65535u;
+        dim3 const grid(g.n_padded / 32, depth_blocks);
+        if (dtype == kF64) hipLaunchKernelGGL(pack_wide_kernel<true>, grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, out, h, k_first);
+        else hipLaunchKernelGGL(pack_wide_kernel<false>, grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, out, h, k_first);
+        hipError_t const status = hipGetLastError();
+        if (status != hipSuccess) return status;
+    }
     double *norms = out + (uint64_t)g.n_padded * g.k_padded;
     dim3 const norms_grid((g.n_padded + 3) / 4);
     if (dtype == kF64) hipLaunchKernelGGL(wide_norms_kernel<true>, norms_grid, dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n, g.k, g.n_padded, norms);
@@ -565,15 +568,25 @@ hipError_t wide_product(int dtype, void const *a, void const *b_packed, void *c,
     g.a = (uint8_t const *)a, g.b = (double const *)((uint8_t const *)b_packed + sizeof(PackedHeader)), g.c = (uint8_t *)c;
     g.a_stride = a_stride, g.c_stride = c_stride;
     g.m = (uint32_t)m, g.n = geo.n, g.k = geo.k, g.n_padded = geo.n_padded, g.k_padded = geo.k_padded;
-    g.tri_shift = shift, g.tri_mask = tri_mask, g.metric = metric;
-    dim3 const grid(geo.n_padded / kWideTile, (uint32_t)((m + kWideTile - 1) / kWideTile));
-    if (grid.y > 65535) return hipErrorInvalidValue;
-    dim3 const matrix_grid(geo.n_padded / kMatrixCols, (uint32_t)((m + kMatrixRows - 1) / kMatrixRows));
-    if (dtype == kF64 && metric) hipLaunchKernelGGL(dots_f64_compensated_kernel<true>, grid, dim3(256), 0, stream, g);
-    else if (dtype == kF64) hipLaunchKernelGGL(dots_f64_compensated_kernel<false>, grid, dim3(256), 0, stream, g);
-    else if (metric) hipLaunchKernelGGL(dots_f32_matrix_kernel<true>, matrix_grid, dim3(512), 0, stream, g);
-    else hipLaunchKernelGGL(dots_f32_matrix_kernel<false>, matrix_grid, dim3(512), 0, stream, g);
-    return hipGetLastError();
+    g.tri_mask = tri_mask, g.metric = metric;
+    // The second grid dimension holds 65535 workgroups: taller products go band by band (a whole number of tiles of
+    // both kernels each; a band's rows start `first` below the diagonal's origin).
+    uint64_t const band = 32767ull * kMatrixRows;
+    static_assert((32767ull * kMatrixRows) % kWideTile == 0 && 32767ull * kMatrixRows / kWideTile <= 65535, "a band is whole tiles of both kernels");
+    for (uint64_t first = 0; first < m; first += band) {
+        uint64_t const rows = m - first < band ? m - first : band;
+        g.a = (uint8_t const *)a + first * a_stride, g.c = (uint8_t *)c + first * c_stride;
+        g.m = (uint32_t)rows, g.tri_shift = shift + (uint32_t)first;
+        dim3 const grid(geo.n_padded / kWideTile, (uint32_t)((rows + kWideTile - 1) / kWideTile));
+        dim3 const matrix_grid(geo.n_padded / kMatrixCols, (uint32_t)((rows + kMatrixRows - 1) / kMatrixRows));
+        if (dtype == kF64 && metric) hipLaunchKernelGGL(dots_f64_compensated_kernel<true>, grid, dim3(256), 0, stream, g);
+        else if (dtype == kF64) hipLaunchKernelGGL(dots_f64_compensated_kernel<false>, grid, dim3(256), 0, stream, g);
+        else if (metric) hipLaunchKernelGGL(dots_f32_matrix_kernel<true>, matrix_grid, dim3(512), 0, stream, g);
+        else hipLaunchKernelGGL(dots_f32_matrix_kernel<false>, matrix_grid, dim3(512), 0, stream, g);
+        hipError_t const status = hipGetLastError();
+        if (status != hipSuccess) return status;
+    }
+    return hipSuccess;
 }
 
 } // namespace nk_gfx950

@@ -52,6 +52,21 @@ def test_shapes_bit_exact(oracle, dtype, kind):
         assert got.dtype == np.float64 and same_bits(got, oracle.dots_packed(dtype, a, b)), f"{dtype} {kind} {m}x{n}x{k}"
 
 
+@pytest.mark.parametrize("dtype", WIDE_DTYPES)
+def test_past_one_grid_of_workgroups(oracle, dtype):
+    """Rows deeper than 65535 x 32 values and products taller than 65535 tiles take several launches inside one call (the
+    reference has no such bound: dots/serial.h:2458-2491): a depth of 2,100,001 on 2 x 3 outputs, bit for bit against the
+    serial restatement; 4,200,000 rows of depth 3 against one column, bit for bit against a plain f64 product of small
+    integers, and the symmetric form of the same call shape for its diagonal bookkeeping across bands."""
+    rng = np.random.default_rng(905)
+    a, b = support.random_matrix(oracle, dtype, 2, 2_100_001, rng), support.random_matrix(oracle, dtype, 3, 2_100_001, rng)
+    assert same_bits(gpu_dots(dtype, a, b), oracle.dots_packed(dtype, a, b))
+    tall = rng.integers(-50, 50, (4_200_000, 3)).astype(support.STORAGE[dtype])
+    one = rng.integers(-50, 50, (1, 3)).astype(support.STORAGE[dtype])
+    got = gpu_dots(dtype, tall, one)
+    assert np.array_equal(got, tall.astype(np.float64) @ one.astype(np.float64).T)
+
+
 def test_closed_forms():
     """Small integers: exact in both kinds. f64: 1e100 + 1 - 1e100 + 1.5 = 2.5, which a plain f64 sum gets wrong."""
     rng = np.random.default_rng(901)
