@@ -66,6 +66,7 @@ struct GemmArgs {
     // Store-bound shapes: workgroup b starts b * stagger_ticks / gridDim.x ticks of the 100 MHz clock late, so that the
     // compute phases of some compute units fall into the store phases of others (0: all start together).
     uint32_t stagger_ticks;
+    uint32_t store_policy; // 0: by the alignment of C's rows; 1: past the caches; 2: through them (test hook)
     uint32_t tile_count;       // tiles_m * tiles_n, or the length of the list
     uint32_t const *tile_list; // (tile row, tile column) pairs in walking order, or NULL for the full grid
 };
@@ -1102,6 +1103,10 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     auto add_row_norm = [&](int i, norm_t value, uint32_t set) {
         __hip_atomic_fetch_add(&norm_part[set + i * NT + tid], value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
+    // u8 only: the stages of a tile that fetch nothing past its end run in a loop of their own, without the scalar work of
+    // choosing between this tile's descriptors and the next one's (measured: u8 1024 x 1,048,576 x 768 1.69 -> 1.45 ms,
+    // u8 8192^3 0.53 -> 0.50 ms; the other types lose 1-9 % to the second copy of the loop, so they keep the single one).
+    constexpr bool kPeel = T::kUnsigned;
     v4i a_reg[2][kLoads];
     v4i b_reg[2][TN][4];
     v4i af[2][TM];
@@ -1281,24 +1286,27 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // One stage of the steady state; `P` = stage parity = LDS buffer = register slot. Stages s+2 and
     // s+3 are fetched here; past the tile's end they are the first stages of `nxt` (the next tile, or
     // this one again when nothing follows: loads of valid memory that nobody uses).
-    auto stage = [&](auto parity_tag, uint32_t s) {
+    // `wrap_tag`: 0 for a stage with three more stages of its tile behind it (kPeel): everything it fetches is this
+    // tile's, and the choice between the two tiles' descriptors is left out.
+    auto stage = [&](auto parity_tag, uint32_t s, auto wrap_tag) {
         constexpr int P = decltype(parity_tag)::value;
+        constexpr bool may_wrap = decltype(wrap_tag)::value != 0 || !kPeel;
         // vector operations behind each MFMA of the k-steps that widen in place: their share of half the chunks
         constexpr int kSpread = T::kPrewiden ? (kLoads * 28 + TM * TN - 1) / (TM * TN) : 0;
-        bool const wrap2 = s + 2 >= fast, wrap3 = s + 3 >= fast;
+        bool const wrap2 = may_wrap && s + 2 >= fast, wrap3 = may_wrap && s + 3 >= fast;
         uint32_t const s2 = wrap2 ? s + 2 - fast : s + 2, s3 = wrap3 ? s + 3 - fast : s + 3;
         TileView const &a2 = wrap2 ? nxt : cur, &a3 = wrap3 ? nxt : cur, &b2 = a2;
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
         multiply(slot_c<P>(), slot_c<0>());
         load_b(b2, s2, slot_c<P>(), slot_c<0>()), load_a(a2, s2, slot_c<P>(), slot_c<2>());
-        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<0>());
+        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), !may_wrap || s + 1 < fast ? s + 1 : 0u, slot_c<0>());
         schedule_k_step(slot_c<0>(), slot_c<kSpread>());
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
         multiply(slot_c<P>(), slot_c<1>());
         load_b(b2, s2, slot_c<P>(), slot_c<1>()), load_a(a2, s2, slot_c<P>(), slot_c<3>());
-        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<1>());
+        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), !may_wrap || s + 1 < fast ? s + 1 : 0u, slot_c<1>());
         schedule_k_step(slot_c<0>(), slot_c<kSpread>());
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
@@ -1306,7 +1314,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         load_b(b2, s2, slot_c<P>(), slot_c<2>());
         // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
         // at the previous barrier); then its registers start being refilled with A(s+3).
-        store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, s + 1 < fast ? 1u : 0u, slot_c<T::kPrewiden ? 1 : 0>());
+        bool const mine = !may_wrap || s + 1 < fast;
+        store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), mine ? s + 1 : 0u, mine ? 1u : 0u, slot_c<T::kPrewiden ? 1 : 0>());
         load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
         schedule_k_step(slot_c<1>(), slot_c<0>());
         __builtin_amdgcn_sched_barrier(0);
@@ -1368,9 +1377,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             if (across || fast > 0) { // (always, when the pipeline runs across tiles: the host checked)
                 if constexpr (!across) prime();
                 uint32_t until_fold = g.chunk_stages;
-                for (uint32_t s = 0; s < fast; s += 2) {
-                    stage(slot_c<0>(), s);
-                    stage(slot_c<1>(), s + 1);
+                auto fold_when_due = [&]() {
                     if constexpr (kChunked) {
                         until_fold -= 2;
                         if (until_fold == 0) {
@@ -1379,6 +1386,17 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                             until_fold = g.chunk_stages;
                         }
                     }
+                };
+                uint32_t s = 0;
+                for (; kPeel && s + 4 < fast; s += 2) { // (all but the last two pairs: nothing they fetch lies past the tile)
+                    stage(slot_c<0>(), s, slot_c<0>());
+                    stage(slot_c<1>(), s + 1, slot_c<0>());
+                    fold_when_due();
+                }
+                for (; s < fast; s += 2) {
+                    stage(slot_c<0>(), s, slot_c<1>());
+                    stage(slot_c<1>(), s + 1, slot_c<1>());
+                    fold_when_due();
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -1468,12 +1486,10 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             }
             sums_here ^= (uint32_t)(kLoads * NT);
         }
-        // Stores: past the caches (`nt`): the output is written once and not read here, and the caches are left to the
-        // operands (measured on one box, same run: bf16 8192^3 1.047 -> 0.972 ms, e4m3 1.027 -> 0.933 ms, i8 0.526 ->
-        // 0.518 ms, i8 1024 x 1,048,576 x 768 1.455 -> 1.395 ms). A scalar base plus one 32-bit per-lane offset,
-        // through an explicitly global pointer. (A store through a generic pointer counts as an LDS operation as
-        // well, and with such stores in flight the loads prefetched for the next tile could only be waited for all
-        // at once.) Tiles that touch the matrix edge take the masked copy of the loop.
+        // Stores: a scalar base plus one 32-bit per-lane offset, through an explicitly global pointer. (A store
+        // through a generic pointer counts as an LDS operation as well, and with such stores in flight the loads
+        // prefetched for the next tile could only be waited for all at once.) Tiles that touch the matrix edge take
+        // the masked copy of the loop.
         // Of a triangular grid, a wavefront's part of a tile is stored whole (all of it right of the diagonal), not
         // at all (all of it left), or through the masked copy.
         // What only the stores need is read from the kernel's arguments again, here, rather than held in a dozen
@@ -1481,15 +1497,27 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         typedef __attribute__((address_space(4))) GemmArgs const late_args_t;
         late_args_t *late = (late_args_t *)__builtin_amdgcn_kernarg_segment_ptr();
         asm volatile("" : "+s"(late));
+        // Stores go past the caches (`nt`): the output is written once and not read here, and the caches are left to the
+        // operands (measured on one box, same run: bf16 8192^3 1.047 -> 0.972 ms, e4m3 1.027 -> 0.933 ms, i8 0.526 ->
+        // 0.518 ms, i8 1024 x 1,048,576 x 768 1.455 -> 1.395 ms). Except where the rows of C do not start on 128-byte
+        // lines and the product is not deep: a 128-byte run of a row then straddles two lines and would reach the
+        // memory as two partial writes; through the L2 the parts of a line written by neighbouring wavefronts meet
+        // first (measured, i8, nt -> plain: 8192 x 8191 x 1000
+        // 0.199 -> 0.146 ms, 4096 x 4095 x 4096 0.099 -> 0.077, 1024 x 1,000,001 x 768 3.99 -> 1.92 ms; bf16 4096 x 4095 x
+        // 4096 0.155 -> 0.143, but 8192 x 8191 x 8192 0.97 -> 1.04: a deep product wants its L2 for the operands).
+        // The distance kinds keep `nt` (i8 angular 1024 x 1,000,001 x 768: 2.57 against 2.70 ms).
+        bool const lines = (((uint64_t)late->c | late->c_stride) & 127) == 0;
+        bool const streamed = NORMS || (late->store_policy ? late->store_policy == 1 : lines || stages > 64);
         // (the distance kinds force the diagonal to zero in the masked copy only: a part of a tile that holds a
         // diagonal element, even its corner alone, is not interior for them)
         bool const interior = row0 + BM <= late->m && col0 + 32 * TN <= late->n &&
                               (((row0 + (BM - 1) + (NORMS ? 1u : 0u) + late->tri_shift) & late->tri_mask) <= col0);
         bool const nothing = ((row0 + late->tri_shift) & late->tri_mask) > col0 + (32 * TN - 1);
         global_u8_t *c_tile = (global_u8_t *)late->c + (uint64_t)row0 * late->c_stride + (uint64_t)col0 * 4;
-        auto store_all = [&](auto masked_tag, auto metric_tag) {
+        auto store_all = [&](auto masked_tag, auto metric_tag, auto streamed_tag) {
             constexpr bool masked = decltype(masked_tag)::value != 0;
             constexpr int metric = decltype(metric_tag)::value;
+            constexpr bool past_caches = decltype(streamed_tag)::value != 0;
             uint64_t const row_step = late->c_stride;
             // Lane l holds column l % 32; register v holds row 8 * (v / 4) + 4 * (l / 32) + v % 4.
             uint32_t const lane_offset = 4 * half * (uint32_t)late->c_stride + col_in_tile * 4;
@@ -1531,8 +1559,14 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                             // a vector's distance from itself is exactly 0 (dots/serial.h:2871-2876)
                             if (metric != 0 && r_fixed - j * 32 == diagonal) bits = 0;
                         }
-                        if (keep)
-                            __builtin_nontemporal_store(bits, (global_u32_t *)(row_base + lane_offset));
+                        // Whole tiles of whole lines go past the caches. Anything else is left to the L2 to put together:
+                        // a 128-byte run of a row that straddles two lines would reach the memory as two partial
+                        // writes (measured, i8, C rows of 8191 and 1,000,001 columns: 8192 x 8191 x 1000 0.218 -> 0.147
+                        // ms, 4096 x 4095 x 4096 0.116 -> 0.078, 1024 x 1,000,001 x 768 4.00 -> 1.91 ms).
+                        if (keep) {
+                            if (past_caches) __builtin_nontemporal_store(bits, (global_u32_t *)(row_base + lane_offset));
+                            else *(global_u32_t *)(row_base + lane_offset) = bits;
+                        }
                         row_base += (v % 4 == 3 ? 5 : 1) * row_step;
                         asm volatile("" : "+s"(row_base));
                     }
@@ -1542,21 +1576,22 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 }
             }
         };
-        if (nothing) {}
-        else if constexpr (NORMS) { // which distance is a run-time choice: one kernel serves both
-            if (late->metric == 2) {
-                if (interior) store_all(slot_c<0>(), slot_c<2>());
-                else store_all(slot_c<1>(), slot_c<2>());
+        auto store_as = [&](auto metric_tag) {
+            if (interior) {
+                if (NORMS || streamed) store_all(slot_c<0>(), metric_tag, slot_c<1>());
+                else if constexpr (!NORMS) store_all(slot_c<0>(), metric_tag, slot_c<0>());
             }
             else {
-                if (interior) store_all(slot_c<0>(), slot_c<1>());
-                else store_all(slot_c<1>(), slot_c<1>());
+                if (NORMS || streamed) store_all(slot_c<1>(), metric_tag, slot_c<1>());
+                else if constexpr (!NORMS) store_all(slot_c<1>(), metric_tag, slot_c<0>());
             }
+        };
+        if (nothing) {}
+        else if constexpr (NORMS) { // which distance is a run-time choice: one kernel serves both
+            if (late->metric == 2) store_as(slot_c<2>());
+            else store_as(slot_c<1>());
         }
-        else {
-            if (interior) store_all(slot_c<0>(), slot_c<0>());
-            else store_all(slot_c<1>(), slot_c<0>());
-        }
+        else store_as(slot_c<0>());
     }
 }
 
@@ -1650,7 +1685,8 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
         g.stagger_ticks = (uint32_t)(round_bytes / 5.5e12 * 1e8);
     }
     int const forced = forced_tile_config();
-    if (forced >> 8) g.stagger_ticks = (uint32_t)(forced >> 8) - 1; // (test hook: bits 8.. = ticks + 1)
+    if ((forced >> 8) & 0xFFFFF) g.stagger_ticks = (uint32_t)((forced >> 8) & 0xFFFFF) - 1; // (test hook: bits 8..27 = ticks + 1)
+    g.store_policy = (uint32_t)(forced >> 28) & 3;                                          // (test hook: bits 28..29)
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, stream, g);
     return hipGetLastError();
 }

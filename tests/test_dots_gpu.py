@@ -120,6 +120,20 @@ def test_small_shapes_every_tile_config(oracle, dtype, config):
         check(oracle, dtype, a, b, config, f"{dtype} {m}x{n}x{k} config {config}")
 
 
+@pytest.mark.parametrize("dtype", ["i8", "u8", "bf16", "e4m3"])
+@pytest.mark.parametrize("store", [1, 2])
+def test_both_kinds_of_store(oracle, dtype, store):
+    """Outputs stored past the caches (what rows of C on 128-byte lines get) and through them (what other rows get),
+    each forced (bits 28..29 of the test hook) over whole tiles and edge tiles of aligned and unaligned rows."""
+    rng = np.random.default_rng(300 + store)
+    for config, (m, n, k) in ((4, (200, 300, 260)), (4, (192, 256, 128)), (3, (260, 257, 130)), (2, (300, 544, 200)), (0, (130, 96, 70))):
+        if config == 1 and dtype not in ("i8", "u8"):
+            continue
+        a = support.random_matrix(oracle, dtype, m, k, rng)
+        b = support.random_matrix(oracle, dtype, n, k, rng)
+        check(oracle, dtype, a, b, config | (store << 28), f"{dtype} {m}x{n}x{k} config {config} store {store}")
+
+
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
 def test_float_input_families(oracle, dtype):
     rng = np.random.default_rng(5)
