@@ -1104,10 +1104,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     auto add_row_norm = [&](int i, norm_t value, uint32_t set) {
         __hip_atomic_fetch_add(&norm_part[set + i * NT + tid], value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
-    // u8 only: the stages of a tile that fetch nothing past its end run in a loop of their own, without the scalar work of
-    // choosing between this tile's descriptors and the next one's (measured: u8 1024 x 1,048,576 x 768 1.69 -> 1.45 ms,
-    // u8 8192^3 0.53 -> 0.50 ms; the other types lose 1-9 % to the second copy of the loop, so they keep the single one).
-    constexpr bool kPeel = T::kUnsigned;
     v4i a_reg[2][kLoads];
     v4i b_reg[2][TN][4];
     v4i af[2][TM];
@@ -1314,13 +1310,10 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // One stage of the steady state; `P` = stage parity = LDS buffer = register slot. Stages s+2 and
     // s+3 are fetched here; past the tile's end they are the first stages of `nxt` (the next tile, or
     // this one again when nothing follows: loads of valid memory that nobody uses).
-    // `wrap_tag`: 0 for a stage with three more stages of its tile behind it (kPeel): everything it fetches is this
-    // tile's, and the choice between the two tiles' descriptors is left out.
     // DEFER: behind k-step q of a tile's stage s < 4, eight results of block 2 s + q / 2 of the held tile are stored
     // (the block has to be known at compile time: s is P or P + 2).
-    auto stage = [&](auto parity_tag, uint32_t s, auto wrap_tag) {
+    auto stage = [&](auto parity_tag, uint32_t s) {
         constexpr int P = decltype(parity_tag)::value;
-        constexpr bool may_wrap = decltype(wrap_tag)::value != 0 || !kPeel;
         auto drain_behind = [&](auto q_tag) {
             constexpr int q = decltype(q_tag)::value;
             if constexpr (DEFER) {
@@ -1333,21 +1326,21 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         };
         // vector operations behind each MFMA of the k-steps that widen in place: their share of half the chunks
         constexpr int kSpread = T::kPrewiden ? (kLoads * 28 + TM * TN - 1) / (TM * TN) : 0;
-        bool const wrap2 = may_wrap && s + 2 >= fast, wrap3 = may_wrap && s + 3 >= fast;
+        bool const wrap2 = s + 2 >= fast, wrap3 = s + 3 >= fast;
         uint32_t const s2 = wrap2 ? s + 2 - fast : s + 2, s3 = wrap3 ? s + 3 - fast : s + 3;
         TileView const &a2 = wrap2 ? nxt : cur, &a3 = wrap3 ? nxt : cur, &b2 = a2;
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
         multiply(slot_c<P>(), slot_c<0>());
         load_b(b2, s2, slot_c<P>(), slot_c<0>()), load_a(a2, s2, slot_c<P>(), slot_c<2>());
-        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), !may_wrap || s + 1 < fast ? s + 1 : 0u, slot_c<0>());
+        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<0>());
         schedule_k_step(slot_c<0>(), slot_c<kSpread>());
         drain_behind(slot_c<0>());
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
         multiply(slot_c<P>(), slot_c<1>());
         load_b(b2, s2, slot_c<P>(), slot_c<1>()), load_a(a2, s2, slot_c<P>(), slot_c<3>());
-        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), !may_wrap || s + 1 < fast ? s + 1 : 0u, slot_c<1>());
+        if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<1>());
         schedule_k_step(slot_c<0>(), slot_c<kSpread>());
         drain_behind(slot_c<1>());
         __builtin_amdgcn_sched_barrier(0);
@@ -1356,7 +1349,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         load_b(b2, s2, slot_c<P>(), slot_c<2>());
         // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
         // at the previous barrier); then its registers start being refilled with A(s+3).
-        bool const mine = !may_wrap || s + 1 < fast;
+        bool const mine = s + 1 < fast;
         store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), mine ? s + 1 : 0u, mine ? 1u : 0u, slot_c<T::kPrewiden ? 1 : 0>());
         load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
         schedule_k_step(slot_c<1>(), slot_c<0>());
@@ -1431,15 +1424,9 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                         }
                     }
                 };
-                uint32_t s = 0;
-                for (; kPeel && s + 4 < fast; s += 2) { // (all but the last two pairs: nothing they fetch lies past the tile)
-                    stage(slot_c<0>(), s, slot_c<0>());
-                    stage(slot_c<1>(), s + 1, slot_c<0>());
-                    fold_when_due();
-                }
-                for (; s < fast; s += 2) {
-                    stage(slot_c<0>(), s, slot_c<1>());
-                    stage(slot_c<1>(), s + 1, slot_c<1>());
+                for (uint32_t s = 0; s < fast; s += 2) {
+                    stage(slot_c<0>(), s);
+                    stage(slot_c<1>(), s + 1);
                     fold_when_due();
                 }
                 __builtin_amdgcn_sched_barrier(0);

@@ -14,6 +14,14 @@
  *                                       accumulation of exact products (what the reference's kernels do,
  *                                       dot/serial.h:522-600) and to the same data widened to f16 on the f16 MFMA.
  *                                       --check exits non-zero unless the facts the kernels rely on hold.
+ *      mfma_probes budget               what the rest of a product kernel costs the i8 32 x 32 x 32 loop on a part that
+ *                                       runs at its power limit: idle cycles (s_sleep behind every 16 MFMAs), the
+ *                                       product kernel's LDS fragment reads (8 ds_read_b128 per 16 MFMAs), its global
+ *                                       loads (4 dwordx4 per 16 MFMAs, L2 hits, three iterations ahead), and all of
+ *                                       them; rate, shader clock and the share of cycles the MFMA pipe is busy.
+ *      mfma_probes stream               what the memory takes for the traffic of the retrieval shape (1024 x 1,048,576
+ *                                       x 768, i8 -> i32: 0.75 GiB read, 4 GiB written) with no arithmetic at all:
+ *                                       only written, only read, and both at once by separate workgroups.
  *
  *  Built by the Makefile next to the library (numkong_amd/lib/mfma_probes); bench.py runs the first mode and reports
  *  it under `others.mfma_ceiling`, tests/test_mfma_numerics_gpu.py runs the second.
@@ -229,6 +237,186 @@ static int ceiling_mode(bool json) {
 
 #pragma endregion Ceiling
 
+#pragma region Budget
+
+/**
+ *  The MFMA loop of the 256 x 256 i8 tile (8 x 2 blocks per wavefront) with parts of the product kernel's other work:
+ *  LOADS global dwordx4 loads per 16 MFMAs, issued three iterations ahead into a ring of registers, the first two
+ *  feeding B (all wander over 2 MiB: L2 hits); READS ds_read_b128 per 16 MFMAs, issued one iteration ahead, feeding A;
+ *  SLEEP x 64 idle cycles behind every 16 MFMAs.
+ */
+template <int LOADS, int READS, int SLEEP>
+__global__ __launch_bounds__(256) void budget_kernel(v4i const *operands, int iterations, float *sink, unsigned long long *clocks, v4i const *stream, unsigned stream_mask) {
+    __shared__ v4i lds[4096];
+    for (int i = threadIdx.x; i < 4096; i += 256) lds[i] = operands[i % 1024];
+    __syncthreads();
+    constexpr int RING = 4, L = LOADS > 0 ? LOADS : 1;
+    v4i a[2][8], g[RING][L], b[2];
+    unsigned const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = 0; i < 8; ++i) a[0][i] = a[1][i] = operands[(i * 64 + lane) % 1024];
+    for (int j = 0; j < 2; ++j) b[j] = operands[((8 + j) * 64 + lane) % 1024];
+    for (int r = 0; r < RING; ++r)
+        for (int l = 0; l < L; ++l) g[r][l] = b[l & 1];
+    v16i acc[8][2];
+    for (int i = 0; i < 8; ++i)
+        for (int j = 0; j < 2; ++j)
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+    unsigned long long const cycles0 = clock64(), ticks0 = wall_clock64();
+    unsigned at = (blockIdx.x * 4 + wave) * 64 * LOADS + lane;
+    for (int it = 0; it < iterations; it += RING) {
+#pragma unroll
+        for (int r = 0; r < RING; ++r) {
+            v4i operand_b[2] = {b[0], b[1]};
+            if constexpr (LOADS >= 2) operand_b[0] = g[r][0], operand_b[1] = g[r][1];
+            if constexpr (LOADS > 0) {
+#pragma unroll
+                for (int l = 0; l < LOADS; ++l) g[r][l] = stream[(at + l * 64) & stream_mask];
+                at += 256 * 4 * 64 * LOADS;
+            }
+            if constexpr (READS > 0) {
+#pragma unroll
+                for (int i = 0; i < READS; ++i) a[(r + 1) & 1][i] = lds[(((it + r) & 7) * 512 + i * 64 + lane) & 4095];
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[r & 1][i], operand_b[j], acc[i][j], 0, 0, 0);
+            if constexpr (SLEEP > 0) __builtin_amdgcn_s_sleep(SLEEP);
+        }
+    }
+    unsigned long long const cycles1 = clock64(), ticks1 = wall_clock64();
+    float total = 0;
+    for (int i = 0; i < 8; ++i)
+        for (int j = 0; j < 2; ++j) total += (float)acc[i][j][0];
+    sink[blockIdx.x * 256 + threadIdx.x] = total;
+    if (threadIdx.x == 0) clocks[2 * blockIdx.x] = cycles1 - cycles0, clocks[2 * blockIdx.x + 1] = ticks1 - ticks0;
+}
+
+template <class Kernel>
+static void run_budget(char const *name, Kernel kernel, int units, v4i *operands, float *sink, unsigned long long *clocks, v4i *stream, unsigned mask) {
+    int const iterations = 1500;
+    hipEvent_t begin, end;
+    CHECK(hipEventCreate(&begin));
+    CHECK(hipEventCreate(&end));
+    for (int warm = 0; warm < 20; ++warm) hipLaunchKernelGGL(kernel, dim3(units), dim3(256), 0, 0, operands, iterations, sink, clocks, stream, mask);
+    CHECK(hipEventRecord(begin, 0));
+    for (int launch = 0; launch < 20; ++launch) hipLaunchKernelGGL(kernel, dim3(units), dim3(256), 0, 0, operands, iterations, sink, clocks, stream, mask);
+    CHECK(hipEventRecord(end, 0));
+    CHECK(hipEventSynchronize(end));
+    CHECK(hipGetLastError());
+    float ms = 0;
+    CHECK(hipEventElapsedTime(&ms, begin, end));
+    ms /= 20;
+    std::vector<unsigned long long> host_clocks(2 * units);
+    CHECK(hipMemcpy(host_clocks.data(), clocks, host_clocks.size() * 8, hipMemcpyDeviceToHost));
+    double cycles = 0, ticks = 0;
+    for (int unit = 0; unit < units; ++unit) cycles += (double)host_clocks[2 * unit], ticks += (double)host_clocks[2 * unit + 1];
+    double const tops = 65536.0 * 16 * iterations * 4 * units / (ms * 1e-3) / 1e12;
+    printf("%-58s %8.4f %9.1f %8.3f %8.0f %9.0f %%\n", name, ms, tops, tops / 5000, cycles / ticks * 100.0, 3200.0 * 16 * iterations * units / cycles);
+    CHECK(hipEventDestroy(begin));
+    CHECK(hipEventDestroy(end));
+}
+
+static int budget_mode() {
+    hipDeviceProp_t properties;
+    CHECK(hipGetDeviceProperties(&properties, 0));
+    int const units = properties.multiProcessorCount;
+    v4i *operands, *stream;
+    float *sink;
+    unsigned long long *clocks;
+    size_t const stream_bytes = 2u << 20;
+    CHECK(hipMalloc(&operands, 16384));
+    CHECK(hipMalloc(&stream, stream_bytes));
+    CHECK(hipMalloc(&sink, (size_t)units * 256 * 4));
+    CHECK(hipMalloc(&clocks, (size_t)units * 16));
+    std::vector<uint8_t> data(stream_bytes);
+    for (size_t at = 0; at < data.size(); ++at) data[at] = (uint8_t)next_random();
+    CHECK(hipMemcpy(operands, data.data(), 16384, hipMemcpyHostToDevice));
+    CHECK(hipMemcpy(stream, data.data(), stream_bytes, hipMemcpyHostToDevice));
+    unsigned const mask = (unsigned)(stream_bytes / 16 - 1);
+    printf("i8 32x32x32 MFMA loop on random data with parts of a product kernel's other work, %d compute units (%s), 4 wavefronts each\n", units, properties.gcnArchName);
+    printf("%-58s %8s %9s %8s %8s %10s\n", "per 16 MFMAs of a wavefront", "ms", "TOP/s", "of peak", "MHz", "MFMA busy");
+    run_budget("nothing else", budget_kernel<0, 0, 0>, units, operands, sink, clocks, stream, mask);
+    run_budget("64 idle cycles", budget_kernel<0, 0, 1>, units, operands, sink, clocks, stream, mask);
+    run_budget("128 idle cycles", budget_kernel<0, 0, 2>, units, operands, sink, clocks, stream, mask);
+    run_budget("256 idle cycles", budget_kernel<0, 0, 4>, units, operands, sink, clocks, stream, mask);
+    run_budget("512 idle cycles", budget_kernel<0, 0, 8>, units, operands, sink, clocks, stream, mask);
+    run_budget("4 ds_read_b128", budget_kernel<0, 4, 0>, units, operands, sink, clocks, stream, mask);
+    run_budget("8 ds_read_b128 (the product kernel's)", budget_kernel<0, 8, 0>, units, operands, sink, clocks, stream, mask);
+    run_budget("2 global dwordx4 loads", budget_kernel<2, 0, 0>, units, operands, sink, clocks, stream, mask);
+    run_budget("4 global dwordx4 loads (the product kernel's)", budget_kernel<4, 0, 0>, units, operands, sink, clocks, stream, mask);
+    run_budget("8 ds_read_b128 and 4 global loads", budget_kernel<4, 8, 0>, units, operands, sink, clocks, stream, mask);
+    run_budget("8 ds_read_b128, 4 global loads, 128 idle cycles", budget_kernel<4, 8, 2>, units, operands, sink, clocks, stream, mask);
+    run_budget("nothing else (again)", budget_kernel<0, 0, 0>, units, operands, sink, clocks, stream, mask);
+    return 0;
+}
+
+#pragma endregion Budget
+
+#pragma region Stream
+
+/** `readers_of_8` of every 8 workgroups read `source` once between them, the others write `target` once between them. */
+__global__ __launch_bounds__(256) void stream_kernel(v4i const *source, size_t source_vectors, v4i *target, size_t target_vectors, int readers_of_8, int *sink, int past_caches) {
+    bool const reader = (int)(blockIdx.x % 8) < readers_of_8;
+    uint32_t const share = reader ? readers_of_8 : 8 - readers_of_8;
+    uint32_t const index = blockIdx.x / 8 * share + (reader ? blockIdx.x % 8 : blockIdx.x % 8 - readers_of_8);
+    size_t const count = (size_t)(gridDim.x / 8) * share;
+    if (reader) {
+        v4i mix = {0, 0, 0, 0};
+        for (size_t at = (size_t)index * 256 + threadIdx.x; at < source_vectors; at += count * 256 * 4) {
+            v4i loaded[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) loaded[u] = at + u * count * 256 < source_vectors ? __builtin_nontemporal_load(source + at + u * count * 256) : mix;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) mix ^= loaded[u];
+        }
+        if (mix[0] == 0x12345678) sink[threadIdx.x] = mix[1];
+    }
+    else {
+        v4i const value = {(int)blockIdx.x, 1, 2, 3};
+        for (size_t at = (size_t)index * 256 + threadIdx.x; at < target_vectors; at += count * 256) {
+            if (past_caches) __builtin_nontemporal_store(value, target + at);
+            else target[at] = value;
+        }
+    }
+}
+
+static int stream_mode() {
+    size_t const read_bytes = (size_t)768 << 20, written_bytes = (size_t)4 << 30; // B and C of 1024 x 1,048,576 x 768, i8 -> i32
+    v4i *source, *target;
+    int *sink;
+    CHECK(hipMalloc(&source, read_bytes));
+    CHECK(hipMalloc(&target, written_bytes));
+    CHECK(hipMalloc(&sink, 4096));
+    CHECK(hipMemset(source, 1, read_bytes));
+    hipEvent_t begin, end;
+    CHECK(hipEventCreate(&begin));
+    CHECK(hipEventCreate(&end));
+    printf("0.75 GiB read and 4 GiB written by 8192 workgroups of linear 16-byte accesses, 5 launches after 2\n%-44s %8s %8s %12s\n", "", "ms", "GB/s", "of 8 TB/s");
+    for (int past_caches = 1; past_caches >= 0; --past_caches)
+        for (int readers : {0, 8, 2}) {
+            if (readers == 8 && !past_caches) continue;
+            for (int launch = 0; launch < 7; ++launch) {
+                if (launch == 2) CHECK(hipEventRecord(begin, 0));
+                hipLaunchKernelGGL(stream_kernel, dim3(8192), dim3(256), 0, 0, source, read_bytes / 16, target, written_bytes / 16, readers, sink, past_caches);
+            }
+            CHECK(hipEventRecord(end, 0));
+            CHECK(hipEventSynchronize(end));
+            CHECK(hipGetLastError());
+            float ms = 0;
+            CHECK(hipEventElapsedTime(&ms, begin, end));
+            ms /= 5;
+            double const bytes = (readers ? (double)read_bytes : 0) + (readers < 8 ? (double)written_bytes : 0);
+            char name[96];
+            snprintf(name, sizeof name, "%s%s", readers == 0 ? "written only" : (readers == 8 ? "read only" : "both (2 of 8 workgroups read)"),
+                     readers == 8 ? "" : (past_caches ? ", stores past the caches" : ", plain stores"));
+            printf("%-44s %8.3f %8.0f %12.3f\n", name, ms, bytes / ms / 1e6, bytes / ms / 1e6 / 8000);
+        }
+    return 0;
+}
+
+#pragma endregion Stream
+
 #pragma region Numerics
 
 enum Mode { kLegacyFP8, kLegacyBF8, kScaledFP8, kScaledBF8, kHalf, kBrain, kModes };
@@ -417,6 +605,8 @@ int main(int argc, char **argv) {
     for (int i = 2; i < argc; ++i) json |= !strcmp(argv[i], "--json"), check |= !strcmp(argv[i], "--check");
     if (argc >= 2 && !strcmp(argv[1], "ceiling")) return ceiling_mode(json);
     if (argc >= 2 && !strcmp(argv[1], "numerics")) return numerics_mode(check);
-    fprintf(stderr, "usage: %s ceiling [--json] | numerics [--check]\n", argv[0]);
+    if (argc >= 2 && !strcmp(argv[1], "budget")) return budget_mode();
+    if (argc >= 2 && !strcmp(argv[1], "stream")) return stream_mode();
+    fprintf(stderr, "usage: %s ceiling [--json] | numerics [--check] | budget | stream\n", argv[0]);
     return 2;
 }
