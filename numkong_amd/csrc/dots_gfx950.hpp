@@ -983,9 +983,8 @@ constexpr bool tail_matters_for() {
     return NORMS || T::kUnsigned || !__is_same(typename T::acc_t, v16i);
 }
 
-template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, bool WHOLE = false, bool DEFER = false>
+template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, bool WHOLE = false>
 __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChunked ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
-    static_assert(!DEFER || (ACROSS && !NORMS && !T::kChunked && !T::kUnsigned && TM * TN == 8), "deferred stores: plain integer products, 8 blocks per wavefront");
     typedef typename T::acc_t acc_t;
     constexpr int BM = TM * 32;
     constexpr int NT = 256;
@@ -1130,33 +1129,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     }
     TileView cur, nxt;
     acc_t acc[TM][TN];
-    // DEFER: a finished tile's results move to a second set of registers and are stored during the first four stages
-    // of the workgroup's next tile, eight stores behind every k-step (at least four stages: the host checked), instead of all at once at the end of
-    // the tile. A shallow product is bound by its stores; issued in one go they fill the memory pipeline, the loads
-    // of the next tile queue behind them (vector memory operations of a wavefront complete in order) and its MFMAs
-    // wait (measured: 16 us for the six stages of a 256 x 256 x 768 tile whose MFMAs take 6). The stores go through
-    // a buffer descriptor of the held tile: its scalar offset operand takes the row, one scalar add per store.
-    acc_t held[DEFER ? TM : 1][DEFER ? TN : 1];
-    uint64_t held_at = 0;  // this wavefront's corner of the held tile in C
-    bool holding = false;  // (a tile on the matrix edge is stored at its end, through the masked stores, and not held)
-    uint32_t const c_stride32 = __builtin_amdgcn_readfirstlane((uint32_t)g.c_stride); // (DEFER: the host checked that BM rows of C span less than 4 GiB)
-    uint32_t const store_lane = 4 * (lane >> 5) * c_stride32 + (lane & 31) * 4;
-    auto drain = [&](auto block_tag, auto half_tag) {
-        constexpr int block = decltype(block_tag)::value, eight = decltype(half_tag)::value;
-        constexpr int i = block % TM, j = block / TM;
-        __amdgpu_buffer_rsrc_t const rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)held_at, 0, -1, 0x00020000);
-        // Rows come in runs of 4 that start 8 apart (register v: row 8 * (v / 4) + v % 4 of lanes 0..31; lanes 32..63 are
-        // 4 rows below, which store_lane holds). A running scalar offset: the empty asm keeps the compiler from working
-        // out all the offsets of a tile ahead of time, which the scalar registers have no room for.
-        uint32_t offset = (uint32_t)(i * 32 + 16 * eight) * c_stride32 + j * 128;
-#pragma unroll
-        for (int v = 8 * eight; v < 8 * eight + 8; ++v) {
-            int const element = held[DEFER ? i : 0][DEFER ? j : 0][v];
-            __builtin_amdgcn_raw_buffer_store_b32(element, rsrc, store_lane, offset, 2 /* nt */);
-            offset += (v % 4 == 3 ? 5 : 1) * c_stride32;
-            asm volatile("" : "+s"(offset));
-        }
-    };
     constexpr bool kChunked = T::kChunked;
     Totals<acc_t, TM, TN, kChunked> total; // second-level accumulators of the chunked types (see E4M3)
 
@@ -1303,27 +1275,15 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                     __builtin_amdgcn_sched_group_barrier(0x020, loads > rest ? loads : 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 if constexpr (vector > 0) __builtin_amdgcn_sched_group_barrier(0x002, vector, 0);
-                }
+            }
             if (writes && kLoads > rest) __builtin_amdgcn_sched_group_barrier(0x200, kLoads - rest, 0);
         }
     };
     // One stage of the steady state; `P` = stage parity = LDS buffer = register slot. Stages s+2 and
     // s+3 are fetched here; past the tile's end they are the first stages of `nxt` (the next tile, or
     // this one again when nothing follows: loads of valid memory that nobody uses).
-    // DEFER: behind k-step q of a tile's stage s < 4, eight results of block 2 s + q / 2 of the held tile are stored
-    // (the block has to be known at compile time: s is P or P + 2).
     auto stage = [&](auto parity_tag, uint32_t s) {
         constexpr int P = decltype(parity_tag)::value;
-        auto drain_behind = [&](auto q_tag) {
-            constexpr int q = decltype(q_tag)::value;
-            if constexpr (DEFER) {
-                __builtin_amdgcn_sched_barrier(0);
-                if (holding) {
-                    if (s == (uint32_t)P) drain(slot_c<2 * P + q / 2>(), slot_c<q % 2>());
-                    else if (s == (uint32_t)P + 2) drain(slot_c<2 * (P + 2) + q / 2>(), slot_c<q % 2>());
-                }
-            }
-        };
         // vector operations behind each MFMA of the k-steps that widen in place: their share of half the chunks
         constexpr int kSpread = T::kPrewiden ? (kLoads * 28 + TM * TN - 1) / (TM * TN) : 0;
         bool const wrap2 = s + 2 >= fast, wrap3 = s + 3 >= fast;
@@ -1335,14 +1295,12 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         load_b(b2, s2, slot_c<P>(), slot_c<0>()), load_a(a2, s2, slot_c<P>(), slot_c<2>());
         if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<0>());
         schedule_k_step(slot_c<0>(), slot_c<kSpread>());
-        drain_behind(slot_c<0>());
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
         multiply(slot_c<P>(), slot_c<1>());
         load_b(b2, s2, slot_c<P>(), slot_c<1>()), load_a(a2, s2, slot_c<P>(), slot_c<3>());
         if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<1>());
         schedule_k_step(slot_c<0>(), slot_c<kSpread>());
-        drain_behind(slot_c<1>());
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
         multiply(slot_c<P>(), slot_c<2>());
@@ -1353,7 +1311,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), mine ? s + 1 : 0u, mine ? 1u : 0u, slot_c<T::kPrewiden ? 1 : 0>());
         load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
         schedule_k_step(slot_c<1>(), slot_c<0>());
-        drain_behind(slot_c<2>());
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
@@ -1361,7 +1318,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         multiply(slot_c<P>(), slot_c<3>());
         load_b(b2, s2, slot_c<P>(), slot_c<3>()), load_a(a3, s3, slot_c<P ^ 1>(), slot_c<1>());
         schedule_k_step(slot_c<0>(), slot_c<0>());
-        drain_behind(slot_c<3>());
     };
 
     // Fills the pipeline for a tile: stages 0 and 1 on their way, A(0) in LDS, its first fragments read.
@@ -1607,24 +1563,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 }
             }
         };
-        if constexpr (DEFER) {
-            holding = false; // (whatever was held has been stored during this tile's stages)
-            if (interior && streamed) {
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) held[DEFER ? i : 0][DEFER ? j : 0] = acc[i][j];
-                uint64_t const corner = (uint64_t)late->c + (uint64_t)row0 * late->c_stride + (uint64_t)col0 * 4;
-                // (the same in every lane: said so, a descriptor built from it stays in scalar registers)
-                // (readfirstlane returns a signed int: through uint32_t, or a low word with its top bit set sign-extends
-                // over the high word, which is what made the first builds of this path fault)
-                uint32_t const corner_high = (uint32_t)__builtin_amdgcn_readfirstlane((int)(corner >> 32));
-                uint32_t const corner_low = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)corner);
-                held_at = ((uint64_t)corner_high << 32) | (uint64_t)corner_low;
-                holding = true;
-                continue;
-            }
-        }
         auto store_as = [&](auto metric_tag) {
             if (interior) {
                 if (NORMS || streamed) store_all(slot_c<0>(), metric_tag, slot_c<1>());
@@ -1642,21 +1580,11 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         }
         else store_as(slot_c<0>());
     }
-    if (DEFER && holding) { // the last tile's results
-        drain(slot_c<0>(), slot_c<0>()), drain(slot_c<0>(), slot_c<1>()), drain(slot_c<1>(), slot_c<0>()), drain(slot_c<1>(), slot_c<1>());
-        drain(slot_c<2>(), slot_c<0>()), drain(slot_c<2>(), slot_c<1>()), drain(slot_c<3>(), slot_c<0>()), drain(slot_c<3>(), slot_c<1>());
-        drain(slot_c<4>(), slot_c<0>()), drain(slot_c<4>(), slot_c<1>()), drain(slot_c<5>(), slot_c<0>()), drain(slot_c<5>(), slot_c<1>());
-        drain(slot_c<6>(), slot_c<0>()), drain(slot_c<6>(), slot_c<1>()), drain(slot_c<7>(), slot_c<0>()), drain(slot_c<7>(), slot_c<1>());
-    }
 }
 
 struct TileConfig {
     int tm, tn;
 };
-constexpr uint32_t kDeferStages = 16; // deepest product (in stages of 128 bytes per row) whose stores are deferred
-// SWITCHED OFF: the deferred-store kernels (DEFER) are not built. Their first two builds faulted on the GPU (an address
-// assembled from a sign-extended low word, since corrected in the source above); the corrected build has not run yet.
-constexpr bool kDeferredStores = false;
 // Index 0 is "choose for me"; 1.. are explicit (5: e2m3 only).
 constexpr TileConfig kConfigs[] = {{0, 0}, {8, 2}, {4, 2}, {4, 1}, {2, 1}, {4, 4}};
 constexpr int kConfigCount = sizeof(kConfigs) / sizeof(kConfigs[0]);
@@ -1718,19 +1646,10 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
         if (norms && whole) kernel = dots_packed_kernel<T, TM, TN, true, true, true>;
     }
     else if (norms) return hipErrorInvalidValue;
-    // Shallow integer products of many tiles, rows of C on 128-byte lines: the results of a tile are stored under the
-    // MFMAs of the workgroup's next one (see DEFER in the kernel).
-    bool defer = false;
-    if constexpr (kDeferredStores && T::kDtype == kI8 && TM == 4 && TN == 2) {
-        bool const lines = (((uint64_t)(uintptr_t)g.c | g.c_stride) & 127) == 0;
-        defer = across && !norms && !triangle && lines && stages <= kDeferStages && tiles >= 4 * 256 &&
-                (uint64_t)BM * g.c_stride <= 0xFFFFFFFFull && (((forced_tile_config() >> 28) & 3) == 0);
-        if (defer) kernel = dots_packed_kernel<T, TM, TN, true, false, false, true>;
-    }
     // Persistent grid: as many workgroups as fit on the device at once (queried once per kernel; threads that
     // ask at the same time store the same number).
-    static std::atomic<int> resident_of[16];
-    std::atomic<int> &slot = resident_of[(across ? 1 : 0) + (norms ? 2 : 0) + (whole ? 4 : 0) + (defer ? 8 : 0)];
+    static std::atomic<int> resident_of[8];
+    std::atomic<int> &slot = resident_of[(across ? 1 : 0) + (norms ? 2 : 0) + (whole ? 4 : 0)];
     int resident = slot.load(std::memory_order_relaxed);
     if (!resident) {
         int per_cu = 0;
