@@ -369,6 +369,8 @@ def main():
     parser.add_argument("--no-cpu", action="store_true")
     parser.add_argument("--no-vendor", action="store_true", help="skip the vendor GEMM timings (others.vendor_*)")
     parser.add_argument("--no-ceiling", action="store_true", help="skip the MFMA-only loop (others.mfma_ceiling)")
+    parser.add_argument("--vendor-probe", action="store_true",
+                        help="for rocprofv3 runs: the vendor library's GEMM for --dtype (i8, bf16, f16) and --shape, 10 launches after 5, nothing else")
     parser.add_argument("--probe", action="store_true",
                         help="for rocprofv3 --pmc runs: launch a plain 1 GiB elementwise copy kernel 3 times, then the selected product 3 times, nothing else")
     args = parser.parse_args()
@@ -380,6 +382,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     m, n, k = args.shape
+    if args.vendor_probe:
+        print(json.dumps({f"vendor_{args.dtype}_{m}x{n}x{k}": time_vendor(args.dtype, m, n, k, 10, 5)}))
+        return
     if args.probe:
         source = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").fill_(1)
         target = torch.empty_like(source)
