@@ -1249,6 +1249,12 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[q & 1][i], b);
         }
     };
+    // What staging one chunk of A costs besides its LDS write: vector operations (u8: four exclusive-ors and the byte
+    // sums; the distance kinds: the squares) and LDS adds (one per sum kept). The k-step that stages asks for them
+    // behind its MFMAs, a chunk's worth each; left alone they all land between the last MFMA and the barrier.
+    constexpr bool kIntegerSums = __is_same(typename T::acc_t, v16i);
+    constexpr int kStageVector = (T::kUnsigned ? 8 : 0) + (NORMS ? (kIntegerSums ? 5 : 28) : 0);
+    constexpr int kStageDs = 1 + (T::kUnsigned ? 1 : 0) + (NORMS ? 1 : 0);
     // Scheduling hints for one k-step. Masks: 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write.
     // Fragment reads go one-to-one with the first TM MFMAs; the global loads of the k-step (TN of B
     // and a quarter of A) are spread over the remaining MFMAs; k-step 2 also carries the LDS writes.
@@ -1265,6 +1271,20 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         }
         if constexpr (rest == 0) {
             if (writes) __builtin_amdgcn_sched_group_barrier(0x200, kLoads, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, loads, 0);
+        }
+        else if constexpr (writes && kStageDs > 1) {
+            // The LDS adds are atomics, and the compiler keeps atomics in program order with every other memory
+            // operation, this k-step's loads included (which cannot go early anyway: the second half of the MFMAs
+            // still reads the registers that B's loads refill). So the stage's k-step 2 stages first in program order,
+            // a chunk in front of each MFMA of the second half, and all its loads go behind the last MFMA.
+#pragma unroll
+            for (int i = 0; i < rest; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if constexpr (vector > 0) __builtin_amdgcn_sched_group_barrier(0x002, vector, 0);
+                if (i < kLoads) __builtin_amdgcn_sched_group_barrier(0x080, kStageDs, 0); // (0x080: any LDS operation)
+            }
+            if (kLoads > rest) __builtin_amdgcn_sched_group_barrier(0x080, kStageDs * (kLoads - rest), 0);
             __builtin_amdgcn_sched_group_barrier(0x020, loads, 0);
         }
         else {
@@ -1304,13 +1324,14 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<3>(), slot_c<1>());
         multiply(slot_c<P>(), slot_c<2>());
-        load_b(b2, s2, slot_c<P>(), slot_c<2>());
+        if constexpr (kStageDs == 1) load_b(b2, s2, slot_c<P>(), slot_c<2>());
         // A(s+1), loaded over the last two stages, goes to the other buffer (every wavefront left it
         // at the previous barrier); then its registers start being refilled with A(s+3).
         bool const mine = s + 1 < fast;
         store_a(slot_c<P ^ 1>(), slot_c<P ^ 1>(), mine ? s + 1 : 0u, mine ? 1u : 0u, slot_c<T::kPrewiden ? 1 : 0>());
+        if constexpr (kStageDs > 1) load_b(b2, s2, slot_c<P>(), slot_c<2>()); // (see schedule_k_step)
         load_a(a3, s3, slot_c<P ^ 1>(), slot_c<0>());
-        schedule_k_step(slot_c<1>(), slot_c<0>());
+        schedule_k_step(slot_c<1>(), slot_c<kStageVector>());
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
