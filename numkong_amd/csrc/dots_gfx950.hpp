@@ -1567,10 +1567,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                             // a vector's distance from itself is exactly 0 (dots/serial.h:2871-2876)
                             if (metric != 0 && r_fixed - j * 32 == diagonal) bits = 0;
                         }
-                        // Whole tiles of whole lines go past the caches. Anything else is left to the L2 to put together:
-                        // a 128-byte run of a row that straddles two lines would reach the memory as two partial
-                        // writes (measured, i8, C rows of 8191 and 1,000,001 columns: 8192 x 8191 x 1000 0.218 -> 0.147
-                        // ms, 4096 x 4095 x 4096 0.116 -> 0.078, 1024 x 1,000,001 x 768 4.00 -> 1.91 ms).
                         if (keep) {
                             if (past_caches) __builtin_nontemporal_store(bits, (global_u32_t *)(row_base + lane_offset));
                             else *(global_u32_t *)(row_base + lane_offset) = bits;
