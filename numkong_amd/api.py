@@ -10,6 +10,11 @@ Reference behaviour mirrored here (python/matrix.c):
 
 There is no CPU fallback: if the shared library is missing, loading raises; if a call fails on the
 GPU side, ``NumKongAmdError`` is raised with the library's own message.
+
+Streams: the synchronous calls run on streams the library keeps per host thread. They are blocking streams, so they
+are ordered behind work queued on the legacy default stream (torch's default) and return when the result is
+complete; operands produced on a non-blocking stream of the caller's must be synchronised first, or the ``*_async``
+entry points used with that stream.
 """
 from __future__ import annotations
 
