@@ -392,7 +392,7 @@ static int stream_mode() {
     hipEvent_t begin, end;
     CHECK(hipEventCreate(&begin));
     CHECK(hipEventCreate(&end));
-    printf("0.75 GiB read and 4 GiB written by 8192 workgroups of linear 16-byte accesses, 5 launches after 2\n%-44s %8s %8s %12s\n", "", "ms", "GB/s", "of 8 TB/s");
+    printf("0.75 GiB read and 4 GiB written by 8192 workgroups of linear 16-byte accesses, 5 launches after 2\n%-58s %8s %8s %12s\n", "", "ms", "GB/s", "of 8 TB/s");
     for (int past_caches = 1; past_caches >= 0; --past_caches)
         for (int readers : {0, 8, 2}) {
             if (readers == 8 && !past_caches) continue;
@@ -410,7 +410,7 @@ static int stream_mode() {
             char name[96];
             snprintf(name, sizeof name, "%s%s", readers == 0 ? "written only" : (readers == 8 ? "read only" : "both (2 of 8 workgroups read)"),
                      readers == 8 ? "" : (past_caches ? ", stores past the caches" : ", plain stores"));
-            printf("%-44s %8.3f %8.0f %12.3f\n", name, ms, bytes / ms / 1e6, bytes / ms / 1e6 / 8000);
+            printf("%-58s %8.3f %8.0f %12.3f\n", name, ms, bytes / ms / 1e6, bytes / ms / 1e6 / 8000);
         }
     return 0;
 }
