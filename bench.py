@@ -62,6 +62,7 @@ def measured_traffic(*key):
 
 _TRAFFIC = None
 HEADLINE = ("i8", 8192, 8192, 8192)
+METRIC_DTYPES = ("i8", "bf16", "e4m3")  # the three types BASELINE's metric names, all at the headline shape
 OTHERS = [("bf16", 8192, 8192, 8192, "dots"), ("e4m3", 8192, 8192, 8192, "dots"), ("e5m2", 8192, 8192, 8192, "dots"),
           ("f16", 8192, 8192, 8192, "dots"), ("i8", 8192, 8191, 1000, "dots"), ("f16", 8192, 8191, 1000, "dots"),
           ("bf16", 4096, 4096, 4096, "dots"), ("i8", 2048, 2048, 2048, "dots"),
@@ -248,6 +249,52 @@ def time_gpu(dtype, m, n, k, steps, warmup, metric="dots"):
     return result
 
 
+def time_sync_abi(dtype, m, n, k, calls=200):
+    """The reference-ABI symbol itself (`nk_dots_packed_<T>`: synchronous, pointers classified per call) on operands in
+    device memory: wall-clock per call, next to the device time of the same product through the asynchronous entry
+    point, so that what the drop-in symbol adds to a launch is a number."""
+    import torch
+
+    import numkong_amd as nk
+    from numkong_amd import api
+
+    lib = nk.library()
+    a, b = make_operands(dtype, m, n, k)
+    packed = nk.dots_pack(b, dtype)
+    c = torch.empty((m, n), dtype=torch.int32 if dtype in ("i8", "u8") else torch.float32, device="cuda:0")
+    code, row_bytes = api.DTYPES[dtype][0], a.shape[1] * a.element_size()
+    stream = torch.cuda.current_stream().cuda_stream
+    entry = getattr(lib, f"nk_dots_packed_{dtype}")
+    arguments = (a.data_ptr(), packed.buffer.data_ptr(), c.data_ptr(), m, n, k, row_bytes, n * 4)
+    for _ in range(20):
+        entry(*arguments)
+    torch.cuda.synchronize()
+    begin = time.perf_counter()
+    for _ in range(calls):
+        entry(*arguments)
+    sync_us = (time.perf_counter() - begin) * 1e6 / calls
+    if lib.nk_amd_last_error():
+        raise RuntimeError(lib.nk_amd_last_error().decode())
+
+    def step():
+        if lib.nk_amd_dots_packed_async(code, *arguments, stream):
+            raise RuntimeError(lib.nk_hip_last_error().decode())
+
+    _, times = timed_steps(step, calls, 20)
+    # the same asynchronous launch followed by a wait for it, as a caller of the synchronous symbol would otherwise write
+    begin = time.perf_counter()
+    for _ in range(calls):
+        step()
+        torch.cuda.current_stream().synchronize()
+    launch_and_wait_us = (time.perf_counter() - begin) * 1e6 / calls
+    del a, packed, c
+    torch.cuda.empty_cache()
+    return {"sync_wall_us_per_call": sync_us, "async_kernel_us": times["kernel_ms"] * 1e3,
+            "async_launch_and_wait_us": launch_and_wait_us, "sync_minus_kernel_us": sync_us - times["kernel_ms"] * 1e3,
+            "what": f"nk_dots_packed_{dtype} on device pointers, {calls} calls back to back, wall-clock per call; "
+                    "nk_amd_dots_packed_async's device time per launch; the asynchronous launch plus a stream wait, wall-clock"}
+
+
 def time_vendor(dtype, m, n, k, steps, warmup):
     """The vendor library's GEMM (hipBLASLt through torch) on operands of the same family in the same process: what
     this part gives a tuned kernel of the same shape. Timing only; nothing of it is used by the product."""
@@ -395,7 +442,45 @@ def main():
         time_gpu(args.dtype, m, n, k, 3, 0, args.metric)
         return
     head = time_gpu(args.dtype, m, n, k, args.steps, args.warmup, args.metric)
-    line = {
+    headline = (args.dtype, m, n, k, args.metric) == (*HEADLINE, "dots")
+    # The metric names three types at 8192^3: all three are timed with the full step count, and their figures ride
+    # inside `roofline` and `cpu_baseline` (`by_dtype`), next to the headline's.
+    def brief(r):
+        keep = {"kernel_ms": r["kernel_ms"], "kernel_ms_median": r["kernel_ms_median"], "kernel_ms_min": r["kernel_ms_min"],
+                "achieved": r["roofline"]["achieved"], "peak": r["roofline"]["peak"], "frac": r["roofline"]["frac"],
+                "traffic": r["roofline"]["traffic"]}
+        if "frac_f16" in r["roofline"]:
+            keep["frac_f16"] = r["roofline"]["frac_f16"]
+        return keep
+
+    metric_types = {}
+    if headline:
+        metric_types["i8"] = head
+        for dtype in METRIC_DTYPES[1:]:
+            metric_types[dtype] = time_gpu(dtype, m, n, k, args.steps, args.warmup, "dots")
+        head["roofline"]["by_dtype"] = {dtype: brief(r) for dtype, r in metric_types.items()}
+    line = {}
+    # (`others` goes first: it is long, and what a reader of the end of the line looks for comes after it)
+    if not args.no_others:
+        line["others"] = {}
+        for dtype, om, on, ok, metric in OTHERS:
+            if (dtype, om, on, ok, metric) in [(t, m, n, k, "dots") for t in metric_types]:
+                r = metric_types[dtype]
+            else:
+                r = time_gpu(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2), metric)
+            name = f"{dtype}_{on}x{ok}_{metric}" if metric in SYMMETRIC_KINDS else f"{dtype}_{om}x{on}x{ok}" + ("" if metric == "dots" else "_" + metric)
+            line["others"][name] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"], "kernel_ms_median": r["kernel_ms_median"],
+                                    "kernel_ms_min": r["kernel_ms_min"], "roofline": {key: value for key, value in r["roofline"].items() if key != "by_dtype"}}
+        for dtype, on, ok in PACKS:
+            line["others"][f"pack_{dtype}_{on}x{ok}"] = time_pack(dtype, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2))
+        line["others"]["sync_abi_i8_2048"] = time_sync_abi("i8", 2048, 2048, 2048)
+    if not args.no_vendor:
+        line.setdefault("others", {})
+        for dtype, om, on, ok in VENDOR:
+            line["others"][f"vendor_{dtype}_{om}x{on}x{ok}"] = time_vendor(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2))
+    if not args.no_ceiling:
+        line.setdefault("others", {})["mfma_ceiling"] = mfma_ceiling()
+    line.update({
         "metric": "gso/s and % MFMA peak: i8->i32, bf16->f32, e4m3->f32 packed dots at 8192^3",
         "value": head["gso_per_s"], "unit": "gso/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -406,24 +491,14 @@ def main():
                                 "B packed once outside the timed region, C overwritten")},
         "kernel_ms": head["kernel_ms"], "kernel_ms_median": head["kernel_ms_median"], "kernel_ms_min": head["kernel_ms_min"],
         "roofline": head["roofline"],
-    }
-    if not args.no_others:
-        line["others"] = {}
-        for dtype, om, on, ok, metric in OTHERS:
-            r = time_gpu(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2), metric)
-            name = f"{dtype}_{on}x{ok}_{metric}" if metric in SYMMETRIC_KINDS else f"{dtype}_{om}x{on}x{ok}" + ("" if metric == "dots" else "_" + metric)
-            line["others"][name] = {"gso_per_s": r["gso_per_s"], "kernel_ms": r["kernel_ms"], "kernel_ms_median": r["kernel_ms_median"],
-                                    "kernel_ms_min": r["kernel_ms_min"], "roofline": r["roofline"]}
-        for dtype, on, ok in PACKS:
-            line["others"][f"pack_{dtype}_{on}x{ok}"] = time_pack(dtype, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2))
-    if not args.no_vendor:
-        line.setdefault("others", {})
-        for dtype, om, on, ok in VENDOR:
-            line["others"][f"vendor_{dtype}_{om}x{on}x{ok}"] = time_vendor(dtype, om, on, ok, max(3, args.steps // 2), max(2, args.warmup // 2))
-    if not args.no_ceiling:
-        line.setdefault("others", {})["mfma_ceiling"] = mfma_ceiling()
+    })
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.dtype, m, n, k)
+        if headline:  # the metric's other two types, on a stated share of the rows of A (the kernels are 5-10 times slower)
+            line["cpu_baseline"]["by_dtype"] = {"i8": {key: line["cpu_baseline"][key] for key in ("value", "median", "cores", "kernel_capability", "sample")}}
+            for dtype in METRIC_DTYPES[1:]:
+                other = cpu_baseline(dtype, m, n, k, budget_rows=2048)
+                line["cpu_baseline"]["by_dtype"][dtype] = {key: other[key] for key in ("value", "median", "cores", "kernel_capability", "sample") if key in other}
     print(json.dumps(line))
 
 

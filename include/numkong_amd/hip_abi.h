@@ -53,6 +53,8 @@ int nk_hip_stream_synchronize(void *stream);
  *     priority: ordered against the legacy default stream, independent of each other). NULL on failure.
  *   - `nk_hip_thread_buffer(slot, pinned, bytes, &ptr)`: a staging buffer of at least `bytes` (device memory, or pinned
  *     host memory when `pinned` is non-zero) that lives in slot 0..7 until a larger one is asked for there.
+ *   - `nk_hip_thread_trim(slot_bytes, total_bytes)`: frees the thread's staging buffers larger than `slot_bytes`, then
+ *     all of them if more than `total_bytes` are still held.
  *   - `nk_hip_event_record / _synchronize`, `nk_hip_stream_wait_event`: the thread's events 0..7 (waiting for one
  *     that was never recorded returns at once).
  */
@@ -60,20 +62,31 @@ void *nk_hip_thread_stream(int which);
 int nk_hip_thread_buffer(int slot, int pinned, size_t bytes, void **ptr);
 size_t nk_hip_thread_cached_bytes(void);
 void nk_hip_thread_release(void);
+void nk_hip_thread_trim(size_t slot_bytes, size_t total_bytes);
 int nk_hip_event_record(int which, void *stream);
 int nk_hip_event_synchronize(int which);
 int nk_hip_stream_wait_event(void *stream, int which);
 
 /**
  *  Device copies of packed images that the caller keeps in host memory (what `malloc(nk_dots_packed_size_T(n, k))`
- *  gives a caller of the reference's interface). `find` looks the image up by the number its pack call left in its
- *  header and, when found (returns 1), hands out the device copy and counts the caller as a user until `release`.
- *  `adopt` gives the cache a device copy the caller has just uploaded with `nk_hip_malloc` memory (returns 1: the cache
- *  owns it now, the caller is its first user and calls `release` when done; 0: not taken, the caller frees it).
+ *  gives a caller of the reference's interface), looked up by the number the image's pack call left in its header.
+ *  A cached copy is always complete: it enters the cache only after every transfer into it has finished.
+ *   - `claim`: 1 = cached, `*device_image` is the copy and the caller counts as a user until `release`; 2 = not cached,
+ *     and an entry is now reserved for the caller, who uploads a copy into `nk_hip_malloc` memory, waits for the
+ *     transfers, and calls `publish` (1: the cache owns the copy, the caller is its first user; 0: not taken, the caller
+ *     frees it) or, on failure, `abandon`; other threads that claim the same image meanwhile wait for that upload
+ *     instead of making their own; 0 = not cacheable (no header, over the budget, every entry in use): the caller
+ *     works with a private copy and frees it.
+ *   - `find`: the lookup alone, never waits (1 = cached and counted as a user).
+ *   - `adopt`: hands the cache a complete copy made some other way (the pack call's own output); 1 = taken, the caller
+ *     is its first user; 0 = not taken (also when a copy of the same image is cached already), the caller frees it.
  *  Copies nobody is using are dropped, least recently used first, beyond 4 images or NK_AMD_IMAGE_CACHE_BYTES
  *  (default 8 GiB); `clear` drops all of them.
  */
 int nk_hip_image_cache_find(void const *host_image, size_t total_bytes, void **device_image);
+int nk_hip_image_cache_claim(void const *host_image, size_t total_bytes, void **device_image);
+int nk_hip_image_cache_publish(void const *host_image, size_t total_bytes, void *device_image);
+void nk_hip_image_cache_abandon(void const *host_image, size_t total_bytes);
 int nk_hip_image_cache_adopt(void const *host_image, size_t total_bytes, void *device_image);
 void nk_hip_image_cache_release(void *device_image);
 void nk_hip_image_cache_clear(void);

@@ -13,8 +13,10 @@ GPU side, ``NumKongAmdError`` is raised with the library's own message.
 
 Streams: the synchronous calls run on streams the library keeps per host thread. They are blocking streams, so they
 are ordered behind work queued on the legacy default stream (torch's default) and return when the result is
-complete; operands produced on a non-blocking stream of the caller's must be synchronised first, or the ``*_async``
-entry points used with that stream.
+complete. ONLY the legacy default stream is ordered with them: operands produced on any other stream of the
+caller's, blocking or not (blocking streams are ordered against the default stream, not against each other), and
+work this library's own ``*_async`` entry points were given on such a stream, must be synchronised before a
+synchronous call reads them; or the ``*_async`` entry points are used with that stream throughout.
 """
 from __future__ import annotations
 

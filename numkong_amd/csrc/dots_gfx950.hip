@@ -14,6 +14,7 @@
 
 #include <stdlib.h>
 
+#include <initializer_list>
 #include <new>
 
 namespace nk_gfx950 {
@@ -203,6 +204,22 @@ void nk_hip_thread_release(void) {
     if (context) context->release(false);
 }
 
+void nk_hip_thread_trim(size_t slot_bytes, size_t total_bytes) {
+    ThreadContext *context = thread_context();
+    if (!context) return;
+    size_t kept = 0;
+    for (int slot = 0; slot < kThreadSlots; ++slot)
+        for (CachedBuffer *buffer : {&context->device[slot], &context->pinned[slot]}) {
+            if (buffer->bytes > slot_bytes) {
+                if (buffer->ptr) (void)(buffer == &context->pinned[slot] ? hipHostFree(buffer->ptr) : hipFree(buffer->ptr));
+                *buffer = CachedBuffer();
+            }
+            kept += buffer->bytes;
+        }
+    if (kept > total_bytes) context->release(false);
+    (void)hipGetLastError();
+}
+
 int nk_hip_event_record(int which, void *stream) {
     ThreadContext *context = thread_context();
     if (!context || which < 0 || which >= kThreadEvents) return fail_msg("nk_hip_event_record: no such event");
@@ -263,7 +280,8 @@ int nk_hip_stream_synchronize(void *stream) {
  *  with malloc, so every product would have to upload it again; instead the upload is kept and found again by the
  *  number that the pack call left in the image's header (images are opaque: only a pack call changes one, and every
  *  pack call leaves a new number). Least recently used copies that no call is using are dropped beyond 4 entries or
- *  `budget` bytes.
+ *  `budget` bytes. An entry is either ready (`device` set: a complete copy, every transfer into it finished) or
+ *  loading (reserved by the one thread that uploads it; the others that ask for the same image wait for it).
  */
 namespace {
 struct CachedImage {
@@ -271,11 +289,13 @@ struct CachedImage {
     uint32_t dtype, n, k;
     void *device;
     int users;
+    int loading;
 };
 constexpr int kCachedImages = 4;
 CachedImage g_images[kCachedImages];
 uint64_t g_image_clock = 0;
 pthread_mutex_t g_image_lock = PTHREAD_MUTEX_INITIALIZER;
+pthread_cond_t g_image_loaded = PTHREAD_COND_INITIALIZER;
 size_t image_budget() {
     static size_t const budget = [] {
         char const *text = getenv("NK_AMD_IMAGE_CACHE_BYTES");
@@ -288,6 +308,36 @@ bool header_of_host_image(void const *image, size_t total_bytes, PackedHeader &h
     memcpy(&h, image, sizeof(h));
     return h.magic == kMagic && h.version == kVersion && h.nonce != 0 && h.total_bytes == total_bytes;
 }
+/** The entry of this image, ready or loading (the lock is held). */
+CachedImage *entry_of(PackedHeader const &h, size_t total_bytes) {
+    for (CachedImage &entry : g_images)
+        if ((entry.device || entry.loading) && entry.nonce == h.nonce && entry.total_bytes == total_bytes &&
+            entry.dtype == h.dtype && entry.n == h.n && entry.k == h.k)
+            return &entry;
+    return nullptr;
+}
+/** A free entry with `total_bytes` of the budget to go with it, dropping least recently used copies that nobody is
+ *  using (into `dropped`, for the caller to free once the lock is released); NULL when everything is in use. */
+CachedImage *room_for(size_t total_bytes, void *(&dropped)[kCachedImages]) {
+    for (;;) {
+        size_t held = 0;
+        CachedImage *vacant = nullptr, *oldest = nullptr;
+        for (CachedImage &entry : g_images) {
+            if (!entry.device && !entry.loading) { vacant = vacant ? vacant : &entry; continue; }
+            held += entry.total_bytes;
+            if (entry.device && !entry.users && (!oldest || entry.last_use < oldest->last_use)) oldest = &entry;
+        }
+        if (vacant && held + total_bytes <= image_budget()) return vacant;
+        if (!oldest) return nullptr;
+        for (void *&slot : dropped)
+            if (!slot) { slot = oldest->device; break; }
+        oldest->device = nullptr;
+    }
+}
+void free_dropped(void *(&dropped)[kCachedImages]) {
+    for (void *image : dropped)
+        if (image) (void)hipFree(image);
+}
 } // namespace
 
 int nk_hip_image_cache_find(void const *host_image, size_t total_bytes, void **device_image) {
@@ -296,15 +346,65 @@ int nk_hip_image_cache_find(void const *host_image, size_t total_bytes, void **d
     if (!header_of_host_image(host_image, total_bytes, h)) return 0;
     int found = 0;
     pthread_mutex_lock(&g_image_lock);
-    for (CachedImage &entry : g_images)
-        if (entry.device && entry.nonce == h.nonce && entry.total_bytes == total_bytes && entry.dtype == h.dtype &&
-            entry.n == h.n && entry.k == h.k) {
-            entry.users++, entry.last_use = ++g_image_clock;
-            *device_image = entry.device, found = 1;
-            break;
-        }
+    CachedImage *entry = entry_of(h, total_bytes);
+    if (entry && entry->device) {
+        entry->users++, entry->last_use = ++g_image_clock;
+        *device_image = entry->device, found = 1;
+    }
     pthread_mutex_unlock(&g_image_lock);
     return found;
+}
+
+int nk_hip_image_cache_claim(void const *host_image, size_t total_bytes, void **device_image) {
+    PackedHeader h;
+    *device_image = nullptr;
+    if (!header_of_host_image(host_image, total_bytes, h) || total_bytes > image_budget()) return 0;
+    void *dropped[kCachedImages] = {};
+    int outcome = 0;
+    pthread_mutex_lock(&g_image_lock);
+    for (;;) {
+        CachedImage *entry = entry_of(h, total_bytes);
+        if (entry && entry->device) {
+            entry->users++, entry->last_use = ++g_image_clock;
+            *device_image = entry->device, outcome = 1;
+            break;
+        }
+        if (entry) { // another thread is uploading this very image: its copy will do
+            pthread_cond_wait(&g_image_loaded, &g_image_lock);
+            continue;
+        }
+        CachedImage *vacant = room_for(total_bytes, dropped);
+        if (vacant) *vacant = CachedImage {h.nonce, total_bytes, ++g_image_clock, h.dtype, h.n, h.k, nullptr, 1, 1}, outcome = 2;
+        break;
+    }
+    pthread_mutex_unlock(&g_image_lock);
+    free_dropped(dropped);
+    return outcome;
+}
+
+int nk_hip_image_cache_publish(void const *host_image, size_t total_bytes, void *device_image) {
+    PackedHeader h;
+    if (!device_image || !header_of_host_image(host_image, total_bytes, h)) return 0;
+    int published = 0;
+    pthread_mutex_lock(&g_image_lock);
+    CachedImage *entry = entry_of(h, total_bytes);
+    if (entry && entry->loading && !entry->device) {
+        entry->device = device_image, entry->loading = 0, entry->last_use = ++g_image_clock; // (users stays 1: the uploader)
+        published = 1;
+    }
+    pthread_cond_broadcast(&g_image_loaded);
+    pthread_mutex_unlock(&g_image_lock);
+    return published;
+}
+
+void nk_hip_image_cache_abandon(void const *host_image, size_t total_bytes) {
+    PackedHeader h;
+    if (!header_of_host_image(host_image, total_bytes, h)) return;
+    pthread_mutex_lock(&g_image_lock);
+    CachedImage *entry = entry_of(h, total_bytes);
+    if (entry && entry->loading && !entry->device) *entry = CachedImage {};
+    pthread_cond_broadcast(&g_image_loaded); // (one of those waiting takes over the upload)
+    pthread_mutex_unlock(&g_image_lock);
 }
 
 int nk_hip_image_cache_adopt(void const *host_image, size_t total_bytes, void *device_image) {
@@ -313,28 +413,12 @@ int nk_hip_image_cache_adopt(void const *host_image, size_t total_bytes, void *d
     void *dropped[kCachedImages] = {};
     int adopted = 0;
     pthread_mutex_lock(&g_image_lock);
-    // room: a free entry, or the least recently used one that nobody is using; and the byte budget
-    for (;;) {
-        size_t held = 0;
-        CachedImage *vacant = nullptr, *oldest = nullptr;
-        for (CachedImage &entry : g_images) {
-            if (!entry.device) { vacant = vacant ? vacant : &entry; continue; }
-            held += entry.total_bytes;
-            if (!entry.users && (!oldest || entry.last_use < oldest->last_use)) oldest = &entry;
-        }
-        if (vacant && held + total_bytes <= image_budget()) {
-            *vacant = CachedImage {h.nonce, total_bytes, ++g_image_clock, h.dtype, h.n, h.k, device_image, 1};
-            adopted = 1;
-            break;
-        }
-        if (!oldest) break; // everything is in use: the caller keeps its copy for the call and frees it
-        for (void *&slot : dropped)
-            if (!slot) { slot = oldest->device; break; }
-        oldest->device = nullptr;
+    if (!entry_of(h, total_bytes)) { // (a copy of this image that is there already, or on its way, is enough)
+        CachedImage *vacant = room_for(total_bytes, dropped);
+        if (vacant) *vacant = CachedImage {h.nonce, total_bytes, ++g_image_clock, h.dtype, h.n, h.k, device_image, 1, 0}, adopted = 1;
     }
     pthread_mutex_unlock(&g_image_lock);
-    for (void *image : dropped)
-        if (image) (void)hipFree(image);
+    free_dropped(dropped);
     return adopted;
 }
 
@@ -351,8 +435,7 @@ void nk_hip_image_cache_clear(void) {
     for (int i = 0; i < kCachedImages; ++i)
         if (g_images[i].device && !g_images[i].users) dropped[i] = g_images[i].device, g_images[i].device = nullptr;
     pthread_mutex_unlock(&g_image_lock);
-    for (void *image : dropped)
-        if (image) (void)hipFree(image);
+    free_dropped(dropped);
 }
 
 size_t nk_hip_dots_packed_size(int dtype, size_t n, size_t k) {

@@ -89,6 +89,15 @@ int nk_amd_spatials_packed_async(nk_kernel_kind_t kind, nk_dtype_t dtype, void c
     return nk_hip_spatials_packed_async((int)dtype, metric, a, b_packed, c, m, n, k, a_stride, c_stride, stream);
 }
 
+/** Is there a GPU? Asked of the runtime until the answer is yes, then remembered (devices do not go away). */
+static int nk_amd_have_device_(void) {
+    static _Atomic int seen = 0;
+    if (atomic_load_explicit(&seen, memory_order_relaxed)) return 1;
+    if (nk_hip_device_count() <= 0) return 0;
+    atomic_store_explicit(&seen, 1, memory_order_relaxed);
+    return 1;
+}
+
 static nk_size_t nk_amd_packed_size_(nk_dtype_t dtype, nk_size_t n, nk_size_t k) {
     return nk_hip_dots_packed_size((int)dtype, n, k);
 }
@@ -98,15 +107,16 @@ static nk_size_t nk_amd_packed_size_(nk_dtype_t dtype, nk_size_t n, nk_size_t k)
 /*  Plain host memory reaches the GPU through pinned bounce buffers that the calling thread keeps between calls
  *  (hip_abi.h: nk_hip_thread_buffer), in pieces, so that the copy into the bounce buffer, the transfer and whatever the
  *  GPU does with the previous piece overlap. Copies of 16 MiB and more between pageable and pinned memory are split
- *  over a few short-lived helper threads: one core moves about 10 GB/s, the link several times that.
+ *  over a few helper threads (started once, then kept): one core moves about 10 GB/s, the link several times that.
  *  Pinned slots: 0, 1 uploads; 2, 3 downloads; 4, 5 row chunks of A; 6, 7 row chunks of C. Events: the same numbers
  *  for the slot's last transfer (4, 5: everything queued for a row chunk); 6: the packed image is on the device. */
 enum {
     nk_amd_piece_bytes_k = 8u << 20,      /* one bounce-buffer piece of a plain upload or download */
     nk_amd_chunk_bytes_k = 32u << 20,     /* what a row chunk of the product moves in one direction, about */
     nk_amd_parallel_copy_k = 16u << 20,   /* host copies from this size on get helper threads */
-    nk_amd_keep_cached_k = 1u << 30,      /* staging memory a thread may keep between calls */
 };
+static size_t const nk_amd_keep_slot_k = (size_t)256 << 20; /* the largest staging buffer a thread keeps between calls */
+static size_t const nk_amd_keep_cached_k = (size_t)2 << 30; /* all the staging memory a thread may keep between calls */
 enum { nk_amd_slot_a_k = 0, nk_amd_slot_c_k = 2, nk_amd_slot_b_k = 4, nk_amd_slot_image_k = 5, nk_amd_slot_result_k = 6 };
 
 typedef struct {
@@ -115,10 +125,8 @@ typedef struct {
     size_t dst_stride, src_stride, width, rows;
 } nk_amd_copy_job_t_;
 
-static void *nk_amd_copy_worker_(void *raw) {
-    nk_amd_copy_job_t_ const *job = (nk_amd_copy_job_t_ const *)raw;
+static void nk_amd_copy_job_run_(nk_amd_copy_job_t_ const *job) {
     for (size_t row = 0; row < job->rows; ++row) memcpy(job->dst + row * job->dst_stride, job->src + row * job->src_stride, job->width);
-    return NULL;
 }
 
 static int nk_amd_copy_threads_(void) {
@@ -133,7 +141,59 @@ static int nk_amd_copy_threads_(void) {
     return threads;
 }
 
-/** `rows` runs of `width` bytes between host buffers, on this thread and, for large copies, a few helpers. */
+/*  Helper threads for large host copies: started once, on the first large copy, and kept (detached, asleep on a
+ *  condition variable between copies). Callers from any thread queue jobs under one lock and wait for their own. */
+enum { nk_amd_copy_queue_k = 64 };
+typedef struct {
+    nk_amd_copy_job_t_ job;
+    _Atomic int *pending; /* the caller's count of jobs not finished yet */
+} nk_amd_queued_copy_t_;
+static pthread_mutex_t nk_amd_copy_lock_ = PTHREAD_MUTEX_INITIALIZER;
+static pthread_cond_t nk_amd_copy_work_ = PTHREAD_COND_INITIALIZER, nk_amd_copy_done_ = PTHREAD_COND_INITIALIZER;
+static nk_amd_queued_copy_t_ nk_amd_copy_queue_[nk_amd_copy_queue_k];
+static int nk_amd_copy_head_ = 0, nk_amd_copy_count_ = 0, nk_amd_copy_helpers_ = 0;
+
+static void *nk_amd_copy_helper_(void *unused) {
+    (void)unused;
+    pthread_mutex_lock(&nk_amd_copy_lock_);
+    for (;;) {
+        while (!nk_amd_copy_count_) pthread_cond_wait(&nk_amd_copy_work_, &nk_amd_copy_lock_);
+        nk_amd_queued_copy_t_ const taken = nk_amd_copy_queue_[nk_amd_copy_head_];
+        nk_amd_copy_head_ = (nk_amd_copy_head_ + 1) % nk_amd_copy_queue_k, nk_amd_copy_count_--;
+        pthread_mutex_unlock(&nk_amd_copy_lock_);
+        nk_amd_copy_job_run_(&taken.job);
+        pthread_mutex_lock(&nk_amd_copy_lock_);
+        if (atomic_fetch_sub_explicit(taken.pending, 1, memory_order_acq_rel) == 1) pthread_cond_broadcast(&nk_amd_copy_done_);
+    }
+    return NULL;
+}
+
+/** Hands `job` to a helper; 0 when there is none to take it (the caller then copies it itself). */
+static int nk_amd_copy_queue_job_(nk_amd_copy_job_t_ const *job, _Atomic int *pending, int wanted_helpers) {
+    int queued = 0;
+    pthread_mutex_lock(&nk_amd_copy_lock_);
+    while (nk_amd_copy_helpers_ < wanted_helpers) { /* (started on first use, never more than 7) */
+        pthread_t helper;
+        pthread_attr_t attributes;
+        if (pthread_attr_init(&attributes) != 0) break;
+        pthread_attr_setdetachstate(&attributes, PTHREAD_CREATE_DETACHED);
+        int const failed = pthread_create(&helper, &attributes, nk_amd_copy_helper_, NULL);
+        pthread_attr_destroy(&attributes);
+        if (failed) break;
+        nk_amd_copy_helpers_++;
+    }
+    if (nk_amd_copy_helpers_ > 0 && nk_amd_copy_count_ < nk_amd_copy_queue_k) {
+        int const at = (nk_amd_copy_head_ + nk_amd_copy_count_) % nk_amd_copy_queue_k;
+        nk_amd_copy_queue_[at].job = *job, nk_amd_copy_queue_[at].pending = pending;
+        atomic_fetch_add_explicit(pending, 1, memory_order_relaxed);
+        nk_amd_copy_count_++, queued = 1;
+        pthread_cond_signal(&nk_amd_copy_work_);
+    }
+    pthread_mutex_unlock(&nk_amd_copy_lock_);
+    return queued;
+}
+
+/** `rows` runs of `width` bytes between host buffers, on this thread and, for large copies, the helpers. */
 static void nk_amd_copy_rows_(void *dst, size_t dst_stride, void const *src, size_t src_stride, size_t width, size_t rows) {
     if (!width || !rows) return;
     if (dst_stride == width && src_stride == width && width != (1u << 16) && rows > 1) {
@@ -146,20 +206,23 @@ static void nk_amd_copy_rows_(void *dst, size_t dst_stride, void const *src, siz
     int threads = width * rows >= nk_amd_parallel_copy_k ? nk_amd_copy_threads_() : 1;
     if ((size_t)threads > rows) threads = (int)rows;
     nk_amd_copy_job_t_ jobs[8];
-    pthread_t helpers[8];
-    int started[8] = {0};
+    _Atomic int pending = 0;
+    int queued[8] = {0};
     size_t const share = (rows + (size_t)threads - 1) / (size_t)threads;
     for (int t = 0; t < threads; ++t) {
         size_t const first = (size_t)t * share, last = first + share < rows ? first + share : rows;
         jobs[t].dst = (char *)dst + first * dst_stride, jobs[t].src = (char const *)src + first * src_stride;
         jobs[t].dst_stride = dst_stride, jobs[t].src_stride = src_stride, jobs[t].width = width;
         jobs[t].rows = first < last ? last - first : 0;
-        if (t > 0 && jobs[t].rows) started[t] = pthread_create(&helpers[t], NULL, nk_amd_copy_worker_, &jobs[t]) == 0;
+        if (t > 0 && jobs[t].rows) queued[t] = nk_amd_copy_queue_job_(&jobs[t], &pending, threads - 1);
     }
     for (int t = 0; t < threads; ++t)
-        if (t == 0 || !started[t]) nk_amd_copy_worker_(&jobs[t]); /* this thread's share, and any a helper could not take */
-    for (int t = 1; t < threads; ++t)
-        if (started[t]) pthread_join(helpers[t], NULL);
+        if (t == 0 || !queued[t]) nk_amd_copy_job_run_(&jobs[t]); /* this thread's share, and any no helper could take */
+    if (threads > 1) {
+        pthread_mutex_lock(&nk_amd_copy_lock_);
+        while (atomic_load_explicit(&pending, memory_order_acquire) > 0) pthread_cond_wait(&nk_amd_copy_done_, &nk_amd_copy_lock_);
+        pthread_mutex_unlock(&nk_amd_copy_lock_);
+    }
 }
 
 /** Host rows -> device rows on `stream`, through pinned pieces 0 and 1. Returns with the last transfers in flight. */
@@ -222,11 +285,12 @@ static int nk_amd_download_flat_(void *dst, void const *src, size_t bytes, void 
     return status;
 }
 
-/** What a synchronous call leaves behind: nothing in flight, and no more staging memory than a thread should keep. */
+/** What a synchronous call that staged something leaves behind: nothing in flight, and no more staging memory than a
+ *  thread should keep (buffers past 256 MiB each go at once, everything once the thread holds more than 2 GiB). */
 static void nk_amd_settle_(void) {
     (void)nk_hip_stream_synchronize(nk_hip_thread_stream(0));
     (void)nk_hip_stream_synchronize(nk_hip_thread_stream(1));
-    if (nk_hip_thread_cached_bytes() > nk_amd_keep_cached_k) nk_hip_thread_release();
+    nk_hip_thread_trim(nk_amd_keep_slot_k, nk_amd_keep_cached_k);
 }
 
 /**
@@ -234,24 +298,28 @@ static void nk_amd_settle_(void) {
  *  is looked up among the device copies of earlier calls and uploaded on `stream` when it is new; `*owned` is then 1
  *  for a copy this call must free and 2 for one to hand back to the cache (nk_amd_drop_image_).
  */
-static int nk_amd_image_on_device_(void const *b_packed, size_t total, void *stream, void const **device, int *owned) {
+static int nk_amd_image_on_device_(void const *b_packed, int p_kind, size_t total, void *stream, void const **device, int *owned) {
     *owned = 0, *device = b_packed;
-    if (nk_hip_pointer_kind(b_packed) != 0) return 0;
+    if (p_kind != 0) return 0;
     void *copy = NULL;
-    if (nk_hip_image_cache_find(b_packed, total, &copy)) {
+    int const claimed = nk_hip_image_cache_claim(b_packed, total, &copy);
+    if (claimed == 1) {
         *device = copy, *owned = 2;
         return 0;
     }
     int status = nk_hip_malloc(&copy, total);
-    if (status) return status;
-    status = nk_amd_upload_flat_(copy, b_packed, total, stream);
+    if (!status) {
+        status = nk_amd_upload_flat_(copy, b_packed, total, stream);
+        /* a copy that other threads can find must be complete: their streams are not ordered behind this one */
+        if (claimed == 2 || status) status = nk_hip_stream_synchronize(stream) || status;
+        if (status) nk_hip_free(copy);
+    }
     if (status) {
-        (void)nk_hip_stream_synchronize(stream);
-        nk_hip_free(copy);
+        if (claimed == 2) nk_hip_image_cache_abandon(b_packed, total);
         return status;
     }
     *device = copy;
-    *owned = nk_hip_image_cache_adopt(b_packed, total, copy) ? 2 : 1;
+    *owned = claimed == 2 && nk_hip_image_cache_publish(b_packed, total, copy) ? 2 : 1;
     return 0;
 }
 static void nk_amd_drop_image_(void const *device, int owned) {
@@ -269,7 +337,7 @@ static void nk_amd_pack_(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_pack: unsupported dtype or dimensions");
         return;
     }
-    if (nk_hip_device_count() <= 0) {
+    if (!nk_amd_have_device_()) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_pack: no HIP device");
         return;
     }
@@ -302,7 +370,7 @@ static void nk_amd_pack_(nk_dtype_t dtype, void const *b, nk_size_t n, nk_size_t
         if (!status && nk_hip_image_cache_adopt(b_packed, total, staged_p)) nk_hip_image_cache_release(staged_p);
         else nk_hip_free(staged_p);
     }
-    nk_amd_settle_();
+    if (staged_b || staged_p || status) nk_amd_settle_();
 }
 
 /** `metric`: 0 dot products, 1 angular distances, 2 euclidean distances; outputs are 4 bytes wide, 8 for f32 and f64 inputs. */
@@ -312,11 +380,12 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
     if (!m || !n) return;
     size_t const out_bytes = nk_amd_output_bytes_(dtype);
     size_t const total = nk_hip_dots_packed_size((int)dtype, n, k);
-    if (nk_hip_device_count() <= 0) {
+    if (!nk_amd_have_device_()) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_packed: no HIP device");
         nk_amd_fill_error_(c, 0, m, n, c_stride, out_bytes);
         return;
     }
+    /* where each operand lives: asked once per pointer and call */
     int const c_kind = nk_hip_pointer_kind(c);
     if (!total || !b_packed || !c) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_packed: unsupported dtype or dimensions");
@@ -324,25 +393,44 @@ static void nk_amd_packed_(nk_dtype_t dtype, int metric, void const *a, void con
         return;
     }
     int const a_kind = k ? nk_hip_pointer_kind(a) : 1;
-    void *streams[2] = {nk_hip_thread_stream(0), nk_hip_thread_stream(1)};
+    int const p_kind = nk_hip_pointer_kind(b_packed);
+    void *stream = nk_hip_thread_stream(0);
+    if (stream && a_kind != 0 && c_kind != 0 && p_kind != 0) {
+        /* Everything where the GPU reads it: one launch on the thread's first stream, one wait for it. Nothing was
+         * staged, so there is nothing else to wait for or to tidy up. */
+        int status = metric == 0 ? nk_hip_dots_packed_async((int)dtype, a, b_packed, c, m, n, k, a_stride, c_stride, stream)
+                                 : nk_hip_spatials_packed_async((int)dtype, metric, a, b_packed, c, m, n, k, a_stride, c_stride, stream);
+        if (!status) status = nk_hip_stream_synchronize(stream);
+        if (status) {
+            nk_amd_set_error_("nk_dots_packed");
+            (void)nk_hip_stream_synchronize(stream);
+            nk_amd_fill_error_(c, c_kind, m, n, c_stride, out_bytes);
+        }
+        return;
+    }
+    void *streams[2] = {stream, nk_hip_thread_stream(1)};
     void const *device_p = b_packed;
     int image_owned = 0;
     int status = streams[0] && streams[1] ? 0 : -1;
-    if (!status) status = nk_amd_image_on_device_(b_packed, total, streams[0], &device_p, &image_owned);
+    if (!status) status = nk_amd_image_on_device_(b_packed, p_kind, total, streams[0], &device_p, &image_owned);
 
     size_t const row_bytes = nk_amd_row_bytes_(dtype, k);
     size_t const a_pitch = nk_amd_round_up_(row_bytes, 16), c_pitch = nk_amd_round_up_(n * out_bytes, 16);
-    if (!status && a_kind != 0 && c_kind != 0) { /* everything where the GPU reads it: one launch */
+    if (!status && a_kind != 0 && c_kind != 0) { /* only the image was in host memory: one launch behind its upload */
         status = metric == 0 ? nk_hip_dots_packed_async((int)dtype, a, device_p, c, m, n, k, a_stride, c_stride, streams[0])
                              : nk_hip_spatials_packed_async((int)dtype, metric, a, device_p, c, m, n, k, a_stride, c_stride, streams[0]);
     }
     else if (!status) {
         /* Rows of A go up and rows of C come down in chunks, alternating between the thread's two streams, so that
          * the upload of one chunk, the product of the one before it and the copy of the one before that out of its
-         * bounce buffer run at the same time. */
+         * bounce buffer run at the same time. A chunk moves about 32 MiB in its heavier direction, in whole tiles of
+         * the product kernels where that many rows are at least one; rows so long that 64 of them pass 256 MiB (the
+         * largest buffer a thread keeps) go in fewer, down to one at a time. */
         size_t const heavier = (a_kind == 0 ? a_pitch : 0) > (c_kind == 0 ? c_pitch : 0) ? a_pitch : c_pitch;
-        size_t chunk = nk_amd_chunk_bytes_k / (heavier ? heavier : 1);
-        chunk = chunk >= 256 ? chunk / 256 * 256 : 64; /* whole tiles of the product kernels */
+        size_t const pitch = heavier ? heavier : 1;
+        size_t chunk = nk_amd_chunk_bytes_k / pitch;
+        if (chunk >= 256) chunk = chunk / 256 * 256;
+        else if (chunk < 64) chunk = 64 * pitch <= nk_amd_keep_slot_k ? 64 : (nk_amd_keep_slot_k / pitch ? nk_amd_keep_slot_k / pitch : 1);
         if (chunk > m) chunk = m;
         size_t const chunks = (m + chunk - 1) / chunk;
         void *device_a[2] = {NULL, NULL}, *device_c[2] = {NULL, NULL}, *bounce_a[2] = {NULL, NULL}, *bounce_c[2] = {NULL, NULL};
@@ -439,7 +527,7 @@ static void nk_amd_symmetric_(nk_dtype_t dtype, int metric, void const *vectors,
     nk_amd_error_[0] = 0;
     if (!n || !row_count || row_start >= n) return;
     size_t const out_bytes = nk_amd_output_bytes_(dtype);
-    if (nk_hip_device_count() <= 0) {
+    if (!nk_amd_have_device_()) {
         snprintf(nk_amd_error_, sizeof(nk_amd_error_), "nk_dots_symmetric: no HIP device");
         nk_amd_fill_symmetric_error_(result, 0, n, result_stride, out_bytes);
         return;

@@ -32,8 +32,10 @@ void nk_error_pack_(void const *b, nk_size_t n, nk_size_t k, nk_size_t b_stride,
     (void)b, (void)n, (void)k, (void)b_stride, (void)b_packed;
 }
 
-/** Outputs of every dtype on this path are 4 bytes wide, so exactly n * 4 bytes per row are poisoned;
- *  C is assumed host-addressable here because this stub is only reached when no GPU backend is selected. */
+/** The stub of a kind this library has no kernel for (with the GPU backend selected, failures are reported by the
+ *  backend itself, which knows the width of its outputs): n * 4 bytes per row are poisoned, the width of every output
+ *  on this path but the f64 results of f32 and f64 inputs, of which that is the first half of each row. A device
+ *  pointer is filled on the device. */
 void nk_error_dots_(void const *a, void const *b_packed, void *c, nk_size_t m, nk_size_t n, nk_size_t k,
                     nk_size_t a_stride, nk_size_t c_stride) {
     (void)a, (void)b_packed, (void)k, (void)a_stride;

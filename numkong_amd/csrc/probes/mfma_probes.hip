@@ -425,23 +425,27 @@ static char const *const kModeNames[kModes] = {"v_mfma_f32_32x32x16_fp8_fp8", "v
 static int bytes_per_lane(int mode) { return mode <= kLegacyBF8 ? 8 : (mode <= kScaledBF8 ? 32 : 16); }
 static int depth_of(int mode) { return mode <= kLegacyBF8 ? 16 : (mode <= kScaledBF8 ? 64 : 16); }
 
-/** `steps` instructions in a row on one wavefront: operands of step s at a + s * 64 * bytes_per_lane, accumulator from `c`. */
-__global__ __launch_bounds__(64) void mfma_steps_kernel(uint8_t const *a, uint8_t const *b, float const *c, float *out, int mode, int steps) {
+/** `steps` instructions in a row on one wavefront: operands of step s at a + s * 64 * bytes_per_lane, accumulator from `c`.
+ *  One kernel per instruction (the instruction is a compile-time choice: nothing but loads and the one MFMA in the loop).
+ *  `UNIT_SCALES`: the block-scaled form with explicit scales of 2^0 (E8M0 code 127) instead of the plain f8f6f4 form. */
+template <int MODE, bool UNIT_SCALES>
+__global__ __launch_bounds__(64) void mfma_steps_kernel(uint8_t const *a, uint8_t const *b, float const *c, float *out, int steps) {
     int const lane = threadIdx.x;
     v16f acc;
     for (int v = 0; v < 16; ++v) acc[v] = c[lane * 16 + v];
     for (int s = 0; s < steps; ++s) {
-        if (mode <= kLegacyBF8) {
+        if constexpr (MODE <= kLegacyBF8) {
             long const x = *(long const *)(a + ((size_t)s * 64 + lane) * 8), y = *(long const *)(b + ((size_t)s * 64 + lane) * 8);
-            acc = mode == kLegacyFP8 ? __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(x, y, acc, 0, 0, 0) : __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(x, y, acc, 0, 0, 0);
+            acc = MODE == kLegacyFP8 ? __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(x, y, acc, 0, 0, 0) : __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(x, y, acc, 0, 0, 0);
         }
-        else if (mode <= kScaledBF8) {
+        else if constexpr (MODE <= kScaledBF8) {
             v8i const x = *(v8i const *)(a + ((size_t)s * 64 + lane) * 32), y = *(v8i const *)(b + ((size_t)s * 64 + lane) * 32);
-            // (format selectors 0 = fp8, 1 = bf8; scales of zero select the unscaled instruction)
-            acc = mode == kScaledFP8 ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc, 0, 0, 0, 0, 0, 0)
-                                     : __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc, 1, 1, 0, 0, 0, 0);
+            // (format selectors 0 = fp8, 1 = bf8; constant scales of zero make the compiler select the instruction without scales)
+            constexpr int kFormat = MODE == kScaledFP8 ? 0 : 1;
+            if constexpr (UNIT_SCALES) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc, kFormat, kFormat, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+            else acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc, kFormat, kFormat, 0, 0, 0, 0);
         }
-        else if (mode == kHalf) {
+        else if constexpr (MODE == kHalf) {
             v8h const x = *(v8h const *)(a + ((size_t)s * 64 + lane) * 16), y = *(v8h const *)(b + ((size_t)s * 64 + lane) * 16);
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(x, y, acc, 0, 0, 0);
         }
@@ -471,11 +475,21 @@ static float output_at(std::vector<float> const &out, int i, int j) { return out
 
 static uint8_t *g_a, *g_b;
 static float *g_c, *g_out;
-static std::vector<float> run_steps(Operands const &a, Operands const &b, std::vector<float> const &c) {
+static std::vector<float> run_steps(Operands const &a, Operands const &b, std::vector<float> const &c, bool unit_scales = false) {
     CHECK(hipMemcpy(g_a, a.bytes.data(), a.bytes.size(), hipMemcpyHostToDevice));
     CHECK(hipMemcpy(g_b, b.bytes.data(), b.bytes.size(), hipMemcpyHostToDevice));
     CHECK(hipMemcpy(g_c, c.data(), 4096, hipMemcpyHostToDevice));
-    hipLaunchKernelGGL(mfma_steps_kernel, dim3(1), dim3(64), 0, 0, g_a, g_b, g_c, g_out, a.mode, a.steps);
+    CHECK(hipMemset(g_out, 0xFF, 4096));
+    void (*kernel)(uint8_t const *, uint8_t const *, float const *, float *, int) = mfma_steps_kernel<kLegacyFP8, false>;
+    switch (a.mode) {
+    case kLegacyBF8: kernel = mfma_steps_kernel<kLegacyBF8, false>; break;
+    case kScaledFP8: kernel = unit_scales ? mfma_steps_kernel<kScaledFP8, true> : mfma_steps_kernel<kScaledFP8, false>; break;
+    case kScaledBF8: kernel = unit_scales ? mfma_steps_kernel<kScaledBF8, true> : mfma_steps_kernel<kScaledBF8, false>; break;
+    case kHalf: kernel = mfma_steps_kernel<kHalf, false>; break;
+    case kBrain: kernel = mfma_steps_kernel<kBrain, false>; break;
+    default: break;
+    }
+    hipLaunchKernelGGL(kernel, dim3(1), dim3(64), 0, 0, g_a, g_b, g_c, g_out, a.steps);
     CHECK(hipGetLastError());
     std::vector<float> out(1024);
     CHECK(hipMemcpy(out.data(), g_out, 4096, hipMemcpyDeviceToHost));
@@ -522,7 +536,7 @@ struct ErrorStats {
 /** 32 x 32 e4m3 dot products of depth `depth`, N(0, 1) scaled to half the largest finite value with 1 % zeros (the
  *  benchmark's fp8 family): normwise error |c - truth| / sum|a b| of the given matrix-core route against the f64 truth. */
 static ErrorStats depth_error(int mode, int depth, std::vector<uint8_t> const &a_codes, std::vector<uint8_t> const &b_codes, std::vector<double> const &truth,
-                              std::vector<double> const &magnitude) {
+                              std::vector<double> const &magnitude, bool unit_scales = false) {
     int const per = depth_of(mode), steps = depth / per;
     Operands a(mode, steps), b(mode, steps);
     for (int row = 0; row < 32; ++row)
@@ -531,7 +545,7 @@ static ErrorStats depth_error(int mode, int depth, std::vector<uint8_t> const &a
             a.set(k / per, row, k % per, mode == kHalf ? f16_of(e4m3_value(x)) : x);
             b.set(k / per, row, k % per, mode == kHalf ? f16_of(e4m3_value(y)) : y);
         }
-    std::vector<float> const out = run_steps(a, b, std::vector<float>(1024, 0.0f));
+    std::vector<float> const out = run_steps(a, b, std::vector<float>(1024, 0.0f), unit_scales);
     ErrorStats stats = {0, 0};
     for (int i = 0; i < 32; ++i)
         for (int j = 0; j < 32; ++j) {
@@ -583,15 +597,16 @@ static int numerics_mode(bool check) {
         }
     printf("\ne4m3 dot products of depth %d, 32 x 32 outputs, normwise error against the f64 truth (mean, max):\n", depth);
     printf("%-56s %.3e %.3e\n", "f32 sums of exact products (reference, dot/serial.h:522-600)", serial.mean, serial.max);
-    ErrorStats const routes[3] = {depth_error(kLegacyFP8, depth, a_codes, b_codes, truth, magnitude), depth_error(kScaledFP8, depth, a_codes, b_codes, truth, magnitude),
-                                  depth_error(kHalf, depth, a_codes, b_codes, truth, magnitude)};
-    char const *const route_names[3] = {"v_mfma_f32_32x32x16_fp8_fp8, one accumulator", "v_mfma_scale_f32_32x32x64_f8f6f4, one accumulator",
-                                        "widened to f16, v_mfma_f32_32x32x16_f16, one accumulator"};
-    for (int route = 0; route < 3; ++route)
+    constexpr int kRoutes = 4;
+    ErrorStats const routes[kRoutes] = {depth_error(kLegacyFP8, depth, a_codes, b_codes, truth, magnitude), depth_error(kScaledFP8, depth, a_codes, b_codes, truth, magnitude),
+                                        depth_error(kScaledFP8, depth, a_codes, b_codes, truth, magnitude, true), depth_error(kHalf, depth, a_codes, b_codes, truth, magnitude)};
+    char const *const route_names[kRoutes] = {"v_mfma_f32_32x32x16_fp8_fp8, one accumulator", "v_mfma_f32_32x32x64_f8f6f4, one accumulator",
+                                              "v_mfma_scale_f32_32x32x64_f8f6f4, scales 2^0, one acc.", "widened to f16, v_mfma_f32_32x32x16_f16, one accumulator"};
+    for (int route = 0; route < kRoutes; ++route)
         printf("%-56s %.3e %.3e   = %.1f x, %.1f x the reference's (gate: 2 x)\n", route_names[route], routes[route].mean, routes[route].max,
                routes[route].mean / serial.mean, routes[route].max / serial.max);
     if (check) {
-        if (!(routes[2].mean < routes[0].mean && routes[2].mean < routes[1].mean)) ++failures, printf("UNEXPECTED: the f16 route is not the more accurate one\n");
+        if (!(routes[3].mean < routes[0].mean && routes[3].mean < routes[1].mean && routes[3].mean < routes[2].mean)) ++failures, printf("UNEXPECTED: the f16 route is not the more accurate one\n");
         if (!(kept[kLegacyFP8][0] < 23 && kept[kScaledFP8][0] < 23)) printf("NOTE: the fp8 forms keep full f32 precision on this part: the f16 detour is no longer needed\n");
         printf(failures ? "FAILED\n" : "ok\n");
     }

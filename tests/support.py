@@ -267,7 +267,8 @@ def ulp_distance_f32(actual: np.ndarray, expected: np.ndarray) -> np.ndarray:
     return np.abs(ordered(actual) - ordered(expected))
 
 
-ULP_TABLE_HEADER = f"{'kernel':<40s} {'max abs err':>12s} {'max rel err':>12s} {'mean ulp':>10s} {'max ulp':>12s} {'exact':>10s}"
+ULP_TABLE_HEADER = (f"{'kernel':<40s} {'max abs err':>12s} {'max rel err':>12s} {'mean rel err':>12s} {'mean ulp':>10s} {'max ulp':>12s} "
+                    f"{'exact':>10s}")
 
 
 def ulp_table_row(name: str, actual: np.ndarray, truth: np.ndarray) -> str:
@@ -282,8 +283,8 @@ def ulp_table_row(name: str, actual: np.ndarray, truth: np.ndarray) -> str:
     absolute = np.abs(got.astype(np.float64) - want.astype(np.float64))
     relative = np.where(want != 0, absolute / np.maximum(np.abs(want.astype(np.float64)), 1e-300), absolute)
     ulps = ulp_distance_f32(got, want)
-    return (f"{name:<40s} {absolute.max():12.2e} {relative.max():12.2e} {ulps.mean():10.1f} {int(ulps.max()):12d} "
-            f"{int((ulps == 0).sum()):10d}")
+    return (f"{name:<40s} {absolute.max():12.2e} {relative.max():12.2e} {relative.mean():12.2e} {ulps.mean():10.1f} "
+            f"{int(ulps.max()):12d} {int((ulps == 0).sum()):10d}")
 
 
 def load_oracle() -> Oracle:

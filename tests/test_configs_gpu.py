@@ -13,7 +13,7 @@ torch = pytest.importorskip("torch")
 
 import numkong_amd as nk  # noqa: E402
 from tests import support  # noqa: E402
-from tests.test_dots_gpu import DEV, assert_float_gate, best_dispatch, to_gpu  # noqa: E402
+from tests.test_dots_gpu import DEV, assert_float_gate, assert_relative_gate, best_dispatch, to_gpu  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 
@@ -68,6 +68,7 @@ def sampled_oracle_gate(oracle, dtype, a, b, c, rows, cols, label=None):
     if dispatched is not None:
         ULP_ROWS.append(support.ulp_table_row(f"dots_packed_{dtype} (host dispatch) {shape}", dispatched, truth))
     assert_float_gate(dtype, got, serial, truth, magnitude, f"{dtype} sample", dispatched)
+    assert_relative_gate(got, (("serial", serial), ("dispatched", dispatched)), truth, magnitude, f"{dtype} sample {shape}")
 
 
 def tiling_invariance(dtype, a, packed, c):

@@ -96,6 +96,30 @@ def assert_float_gate(dtype, got, serial, truth, magnitude, where="", dispatched
                                         f"worst {e_gpu[worst]:.3e} against its reference's {e_ref[worst]:.3e} {where}")
 
 
+def assert_relative_gate(got, references, truth, magnitude, where=""):
+    """The same comparison with each error taken relative to the result itself, e = |c - truth| / |truth|: the mean
+    within twice the reference kernel's, and the maximum within twice the reference kernel's or, where that kernel
+    happens to land on the truth, twice the per-element floor of assert_float_gate at the sample's worst-conditioned
+    element. An element's relative error is its normwise error times kappa = sum|a*b| / |truth|, the same factor for
+    every kernel, and kappa has a heavy tail (a sum of thousands of products that nearly cancels): both statistics are
+    carried by the few outputs nearest to zero, so this gate is for samples of thousands of outputs and says little that
+    the per-element bound has not said already."""
+    for name, ref in references:
+        if ref is None:
+            continue
+        use = np.isfinite(truth) & (truth != 0) & np.isfinite(ref) & np.isfinite(got)
+        if not use.any():
+            continue
+        size = np.abs(truth[use])
+        e_gpu = np.abs(got[use].astype(np.float64) - truth[use]) / size
+        e_ref = np.abs(ref[use].astype(np.float64) - truth[use]) / size
+        kappa = magnitude[use] / size
+        floor = PER_ELEMENT_FLOOR * U * kappa.max()
+        assert e_gpu.mean() <= 2 * e_ref.mean() + U * kappa.mean() / np.sqrt(e_gpu.size), (
+            f"mean relative error {e_gpu.mean():.3e} vs {name} {e_ref.mean():.3e} {where}")
+        assert e_gpu.max() <= 2 * max(e_ref.max(), floor), f"max relative error {e_gpu.max():.3e} vs {name} {e_ref.max():.3e} {where}"
+
+
 def check(oracle, dtype, a, b, config=0, where=""):
     got = gpu_dots(dtype, a, b, config)
     if dtype in ("i8", "u8"):

@@ -107,6 +107,50 @@ def test_row_tiles_from_eight_threads_host_operands(oracle, dtype):
         assert np.array_equal(whole.view(np.uint32), nk.dots_packed(to_gpu(a), nk.dots_pack(to_gpu(b), dtype)).cpu().numpy().view(np.uint32))
 
 
+@pytest.mark.parametrize("dtype", ["i8", "bf16"])
+def test_eight_threads_miss_the_image_cache_at_once(oracle, dtype):
+    """A host image that no earlier call has uploaded (packed on the device, then copied to the host): the first calls
+    from eight threads all miss the cache of device copies together. One of them uploads the image, the others wait for
+    that copy, and nobody may multiply with a copy whose transfers are still in flight. The image is large enough to go
+    up in several pieces."""
+    m, n, k = 512, 4100, 4096 if dtype == "i8" else 2048
+    rng = np.random.default_rng(913)
+    a = support.random_matrix(oracle, dtype, m, k, rng)
+    b = support.random_matrix(oracle, dtype, n, k, rng)
+    lib = nk.library()
+    entry = getattr(lib, f"nk_dots_packed_{dtype}")
+    expected = nk.dots_packed(to_gpu(a), nk.dots_pack(to_gpu(b), dtype)).cpu().numpy()
+    for attempt in range(3):
+        lib.nk_hip_image_cache_clear()
+        image = nk.dots_pack(to_gpu(b), dtype).buffer.cpu().numpy()  # a fresh number in its header every time
+        assert image.nbytes > 16 << 20
+        pieces = np.full((m, n), -1, np.int32).view(support.OUTPUT[dtype])
+        start = threading.Barrier(THREADS)
+
+        def call(first, count):
+            entry(a.ctypes.data + first * a.strides[0], image.ctypes.data, pieces.ctypes.data + first * pieces.strides[0],
+                  count, n, k, a.strides[0], pieces.strides[0])
+
+        failures = []
+
+        def worker(index):
+            lib.nk_configure_thread(ctypes.c_uint64(lib.nk_capabilities()))
+            start.wait()
+            call(index * TILE, TILE)
+            message = lib.nk_amd_last_error()
+            if message:
+                failures.append(message.decode())
+
+        threads = [threading.Thread(target=worker, args=(index,)) for index in range(THREADS)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert not failures, failures[:3]
+        assert np.array_equal(pieces.view(np.uint32), expected.view(np.uint32)), f"{dtype} attempt {attempt}"
+    lib.nk_hip_image_cache_clear()
+
+
 def test_tile_config_hook_is_per_thread():
     """The test hook that forces a tile shape reaches the calling thread's launches only."""
     lib = nk.library()

@@ -57,7 +57,8 @@ def test_past_one_grid_of_workgroups(oracle, dtype):
     """Rows deeper than 65535 x 32 values and products taller than 65535 tiles take several launches inside one call (the
     reference has no such bound: dots/serial.h:2458-2491): a depth of 2,100,001 on 2 x 3 outputs, bit for bit against the
     serial restatement; 4,200,000 rows of depth 3 against one column, bit for bit against a plain f64 product of small
-    integers, and the symmetric form of the same call shape for its diagonal bookkeeping across bands."""
+    integers. (The symmetric kinds cannot reach a second band: a window of more than 4,194,176 rows of a result that
+    wide does not fit any memory, so the per-band shift of their diagonal is exercised by no test.)"""
     rng = np.random.default_rng(905)
     a, b = support.random_matrix(oracle, dtype, 2, 2_100_001, rng), support.random_matrix(oracle, dtype, 3, 2_100_001, rng)
     assert same_bits(gpu_dots(dtype, a, b), oracle.dots_packed(dtype, a, b))
