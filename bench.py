@@ -12,7 +12,7 @@ Every step sits between two events of its own on the launch stream: `kernel_ms` 
 `kernel_ms_median` and `kernel_ms_min` come from the per-step pairs (include/numkong/dots/README.md:127-135 quotes
 medians). `others` also holds, measured in the same process on the same box: the vendor library's GEMM on the same
 operands (`vendor_*`: torch._int_mm / torch.matmul, which run hipBLASLt; timing only) and the rate an MFMA-only loop
-sustains (`mfma_ceiling`, numkong_amd/lib/mfma_probes), so that a reader can tell the kernel from the part.
+sustains (`mfma_ceiling`, tests/probes/mfma_probes), so that a reader can tell the kernel from the part.
 
 The symmetric kinds (`--metric symmetric`, `symmetric-angular`, `symmetric-euclidean`; N vectors of depth K, M is
 ignored) time the whole call as the reference's benchmark does (bench/bench.hpp:397-438): packing the vectors,
@@ -317,12 +317,12 @@ def time_vendor(dtype, m, n, k, steps, warmup):
 
 
 def mfma_ceiling():
-    """The rate an MFMA-only loop sustains on this box (numkong_amd/lib/mfma_probes ceiling), as a child process."""
+    """The rate an MFMA-only loop sustains on this box (tests/probes/mfma_probes ceiling), as a child process."""
     import subprocess
 
-    probe = os.path.join(ROOT, "numkong_amd", "lib", "mfma_probes")
+    probe = os.path.join(ROOT, "tests", "probes", "mfma_probes")
     if not os.path.exists(probe):
-        return {"error": "numkong_amd/lib/mfma_probes is not built"}
+        return {"error": "tests/probes/mfma_probes is not built"}
     try:
         done = subprocess.run([probe, "ceiling", "--json"], capture_output=True, text=True, timeout=120)
         return json.loads(done.stdout) if done.returncode == 0 else {"error": done.stderr[-300:]}

@@ -71,10 +71,10 @@
  *      nk_reduce_moments_{f32,f64}_serial; distances against nk_{angulars,euclideans}_{packed,symmetric}_{f32,f64}_serial
  *      to 16 units of 2^-53 (their norms come from the host-dispatched moments), and against closed forms.
  *
- *  Parity unpinned: the per-column norms of FLOAT types in the serial packed image as stored bytes (the
- *  reference computes them with the host-dispatched nk_reduce_moments_*, whose summation order is not restated
- *  here). They are not read by dots_packed; nko_serial_pack writes zeros there and the tests compare header +
- *  rows only. nko_serial_spatials takes its norms from the unpacked rows instead.
+ *  The per-column norms behind the rows of the serial packed image (dots/serial.h:326-332) are the sums of squares
+ *  above: the reference takes them from whatever nk_reduce_moments_<T> its dispatch table holds, so the image is
+ *  pinned byte for byte, norms included, against nk_dots_pack_<T>_serial with that table set to the serial kernels
+ *  (nk_dispatch_table_update), and header + rows against it under any table. Nothing here is "parity unpinned".
  */
 #include <math.h>
 #include <stddef.h>
@@ -311,6 +311,8 @@ NKO_API size_t nko_serial_packed_size(int dtype, size_t columns, size_t depth) {
     return 64 + columns * serial_padded_depth(dtype, depth) * serial_packed_element_bytes(dtype) + columns * 4;
 }
 
+static uint32_t row_sumsq_bits(int dtype, void const *row, size_t depth);
+
 NKO_API void nko_serial_pack(int dtype, void const *b, size_t columns, size_t depth, size_t b_stride, void *packed) {
     size_t const padded = serial_padded_depth(dtype, depth);
     size_t const width = serial_packed_element_bytes(dtype);
@@ -326,18 +328,9 @@ NKO_API void nko_serial_pack(int dtype, void const *b, size_t columns, size_t de
             for (size_t l = 0; l < depth; ++l) ((float *)target)[l] = nko_f16_to_f32(((uint16_t const *)source)[l]);
         else memcpy(target, source, depth * width);
     }
+    /* the norms behind the rows: u32 for the integers, f32 for the floats (dots/serial.h:124-164, 326-332) */
     uint32_t *norms = (uint32_t *)(rows + columns * padded * width);
-    for (size_t j = 0; j < columns; ++j) {
-        uint64_t sum_of_squares = 0;
-        if (dtype == NKO_I8 || dtype == NKO_U8) {
-            unsigned char const *source = (unsigned char const *)b + j * b_stride;
-            for (size_t l = 0; l < depth; ++l) {
-                int64_t const v = dtype == NKO_I8 ? (int64_t)((int8_t const *)source)[l] : (int64_t)source[l];
-                sum_of_squares += (uint64_t)(v * v);
-            }
-        }
-        norms[j] = (uint32_t)sum_of_squares; /* float dtypes: zeros, see "parity unpinned" in the file header */
-    }
+    for (size_t j = 0; j < columns; ++j) norms[j] = row_sumsq_bits(dtype, (unsigned char const *)b + j * b_stride, depth);
 }
 
 #pragma endregion Serial packed layout

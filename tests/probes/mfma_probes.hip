@@ -1,7 +1,9 @@
 /**
  *  @brief What the matrix cores of this GPU do, measured: the rate an MFMA-only loop sustains, and how the fp8, f16
  *         and bf16 forms round. The product kernels are designed around these facts; this program states them.
- *  @file numkong_amd/csrc/probes/mfma_probes.hip
+ *  @file tests/probes/mfma_probes.hip
+ *
+ *  Measurement code, not part of the library: nothing under numkong_amd/ builds, links or loads it.
  *
  *      mfma_probes ceiling [--json]     every MFMA form the kernels could use, fed from registers only, in the 8 x 2
  *                                       block arrangement of the 256 x 256 product tile, on random and on zero data:
@@ -23,8 +25,9 @@
  *                                       x 768, i8 -> i32: 0.75 GiB read, 4 GiB written) with no arithmetic at all:
  *                                       only written, only read, and both at once by separate workgroups.
  *
- *  Built by the Makefile next to the library (numkong_amd/lib/mfma_probes); bench.py runs the first mode and reports
- *  it under `others.mfma_ceiling`, tests/test_mfma_numerics_gpu.py runs the second.
+ *  Built by the Makefile next to it (tests/probes/mfma_probes); bench.py runs the first mode and reports it under
+ *  `others.mfma_ceiling`, tests/test_mfma_numerics_gpu.py runs the second, and the last two are the commands behind the
+ *  summaries profiles/mfma_budget.txt and profiles/memory_stream.txt.
  */
 #include <hip/hip_runtime.h>
 

@@ -10,6 +10,7 @@ Checks, in the order of strength:
     products from numpy int64, powers of two, f64 matmul of decoded inputs.
 NaN payloads are never compared: the reference's own cast backends disagree on them.
 """
+import ctypes
 import os
 
 import numpy as np
@@ -139,7 +140,15 @@ def test_serial_layout_and_product_match_reference(oracle, reference, dtype):
             body = 64 + n * padded * (4 if dtype == "f16" else a.itemsize)
             assert np.array_equal(mine[:body], theirs[:body])
             if dtype in ("i8", "u8"):
-                assert np.array_equal(mine, theirs[: len(mine)])  # integer norms too
+                assert np.array_equal(mine, theirs[: len(mine)])  # integer norms too: every backend's are exact
+            else:
+                # The float norms behind the rows come from the reduce kernel in the reference's dispatch table
+                # (dots/serial.h:124-143): with the table set to the serial kernels the whole image is pinned.
+                reference.lib.nk_dispatch_table_update(ctypes.c_uint64(support.CAP_SERIAL))
+                try:
+                    assert np.array_equal(mine, reference.pack(dtype, b)[: len(mine)])
+                finally:
+                    reference.lib.nk_dispatch_table_update(ctypes.c_uint64(reference.capabilities))
             assert same_floats(oracle.dots_packed(dtype, a, b).view(np.float32), reference.dots_packed(dtype, a, b).view(np.float32))
 
 
