@@ -480,41 +480,32 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
         if ((e = hipGetLastError()) != hipSuccess) return fail(e, "write_header_kernel");
     }
     if (g.n_tiles && g.k_chunks) {
-        uint64_t const blocks = (uint64_t)g.n_tiles * (g.k_chunks / kStageChunks);
-        if (blocks > 0x7FFFFFFFull) return fail_msg("nk_hip_dots_pack: matrix too large");
         uint32_t const xr = dtype == kU8 ? 0x80808080u : 0u;
-        void (*kernel)(uint8_t const *, uint64_t, uint32_t, uint64_t, uint32_t, uint8_t *, int, uint32_t, PackedHeader) = pack_kernel<0>;
+        // by how the source is widened and by what the image then holds (see pack_kernel)
+        typedef void (*pack_fn)(uint8_t const *, uint64_t, uint32_t, uint64_t, uint32_t, uint32_t, uint8_t *, uint32_t *,
+                                uint32_t *, int, uint32_t, int, PackedHeader);
+        pack_fn kernel = nullptr;
         switch (widen_kind_of(dtype, k)) {
-        case 1: kernel = pack_kernel<1>; break;
-        case 2: kernel = pack_kernel<2>; break;
-        case 3: kernel = pack_kernel<3>; break;
-        case 4: kernel = pack_kernel<4>; break;
-        case 5: kernel = pack_kernel<5>; break;
-        case 6: kernel = pack_kernel<6>; break;
-        case 7: kernel = pack_kernel<7>; break;
-        case 8: kernel = pack_kernel<8>; break;
-        default: break;
+        case 0: kernel = dtype == kI8 ? pack_kernel<0, 0> : (dtype == kU8 ? pack_kernel<0, 1> : (dtype == kBF16 ? pack_kernel<0, 2> : pack_kernel<0, 3>)); break;
+        case 1: kernel = pack_kernel<1, 3>; break;
+        case 2: kernel = pack_kernel<2, 3>; break;
+        case 3: kernel = pack_kernel<3, 0>; break;
+        case 4: kernel = pack_kernel<4, 3>; break;
+        case 5: kernel = pack_kernel<5, 0>; break;
+        case 6: kernel = pack_kernel<6, 0>; break;
+        case 7: kernel = pack_kernel<7, 4>; break;
+        default: kernel = pack_kernel<8, 3>; break;
         }
-        hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t const *)b, (uint64_t)b_stride,
-                           g.n, g.k_src_bytes, g.k_chunks, data, widest_load(b, b_stride), xr, h);
+        hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(kPackThreads), 0, stream, (uint8_t const *)b, (uint64_t)b_stride, g.n,
+                           g.k_src_bytes, g.k_chunks, g.k, data, sums, norms, widest_load(b, b_stride), xr, terms ? 1 : 0, h);
         e = hipGetLastError();
         if (e != hipSuccess) return fail(e, "pack_kernel");
     }
-    if (g.n_tiles && terms) {
-        if (g.k_chunks && dtype != kU1) { // (the 1-bit type has the dot-product kinds only, which read no terms: zeros)
-            // by what the image holds: signed bytes (i8, the widened 4-bit types and bits, e2m3 as 8 x its values), offset u8, bf16, f16 (and what is widened to it)
-            auto kernel = dtype == kI8 || dtype == kI4 || dtype == kU4 || (dtype == kE2M3 && e2m3_as_integers(k))
-                              ? column_terms_kernel<0>
-                              : (dtype == kU8 ? column_terms_kernel<1> : (dtype == kBF16 ? column_terms_kernel<2> : column_terms_kernel<3>));
-            hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(32 * kColumnParts), 0, stream, (uint8_t const *)data, g.k_chunks, g.k, sums, norms);
-        }
-        else {
-            uint64_t const count = 2 * (uint64_t)g.n_tiles * kTileRows; // both arrays, back to back
-            hipLaunchKernelGGL(fill_u32_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, stream, sums, count,
-                               0u);
-        }
+    else if (g.n_tiles && terms) { // no depth at all: the terms are zeros
+        uint64_t const count = 2 * (uint64_t)g.n_tiles * kTileRows; // both arrays, back to back
+        hipLaunchKernelGGL(fill_u32_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, stream, sums, count, 0u);
         e = hipGetLastError();
-        if (e != hipSuccess) return fail(e, "column_terms_kernel");
+        if (e != hipSuccess) return fail(e, "fill_u32_kernel");
     }
     return 0;
 }

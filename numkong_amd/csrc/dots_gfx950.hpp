@@ -404,46 +404,6 @@ inline int widen_kind_of(int dtype, size_t k) {
 
 #pragma region Packing
 
-/**
- *  One thread per 16-byte chunk of the image. A block of 256 threads covers 32 rows x 8 chunks: reads are
- *  128 (64 for the widened types) contiguous bytes per row, writes are eight 512-byte runs. WIDEN: 0 copies the
- *  elements, 3 rewrites e2m3 bytes as i8 values in place, 7 copies the 16 bits of a chunk of the 1-bit type as they
- *  are (eight 64-byte runs), otherwise the kind of widen_chunk (8 source bytes per chunk).
- */
-template <int WIDEN>
-__global__ __launch_bounds__(256) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
-                                                   uint64_t k_src_bytes, uint32_t k_chunks, uint8_t *__restrict__ data,
-                                                   int avec, uint32_t xr, PackedHeader header) {
-    constexpr int kSrcChunk = WIDEN == 0 || WIDEN == 3 ? 16 : (WIDEN == 7 ? 2 : 8);
-    constexpr int kImageChunk = WIDEN == 7 ? 2 : kChunkBytes;
-    if (blockIdx.x == 0 && threadIdx.x == 0) *(PackedHeader *)(data - sizeof(PackedHeader)) = header; // (64 bytes in front of the tiles)
-    uint32_t const groups = k_chunks / kStageChunks;
-    uint32_t const tile = blockIdx.x / groups;
-    uint32_t const group = blockIdx.x % groups;
-    uint32_t const r = threadIdx.x >> 3;
-    uint32_t const c = group * kStageChunks + (threadIdx.x & 7);
-    uint64_t const row = (uint64_t)tile * kTileRows + r;
-    int64_t const left = (int64_t)k_src_bytes - (int64_t)c * kSrcChunk;
-    int const valid = row < n ? (int)(left > kSrcChunk ? kSrcChunk : (left < 0 ? 0 : left)) : 0;
-    v4i v = {0, 0, 0, 0};
-    if (valid > 0) {
-        uint8_t const *src = b + row * b_stride + (uint64_t)c * kSrcChunk;
-        if ((WIDEN == 0 || WIDEN == 3) && valid == 16 && avec >= 16) {
-            v = *(v4i const *)src;
-            v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
-        }
-        else { v = load_chunk_guarded(src, valid, avec, xr); }
-        if constexpr (WIDEN == 3) {
-#pragma unroll
-            for (int w = 0; w < 4; ++w) v[w] = (int)widen_e2m3x4((uint32_t)v[w]);
-        }
-        else if constexpr (WIDEN != 0 && WIDEN != 7) v = widen_chunk<WIDEN>((uint32_t)v[0], (uint32_t)v[1]);
-    }
-    uint8_t *at = data + (((uint64_t)tile * k_chunks + c) * kTileRows + r) * kImageChunk;
-    if constexpr (WIDEN == 7) *(uint16_t *)at = (uint16_t)v[0];
-    else *(v4i *)at = v;
-}
-
 /** Sum of the squares of the 8 values of a 16-byte chunk of bf16 (f32 = bits << 16) or f16, in f64. */
 template <bool BF16_VALUES>
 __device__ __forceinline__ double chunk_sumsq_f64(v4i v) {
@@ -467,29 +427,64 @@ __device__ __forceinline__ double chunk_sumsq_f64(v4i v) {
 }
 
 /**
- *  Per-column terms, from the packed tiles: the u8 compensation term (128 * sum of the signed packed bytes of
- *  the row, mod 2^32; zero for the other types) and the column's sum of squares, which the angular and
- *  euclidean products need (reference: the norms behind the packed rows, dots/serial.h:326-332): exact mod
- *  2^32 for the integer types, accumulated in f64 and rounded once to f32 for the float types.
- *  Sixteen wavefronts per tile (a tile is all the parallelism a workgroup has, and 8192 rows are only 256 tiles):
- *  lane l of wavefront w owns row l % 32 and every 32nd chunk starting at 2 w + l / 32.
- *  KIND: 0 i8, 1 u8, 2 bf16, 3 f16 (and fp8, stored widened to f16).
+ *  Packing, one pass: a workgroup of 1024 threads takes one 32-row tile through the whole depth, 32 chunks of every
+ *  row per step (thread t: row (t / 8) % 32, chunk 8 * (t / 256) + t % 8 of the step, so 8 neighbouring threads read
+ *  128 (64, 16) contiguous source bytes of a row and 8 neighbouring rows write a 128-byte run of the image), and keeps
+ *  the per-column terms of what it writes in registers on the way: the u8 compensation term (128 * the sum of the
+ *  signed packed bytes of the row, mod 2^32; zero for the other types) and the column's sum of squares, which the
+ *  angular and euclidean kinds need (reference: the norms behind the packed rows, dots/serial.h:326-332): exact mod
+ *  2^32 for the integer types, accumulated in f64 and rounded once to f32 for the float types. A thread always works
+ *  on the same row and on the chunks of one residue mod 32; the 32 partial sums of a row are added in ascending
+ *  order of that residue, so the terms do not depend on anything but the row.
+ *  WIDEN: 0 copies the elements, 3 rewrites e2m3 bytes as i8 values in place, 7 copies the 16 bits of a chunk of the
+ *  1-bit type as they are, otherwise the kind of widen_chunk (8 source bytes per chunk).
+ *  KIND, by what the image holds: 0 signed bytes (i8, the widened 4-bit types, e2m3 as 8 x its values), 1 u8 stored
+ *  with its offset, 2 bf16, 3 f16 (and what is widened to it), 4 bits (no terms: zeros).
+ *  `terms` == 0: the tiles only (callers that will never read the terms).
  */
-constexpr int kColumnParts = 32; // 32-lane groups of a workgroup of column_terms_kernel, each with a share of the chunks
-template <int KIND>
-__global__ __launch_bounds__(32 * kColumnParts) void column_terms_kernel(uint8_t const *__restrict__ data, uint32_t k_chunks, uint32_t k,
-                                                           uint32_t *__restrict__ sums, uint32_t *__restrict__ norms) {
-    __shared__ int part_sum[kColumnParts][32];
-    __shared__ uint32_t part_squares[kColumnParts][32];
-    __shared__ double part_f64[kColumnParts][32];
+constexpr int kPackThreads = 1024;
+constexpr int kPackChunks = kPackThreads / kTileRows; // chunks of every row per step of a workgroup
+template <int WIDEN, int KIND>
+__global__ __launch_bounds__(kPackThreads) void pack_kernel(uint8_t const *__restrict__ b, uint64_t b_stride, uint32_t n,
+                                                            uint64_t k_src_bytes, uint32_t k_chunks, uint32_t k,
+                                                            uint8_t *__restrict__ data, uint32_t *__restrict__ sums,
+                                                            uint32_t *__restrict__ norms, int avec, uint32_t xr, int terms,
+                                                            PackedHeader header) {
+    constexpr int kSrcChunk = WIDEN == 0 || WIDEN == 3 ? 16 : (WIDEN == 7 ? 2 : 8);
+    constexpr int kImageChunk = WIDEN == 7 ? 2 : kChunkBytes;
+    __shared__ int part_sum[kPackChunks][kTileRows];
+    __shared__ uint32_t part_squares[kPackChunks][kTileRows];
+    __shared__ double part_f64[kPackChunks][kTileRows];
+    if (blockIdx.x == 0 && threadIdx.x == 0) *(PackedHeader *)(data - sizeof(PackedHeader)) = header; // (64 bytes in front of the tiles)
     uint32_t const tile = blockIdx.x;
-    uint32_t const first = threadIdx.x >> 5, row = threadIdx.x & 31; // chunk residue mod 32, row of the tile
-    uint8_t const *base = data + (uint64_t)tile * k_chunks * kTileChunkBytes + row * kChunkBytes;
+    uint32_t const r = (threadIdx.x >> 3) & 31;
+    uint32_t const part = ((threadIdx.x >> 8) << 3) | (threadIdx.x & 7); // chunk of the step = residue of the chunk mod 32
+    uint64_t const row = (uint64_t)tile * kTileRows + r;
+    uint8_t const *source = b + row * b_stride;
+    uint8_t *target = data + ((uint64_t)tile * k_chunks * kTileRows + r) * kImageChunk;
     int sum = 0;
     uint32_t squares = 0;
     double squares_f64 = 0;
     auto take = [&](uint32_t c) {
-        v4i const v = *(v4i const *)(base + (uint64_t)c * kTileChunkBytes);
+        int64_t const left = (int64_t)k_src_bytes - (int64_t)c * kSrcChunk;
+        int const valid = row < n ? (int)(left > kSrcChunk ? kSrcChunk : (left < 0 ? 0 : left)) : 0;
+        v4i v = {0, 0, 0, 0};
+        if (valid > 0) {
+            uint8_t const *src = source + (uint64_t)c * kSrcChunk;
+            if ((WIDEN == 0 || WIDEN == 3) && valid == 16 && avec >= 16) {
+                v = __builtin_nontemporal_load((v4i const *)src); // (read once)
+                v[0] ^= (int)xr, v[1] ^= (int)xr, v[2] ^= (int)xr, v[3] ^= (int)xr;
+            }
+            else { v = load_chunk_guarded(src, valid, avec, xr); }
+            if constexpr (WIDEN == 3) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) v[w] = (int)widen_e2m3x4((uint32_t)v[w]);
+            }
+            else if constexpr (WIDEN != 0 && WIDEN != 7) v = widen_chunk<WIDEN>((uint32_t)v[0], (uint32_t)v[1]);
+        }
+        uint8_t *at = target + (uint64_t)c * (kTileRows * kImageChunk);
+        if constexpr (WIDEN == 7) *(uint16_t *)at = (uint16_t)v[0];
+        else *(v4i *)at = v;
         if (KIND == 0) {
 #pragma unroll
             for (int w = 0; w < 4; ++w) squares = (uint32_t)__builtin_amdgcn_sdot4(v[w], v[w], (int)squares, false);
@@ -501,25 +496,22 @@ __global__ __launch_bounds__(32 * kColumnParts) void column_terms_kernel(uint8_t
                 squares = (uint32_t)__builtin_amdgcn_sdot4(v[w], v[w], (int)squares, false);
             }
         }
-        else { squares_f64 += chunk_sumsq_f64<KIND == 2>(v); }
+        else if (KIND == 2 || KIND == 3) { squares_f64 += chunk_sumsq_f64<KIND == 2>(v); }
     };
-    if (KIND < 2) { // four loads in flight per lane (i8 8192 x 8192: the whole pack 42 -> 32 us); the f64 chain of the floats gains nothing from it
 #pragma unroll 4
-        for (uint32_t c = first; c < k_chunks; c += kColumnParts) take(c);
-    }
-    else {
-        for (uint32_t c = first; c < k_chunks; c += kColumnParts) take(c);
-    }
-    part_sum[first][row] = sum, part_squares[first][row] = squares, part_f64[first][row] = squares_f64;
+    for (uint32_t c = part; c < k_chunks; c += kPackChunks) take(c);
+    if (!terms) return;
+    part_sum[part][r] = sum, part_squares[part][r] = squares, part_f64[part][r] = squares_f64;
     __syncthreads();
-    if (threadIdx.x < 32) {
+    if (threadIdx.x < kTileRows) {
+        uint32_t const mine = threadIdx.x;
         sum = 0, squares = 0, squares_f64 = 0;
 #pragma unroll
-        for (int part = 0; part < kColumnParts; ++part) sum += part_sum[part][row], squares += part_squares[part][row], squares_f64 += part_f64[part][row];
+        for (int p = 0; p < kPackChunks; ++p) sum += part_sum[p][mine], squares += part_squares[p][mine], squares_f64 += part_f64[p][mine];
         // u8 is stored as b - 128 (and its padding as 0): sum(b^2) = sum((b - 128)^2) + 256 * sum(b - 128) + 128^2 * k
         if (KIND == 1) squares += 256u * (uint32_t)sum + 16384u * k;
-        sums[(uint64_t)tile * kTileRows + row] = (uint32_t)sum * 128u;
-        norms[(uint64_t)tile * kTileRows + row] = KIND < 2 ? squares : __builtin_bit_cast(uint32_t, (float)squares_f64);
+        sums[(uint64_t)tile * kTileRows + mine] = (uint32_t)sum * 128u;
+        norms[(uint64_t)tile * kTileRows + mine] = KIND < 2 ? squares : (KIND == 4 ? 0u : __builtin_bit_cast(uint32_t, (float)squares_f64));
     }
 }
 
@@ -800,6 +792,33 @@ __device__ __forceinline__ uint32_t distance_from_dot(uint32_t dot_bits, float q
     return __builtin_bit_cast(uint32_t, result);
 }
 
+/** The hardware's reciprocal square root (good to about a unit in the last place) refined by one Newton step with a
+ *  fused residual. Zero gives NaN (infinity times zero), which is what angular_from_factors wants of it. */
+__device__ __forceinline__ float refined_rsqrt(float x) {
+    float const root = __builtin_amdgcn_rsqf(x);
+    float const residual = __builtin_fmaf(-(x * root), root, 1.0f);
+    return __builtin_fmaf(root * 0.5f, residual, root);
+}
+
+/**
+ *  The angular distance where it is cheap: 1 - dot * (rq * rt), with rq and rt the refined reciprocal square roots of
+ *  the row's and the column's sums of squares, taken once per row and once per column of a tile instead of once per
+ *  output. Three roundings of relative size 2^-24 enter the cosine instead of the one and a half of the full
+ *  finaliser, so the form is only used where the cosine is at most a quarter in magnitude (`*cheap`): its error is
+ *  then under a unit of 2^-24, below the rounding of the result itself (1 - cos lies in [0.75, 1.25] there). Zero or
+ *  overflowed sums of squares make the factors NaN or infinite and fail the test. Everything else, identical rows
+ *  above all, takes distance_from_dot.
+ */
+template <class T>
+__device__ __forceinline__ float angular_from_factors(uint32_t dot_bits, float row_factor, float column_factor, bool *cheap) {
+    float const dot = T::kDtype == kI8 || T::kDtype == kI4
+                          ? (float)(int)dot_bits
+                          : (T::kDtype == kU8 || T::kDtype == kU4 ? (float)dot_bits : __builtin_bit_cast(float, dot_bits));
+    float const scale = row_factor * column_factor;
+    *cheap = __builtin_fabsf(dot * scale) <= 0.25f; // (false for NaN)
+    return __builtin_fmaf(-dot, scale, 1.0f);
+}
+
 #pragma endregion Element types
 
 #pragma region Packed product
@@ -996,6 +1015,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     __shared__ uint32_t row_part[T::kUnsigned ? 2 * BM * kStageChunks : 1]; // u8 only: the partial sums behind them
     typedef typename T::norm_t norm_t;
     __shared__ __attribute__((aligned(16))) uint32_t row_norms[NORMS ? BM : 4]; // distances only: sum of squares of each A row
+    __shared__ __attribute__((aligned(16))) float row_factors[NORMS ? BM : 4];  // ... and its refined reciprocal square root
     __shared__ norm_t norm_part[NORMS ? 2 * BM * kStageChunks : 1];              // ... and the partial sums behind them
 
     uint32_t const tid = threadIdx.x, lane = tid & 63;
@@ -1484,6 +1504,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                     if constexpr (sizeof(norm_t) == 8) bits = __builtin_bit_cast(uint32_t, (float)sum); // f64 -> f32, once
                     else bits = (uint32_t)sum;
                     row_norms[tid] = __builtin_bit_cast(uint32_t, norm_as_f32<T>(bits));
+                    row_factors[tid] = refined_rsqrt(norm_as_f32<T>(bits));
                 }
             }
             __syncthreads();
@@ -1542,7 +1563,10 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 // scalar registers overflow).
                 global_u8_t *row_base = c_tile + j * 128;
                 v4i row_term4 = {0, 0, 0, 0}, row_norm4 = {0, 0, 0, 0};
+                typedef float v4f __attribute__((ext_vector_type(4)));
+                v4f row_factor4 = {0, 0, 0, 0};
                 float const col_value = metric != 0 ? norm_as_f32<T>(col_norm[j]) : 0.0f;
+                float const col_factor = metric == 1 ? refined_rsqrt(col_value) : 0.0f;
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -1556,10 +1580,24 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                             if (v % 4 == 0) row_term4 = *(v4i const *)&row_terms[i * 32 + 8 * (v / 4) + 4 * half];
                             bits += (uint32_t)row_term4[v % 4] + col_term[j];
                         }
-                        if (metric != 0) {
+                        if (metric == 1) {
+                            // the cheap form where it is good enough (almost everywhere on vectors that are not near
+                            // copies of each other), the full finaliser for the lanes where it is not
+                            if (v % 4 == 0) row_factor4 = *(v4f const *)&row_factors[i * 32 + 8 * (v / 4) + 4 * half];
+                            bool cheap;
+                            float const quick = angular_from_factors<T>(bits, row_factor4[v % 4], col_factor, &cheap);
+                            uint32_t result = __builtin_bit_cast(uint32_t, quick);
+                            if (__builtin_amdgcn_ballot_w64(!cheap) != 0) { // (uniform: the wavefront branches as one)
+                                int const row_bits = *(int const *)&row_norms[i * 32 + 8 * (v / 4) + 4 * half + v % 4];
+                                uint32_t const full = distance_from_dot<T, 1>(bits, __builtin_bit_cast(float, row_bits), col_value);
+                                result = cheap ? result : full;
+                            }
+                            bits = result;
+                        }
+                        else if (metric != 0) {
                             if (v % 4 == 0) row_norm4 = *(v4i const *)&row_norms[i * 32 + 8 * (v / 4) + 4 * half];
                             int const row_bits = row_norm4[v % 4];
-                            bits = distance_from_dot<T, metric == 2 ? 2 : 1>(bits, __builtin_bit_cast(float, row_bits), col_value);
+                            bits = distance_from_dot<T, 2>(bits, __builtin_bit_cast(float, row_bits), col_value);
                         }
                         bool keep = true;
                         if (masked) {
