@@ -577,6 +577,11 @@ struct I8 {
     static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
     }
+    /** The same with nothing to add to: the first product of a sum (the zero is an operand of the instruction). */
+    static __device__ __forceinline__ void mma_fresh(acc_t &acc, v4i a, v4i b) {
+        acc_t const zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, zero, 0, 0, 0);
+    }
 };
 struct U8 : I8 {
     static constexpr int kDtype = kU8;
@@ -620,6 +625,11 @@ struct BF16 {
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), acc, 0,
                                                       0, 0);
     }
+    static __device__ __forceinline__ void mma_fresh(acc_t &acc, v4i a, v4i b) {
+        acc_t const zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), zero, 0,
+                                                      0, 0);
+    }
 };
 struct F16 {
     static constexpr bool kChunked = kHalfChunked;
@@ -661,6 +671,11 @@ struct F16 {
     }
     static __device__ __forceinline__ void mma(acc_t &acc, v4i a, v4i b) {
         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), acc, 0, 0,
+                                                     0);
+    }
+    static __device__ __forceinline__ void mma_fresh(acc_t &acc, v4i a, v4i b) {
+        acc_t const zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), zero, 0, 0,
                                                      0);
     }
 };
@@ -850,6 +865,10 @@ struct Totals {
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
             }
     }
+    __device__ __forceinline__ void clear_block(int i, int j) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) value[i][j][v] = 0;
+    }
     __device__ __forceinline__ auto finish(acc_t const (&acc)[TM][TN], int i, int j, int v) const {
         return acc[i][j][v] + value[i][j][v];
     }
@@ -858,6 +877,7 @@ template <class acc_t, int TM, int TN>
 struct Totals<acc_t, TM, TN, false> {
     __device__ __forceinline__ void clear() {}
     __device__ __forceinline__ void fold(acc_t (&)[TM][TN]) {}
+    __device__ __forceinline__ void clear_block(int, int) {}
     __device__ __forceinline__ auto finish(acc_t const (&acc)[TM][TN], int i, int j, int v) const { return acc[i][j][v]; }
 };
 
@@ -1156,7 +1176,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     auto load_a = [&](TileView const &view, uint32_t s, auto slot_tag, auto part_tag) {
         constexpr int slot = decltype(slot_tag)::value, part = decltype(part_tag)::value;
         __amdgpu_buffer_rsrc_t const rsrc = a_rsrc_of(view);
-        uint32_t const stage_offset = s * kSrcStage;
+        uint32_t const stage_offset = __builtin_amdgcn_readfirstlane(s * kSrcStage); // (the same in all lanes: see load_b)
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             if (i * 4 / kLoads != part) continue;
@@ -1244,13 +1264,13 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         __amdgpu_buffer_rsrc_t const rsrc = b_rsrc_of(view);
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
+            // (the same in all lanes; saying so keeps the offset a scalar operand where the compiler has lost track of it,
+            // instead of a loop over the lanes' values)
+            uint32_t const tile_offset = __builtin_amdgcn_readfirstlane(view.b_tile[j] + s * (kStageChunks * kImageTileChunk));
             if constexpr (T::kImageChunk == 2) // (sixteen bits per lane: the rest of the register is never looked at)
-                b_reg[slot][j][q][0] = (int)(uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, b_lane + q * 2 * kImageTileChunk,
-                                                                                           view.b_tile[j] + s * (kStageChunks * kImageTileChunk), 0);
+                b_reg[slot][j][q][0] = (int)(uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, b_lane + q * 2 * kImageTileChunk, tile_offset, 0);
             else
-                b_reg[slot][j][q] = __builtin_bit_cast(
-                    v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_lane + q * 2 * kImageTileChunk,
-                                                               view.b_tile[j] + s * (kStageChunks * kImageTileChunk), 0));
+                b_reg[slot][j][q] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_lane + q * 2 * kImageTileChunk, tile_offset, 0));
         }
     };
     auto read_frags = [&](auto buffer_tag, auto q_tag, auto parity_tag) {
@@ -1267,6 +1287,20 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             v4i const b = T::operand_b(b_reg[slot][j][q]);
 #pragma unroll
             for (int i = 0; i < TM; ++i) T::mma(acc[i][j], af[q & 1][i], b);
+        }
+    };
+    // The same for the first k-step of a tile: its MFMAs start the sums from a zero operand, so that no accumulator is
+    // ever cleared (the totals of the chunked types are, a block's in front of its MFMA).
+    auto multiply_fresh = [&](auto slot_tag, auto q_tag) {
+        constexpr int slot = decltype(slot_tag)::value, q = decltype(q_tag)::value;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            v4i const b = T::operand_b(b_reg[slot][j][q]);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                total.clear_block(i, j);
+                T::mma_fresh(acc[i][j], af[q & 1][i], b);
+            }
         }
     };
     // What staging one chunk of A costs besides its LDS write: vector operations (u8: four exclusive-ors and the byte
@@ -1319,11 +1353,25 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             if (writes && kLoads > rest) __builtin_amdgcn_sched_group_barrier(0x200, kLoads - rest, 0);
         }
     };
+    // The first k-step of a tile of the chunked types: in front of every MFMA the 16 zeros of its block's total;
+    // fragment reads and loads as in any k-step without LDS writes.
+    auto schedule_fresh_k_step = [&]() {
+        constexpr int loads = TN + (kLoads >= 4 ? kLoads / 4 : 1);
+#pragma unroll
+        for (int i = 0; i < TM * TN; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);
+            if (i < TM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i >= TM && i - TM < loads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        if (TM * TN - TM < loads) __builtin_amdgcn_sched_group_barrier(0x020, loads - (TM * TN - TM), 0);
+    };
     // One stage of the steady state; `P` = stage parity = LDS buffer = register slot. Stages s+2 and
     // s+3 are fetched here; past the tile's end they are the first stages of `nxt` (the next tile, or
     // this one again when nothing follows: loads of valid memory that nobody uses).
-    auto stage = [&](auto parity_tag, uint32_t s) {
+    auto stage = [&](auto parity_tag, uint32_t s, auto entry_tag) __attribute__((always_inline)) {
         constexpr int P = decltype(parity_tag)::value;
+        constexpr int entry = decltype(entry_tag)::value; // 0: in the middle of a sum; 2: the first stage of a tile
         // vector operations behind each MFMA of the k-steps that widen in place: their share of half the chunks
         constexpr int kSpread = T::kPrewiden ? (kLoads * 28 + TM * TN - 1) / (TM * TN) : 0;
         bool const wrap2 = s + 2 >= fast, wrap3 = s + 3 >= fast;
@@ -1331,10 +1379,12 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         TileView const &a2 = wrap2 ? nxt : cur, &a3 = wrap3 ? nxt : cur, &b2 = a2;
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<1>(), slot_c<1>());
-        multiply(slot_c<P>(), slot_c<0>());
+        if constexpr (entry == 2) multiply_fresh(slot_c<P>(), slot_c<0>());
+        else multiply(slot_c<P>(), slot_c<0>());
         load_b(b2, s2, slot_c<P>(), slot_c<0>()), load_a(a2, s2, slot_c<P>(), slot_c<2>());
         if constexpr (T::kPrewiden) prewiden(slot_c<P ^ 1>(), s + 1 < fast ? s + 1 : 0u, slot_c<0>());
-        schedule_k_step(slot_c<0>(), slot_c<kSpread>());
+        if constexpr (entry == 2 && kChunked) schedule_fresh_k_step();
+        else schedule_k_step(slot_c<0>(), slot_c<kSpread>());
         __builtin_amdgcn_sched_barrier(0);
         read_frags(slot_c<P>(), slot_c<2>(), slot_c<0>());
         multiply(slot_c<P>(), slot_c<1>());
@@ -1389,12 +1439,6 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         nxt = view_of(has_next ? tile + gridDim.x : tile);
         uint32_t const row0 = cur.row0, col0 = cur.col0;
 
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
         // u8: the column terms of this tile are fetched now and used in the epilogue, so that nothing has to
         // wait for them (a wait for a load is a wait for every store issued before it).
         uint32_t col_term[TN], col_norm[TN];
@@ -1405,13 +1449,15 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
             if constexpr (T::kUnsigned) col_term[j] = col_terms[(uint64_t)t * kTileRows + (lane & 31)];
             if constexpr (NORMS) col_norm[j] = col_norms[(uint64_t)t * kTileRows + (lane & 31)];
         }
-        total.clear();
 
         {
             if (across || fast > 0) { // (always, when the pipeline runs across tiles: the host checked)
                 if constexpr (!across) prime();
+                // Nothing is cleared at the start of a tile: in its first k-step the first MFMA of every block takes a
+                // zero operand (and the totals of the chunked types are zeroed next to it). Chunked types: every
+                // `chunk_stages` stages the running sums go into the totals.
                 uint32_t until_fold = g.chunk_stages;
-                auto fold_when_due = [&]() {
+                auto fold_when_due = [&]() __attribute__((always_inline)) {
                     if constexpr (kChunked) {
                         until_fold -= 2;
                         if (until_fold == 0) {
@@ -1421,9 +1467,12 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                         }
                     }
                 };
-                for (uint32_t s = 0; s < fast; s += 2) {
-                    stage(slot_c<0>(), s);
-                    stage(slot_c<1>(), s + 1);
+                stage(slot_c<0>(), 0u, slot_c<2>());
+                stage(slot_c<1>(), 1u, slot_c<0>());
+                fold_when_due();
+                for (uint32_t s = 2; s < fast; s += 2) {
+                    stage(slot_c<0>(), s, slot_c<0>());
+                    stage(slot_c<1>(), s + 1, slot_c<0>());
                     fold_when_due();
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -1431,6 +1480,13 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
 
             // Remaining stages: the ragged end of K, or everything when A cannot be read with vector loads.
             if (!across && fast < stages) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+                total.clear();
                 uint8_t const *a_tile = g.a + (uint64_t)row0 * g.a_stride;
                 uint32_t a_slow[kLoads]; // rows clamped to the last one: plain loads have no descriptor to stop them
 #pragma unroll
@@ -1772,6 +1828,15 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream, TriangleScratch const *
         // (measured on 1024 x 1,048,576 x 768: 2.17 against 2.33 ms angular, 1.98 against 2.07 ms euclidean).
         if (args.metric != 0 && best < 3 && args.k_chunks / kStageChunks <= 8 && tiles_of(args, 3) >= 256) best = 3;
         if (T::kChunked && best == 1) best = 2; // two accumulator sets do not fit the 256 x 256 tile
+        // Shallow products into rows of C that do not start on 128-byte lines: the stores go through the L2 (see the
+        // epilogue) and take long enough to matter, and three small workgroups per compute unit overlap one's stores
+        // with the others' loops, which one large tile cannot (measured, 64 x 128 against the tile chosen above: i8
+        // 8192 x 8191 x 1000 0.129 against 0.142 ms, x 512 0.085 against 0.101; f16 8192 x 8191 x 1000 0.239 against
+        // 0.280; i8 4096 x 4095 x 1000 0.036 against 0.039; deeper products and aligned rows lose by it).
+        bool const lines = (((uintptr_t)args.c | args.c_stride) & 127) == 0;
+        if (!lines && !triangle && args.metric == 0 && best < 4 && args.k_chunks / kStageChunks <= (T::kChunked ? 16u : 8u) &&
+            tiles_of(args, 4) >= 256)
+            best = 4;
         // e2m3 pays 13 vector operations for every dword of A it stages: a 128 x 512 tile (every wavefront 128 x 128)
         // stages half as much A per MFMA as 256 x 256 (8192^3: 0.51 against 0.59 ms; for i8 itself the two are equal)
         if (T::kDtype == kE2M3 && !triangle && args.metric == 0 && first == 1 && tiles_of(args, 5) >= 256) best = 5;
