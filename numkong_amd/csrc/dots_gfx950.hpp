@@ -1826,7 +1826,21 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream, TriangleScratch const *
         // Distances over a shallow depth are bound by the epilogue (a finaliser and a store per output): two
         // workgroups per CU of 128 x 128 tiles overlap it with the other's loop better than one large tile does
         // (measured on 1024 x 1,048,576 x 768: 2.17 against 2.33 ms angular, 1.98 against 2.07 ms euclidean).
-        if (args.metric != 0 && best < 3 && args.k_chunks / kStageChunks <= 8 && tiles_of(args, 3) >= 256) best = 3;
+        // Since then the angular finaliser has become cheap where the cosine is small, and what is left of an epilogue's
+        // cost is its length: the code of TM x TN x 16 finalisers and stores does not fit the instruction cache for the
+        // large tiles. Measured, shallow depths (best shape against the others, ms): i8 angular 1024 x 1,048,576 x 768
+        // 128 x 256 1.73, 256 x 256 1.78, 128 x 128 1.90, 64 x 128 2.09, but 8192 x 131,072 x 768 and 8192 x 8192 x
+        // 1024 128 x 128 (1.42 against 1.55; 0.114 against 0.120); u8 128 x 128 (2.29 against 2.54 and 2.91); bf16
+        // angular 1024 x 524,288 x 768 64 x 128 1.58 against 1.72 (128 x 128) and 2.18 (128 x 256), 8192 x 8192 x 1024
+        // 0.198 against 0.267 and 0.319, and still 3.39 against 3.77 at depth 2048; f16 and e4m3 likewise.
+        uint32_t const depth_stages = args.k_chunks / kStageChunks;
+        if (args.metric != 0 && T::kChunked) {
+            if (depth_stages <= 32 && tiles_of(args, 4) >= 256) best = 4;
+        }
+        else if (args.metric != 0 && depth_stages <= 8) {
+            if (!T::kUnsigned && args.m <= 2048 && best < 2 && tiles_of(args, 2) >= 256) best = 2;
+            else if (best < 3 && tiles_of(args, 3) >= 256) best = 3;
+        }
         if (T::kChunked && best == 1) best = 2; // two accumulator sets do not fit the 256 x 256 tile
         // Shallow products into rows of C that do not start on 128-byte lines: the stores go through the L2 (see the
         // epilogue) and take long enough to matter, and three small workgroups per compute unit overlap one's stores
