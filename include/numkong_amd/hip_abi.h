@@ -156,8 +156,9 @@ int nk_hip_fill_rows_async(void *c, size_t m, size_t n, size_t c_stride, uint32_
 /** TEST HOOK, not part of the product interface: forces the tile shape of the calling thread's launches (0 = the
  *  heuristic picks; 1..5 = 256x256, 128x256, 128x128, 64x128, 128x512; bit 7: a forced shape may still split a
  *  triangle; bits 8..27: spread of the workgroups' start times in 10 ns ticks, plus one; bits 28..29: 1 = outputs
- *  stored past the caches, 2 = through them, whatever the alignment of C). The tests use it to run every shape and
- *  both kinds of store over the same small cases; thread-local, so it never reaches another thread's calls. */
+ *  stored past the caches, 2 = through them, whatever the alignment of C; bit 30: A is staged through registers also
+ *  where it would go straight into LDS). The tests use it to run every shape, both kinds of store and both kinds of
+ *  staging over the same cases; thread-local, so it never reaches another thread's calls. */
 void nk_hip_set_tile_config(int config);
 
 /** Thread-local text of the last failure in this layer ("" if none). */

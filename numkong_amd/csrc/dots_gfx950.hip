@@ -708,7 +708,7 @@ int nk_hip_symmetric_static_async(int dtype, int metric, void const *vectors, si
 }
 
 void nk_hip_set_tile_config(int config) {
-    t_forced_config = config; // (bits 0..6 the shape; bit 7: a forced shape may still hand the narrow end of a triangle to small tiles; bits 8..27: start spread in 10 ns ticks + 1; bits 28..29: kind of store)
+    t_forced_config = config; // (bits 0..6 the shape; bit 7: a forced shape may still hand the narrow end of a triangle to small tiles; bits 8..27: start spread in 10 ns ticks + 1; bits 28..29: kind of store; bit 30: no staging straight into LDS)
 }
 
 char const *nk_hip_last_error(void) { return g_last_error; }

@@ -47,7 +47,22 @@
 /** What crosses translation units: the product's arguments, its scratch memory, one launcher per element type. */
 namespace nk_gfx950 {
 
-constexpr uint32_t kTileBand = 8; // tile rows per band of the walk over the tile grid
+// Tile rows per band of the walk over the tile grid. An XCD works on 32 tiles at a time, a band's height times as many
+// columns: 8 x 4 is the shape with the smallest perimeter for the 256 x 256 and the 128 x 256 tile alike, and the
+// perimeter is what the XCD's L2 fetches per sweep of the depth (measured at 8192^3, bytes read per launch: bf16 2.18 GB
+// with 8, 2.75 GB with 4 or 16, 5.28 GB with 2; i8 0.82 GB with 8 or 4, 1.22 GB with 2 or 16). NK_TILE_BAND overrides it
+// for such measurements (make EXTRA=-DNK_TILE_BAND=4).
+#ifndef NK_TILE_BAND
+#define NK_TILE_BAND 8
+#endif
+constexpr uint32_t kTileBand = NK_TILE_BAND;
+#ifndef NK_DIRECT_STAGING
+#define NK_DIRECT_STAGING 1
+#endif
+#ifndef NK_DIRECT_CHUNKED
+#define NK_DIRECT_CHUNKED 0
+#endif
+constexpr bool kDirectStaging = NK_DIRECT_STAGING != 0; // A straight into LDS where that applies (see dots_packed_kernel)
 
 struct GemmArgs {
     uint8_t const *a;
@@ -1022,7 +1037,24 @@ constexpr bool tail_matters_for() {
     return NORMS || T::kUnsigned || !__is_same(typename T::acc_t, v16i);
 }
 
-template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, bool WHOLE = false>
+/** 16 bytes per lane from a buffer straight into LDS at `dst` + 16 x lane (`dst` the same in all lanes). A function of
+ *  its own: the host pass does not know the instruction, and from inside a lambda of a kernel it would take the kernel's
+ *  host side with it. */
+typedef __attribute__((address_space(3))) void lds_void_t;
+__device__ __forceinline__ void fetch_to_lds(__amdgpu_buffer_rsrc_t rsrc, lds_void_t *dst, uint32_t lane_offset, uint32_t offset) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, dst, 16, lane_offset, offset, 0, 0);
+}
+
+/**
+ *  DIRECT: A goes from memory straight into LDS (`buffer_load_dwordx4 ... lds`: 64 lanes x 16 bytes land in 1 KiB of LDS
+ *  in lane order, so a lane fetches the chunk that belongs at its position of the swizzled row), not through registers
+ *  and `ds_write`. LDS is then a ring of four stages, each an array of its own (the compiler tracks what such a load
+ *  writes per array, and only so do the waits for one stage's loads not wait for the next stages' as well); a stage's
+ *  loads are issued three stages ahead, and one trip of the loop is four stages. For types that reach LDS as they are
+ *  in memory, depths of a whole number of trips, the pipelined kernel across tiles, dot products only (the host
+ *  checks).
+ */
+template <class T, int TM, int TN, bool ACROSS, bool NORMS = false, bool WHOLE = false, bool DIRECT = false>
 __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChunked ? 2 : 1))) void dots_packed_kernel(GemmArgs g) {
     typedef typename T::acc_t acc_t;
     constexpr int BM = TM * 32;
@@ -1030,7 +1062,13 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     constexpr int kStageLds = BM * kStageBytes;
     constexpr int kLoads = BM * kStageChunks / NT; // 16-byte LDS chunks per thread per stage = TM
     constexpr int kSrcStage = kStageChunks * T::kSrcChunk; // source bytes of A per row per stage
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStageLds];
+    static_assert(!DIRECT || (ACROSS && !NORMS && !T::kUnsigned && !T::kPrewiden && T::kSrcChunk == 16 && T::kImageChunk == 16),
+                  "straight into LDS: only what needs nothing done to it on the way");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[DIRECT ? 16 : 2 * kStageLds];
+    __shared__ __attribute__((aligned(1024))) uint8_t ring0[DIRECT ? kStageLds : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t ring1[DIRECT ? kStageLds : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t ring2[DIRECT ? kStageLds : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t ring3[DIRECT ? kStageLds : 16];
     __shared__ __attribute__((aligned(16))) uint32_t row_terms[T::kUnsigned ? BM : 4]; // u8 only: 128 * (sum of the bytes of each A row of the tile)
     __shared__ uint32_t row_part[T::kUnsigned ? 2 * BM * kStageChunks : 1]; // u8 only: the partial sums behind them
     typedef typename T::norm_t norm_t;
@@ -1273,10 +1311,14 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                 b_reg[slot][j][q] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_lane + q * 2 * kImageTileChunk, tile_offset, 0));
         }
     };
+    auto ring_of = [&](auto index_tag) -> uint8_t * {
+        constexpr int index = decltype(index_tag)::value & 3;
+        return index == 0 ? ring0 : (index == 1 ? ring1 : (index == 2 ? ring2 : ring3));
+    };
     auto read_frags = [&](auto buffer_tag, auto q_tag, auto parity_tag) {
         constexpr int buffer = decltype(buffer_tag)::value, q = decltype(q_tag)::value,
                       parity = decltype(parity_tag)::value;
-        uint8_t const *src = lds + buffer * kStageLds + a_frag[q];
+        uint8_t const *src = (DIRECT ? ring_of(buffer_tag) : lds + buffer * kStageLds) + a_frag[q];
 #pragma unroll
         for (int i = 0; i < TM; ++i) af[parity][i] = *(v4i const *)(src + i * 32 * kStageBytes);
     };
@@ -1411,6 +1453,107 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
         schedule_k_step(slot_c<0>(), slot_c<0>());
     };
 
+    // ---- A straight into LDS (DIRECT) ----
+    // Fetch t of a wavefront brings the 8 rows from 8 * (4 t + wave) on: lane l lands at row l / 8, position l % 8 of
+    // the 1 KiB that starts there, so it fetches the chunk that the swizzle puts at that position.
+    uint32_t a_direct[DIRECT ? kLoads : 1];
+    if constexpr (DIRECT) {
+#pragma unroll
+        for (int t = 0; t < kLoads; ++t) {
+            uint32_t const r = 8 * (4 * t + wave) + (lane >> 3);
+            a_direct[t] = r * (uint32_t)g.a_stride + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+        }
+    }
+    auto fetch_a = [&](TileView const &view, uint32_t s, auto ring_tag, auto part_tag) __attribute__((always_inline)) {
+        constexpr int part = decltype(part_tag)::value;
+        __amdgpu_buffer_rsrc_t const rsrc = a_rsrc_of(view);
+        uint32_t const stage_offset = __builtin_amdgcn_readfirstlane(s * kSrcStage);
+        uint8_t *stage_base = ring_of(ring_tag);
+#pragma unroll
+        for (int t = 0; t < kLoads; ++t) {
+            if (t * 4 / kLoads != part) continue;
+            fetch_to_lds(rsrc, (lds_void_t *)(stage_base + (4 * t + wave) * 1024), a_direct[DIRECT ? t : 0], stage_offset);
+        }
+    };
+    auto fetch_a_all = [&](TileView const &view, uint32_t s, auto ring_tag) __attribute__((always_inline)) {
+        fetch_a(view, s, ring_tag, slot_c<0>()), fetch_a(view, s, ring_tag, slot_c<1>());
+        fetch_a(view, s, ring_tag, slot_c<2>()), fetch_a(view, s, ring_tag, slot_c<3>());
+    };
+    // Every wavefront waits for its own fetches into a stage (the compiler puts that wait in front of any read of the
+    // stage's array: one word is read for the purpose), then all meet: after that the stage is whole for everybody.
+    // No fence: a fence would wait for the fetches of the later stages as well. The waits for the fragment reads
+    // that are still in flight come with the word read (LDS answers in order).
+    auto stage_arrived = [&](auto ring_tag) __attribute__((always_inline)) {
+        __builtin_amdgcn_sched_barrier(0);
+        typedef __attribute__((address_space(3))) uint32_t const lds_u32_t;
+        uint32_t const word = *(lds_u32_t *)(ring_of(ring_tag) + lane * 4);
+        asm volatile("" ::"v"(word) : "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // One stage: `R` = its place in the ring, `P` = the register slot of its B (stage parity). A(s+3) is fetched into
+    // the ring stage that the barrier of the stage before has freed; B(s+2) into the registers just used.
+    auto schedule_direct_k_step = [&]() {
+        constexpr int loads = TN + (kLoads >= 4 ? kLoads / 4 : 1);
+        constexpr int rest = TM * (TN - 1);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        if constexpr (rest == 0) __builtin_amdgcn_sched_group_barrier(0x020, loads, 0);
+        else {
+#pragma unroll
+            for (int i = 0; i < rest; ++i) {
+                if (i * loads / (rest ? rest : 1) != (i + 1) * loads / (rest ? rest : 1) || (loads > rest && i == 0))
+                    __builtin_amdgcn_sched_group_barrier(0x020, loads > rest ? loads : 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+        }
+    };
+    auto stage_direct = [&](auto ring_tag, uint32_t s, auto entry_tag) __attribute__((always_inline)) {
+        constexpr int R = decltype(ring_tag)::value & 3, P = R & 1;
+        constexpr int entry = decltype(entry_tag)::value;
+        bool const wrap2 = s + 2 >= fast, wrap3 = s + 3 >= fast;
+        uint32_t const s2 = wrap2 ? s + 2 - fast : s + 2, s3 = wrap3 ? s + 3 - fast : s + 3;
+        TileView const &b2 = wrap2 ? nxt : cur, &a3 = wrap3 ? nxt : cur;
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(slot_c<R>(), slot_c<1>(), slot_c<1>());
+        if constexpr (entry == 2) multiply_fresh(slot_c<P>(), slot_c<0>());
+        else multiply(slot_c<P>(), slot_c<0>());
+        load_b(b2, s2, slot_c<P>(), slot_c<0>()), fetch_a(a3, s3, slot_c<R + 3>(), slot_c<0>());
+        if constexpr (entry == 2 && kChunked) schedule_fresh_k_step();
+        else schedule_direct_k_step();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(slot_c<R>(), slot_c<2>(), slot_c<0>());
+        multiply(slot_c<P>(), slot_c<1>());
+        load_b(b2, s2, slot_c<P>(), slot_c<1>()), fetch_a(a3, s3, slot_c<R + 3>(), slot_c<1>());
+        schedule_direct_k_step();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(slot_c<R>(), slot_c<3>(), slot_c<1>());
+        multiply(slot_c<P>(), slot_c<2>());
+        load_b(b2, s2, slot_c<P>(), slot_c<2>()), fetch_a(a3, s3, slot_c<R + 3>(), slot_c<2>());
+        schedule_direct_k_step();
+        stage_arrived(slot_c<R + 1>());
+        read_frags(slot_c<R + 1>(), slot_c<0>(), slot_c<0>());
+        multiply(slot_c<P>(), slot_c<3>());
+        load_b(b2, s2, slot_c<P>(), slot_c<3>()), fetch_a(a3, s3, slot_c<R + 3>(), slot_c<3>());
+        schedule_direct_k_step();
+    };
+    auto prime_direct = [&]() {
+        __syncthreads();
+        fetch_a_all(cur, 0, slot_c<0>());
+        load_b(cur, 0, slot_c<0>(), slot_c<0>()), load_b(cur, 0, slot_c<0>(), slot_c<1>());
+        load_b(cur, 0, slot_c<0>(), slot_c<2>()), load_b(cur, 0, slot_c<0>(), slot_c<3>());
+        fetch_a_all(cur, 1, slot_c<1>());
+        load_b(cur, 1, slot_c<1>(), slot_c<0>()), load_b(cur, 1, slot_c<1>(), slot_c<1>());
+        load_b(cur, 1, slot_c<1>(), slot_c<2>()), load_b(cur, 1, slot_c<1>(), slot_c<3>());
+        fetch_a_all(cur, 2, slot_c<2>());
+        stage_arrived(slot_c<0>());
+        read_frags(slot_c<0>(), slot_c<0>(), slot_c<0>());
+    };
+
     // Fills the pipeline for a tile: stages 0 and 1 on their way, A(0) in LDS, its first fragments read.
     auto prime = [&]() {
         __syncthreads(); // the previous tile's last fragment reads are done
@@ -1430,7 +1573,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     };
     if constexpr (across) {
         cur = view_of(blockIdx.x);
-        prime();
+        if constexpr (DIRECT) prime_direct();
+        else prime();
     }
 
     for (uint32_t tile = blockIdx.x; tile < tile_count; tile += gridDim.x) {
@@ -1467,13 +1611,39 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                         }
                     }
                 };
-                stage(slot_c<0>(), 0u, slot_c<2>());
-                stage(slot_c<1>(), 1u, slot_c<0>());
-                fold_when_due();
-                for (uint32_t s = 2; s < fast; s += 2) {
-                    stage(slot_c<0>(), s, slot_c<0>());
-                    stage(slot_c<1>(), s + 1, slot_c<0>());
+                if constexpr (DIRECT) { // (four stages a trip: the host checked that the depth, and a chunk, are whole trips)
+                    auto fold_after_trip = [&]() __attribute__((always_inline)) {
+                        if constexpr (kChunked) {
+                            until_fold -= 4;
+                            if (until_fold == 0) {
+                                __builtin_amdgcn_sched_barrier(0);
+                                total.fold(acc);
+                                until_fold = g.chunk_stages;
+                            }
+                        }
+                    };
+                    stage_direct(slot_c<0>(), 0u, slot_c<2>());
+                    stage_direct(slot_c<1>(), 1u, slot_c<0>());
+                    stage_direct(slot_c<2>(), 2u, slot_c<0>());
+                    stage_direct(slot_c<3>(), 3u, slot_c<0>());
+                    fold_after_trip();
+                    for (uint32_t s = 4; s < fast; s += 4) {
+                        stage_direct(slot_c<0>(), s, slot_c<0>());
+                        stage_direct(slot_c<1>(), s + 1, slot_c<0>());
+                        stage_direct(slot_c<2>(), s + 2, slot_c<0>());
+                        stage_direct(slot_c<3>(), s + 3, slot_c<0>());
+                        fold_after_trip();
+                    }
+                }
+                else {
+                    stage(slot_c<0>(), 0u, slot_c<2>());
+                    stage(slot_c<1>(), 1u, slot_c<0>());
                     fold_when_due();
+                    for (uint32_t s = 2; s < fast; s += 2) {
+                        stage(slot_c<0>(), s, slot_c<0>());
+                        stage(slot_c<1>(), s + 1, slot_c<0>());
+                        fold_when_due();
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -1752,6 +1922,16 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
     if constexpr (tail_matters_for<T, false>()) {
         if (whole) kernel = dots_packed_kernel<T, TM, TN, true, false, true>;
     }
+    // A straight into LDS (see the kernel): the 256 x 256 tile of the types that reach LDS as they are, depths of whole
+    // trips of four stages (measured, i8 8192^3, alternating in one session: 0.438 -> 0.419 ms, 0.473 -> 0.425 ms)
+    bool direct = false;
+    if constexpr (kDirectStaging && !T::kUnsigned && !T::kPrewiden && T::kSrcChunk == 16 && T::kImageChunk == 16 &&
+                  ((TM == 8 && TN == 2) || (NK_DIRECT_CHUNKED && TM == 4 && TN == 2 && T::kChunked))) {
+        direct = across && !norms && stages % 4 == 0 && stages >= 8 && (whole || !tail_matters_for<T, false>()) &&
+                 (!T::kChunked || g.chunk_stages % 4 == 0) &&
+                 (g.avec >= 16) && !(forced_tile_config() & 0x40000000);
+        if (direct) kernel = dots_packed_kernel<T, TM, TN, true, false, tail_matters_for<T, false>(), true>;
+    }
     if constexpr (T::kDistances) {
         if (norms) kernel = across ? dots_packed_kernel<T, TM, TN, true, true> : dots_packed_kernel<T, TM, TN, false, true>;
         if (norms && whole) kernel = dots_packed_kernel<T, TM, TN, true, true, true>;
@@ -1759,8 +1939,8 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
     else if (norms) return hipErrorInvalidValue;
     // Persistent grid: as many workgroups as fit on the device at once (queried once per kernel; threads that
     // ask at the same time store the same number).
-    static std::atomic<int> resident_of[8];
-    std::atomic<int> &slot = resident_of[(across ? 1 : 0) + (norms ? 2 : 0) + (whole ? 4 : 0)];
+    static std::atomic<int> resident_of[9];
+    std::atomic<int> &slot = resident_of[direct ? 8 : (across ? 1 : 0) + (norms ? 2 : 0) + (whole ? 4 : 0)];
     int resident = slot.load(std::memory_order_relaxed);
     if (!resident) {
         int per_cu = 0;

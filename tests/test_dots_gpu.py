@@ -158,6 +158,29 @@ def test_both_kinds_of_store(oracle, dtype, store):
         check(oracle, dtype, a, b, config | (store << 28), f"{dtype} {m}x{n}x{k} config {config} store {store}")
 
 
+def test_staging_straight_into_lds():
+    """i8 at the 256 x 256 tile takes A from memory straight into LDS (a ring of four stages, four stages a trip of the
+    loop) when the depth is a whole number of trips; bit 30 of the test hook keeps the staging through registers. Both
+    must equal the exact product: tiles off the edges of A and B, a padded A, one tile and several tiles per workgroup
+    (the pipeline runs on across them), and depths of two to sixteen trips."""
+    rng = np.random.default_rng(77)
+    for m, n, k, pad in ((300, 515, 1024, 0), (257, 1000, 1536, 16), (1024, 256, 4096, 0), (2100, 33000, 2048, 0), (70000, 300, 1024, 32)):
+        a_wide = rng.integers(-128, 128, (m, k + pad), dtype=np.int8)
+        b = rng.integers(-128, 128, (n, k), dtype=np.int8)
+        ga, packed = to_gpu(a_wide)[:, :k], nk.dots_pack(to_gpu(b), "i8")
+        results = []
+        for hook in (1, 1 | (1 << 30)):
+            nk.library().nk_hip_set_tile_config(hook)
+            try:
+                results.append(nk.dots_packed(ga, packed))
+            finally:
+                nk.library().nk_hip_set_tile_config(0)
+        assert torch.equal(results[0], results[1]), f"{m}x{n}x{k}"
+        rows = torch.from_numpy(rng.choice(m, min(m, 300), replace=False)).to(DEV)
+        exact = ga[rows].double() @ to_gpu(b).double().T
+        assert torch.equal(results[0][rows].double(), exact), f"{m}x{n}x{k}"
+
+
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
 def test_float_input_families(oracle, dtype):
     rng = np.random.default_rng(5)
