@@ -59,9 +59,6 @@ constexpr uint32_t kTileBand = NK_TILE_BAND;
 #ifndef NK_DIRECT_STAGING
 #define NK_DIRECT_STAGING 1
 #endif
-#ifndef NK_DIRECT_CHUNKED
-#define NK_DIRECT_CHUNKED 0
-#endif
 constexpr bool kDirectStaging = NK_DIRECT_STAGING != 0; // A straight into LDS where that applies (see dots_packed_kernel)
 
 struct GemmArgs {
@@ -1922,11 +1919,13 @@ hipError_t launch_one(GemmArgs &g, hipStream_t stream, TriangleScratch const *tr
     if constexpr (tail_matters_for<T, false>()) {
         if (whole) kernel = dots_packed_kernel<T, TM, TN, true, false, true>;
     }
-    // A straight into LDS (see the kernel): the 256 x 256 tile of the types that reach LDS as they are, depths of whole
-    // trips of four stages (measured, i8 8192^3, alternating in one session: 0.438 -> 0.419 ms, 0.473 -> 0.425 ms)
+    // A straight into LDS (see the kernel): the largest tile of the types that reach LDS as they are, depths of whole
+    // trips of four stages, and for the two-accumulator types folds that fall between trips (measured at 8192^3,
+    // alternating in one session: i8 0.438 -> 0.419 ms, bf16 0.930 -> 0.902, f16 0.997 -> 0.968; with a fold after every
+    // second stage of the trip instead, the compiler ran out of registers in the folds and bf16 took 1.10 ms)
     bool direct = false;
     if constexpr (kDirectStaging && !T::kUnsigned && !T::kPrewiden && T::kSrcChunk == 16 && T::kImageChunk == 16 &&
-                  ((TM == 8 && TN == 2) || (NK_DIRECT_CHUNKED && TM == 4 && TN == 2 && T::kChunked))) {
+                  ((TM == 8 && TN == 2) || (TM == 4 && TN == 2 && T::kChunked))) {
         direct = across && !norms && stages % 4 == 0 && stages >= 8 && (whole || !tail_matters_for<T, false>()) &&
                  (!T::kChunked || g.chunk_stages % 4 == 0) &&
                  (g.avec >= 16) && !(forced_tile_config() & 0x40000000);

@@ -159,7 +159,7 @@ def test_both_kinds_of_store(oracle, dtype, store):
 
 
 def test_staging_straight_into_lds():
-    """i8 at the 256 x 256 tile takes A from memory straight into LDS (a ring of four stages, four stages a trip of the
+    """i8 at the 256 x 256 tile (bf16 and f16 at 128 x 256) takes A from memory straight into LDS (a ring of four stages, four stages a trip of the
     loop) when the depth is a whole number of trips; bit 30 of the test hook keeps the staging through registers. Both
     must equal the exact product: tiles off the edges of A and B, a padded A, one tile and several tiles per workgroup
     (the pipeline runs on across them), and depths of two to sixteen trips."""
@@ -179,6 +179,23 @@ def test_staging_straight_into_lds():
         rows = torch.from_numpy(rng.choice(m, min(m, 300), replace=False)).to(DEV)
         exact = ga[rows].double() @ to_gpu(b).double().T
         assert torch.equal(results[0][rows].double(), exact), f"{m}x{n}x{k}"
+    # bf16 and f16 at their largest tile (128 x 256) do the same when their folds fall between trips: same bits either way
+    oracle = support.load_oracle()
+    for dtype, (m, n, k) in (("bf16", (300, 515, 2048)), ("f16", (1100, 9000, 4096)), ("bf16", (2100, 16500, 2048))):
+        a, b = support.random_matrix(oracle, dtype, m, k, rng), support.random_matrix(oracle, dtype, n, k, rng)
+        ga, packed = to_gpu(a), nk.dots_pack(to_gpu(b), dtype)
+        results = []
+        for hook in (2, 2 | (1 << 30)):
+            nk.library().nk_hip_set_tile_config(hook)
+            try:
+                results.append(nk.dots_packed(ga, packed))
+            finally:
+                nk.library().nk_hip_set_tile_config(0)
+        assert torch.equal(results[0].view(torch.int32), results[1].view(torch.int32)), f"{dtype} {m}x{n}x{k}"
+        sample = np.sort(rng.choice(m, 40, replace=False))
+        truth, magnitude = oracle.truth(dtype, a[sample], b[:500])
+        assert_float_gate(dtype, results[0][torch.from_numpy(sample).to(DEV)][:, :500].cpu().numpy(), oracle.dots_packed(dtype, a[sample], b[:500]),
+                          truth, magnitude, f"{dtype} {m}x{n}x{k} straight into LDS")
 
 
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
