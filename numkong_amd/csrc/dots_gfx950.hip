@@ -487,7 +487,7 @@ static int pack_async(int dtype, void const *b, size_t n, size_t k, size_t b_str
         pack_fn kernel = nullptr;
         switch (widen_kind_of(dtype, k)) {
         case 0: kernel = dtype == kI8 ? pack_kernel<0, 0> : (dtype == kU8 ? pack_kernel<0, 1> : (dtype == kBF16 ? pack_kernel<0, 2> : pack_kernel<0, 3>)); break;
-        case 1: kernel = pack_kernel<1, 3>; break;
+        case 1: kernel = kE4M3ViaBF16 ? pack_kernel<1, 2> : pack_kernel<1, 3>; break;
         case 2: kernel = pack_kernel<2, 3>; break;
         case 3: kernel = pack_kernel<3, 0>; break;
         case 4: kernel = pack_kernel<4, 3>; break;

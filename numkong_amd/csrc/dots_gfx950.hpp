@@ -37,6 +37,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <type_traits>
 #include <stddef.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -292,10 +293,26 @@ __device__ __forceinline__ uint32_t sum_bytes_u8(v4i v) {
     return s;
 }
 
-/** Eight OCP fp8 values (two dwords) -> eight f16 values, exact for every code incl. subnormals, Inf, NaN. */
+#ifndef NK_E4M3_VIA_BF16
+#define NK_E4M3_VIA_BF16 0
+#endif
+/** e4m3 widened to bf16 and run on the bf16 MFMA instead of f16 (every e4m3 value is a bf16 value as well). */
+constexpr bool kE4M3ViaBF16 = NK_E4M3_VIA_BF16 != 0;
+
+/** Eight OCP fp8 values (two dwords) -> eight f16 values (e4m3 optionally bf16 values), exact for every code incl.
+ *  subnormals, Inf, NaN. */
 template <bool E5M2>
 __device__ __forceinline__ v4i widen_fp8x8(uint32_t lo, uint32_t hi) {
     typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+    if constexpr (!E5M2 && kE4M3ViaBF16) {
+        typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+        v2bf const q0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false), q1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+        v2bf const q2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false), q3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+        v4i wide;
+        wide[0] = __builtin_bit_cast(int, q0), wide[1] = __builtin_bit_cast(int, q1);
+        wide[2] = __builtin_bit_cast(int, q2), wide[3] = __builtin_bit_cast(int, q3);
+        return wide;
+    }
     v2h p0, p1, p2, p3;
     if (E5M2) {
         p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(lo, 1.0f, false);
@@ -692,12 +709,16 @@ struct F16 {
     }
 };
 /** fp8 runs widened to f16 (exact), on the f16 MFMA; see widen_fp8x8. */
-struct E4M3 : F16 {
+struct E4M3 : std::conditional<kE4M3ViaBF16, BF16, F16>::type {
+    typedef std::conditional<kE4M3ViaBF16, BF16, F16>::type base_t;
     static constexpr bool kChunked = true;
     static constexpr int kDtype = kE4M3;
     static constexpr int kSrcChunk = 8;
     static __device__ __forceinline__ v4i widen(v4i v) { return widen_fp8x8<false>((uint32_t)v[0], (uint32_t)v[1]); }
-    static __device__ __forceinline__ norm_t sumsq(v4i, v4i wide) { return sumsq_of_normals(wide); } // smallest value 2^-9
+    static __device__ __forceinline__ base_t::norm_t sumsq(v4i raw, v4i wide) {
+        if constexpr (kE4M3ViaBF16) return BF16::sumsq(raw, wide);
+        else return F16::sumsq_of_normals(wide); // smallest value 2^-9: no f16 denormals
+    }
 };
 struct E5M2 : F16 {
     static constexpr bool kChunked = true;

@@ -59,12 +59,13 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 #pragma region Ceiling
 
-enum Form { kI8Large, kI8Small, kBF16Large, kBF16Small, kF16Large, kFP8Legacy, kFP8Scaled, kForms };
+enum Form { kI8Large, kI8Small, kBF16Large, kBF16Small, kF16Large, kFP8Legacy, kFP8Scaled, kF16OfE4M3, kBF16OfE4M3, kForms };
 static char const *const kFormNames[kForms] = {"i8 32x32x32", "i8 16x16x64", "bf16 32x32x16", "bf16 16x16x32",
-                                               "f16 32x32x16", "fp8 32x32x16 (legacy)", "fp8 32x32x64 (f8f6f4)"};
+                                               "f16 32x32x16", "fp8 32x32x16 (legacy)", "fp8 32x32x64 (f8f6f4)",
+                                               "f16 32x32x16 on e4m3 values", "bf16 32x32x16 on e4m3 values"};
 static double const kFormOps[kForms] = {2.0 * 32 * 32 * 32, 2.0 * 16 * 16 * 64, 2.0 * 32 * 32 * 16, 2.0 * 16 * 16 * 32,
-                                        2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 64};
-static double const kFormPeak[kForms] = {5000, 5000, 2500, 2500, 2500, 5000, 5000}; // published dense peaks, T(FL)OP/s
+                                        2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 64, 2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 16};
+static double const kFormPeak[kForms] = {5000, 5000, 2500, 2500, 2500, 5000, 5000, 2500, 2500}; // published dense peaks, T(FL)OP/s
 
 /**
  *  One workgroup of four wavefronts per compute unit, every wavefront 256 accumulator registers: ROWS x COLS blocks,
@@ -73,7 +74,7 @@ static double const kFormPeak[kForms] = {5000, 5000, 2500, 2500, 2500, 5000, 500
  */
 template <int FORM>
 __global__ __launch_bounds__(256) void mfma_only_kernel(v8i const *operands, int iterations, float *sink, unsigned long long *clocks) {
-    constexpr bool kLarge = FORM == kI8Large || FORM == kBF16Large || FORM == kF16Large || FORM == kFP8Legacy || FORM == kFP8Scaled;
+    constexpr bool kLarge = FORM != kI8Small && FORM != kBF16Small;
     constexpr int ROWS = 8, COLS = kLarge ? 2 : 8;
     v8i a[ROWS], b[COLS];
     for (int i = 0; i < ROWS; ++i) a[i] = operands[(i * 64 + (threadIdx.x & 63)) % 1024];
@@ -93,9 +94,9 @@ __global__ __launch_bounds__(256) void mfma_only_kernel(v8i const *operands, int
                 long const a2 = ((long)a[i][1] << 32) | (unsigned)a[i][0], b2 = ((long)b[j][1] << 32) | (unsigned)b[j][0];
                 if constexpr (FORM == kI8Large) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, b4, acc[i][j], 0, 0, 0);
                 if constexpr (FORM == kI8Small) acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a4, b4, acc[i][j], 0, 0, 0);
-                if constexpr (FORM == kBF16Large) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a4), __builtin_bit_cast(v8bf, b4), acc[i][j], 0, 0, 0);
+                if constexpr (FORM == kBF16Large || FORM == kBF16OfE4M3) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a4), __builtin_bit_cast(v8bf, b4), acc[i][j], 0, 0, 0);
                 if constexpr (FORM == kBF16Small) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a4), __builtin_bit_cast(v8bf, b4), acc[i][j], 0, 0, 0);
-                if constexpr (FORM == kF16Large) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a4), __builtin_bit_cast(v8h, b4), acc[i][j], 0, 0, 0);
+                if constexpr (FORM == kF16Large || FORM == kF16OfE4M3) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a4), __builtin_bit_cast(v8h, b4), acc[i][j], 0, 0, 0);
                 if constexpr (FORM == kFP8Legacy) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a2, b2, acc[i][j], 0, 0, 0);
                 if constexpr (FORM == kFP8Scaled) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i], b[j], acc[i][j], 0, 0, 0, 0, 0, 0);
             }
@@ -149,7 +150,8 @@ static uint8_t e4m3_of(float f) {
     return (uint8_t)(best | (f < 0 ? 0x80 : 0));
 }
 
-/** 16 KiB of operand data in the element type of `form`: full-range integers, N(0, 1) floats, or zeros. */
+/** 16 KiB of operand data in the element type of `form`: full-range integers, N(0, 1) floats (for the last two forms
+ *  rounded to e4m3 first: what the fp8 product kernels feed the f16 instruction, few mantissa bits set), or zeros. */
 static std::vector<uint8_t> operand_data(int form, bool zeros) {
     std::vector<uint8_t> data(1024 * 32, 0);
     if (zeros) return data;
@@ -157,7 +159,8 @@ static std::vector<uint8_t> operand_data(int form, bool zeros) {
         if (form == kI8Large || form == kI8Small) data[at] = (uint8_t)next_random(), data[at + 1] = (uint8_t)next_random();
         else if (form == kFP8Legacy || form == kFP8Scaled) data[at] = e4m3_of((float)next_normal()), data[at + 1] = e4m3_of((float)next_normal());
         else {
-            uint16_t const bits = form == kF16Large ? f16_of((float)next_normal()) : bf16_of((float)next_normal());
+            float const value = form == kF16OfE4M3 || form == kBF16OfE4M3 ? e4m3_value(e4m3_of((float)next_normal())) : (float)next_normal();
+            uint16_t const bits = form == kF16Large || form == kF16OfE4M3 ? f16_of(value) : bf16_of(value);
             memcpy(&data[at], &bits, 2);
         }
     }
@@ -220,9 +223,11 @@ static int ceiling_mode(bool json) {
         results[kF16Large][zeros] = run_ceiling<kF16Large>(zeros, units, operands, sink, clocks);
         results[kFP8Legacy][zeros] = run_ceiling<kFP8Legacy>(zeros, units, operands, sink, clocks);
         results[kFP8Scaled][zeros] = run_ceiling<kFP8Scaled>(zeros, units, operands, sink, clocks);
+        results[kF16OfE4M3][zeros] = run_ceiling<kF16OfE4M3>(zeros, units, operands, sink, clocks);
+        results[kBF16OfE4M3][zeros] = run_ceiling<kBF16OfE4M3>(zeros, units, operands, sink, clocks);
     }
     if (json) printf("{\"compute_units\": %d, \"device\": \"%s\", \"forms\": {", units, properties.gcnArchName);
-    else printf("MFMA-only loop, %d compute units (%s), 4 wavefronts each, 20 launches after 20 warm-up launches\n%-24s %-7s %9s %10s %8s %8s %12s\n", units,
+    else printf("MFMA-only loop, %d compute units (%s), 4 wavefronts each, 20 launches after 20 warm-up launches\n%-30s %-7s %9s %10s %8s %8s %12s\n", units,
                 properties.gcnArchName, "instruction", "data", "ms", "T(FL)OP/s", "of peak", "MHz", "cycles/MFMA");
     for (int form = 0; form < kForms; ++form)
         for (int zeros = 0; zeros < 2; ++zeros) {
@@ -231,7 +236,7 @@ static int ceiling_mode(bool json) {
                 printf("%s\"%s, %s\": {\"tops\": %.1f, \"frac_of_peak\": %.4f, \"mhz\": %.0f, \"cycles_per_mfma\": %.2f}", form + zeros ? ", " : "",
                        kFormNames[form], zeros ? "zeros" : "random", r.tops, r.tops / kFormPeak[form], r.mhz, r.cycles_per_mfma);
             else
-                printf("%-24s %-7s %9.4f %10.1f %8.3f %8.0f %12.2f\n", kFormNames[form], zeros ? "zeros" : "random", r.ms, r.tops, r.tops / kFormPeak[form], r.mhz,
+                printf("%-30s %-7s %9.4f %10.1f %8.3f %8.0f %12.2f\n", kFormNames[form], zeros ? "zeros" : "random", r.ms, r.tops, r.tops / kFormPeak[form], r.mhz,
                        r.cycles_per_mfma);
         }
     if (json) printf("}}\n");
