@@ -1431,12 +1431,15 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
     // One stage of the steady state; `P` = stage parity = LDS buffer = register slot. Stages s+2 and
     // s+3 are fetched here; past the tile's end they are the first stages of `nxt` (the next tile, or
     // this one again when nothing follows: loads of valid memory that nobody uses).
-    auto stage = [&](auto parity_tag, uint32_t s, auto entry_tag) __attribute__((always_inline)) {
+    // `inside`: how many of the stages s + 2, s + 3 are known to be this tile's (a tile's first two stages, whose numbers
+    // are constants and which the host guarantees two or three more: see stage_direct).
+    auto stage = [&](auto parity_tag, uint32_t s, auto entry_tag, auto inside_tag) __attribute__((always_inline)) {
         constexpr int P = decltype(parity_tag)::value;
         constexpr int entry = decltype(entry_tag)::value; // 0: in the middle of a sum; 2: the first stage of a tile
+        constexpr int inside = ACROSS ? decltype(inside_tag)::value : 0; // (without ACROSS a tile may have two stages only)
         // vector operations behind each MFMA of the k-steps that widen in place: their share of half the chunks
         constexpr int kSpread = T::kPrewiden ? (kLoads * 28 + TM * TN - 1) / (TM * TN) : 0;
-        bool const wrap2 = s + 2 >= fast, wrap3 = s + 3 >= fast;
+        bool const wrap2 = inside < 1 && s + 2 >= fast, wrap3 = inside < 2 && s + 3 >= fast;
         uint32_t const s2 = wrap2 ? s + 2 - fast : s + 2, s3 = wrap3 ? s + 3 - fast : s + 3;
         TileView const &a2 = wrap2 ? nxt : cur, &a3 = wrap3 ? nxt : cur, &b2 = a2;
         __builtin_amdgcn_sched_barrier(0);
@@ -1660,12 +1663,12 @@ __global__ __launch_bounds__(256, (TM * TN <= 2 ? 3 : (TM * TN <= 4 && !T::kChun
                     }
                 }
                 else {
-                    stage(slot_c<0>(), 0u, slot_c<2>());
-                    stage(slot_c<1>(), 1u, slot_c<0>());
+                    stage(slot_c<0>(), 0u, slot_c<2>(), slot_c<2>()); // (with ACROSS at least four stages: the host checked)
+                    stage(slot_c<1>(), 1u, slot_c<0>(), slot_c<1>());
                     fold_when_due();
                     for (uint32_t s = 2; s < fast; s += 2) {
-                        stage(slot_c<0>(), s, slot_c<0>());
-                        stage(slot_c<1>(), s + 1, slot_c<0>());
+                        stage(slot_c<0>(), s, slot_c<0>(), slot_c<0>());
+                        stage(slot_c<1>(), s + 1, slot_c<0>(), slot_c<0>());
                         fold_when_due();
                     }
                 }
@@ -2059,7 +2062,8 @@ hipError_t launch_typed(GemmArgs &g, hipStream_t stream, TriangleScratch const *
             best = 4;
         // e2m3 pays 13 vector operations for every dword of A it stages: a 128 x 512 tile (every wavefront 128 x 128)
         // stages half as much A per MFMA as 256 x 256 (8192^3: 0.51 against 0.59 ms; for i8 itself the two are equal)
-        if (T::kDtype == kE2M3 && !triangle && args.metric == 0 && first == 1 && tiles_of(args, 5) >= 256) best = 5;
+        // (not the f16 route of very deep rows: its two accumulator sets do not fit that tile)
+        if (T::kDtype == kE2M3 && !T::kChunked && !triangle && args.metric == 0 && first == 1 && tiles_of(args, 5) >= 256) best = 5;
         return best;
     };
     if (chosen_here) config = choose(g, 1);

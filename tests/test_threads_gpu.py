@@ -173,3 +173,85 @@ def test_tile_config_hook_is_per_thread():
     finally:
         lib.nk_hip_set_tile_config(0)
     assert torch.equal(results["mine"], expected) and torch.equal(results["other"], expected)
+
+
+def test_staging_buffers_are_kept_and_trimmed():
+    """A thread's staging buffers stay between calls; `nk_hip_thread_trim` gives back the slots larger than its first
+    argument, then everything if more than its second is still held; a host-pointer product afterwards works as
+    before (gfx950.c keeps 256 MiB per slot and 2 GiB per thread this way)."""
+    lib = nk.library()
+    lib.nk_hip_thread_buffer.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]
+    lib.nk_hip_thread_buffer.restype = ctypes.c_int
+    lib.nk_hip_thread_cached_bytes.restype = ctypes.c_size_t
+    lib.nk_hip_thread_trim.argtypes = [ctypes.c_size_t, ctypes.c_size_t]
+    lib.nk_hip_thread_trim.restype = None
+    lib.nk_hip_thread_release.restype = None
+    lib.nk_hip_thread_release()
+    assert lib.nk_hip_thread_cached_bytes() == 0
+    small, large, again = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+    assert lib.nk_hip_thread_buffer(0, 0, 1 << 20, ctypes.byref(small)) == 0 and small.value
+    assert lib.nk_hip_thread_buffer(1, 1, 3 << 20, ctypes.byref(large)) == 0 and large.value
+    held = lib.nk_hip_thread_cached_bytes()
+    assert held >= (1 << 20) + (3 << 20)
+    assert lib.nk_hip_thread_buffer(0, 0, 1 << 19, ctypes.byref(again)) == 0 and again.value == small.value  # kept, not regrown
+    assert lib.nk_hip_thread_cached_bytes() == held
+    lib.nk_hip_thread_trim(2 << 20, 1 << 30)  # the 3 MiB slot goes, the 1 MiB slot stays
+    assert (1 << 20) <= lib.nk_hip_thread_cached_bytes() < (3 << 20)
+    lib.nk_hip_thread_trim(1 << 30, 1 << 19)  # more than the total cap is still held: everything goes
+    assert lib.nk_hip_thread_cached_bytes() == 0
+    rng = np.random.default_rng(914)
+    a = rng.integers(-128, 128, (70, 200), dtype=np.int8)
+    b = rng.integers(-128, 128, (90, 200), dtype=np.int8)
+    packed = nk.dots_pack(to_gpu(b), "i8").buffer.cpu().numpy()
+    c = np.full((70, 90), -1, np.int32)
+    lib.nk_dots_packed_i8(a.ctypes.data, packed.ctypes.data, c.ctypes.data, 70, 90, 200, a.strides[0], c.strides[0])
+    assert not lib.nk_amd_last_error()
+    assert np.array_equal(c.astype(np.int64), a.astype(np.int64) @ b.astype(np.int64).T)
+    assert lib.nk_hip_thread_cached_bytes() > 0
+    lib.nk_hip_thread_release()
+    lib.nk_hip_image_cache_clear()
+
+
+def test_image_cache_claim_abandon_publish():
+    """The life of a cache entry as the host layer drives it: the first claim of an unknown image reserves it (2), an
+    abandoned reservation leaves no trace, a published copy is found by later claims (1) until the cache is cleared."""
+    lib = nk.library()
+    for name in ("nk_hip_image_cache_claim", "nk_hip_image_cache_find"):
+        getattr(lib, name).argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]
+        getattr(lib, name).restype = ctypes.c_int
+    lib.nk_hip_image_cache_publish.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    lib.nk_hip_image_cache_publish.restype = ctypes.c_int
+    lib.nk_hip_image_cache_abandon.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    lib.nk_hip_image_cache_abandon.restype = None
+    lib.nk_hip_image_cache_release.argtypes = [ctypes.c_void_p]
+    lib.nk_hip_image_cache_release.restype = None
+    lib.nk_hip_image_cache_clear()
+    rng = np.random.default_rng(915)
+    b = rng.integers(-128, 128, (64, 128), dtype=np.int8)
+    packed = nk.dots_pack(to_gpu(b), "i8")
+    image = packed.buffer.cpu().numpy()
+    where = ctypes.c_void_p()
+    assert lib.nk_hip_image_cache_find(image.ctypes.data, image.nbytes, ctypes.byref(where)) == 0
+    assert lib.nk_hip_image_cache_claim(image.ctypes.data, image.nbytes, ctypes.byref(where)) == 2 and not where.value
+    lib.nk_hip_image_cache_abandon(image.ctypes.data, image.nbytes)
+    assert lib.nk_hip_image_cache_find(image.ctypes.data, image.nbytes, ctypes.byref(where)) == 0
+    assert lib.nk_hip_image_cache_claim(image.ctypes.data, image.nbytes, ctypes.byref(where)) == 2
+    # the cache owns what is published to it and frees it when the entry goes: give it memory of the library's own
+    lib.nk_hip_malloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
+    copy = ctypes.c_void_p()
+    assert lib.nk_hip_malloc(ctypes.byref(copy), image.nbytes) == 0
+    lib.nk_hip_memcpy_h2d.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    assert lib.nk_hip_memcpy_h2d(copy, image.ctypes.data, image.nbytes, None) == 0
+    torch.cuda.synchronize()
+    assert lib.nk_hip_image_cache_publish(image.ctypes.data, image.nbytes, copy) == 1
+    lib.nk_hip_image_cache_release(copy)  # the uploader's own use of it
+    assert lib.nk_hip_image_cache_claim(image.ctypes.data, image.nbytes, ctypes.byref(where)) == 1 and where.value == copy.value
+    lib.nk_hip_image_cache_release(where)
+    # a product with the host image now runs against that copy
+    a = rng.integers(-128, 128, (40, 128), dtype=np.int8)
+    c = np.full((40, 64), -1, np.int32)
+    lib.nk_dots_packed_i8(a.ctypes.data, image.ctypes.data, c.ctypes.data, 40, 64, 128, a.strides[0], c.strides[0])
+    assert not lib.nk_amd_last_error()
+    assert np.array_equal(c.astype(np.int64), a.astype(np.int64) @ b.astype(np.int64).T)
+    lib.nk_hip_image_cache_clear()
+    assert lib.nk_hip_image_cache_find(image.ctypes.data, image.nbytes, ctypes.byref(where)) == 0
