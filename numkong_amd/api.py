@@ -165,6 +165,23 @@ class PackedMatrix:
         return dots_packed(a, self)
 
 
+def _inferred_dtype(t) -> str:
+    """The packing dtype of a tensor whose element type says it (the reference's ``dtype=None``, python/matrix.c:632-647);
+    the sub-byte and 6-bit types have no tensor type of their own and must be named."""
+    import torch
+
+    names = {torch.int8: "i8", torch.uint8: "u8", torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32",
+             torch.float64: "f64"}
+    for attribute, name in (("float8_e4m3fn", "e4m3"), ("float8_e5m2", "e5m2")):
+        if hasattr(torch, attribute):
+            names[getattr(torch, attribute)] = name
+    if not isinstance(t, torch.Tensor) and hasattr(t, "__dlpack__"):
+        t = torch.from_dlpack(t)
+    if not isinstance(t, torch.Tensor) or t.dtype not in names:
+        raise TypeError("dtype cannot be inferred from this input; name one of " + str(sorted(DTYPES)))
+    return names[t.dtype]
+
+
 def _as_matrix(t, dtype: str, what: str):
     import torch
 
@@ -185,10 +202,13 @@ def _as_matrix(t, dtype: str, what: str):
     return t
 
 
-def dots_pack(b, dtype: str) -> PackedMatrix:
-    """Pack row-major ``b`` (width x depth, raw element bits in a same-width torch dtype)."""
+def dots_pack(b, dtype: str = None) -> PackedMatrix:
+    """Pack row-major ``b`` (width x depth, raw element bits in a same-width torch dtype); ``dtype`` defaults to the
+    tensor's own element type."""
     import torch
 
+    if dtype is None:
+        dtype = _inferred_dtype(b)
     b = _as_matrix(b, dtype, "b")
     width, depth = int(b.shape[0]), int(b.shape[1]) * DTYPES[dtype][3]
     size = dots_packed_size(dtype, width, depth)
@@ -292,23 +312,30 @@ def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_r
     return out
 
 
-def dots_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
+def dots_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None):
     """Upper triangle (diagonal included) of ``vectors @ vectors.T`` for the rows ``[start_row, end_row)``, widened as
-    in ``dots_packed``; the rest of ``out`` is left as it was (zeros when allocated here)."""
+    in ``dots_packed``; the rest of ``out`` is left as it was (zeros when allocated here). ``dtype`` defaults to the
+    tensor's own element type."""
+    if dtype is None:
+        dtype = _inferred_dtype(vectors)
     if dtype not in DTYPES:
         raise TypeError(f"unsupported dtype {dtype!r}; expected one of {sorted(DTYPES)}")
     return _symmetric("nk_dots_symmetric_", DTYPES[dtype][2], vectors, dtype, out, start_row, end_row)
 
 
-def angulars_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
+def angulars_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None):
     """Upper triangle of the pairwise angular distances as float32 (float64 for f32 and f64 inputs); the diagonal is
     exactly 0."""
+    if dtype is None:
+        dtype = _inferred_dtype(vectors)
     _needs_distances(dtype)
     return _symmetric("nk_angulars_symmetric_", _distance_dtype(dtype), vectors, dtype, out, start_row, end_row)
 
 
-def euclideans_symmetric(vectors, dtype: str, out=None, start_row=None, end_row=None):
+def euclideans_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None):
     """Upper triangle of the pairwise euclidean distances as float32 (float64 for f32 and f64 inputs); the diagonal is
     exactly 0."""
+    if dtype is None:
+        dtype = _inferred_dtype(vectors)
     _needs_distances(dtype)
     return _symmetric("nk_euclideans_symmetric_", _distance_dtype(dtype), vectors, dtype, out, start_row, end_row)

@@ -59,3 +59,24 @@ def test_python_packed_matrix_operator_and_dlpack(oracle):
 
     again = nk.dots_packed(Exporter(ga), nk.dots_pack(Exporter(gb), "i8"))
     assert np.array_equal(again.cpu().numpy(), expected)
+
+
+@pytest.mark.gpu
+def test_python_dtype_is_inferred_from_the_tensor(oracle):
+    """``dots_pack(b)`` and the symmetric calls without a dtype take it from the tensor's element type, as the
+    reference's ``dtype=None`` does (python/matrix.c:632-647); the types that have no tensor type must be named."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(92)
+    a, b = support.random_matrix(oracle, "bf16", 20, 96, rng), support.random_matrix(oracle, "bf16", 30, 96, rng)
+    ga, gb = torch.from_numpy(a).to("cuda:0").view(torch.bfloat16), torch.from_numpy(b).to("cuda:0").view(torch.bfloat16)
+    packed = nk.dots_pack(gb)
+    assert packed.dtype == "bf16"
+    named = nk.dots_packed(torch.from_numpy(a).to("cuda:0"), nk.dots_pack(torch.from_numpy(b).to("cuda:0"), "bf16"))
+    assert torch.equal(nk.dots_packed(ga, packed), named)
+    bytes_ = torch.from_numpy(rng.integers(0, 256, (12, 64), dtype=np.uint8)).to("cuda:0")
+    assert nk.dots_pack(bytes_).dtype == "u8"
+    signed = torch.from_numpy(rng.integers(-128, 128, (12, 64), dtype=np.int8)).to("cuda:0")
+    assert torch.equal(nk.dots_symmetric(signed), nk.dots_symmetric(signed, "i8"))
+    assert torch.equal(nk.angulars_symmetric(ga), nk.angulars_symmetric(torch.from_numpy(a).to("cuda:0"), "bf16"))
+    with pytest.raises(TypeError):
+        nk.dots_pack(torch.zeros((4, 8), dtype=torch.int32, device="cuda:0"))
