@@ -160,6 +160,14 @@ class PackedMatrix:
         """(width, depth), as the reference's PackedMatrix reports it."""
         return (self.width, self.depth)
 
+    @classmethod
+    def packed_size(cls, width: int, depth: int, dtype: str = None) -> int:
+        """Bytes of the packed image for a shape and dtype: the reference's ``PackedMatrix.packed_size(width, depth, /,
+        dtype)`` (python/matrix.c:75-129), which asks for the dtype as well."""
+        if dtype is None:
+            raise TypeError("packed_size() requires 'dtype' argument")
+        return dots_packed_size(dtype, int(width), int(depth))
+
     def __rmatmul__(self, a):
         """``a @ packed`` is ``dots_packed(a, packed)``: the reference's ``Tensor @ PackedMatrix`` (python/matrix.c:324-490)."""
         return dots_packed(a, self)

@@ -44,6 +44,7 @@ def test_python_packed_matrix_operator_and_dlpack(oracle):
     ga, gb = torch.from_numpy(a).to("cuda:0"), torch.from_numpy(b).to("cuda:0")
     packed = nk.dots_pack(gb, "i8")
     assert packed.shape == (21, 100) and packed.nbytes == nk.dots_packed_size("i8", 21, 100)
+    assert type(packed).packed_size(21, 100, dtype="i8") == packed.nbytes and (packed.width, packed.depth, packed.dtype) == (21, 100, "i8")
     expected = a.astype(np.int64) @ b.astype(np.int64).T
     assert np.array_equal((ga @ packed).cpu().numpy(), expected)
 
