@@ -229,7 +229,7 @@ def dots_pack(b, dtype: str = None) -> PackedMatrix:
     return PackedMatrix(dtype, width, depth, buffer)
 
 
-def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out):
+def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out, start_row=None, end_row=None):
     import torch
 
     if not isinstance(packed, PackedMatrix):
@@ -252,17 +252,27 @@ def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out):
             raise ValueError("out rows must be contiguous")
     a_stride = int(a.stride(0)) * a.element_size() if height > 1 else int(a.shape[1]) * a.element_size()
     c_stride = int(out.stride(0)) * out.element_size() if height > 1 else packed.width * out.element_size()
-    getattr(library(), stem + packed.dtype)(
-        a.data_ptr(), packed.buffer.data_ptr(), out.data_ptr(), height, packed.width, depth, a_stride, c_stride
-    )
+    # rows [start_row, end_row) of a, into the same rows of out; the others are left as they were
+    # (reference: python/matrix.c:453-464)
+    first = 0 if start_row is None or int(start_row) < 0 else int(start_row)
+    last = height if end_row is None or int(end_row) < 0 else int(end_row)
+    if first > height or last > height or first > last:
+        raise ValueError(f"Invalid row range [{first}, {last}) for matrix with {height} rows")
+    if last > first:
+        getattr(library(), stem + packed.dtype)(
+            a.data_ptr() + first * a_stride, packed.buffer.data_ptr(), out.data_ptr() + first * c_stride, last - first,
+            packed.width, depth, a_stride, c_stride
+        )
     _check(stem + packed.dtype)
     return out
 
 
-def dots_packed(a, packed: PackedMatrix, out=None):
-    """``C[height x width] = a @ B.T`` with widened accumulators; ``out`` (optional) is overwritten."""
+def dots_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None):
+    """``C[height x width] = a @ B.T`` with widened accumulators; ``out`` (optional) is overwritten. With ``start_row``
+    / ``end_row`` only those rows of ``a`` are multiplied, into the same rows of ``out`` (reference:
+    ``dots_packed(a, b, /, *, out=None, start_row=None, end_row=None)``, python/matrix.c:780-796)."""
     return _packed_product("nk_dots_packed_", DTYPES[packed.dtype][2] if isinstance(packed, PackedMatrix) else "float32",
-                           a, packed, out)
+                           a, packed, out, start_row, end_row)
 
 
 def _needs_distances(dtype: str) -> None:
@@ -275,20 +285,22 @@ def _distance_dtype(dtype) -> str:
     return "float64" if dtype in ("f32", "f64") else "float32"
 
 
-def angulars_packed(a, packed: PackedMatrix, out=None):
+def angulars_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None):
     """Angular distances ``1 - cos(a_i, b_j)`` as float32, float64 for f32 and f64 inputs (reference:
     ``nk_angulars_packed_<dtype>``)."""
     if isinstance(packed, PackedMatrix):
         _needs_distances(packed.dtype)
-    return _packed_product("nk_angulars_packed_", _distance_dtype(getattr(packed, "dtype", None)), a, packed, out)
+    return _packed_product("nk_angulars_packed_", _distance_dtype(getattr(packed, "dtype", None)), a, packed, out,
+                           start_row, end_row)
 
 
-def euclideans_packed(a, packed: PackedMatrix, out=None):
+def euclideans_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None):
     """Euclidean distances ``|a_i - b_j|`` as float32, float64 for f32 and f64 inputs (reference:
     ``nk_euclideans_packed_<dtype>``)."""
     if isinstance(packed, PackedMatrix):
         _needs_distances(packed.dtype)
-    return _packed_product("nk_euclideans_packed_", _distance_dtype(getattr(packed, "dtype", None)), a, packed, out)
+    return _packed_product("nk_euclideans_packed_", _distance_dtype(getattr(packed, "dtype", None)), a, packed, out,
+                           start_row, end_row)
 
 
 def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_row, end_row):

@@ -60,6 +60,14 @@ def test_python_packed_matrix_operator_and_dlpack(oracle):
 
     again = nk.dots_packed(Exporter(ga), nk.dots_pack(Exporter(gb), "i8"))
     assert np.array_equal(again.cpu().numpy(), expected)
+    # a window of rows, as the reference's start_row / end_row: the other rows of out stay as they were
+    window = torch.full((33, 21), -7, dtype=torch.int32, device="cuda:0")
+    assert nk.dots_packed(ga, packed, out=window, start_row=5, end_row=20) is window
+    kept = np.full((33, 21), -7, np.int64)
+    kept[5:20] = expected[5:20]
+    assert np.array_equal(window.cpu().numpy(), kept)
+    with pytest.raises(ValueError):
+        nk.dots_packed(ga, packed, start_row=20, end_row=5)
 
 
 @pytest.mark.gpu
