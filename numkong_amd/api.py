@@ -11,6 +11,11 @@ Reference behaviour mirrored here (python/matrix.c):
 There is no CPU fallback: if the shared library is missing, loading raises; if a call fails on the
 GPU side, ``NumKongAmdError`` is raised with the library's own message.
 
+Operands may live in GPU memory (torch CUDA tensors, DLPack exporters) or in host memory (numpy arrays, torch CPU
+tensors: what a caller of the reference has). Host operands are staged by the library (pinned buffers, two streams;
+a packed image in host memory is uploaded once and found again by the number in its header); the result is then a
+host array of the same kind as ``a``. The arithmetic always runs on the GPU.
+
 Streams: the synchronous calls run on streams the library keeps per host thread. They are blocking streams, so they
 are ordered behind work queued on the legacy default stream (torch's default) and return when the result is
 complete. ONLY the legacy default stream is ordered with them: operands produced on any other stream of the
@@ -144,7 +149,10 @@ def dots_packed_size(dtype: str, width: int, depth: int) -> int:
 
 @dataclass
 class PackedMatrix:
-    """B packed for the GPU kernels; ``buffer`` is a uint8 CUDA tensor holding the relocatable image."""
+    """B packed for the GPU kernels; ``buffer`` is a uint8 tensor holding the relocatable image, in GPU memory when B was
+    there and in host memory otherwise (the library then keeps a device copy, found again by the number in the header)."""
+
+    __array_ufunc__ = None  # numpy: `array @ packed` is this class's to answer (__rmatmul__), not a ufunc over objects
 
     dtype: str
     width: int  # rows of B = columns of C
@@ -183,11 +191,33 @@ def _inferred_dtype(t) -> str:
     for attribute, name in (("float8_e4m3fn", "e4m3"), ("float8_e5m2", "e5m2")):
         if hasattr(torch, attribute):
             names[getattr(torch, attribute)] = name
-    if not isinstance(t, torch.Tensor) and hasattr(t, "__dlpack__"):
-        t = torch.from_dlpack(t)
+    t = _as_tensor(t)
     if not isinstance(t, torch.Tensor) or t.dtype not in names:
         raise TypeError("dtype cannot be inferred from this input; name one of " + str(sorted(DTYPES)))
     return names[t.dtype]
+
+
+def _is_numpy(t) -> bool:
+    return type(t).__module__ == "numpy" and type(t).__name__ == "ndarray"
+
+
+def _as_tensor(t):
+    """A torch view of the operand, without a copy: numpy arrays (host memory), DLPack exporters, tensors as they are."""
+    import torch
+
+    if isinstance(t, torch.Tensor):
+        return t
+    if _is_numpy(t):
+        import numpy
+
+        if t.dtype == numpy.uint16:  # raw bf16 / f16 bits: torch has no arithmetic on uint16 and needs none here
+            t = t.view(numpy.int16)
+        elif t.dtype == numpy.uint32:
+            t = t.view(numpy.int32)
+        return torch.from_numpy(t)
+    if hasattr(t, "__dlpack__"):
+        return torch.from_dlpack(t)  # any DLPack exporter (reference: python/dlpack_interop.c)
+    return t
 
 
 def _as_matrix(t, dtype: str, what: str):
@@ -195,14 +225,11 @@ def _as_matrix(t, dtype: str, what: str):
 
     if dtype not in DTYPES:
         raise TypeError(f"unsupported dtype {dtype!r}; expected one of {sorted(DTYPES)}")
-    if not isinstance(t, torch.Tensor) and hasattr(t, "__dlpack__"):
-        t = torch.from_dlpack(t)  # any DLPack exporter of device memory (reference: python/dlpack_interop.c)
+    t = _as_tensor(t)
     if not isinstance(t, torch.Tensor):
-        raise TypeError(f"{what} must be a torch.Tensor or export DLPack")
+        raise TypeError(f"{what} must be a torch.Tensor, a numpy array or export DLPack")
     if t.dim() != 2:
         raise ValueError(f"{what} must be 2-dimensional, got {t.dim()} dimensions")
-    if not t.is_cuda:
-        raise ValueError(f"{what} must live on the GPU")
     if t.element_size() != DTYPES[dtype][1]:
         raise TypeError(f"{what} has {t.element_size()}-byte elements, dtype {dtype!r} needs {DTYPES[dtype][1]}")
     if t.shape[1] > 1 and t.stride(1) != 1:
@@ -229,27 +256,36 @@ def dots_pack(b, dtype: str = None) -> PackedMatrix:
     return PackedMatrix(dtype, width, depth, buffer)
 
 
-def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out, start_row=None, end_row=None):
+def _result_matrix(out, shape, out_dtype_name: str, like, as_numpy: bool, zeroed: bool):
+    """The tensor the library writes into and what the caller gets back: ``out`` itself when given (a tensor or a
+    numpy array, validated), else a new matrix where ``like`` lives, handed back as a numpy array for numpy operands."""
     import torch
 
+    out_dtype = getattr(torch, out_dtype_name)
+    if out is None:
+        tensor = (torch.zeros if zeroed else torch.empty)(shape, dtype=out_dtype, device=like.device)
+        return tensor, (tensor.numpy() if as_numpy else tensor)
+    tensor = _as_tensor(out)
+    if not isinstance(tensor, torch.Tensor) or tensor.dim() != 2:
+        raise ValueError("out must be a 2-dimensional tensor or array")
+    if tuple(tensor.shape) != tuple(shape):
+        raise ValueError(f"out has shape {tuple(tensor.shape)}, expected {tuple(shape)}")
+    if tensor.dtype != out_dtype:
+        raise TypeError(f"out must have dtype {out_dtype}")
+    if shape[1] > 1 and tensor.stride(1) != 1:
+        raise ValueError("out rows must be contiguous")
+    return tensor, out
+
+
+def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out, start_row=None, end_row=None):
     if not isinstance(packed, PackedMatrix):
         raise TypeError("packed must be a PackedMatrix from dots_pack()")
+    as_numpy = _is_numpy(a)
     a = _as_matrix(a, packed.dtype, "a")
     height, depth = int(a.shape[0]), int(a.shape[1]) * DTYPES[packed.dtype][3]
     if depth != packed.depth:
         raise ValueError(f"depth mismatch: a has {depth} columns, packed matrix has depth {packed.depth}")
-    out_dtype = getattr(torch, out_dtype_name)
-    if out is None:
-        out = torch.empty((height, packed.width), dtype=out_dtype, device=a.device)
-    else:
-        if not isinstance(out, torch.Tensor) or not out.is_cuda or out.dim() != 2:
-            raise ValueError("out must be a 2-dimensional GPU tensor")
-        if tuple(out.shape) != (height, packed.width):
-            raise ValueError(f"out has shape {tuple(out.shape)}, expected {(height, packed.width)}")
-        if out.dtype != out_dtype:
-            raise TypeError(f"out must have dtype {out_dtype}")
-        if packed.width > 1 and out.stride(1) != 1:
-            raise ValueError("out rows must be contiguous")
+    out, result = _result_matrix(out, (height, packed.width), out_dtype_name, a, as_numpy, False)
     a_stride = int(a.stride(0)) * a.element_size() if height > 1 else int(a.shape[1]) * a.element_size()
     c_stride = int(out.stride(0)) * out.element_size() if height > 1 else packed.width * out.element_size()
     # rows [start_row, end_row) of a, into the same rows of out; the others are left as they were
@@ -264,7 +300,7 @@ def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out, sta
             packed.width, depth, a_stride, c_stride
         )
     _check(stem + packed.dtype)
-    return out
+    return result
 
 
 def dots_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None):
@@ -304,23 +340,11 @@ def euclideans_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row
 
 
 def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_row, end_row):
-    import torch
-
+    as_numpy = _is_numpy(vectors)
     vectors = _as_matrix(vectors, dtype, "vectors")
     count, depth = int(vectors.shape[0]), int(vectors.shape[1]) * DTYPES[dtype][3]
-    out_dtype = getattr(torch, out_dtype_name)
-    if out is None:
-        # (the reference leaves what it does not write uninitialised; zeros are easier on the eye)
-        out = torch.zeros((count, count), dtype=out_dtype, device=vectors.device)
-    else:
-        if not isinstance(out, torch.Tensor) or not out.is_cuda or out.dim() != 2:
-            raise ValueError("out must be a 2-dimensional GPU tensor")
-        if tuple(out.shape) != (count, count):
-            raise ValueError(f"out has shape {tuple(out.shape)}, expected {(count, count)}")
-        if out.dtype != out_dtype:
-            raise TypeError(f"out must have dtype {out_dtype}")
-        if count > 1 and out.stride(1) != 1:
-            raise ValueError("out rows must be contiguous")
+    # (the reference leaves what it does not write uninitialised; zeros are easier on the eye)
+    out, result = _result_matrix(out, (count, count), out_dtype_name, vectors, as_numpy, True)
     first = 0 if start_row is None else int(start_row)
     last = count if end_row is None else int(end_row)
     if first < 0 or last < 0 or first > count or last > count or first > last:
@@ -329,7 +353,7 @@ def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_r
     out_stride = int(out.stride(0)) * out.element_size() if count > 1 else count * out.element_size()
     getattr(library(), stem + dtype)(vectors.data_ptr(), count, depth, stride, out.data_ptr(), out_stride, first, last - first)
     _check(stem + dtype)
-    return out
+    return result
 
 
 def dots_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None):

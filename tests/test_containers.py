@@ -89,3 +89,37 @@ def test_python_dtype_is_inferred_from_the_tensor(oracle):
     assert torch.equal(nk.angulars_symmetric(ga), nk.angulars_symmetric(torch.from_numpy(a).to("cuda:0"), "bf16"))
     with pytest.raises(TypeError):
         nk.dots_pack(torch.zeros((4, 8), dtype=torch.int32, device="cuda:0"))
+
+
+@pytest.mark.gpu
+def test_python_host_operands(oracle):
+    """What a caller of the reference has: numpy arrays (and torch CPU tensors) in host memory. The library stages them,
+    the packed image stays in host memory and is uploaded once, results come back as host arrays of the caller's kind."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(93)
+    a = rng.integers(-128, 128, (45, 200), dtype=np.int8)
+    b = rng.integers(-128, 128, (70, 200), dtype=np.int8)
+    expected = a.astype(np.int64) @ b.astype(np.int64).T
+    packed = nk.dots_pack(b)  # dtype from the array
+    assert packed.dtype == "i8" and not packed.buffer.is_cuda and packed.nbytes == nk.dots_packed_size("i8", 70, 200)
+    c = nk.dots_packed(a, packed)
+    assert isinstance(c, np.ndarray) and c.dtype == np.int32 and np.array_equal(c, expected)
+    assert np.array_equal(a @ packed, expected)  # numpy hands the operator to PackedMatrix.__rmatmul__
+    out = np.full((45, 70), -3, np.int32)
+    assert nk.dots_packed(a, packed, out=out, start_row=10, end_row=30) is out
+    assert np.array_equal(out[10:30], expected[10:30]) and (out[:10] == -3).all() and (out[30:] == -3).all()
+    # torch CPU tensors give torch CPU tensors; a host A against an image in GPU memory works as well
+    on_gpu = nk.dots_pack(torch.from_numpy(b).to("cuda:0"))
+    c_cpu = nk.dots_packed(torch.from_numpy(a), on_gpu)
+    assert isinstance(c_cpu, torch.Tensor) and not c_cpu.is_cuda and np.array_equal(c_cpu.numpy(), expected)
+    # raw bf16 bits in a uint16 array: the dtype has to be named; results equal the GPU-resident call bit for bit
+    a16, b16 = support.random_matrix(oracle, "bf16", 33, 128, rng), support.random_matrix(oracle, "bf16", 40, 128, rng)
+    host = nk.dots_packed(a16.view(np.uint16), nk.dots_pack(b16.view(np.uint16), "bf16"))
+    resident = nk.dots_packed(torch.from_numpy(a16).to("cuda:0"), nk.dots_pack(torch.from_numpy(b16).to("cuda:0"), "bf16"))
+    assert host.dtype == np.float32 and np.array_equal(host.view(np.uint32), resident.cpu().numpy().view(np.uint32))
+    gram = nk.dots_symmetric(a)
+    assert isinstance(gram, np.ndarray) and np.array_equal(np.triu(gram), np.triu(a.astype(np.int64) @ a.astype(np.int64).T))
+    distances = nk.angulars_packed(a16.view(np.uint16), nk.dots_pack(b16.view(np.uint16), "bf16"))
+    on_device = nk.angulars_packed(torch.from_numpy(a16).to("cuda:0"), nk.dots_pack(torch.from_numpy(b16).to("cuda:0"), "bf16"))
+    assert np.array_equal(distances.view(np.uint32), on_device.cpu().numpy().view(np.uint32))
+    nk.library().nk_hip_image_cache_clear()
