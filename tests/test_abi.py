@@ -195,8 +195,13 @@ def test_python_mirror_validates_arguments():
     import torch
 
     cpu = torch.zeros(4, 4, dtype=torch.int8)
+    if not torch.cuda.is_available():  # host operands are staged by the library: without a GPU it says so, it never computes
+        with pytest.raises(nk.NumKongAmdError, match="no HIP device"):
+            nk.dots_pack(cpu, "i8")
+        with pytest.raises(nk.NumKongAmdError, match="no HIP device"):
+            nk.dots_symmetric(cpu, "i8")
     with pytest.raises(ValueError):
-        nk.dots_pack(cpu, "i8")  # must live on the GPU
+        nk.dots_pack(torch.zeros(4, 4, 2, dtype=torch.int8), "i8")  # two dimensions
     with pytest.raises(TypeError):
         nk.dots_pack(cpu, "f16c")
     with pytest.raises(TypeError):
@@ -204,7 +209,7 @@ def test_python_mirror_validates_arguments():
     with pytest.raises(TypeError):
         nk.dots_packed(cpu, object())
     with pytest.raises(ValueError):
-        nk.dots_symmetric(cpu, "i8")  # must live on the GPU
+        nk.dots_symmetric(cpu[:, ::2], "i8")  # rows must be contiguous
     with pytest.raises(TypeError):
         nk.angulars_symmetric(cpu, "f16c")
     with pytest.raises(TypeError):
