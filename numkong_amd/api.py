@@ -303,10 +303,12 @@ def _packed_product(stem: str, out_dtype_name, a, packed: PackedMatrix, out, sta
     return result
 
 
-def dots_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None):
+def dots_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None, threads=None):
     """``C[height x width] = a @ B.T`` with widened accumulators; ``out`` (optional) is overwritten. With ``start_row``
     / ``end_row`` only those rows of ``a`` are multiplied, into the same rows of ``out`` (reference:
-    ``dots_packed(a, b, /, *, out=None, start_row=None, end_row=None)``, python/matrix.c:780-796)."""
+    ``dots_packed(a, b, /, *, out=None, start_row=None, end_row=None)``, python/matrix.c:780-796). ``threads``, which
+    the reference's calls also take (python/matrix.c:354-358), is accepted and means nothing here: the rows are spread
+    over the GPU's compute units by the one launch."""
     return _packed_product("nk_dots_packed_", DTYPES[packed.dtype][2] if isinstance(packed, PackedMatrix) else "float32",
                            a, packed, out, start_row, end_row)
 
@@ -321,7 +323,7 @@ def _distance_dtype(dtype) -> str:
     return "float64" if dtype in ("f32", "f64") else "float32"
 
 
-def angulars_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None):
+def angulars_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None, threads=None):
     """Angular distances ``1 - cos(a_i, b_j)`` as float32, float64 for f32 and f64 inputs (reference:
     ``nk_angulars_packed_<dtype>``)."""
     if isinstance(packed, PackedMatrix):
@@ -330,7 +332,7 @@ def angulars_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=N
                            start_row, end_row)
 
 
-def euclideans_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None):
+def euclideans_packed(a, packed: PackedMatrix, out=None, start_row=None, end_row=None, threads=None):
     """Euclidean distances ``|a_i - b_j|`` as float32, float64 for f32 and f64 inputs (reference:
     ``nk_euclideans_packed_<dtype>``)."""
     if isinstance(packed, PackedMatrix):
@@ -356,7 +358,7 @@ def _symmetric(stem: str, out_dtype_name: str, vectors, dtype: str, out, start_r
     return result
 
 
-def dots_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None):
+def dots_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None, threads=None):
     """Upper triangle (diagonal included) of ``vectors @ vectors.T`` for the rows ``[start_row, end_row)``, widened as
     in ``dots_packed``; the rest of ``out`` is left as it was (zeros when allocated here). ``dtype`` defaults to the
     tensor's own element type."""
@@ -367,7 +369,7 @@ def dots_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row
     return _symmetric("nk_dots_symmetric_", DTYPES[dtype][2], vectors, dtype, out, start_row, end_row)
 
 
-def angulars_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None):
+def angulars_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None, threads=None):
     """Upper triangle of the pairwise angular distances as float32 (float64 for f32 and f64 inputs); the diagonal is
     exactly 0."""
     if dtype is None:
@@ -376,7 +378,7 @@ def angulars_symmetric(vectors, dtype: str = None, out=None, start_row=None, end
     return _symmetric("nk_angulars_symmetric_", _distance_dtype(dtype), vectors, dtype, out, start_row, end_row)
 
 
-def euclideans_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None):
+def euclideans_symmetric(vectors, dtype: str = None, out=None, start_row=None, end_row=None, threads=None):
     """Upper triangle of the pairwise euclidean distances as float32 (float64 for f32 and f64 inputs); the diagonal is
     exactly 0."""
     if dtype is None:

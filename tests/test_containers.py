@@ -102,7 +102,7 @@ def test_python_host_operands(oracle):
     expected = a.astype(np.int64) @ b.astype(np.int64).T
     packed = nk.dots_pack(b)  # dtype from the array
     assert packed.dtype == "i8" and not packed.buffer.is_cuda and packed.nbytes == nk.dots_packed_size("i8", 70, 200)
-    c = nk.dots_packed(a, packed)
+    c = nk.dots_packed(a, packed, threads=8)  # (the reference's callers pass it; the GPU has its own parallelism)
     assert isinstance(c, np.ndarray) and c.dtype == np.int32 and np.array_equal(c, expected)
     assert np.array_equal(a @ packed, expected)  # numpy hands the operator to PackedMatrix.__rmatmul__
     out = np.full((45, 70), -3, np.int32)
