@@ -110,12 +110,26 @@ def make_operands(dtype, m, n, k, seed=42):
     return one(m), one(n)
 
 
+# From idle the part takes some tens of milliseconds of load to reach the clocks it then holds (measured, first series of
+# a process against the same series later in it: bf16 4096^3 144 against 120 us per launch, i8 8192^3 455 against 417),
+# and a short series timed from idle reads that ramp instead of the kernel. Every timing here, this library's kernels
+# and the vendor library's alike, is therefore preceded by this much untimed running of the same step (--spin-up-ms;
+# 0 turns it off); the warm-up steps and the timed steps follow as asked for.
+SPIN_UP_MS = 100.0
+
+
 def timed_steps(step, steps, warmup):
-    """`warmup` untimed calls of `step`, then `steps` timed ones, each between two events of its own on torch's
-    current stream (the stream the kernels are launched on). Returns wall ms per step and the device times in ms:
-    mean over the whole region, median and minimum of the per-step pairs."""
+    """Untimed running of `step` until the clocks have settled (SPIN_UP_MS), `warmup` untimed calls, then `steps` timed
+    ones, each between two events of its own on torch's current stream (the stream the kernels are launched on). Returns
+    wall ms per step and the device times in ms: mean over the whole region, median and minimum of the per-step pairs."""
     import torch
 
+    if SPIN_UP_MS > 0:
+        until = time.perf_counter() + SPIN_UP_MS * 1e-3
+        while time.perf_counter() < until:
+            for _ in range(4):
+                step()
+            torch.cuda.synchronize()
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -403,6 +417,7 @@ def cpu_baseline(dtype, m, n, k, budget_rows=8192):
 
 
 def main():
+    global SPIN_UP_MS
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=50)
@@ -412,6 +427,8 @@ def main():
     parser.add_argument("--metric", default="dots", choices=["dots", "angular", "euclidean"] + sorted(SYMMETRIC_KINDS),
                         help="what the timed call computes: the packed product, one of the packed distances on top of it, or "
                              "one of the symmetric kinds over N vectors of depth K")
+    parser.add_argument("--spin-up-ms", type=float, default=SPIN_UP_MS,
+                        help="untimed running of each timed step before its warm-up steps, until the clocks have settled (0: none)")
     parser.add_argument("--no-others", action="store_true")
     parser.add_argument("--no-cpu", action="store_true")
     parser.add_argument("--no-vendor", action="store_true", help="skip the vendor GEMM timings (others.vendor_*)")
@@ -421,6 +438,7 @@ def main():
     parser.add_argument("--probe", action="store_true",
                         help="for rocprofv3 --pmc runs: launch a plain 1 GiB elementwise copy kernel 3 times, then the selected product 3 times, nothing else")
     args = parser.parse_args()
+    SPIN_UP_MS = 0.0 if args.probe or args.vendor_probe else max(0.0, args.spin_up_ms)
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (rows of A or of B shard without "
                  "communication); run with --gpus 1")
@@ -507,6 +525,7 @@ def main():
                                (f"{args.dtype} packed {args.metric} C = A * B^T, M={m} N={n} K={k}, A row-major in HBM, "
                                 "B packed once outside the timed region, C overwritten")},
         "kernel_ms": head["kernel_ms"], "kernel_ms_median": head["kernel_ms_median"], "kernel_ms_min": head["kernel_ms_min"],
+        "spin_up_ms": SPIN_UP_MS,  # untimed running before the warm-up steps of every timing (clock ramp from idle)
         "roofline": head["roofline"],
     })
     if not args.no_cpu:
