@@ -37,6 +37,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <chrono>
 #include <type_traits>
 #include <vector>
 
@@ -181,7 +182,11 @@ static CeilingResult run_ceiling(bool zeros, int units, v8i *operands, float *si
     hipEvent_t begin, end;
     CHECK(hipEventCreate(&begin));
     CHECK(hipEventCreate(&end));
-    for (int warm = 0; warm < 20; ++warm) hipLaunchKernelGGL(mfma_only_kernel<FORM>, dim3(units), dim3(256), 0, 0, operands, iterations, sink, clocks);
+    // (from idle the part ramps its clocks for some tens of milliseconds: 100 ms of the same loop first)
+    for (auto const start = std::chrono::steady_clock::now(); std::chrono::steady_clock::now() - start < std::chrono::milliseconds(100);) {
+        for (int warm = 0; warm < 20; ++warm) hipLaunchKernelGGL(mfma_only_kernel<FORM>, dim3(units), dim3(256), 0, 0, operands, iterations, sink, clocks);
+        CHECK(hipDeviceSynchronize());
+    }
     CHECK(hipEventRecord(begin, 0));
     constexpr int kLaunches = 20;
     for (int launch = 0; launch < kLaunches; ++launch) hipLaunchKernelGGL(mfma_only_kernel<FORM>, dim3(units), dim3(256), 0, 0, operands, iterations, sink, clocks);
@@ -227,7 +232,7 @@ static int ceiling_mode(bool json) {
         results[kBF16OfE4M3][zeros] = run_ceiling<kBF16OfE4M3>(zeros, units, operands, sink, clocks);
     }
     if (json) printf("{\"compute_units\": %d, \"device\": \"%s\", \"forms\": {", units, properties.gcnArchName);
-    else printf("MFMA-only loop, %d compute units (%s), 4 wavefronts each, 20 launches after 20 warm-up launches\n%-30s %-7s %9s %10s %8s %8s %12s\n", units,
+    else printf("MFMA-only loop, %d compute units (%s), 4 wavefronts each, 20 launches after 100 ms of the same loop\n%-30s %-7s %9s %10s %8s %8s %12s\n", units,
                 properties.gcnArchName, "instruction", "data", "ms", "T(FL)OP/s", "of peak", "MHz", "cycles/MFMA");
     for (int form = 0; form < kForms; ++form)
         for (int zeros = 0; zeros < 2; ++zeros) {
