@@ -305,13 +305,67 @@ __global__ __launch_bounds__(256) void budget_kernel(v4i const *operands, int it
     if (threadIdx.x == 0) clocks[2 * blockIdx.x] = cycles1 - cycles0, clocks[2 * blockIdx.x + 1] = ticks1 - ticks0;
 }
 
+/**
+ *  The same tile with the 16 x 16 x 64 instruction: 16 x 4 blocks per wavefront, one trip a 64-deep step (64 MFMAs, the
+ *  work of two trips of the loop above), with twice the loads and reads per trip so that the traffic per operation is
+ *  the same: 2 x LOADS global loads two trips ahead, 2 x READS ds_read_b128 one trip ahead.
+ */
+template <int LOADS, int READS>
+__global__ __launch_bounds__(256) void budget_small_kernel(v4i const *operands, int iterations, float *sink, unsigned long long *clocks, v4i const *stream, unsigned stream_mask) {
+    __shared__ v4i lds[4096];
+    for (int i = threadIdx.x; i < 4096; i += 256) lds[i] = operands[i % 1024];
+    __syncthreads();
+    constexpr int RING = 2, L = LOADS > 0 ? 2 * LOADS : 1;
+    v4i a[2][16], g[RING][L], b[4];
+    unsigned const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = 0; i < 16; ++i) a[0][i] = a[1][i] = operands[(i * 64 + lane) % 1024];
+    for (int j = 0; j < 4; ++j) b[j] = operands[((8 + j) * 64 + lane) % 1024];
+    for (int r = 0; r < RING; ++r)
+        for (int l = 0; l < L; ++l) g[r][l] = b[l & 3];
+    v4i acc[16][4];
+    for (int i = 0; i < 16; ++i)
+        for (int j = 0; j < 4; ++j) acc[i][j] = v4i {0, 0, 0, 0};
+    unsigned long long const cycles0 = clock64(), ticks0 = wall_clock64();
+    unsigned at = (blockIdx.x * 4 + wave) * 64 * L + lane;
+    for (int it = 0; it < iterations; it += 2 * RING) { // (`iterations` counts 32-deep steps, as for the loop above)
+#pragma unroll
+        for (int r = 0; r < RING; ++r) {
+            v4i operand_b[4] = {b[0], b[1], b[2], b[3]};
+            if constexpr (LOADS >= 2) operand_b[0] = g[r][0], operand_b[1] = g[r][1], operand_b[2] = g[r][2], operand_b[3] = g[r][3];
+            if constexpr (LOADS > 0) {
+#pragma unroll
+                for (int l = 0; l < L; ++l) g[r][l] = stream[(at + l * 64) & stream_mask];
+                at += 256 * 4 * 64 * L;
+            }
+            if constexpr (READS > 0) {
+#pragma unroll
+                for (int i = 0; i < 2 * READS; ++i) a[(r + 1) & 1][i] = lds[(((it / 2 + r) & 3) * 1024 + i * 64 + lane) & 4095];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[r & 1][i], operand_b[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    unsigned long long const cycles1 = clock64(), ticks1 = wall_clock64();
+    float total = 0;
+    for (int i = 0; i < 16; ++i)
+        for (int j = 0; j < 4; ++j) total += (float)acc[i][j][0];
+    sink[blockIdx.x * 256 + threadIdx.x] = total;
+    if (threadIdx.x == 0) clocks[2 * blockIdx.x] = cycles1 - cycles0, clocks[2 * blockIdx.x + 1] = ticks1 - ticks0;
+}
+
 template <class Kernel>
 static void run_budget(char const *name, Kernel kernel, int units, v4i *operands, float *sink, unsigned long long *clocks, v4i *stream, unsigned mask) {
     int const iterations = 1500;
     hipEvent_t begin, end;
     CHECK(hipEventCreate(&begin));
     CHECK(hipEventCreate(&end));
-    for (int warm = 0; warm < 20; ++warm) hipLaunchKernelGGL(kernel, dim3(units), dim3(256), 0, 0, operands, iterations, sink, clocks, stream, mask);
+    // (from idle the part ramps its clocks for some tens of milliseconds: 100 ms of the same loop first)
+    for (auto const start = std::chrono::steady_clock::now(); std::chrono::steady_clock::now() - start < std::chrono::milliseconds(100);) {
+        for (int warm = 0; warm < 20; ++warm) hipLaunchKernelGGL(kernel, dim3(units), dim3(256), 0, 0, operands, iterations, sink, clocks, stream, mask);
+        CHECK(hipDeviceSynchronize());
+    }
     CHECK(hipEventRecord(begin, 0));
     for (int launch = 0; launch < 20; ++launch) hipLaunchKernelGGL(kernel, dim3(units), dim3(256), 0, 0, operands, iterations, sink, clocks, stream, mask);
     CHECK(hipEventRecord(end, 0));
@@ -361,6 +415,11 @@ static int budget_mode() {
     run_budget("8 ds_read_b128 and 4 global loads", budget_kernel<4, 8, 0>, units, operands, sink, clocks, stream, mask);
     run_budget("8 ds_read_b128, 4 global loads, 128 idle cycles", budget_kernel<4, 8, 2>, units, operands, sink, clocks, stream, mask);
     run_budget("nothing else (again)", budget_kernel<0, 0, 0>, units, operands, sink, clocks, stream, mask);
+    printf("the same tile with the 16x16x64 instruction (64 MFMAs per 64-deep step; figures per 16 MFMAs of the 32x32x32 loop; MFMA busy at 16 cycles an MFMA)\n");
+    run_budget("16x16x64: nothing else", budget_small_kernel<0, 0>, units, operands, sink, clocks, stream, mask);
+    run_budget("16x16x64: 8 ds_read_b128", budget_small_kernel<0, 8>, units, operands, sink, clocks, stream, mask);
+    run_budget("16x16x64: 4 global dwordx4 loads", budget_small_kernel<4, 0>, units, operands, sink, clocks, stream, mask);
+    run_budget("16x16x64: 8 ds_read_b128 and 4 global loads", budget_small_kernel<4, 8>, units, operands, sink, clocks, stream, mask);
     return 0;
 }
 
